@@ -1,0 +1,101 @@
+"""ctypes binding of the C ABI in include/ao_amd.h (ao_amd/lib/libao_amd.so).
+
+There is no fallback: if the library is missing or a call fails, the error is raised to the
+caller.  torch is imported first so that the library binds to the HIP runtime torch already
+loaded (both have the soname libamdhip64.so.7) and stream handles are shared.
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (must be loaded before the HIP library, see module docstring)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libao_amd.so")
+
+F32, BF16, F16, I32, I64, I8, U8 = 0, 1, 2, 3, 4, 5, 6
+MAP_SYMMETRIC, MAP_ASYMMETRIC = 0, 1
+ZP_INT, ZP_FLOAT = 0, 1
+
+DTYPE_CODE = {
+    torch.float32: F32,
+    torch.bfloat16: BF16,
+    torch.float16: F16,
+    torch.int32: I32,
+    torch.int64: I64,
+    torch.int8: I8,
+    torch.uint8: U8,
+}
+
+_p, _i64, _int, _dbl = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_double
+_i64p = ctypes.POINTER(ctypes.c_int64)
+
+_SIGNATURES = {
+    "ao_amd_abi_version": ([], _int),
+    "ao_amd_last_error": ([], ctypes.c_char_p),
+    "ao_amd_choose_qparams_affine": ([_p, _int, _i64, _i64, _i64, _i64, _i64, _int, _i64, _i64, _dbl, _int, _int, _int, _int, _p, _p, _p], _int),
+    "ao_amd_quantize_affine": ([_p, _int, _i64, _i64, _i64, _i64, _i64, _p, _int, _p, _int, _i64, _i64, _int, _p, _int, _p], _int),
+    "ao_amd_dequantize_affine": ([_p, _int, _i64, _i64, _i64, _i64, _p, _int, _p, _int, _i64, _i64, _int, _p, _int, _p], _int),
+    "ao_amd_int4wo_packed_shape": ([_i64, _i64, _i64, _i64p, _i64p, _i64p, _i64p], _int),
+    "ao_amd_int4wo_quantize_pack": ([_p, _i64, _i64, _i64, _i64, _p, _p, _p], _int),
+    "ao_amd_int4wo_pack": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p], _int),
+    "ao_amd_int4wo_unpack": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _p], _int),
+    "ao_amd_int4wo_dequantize": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
+    "ao_amd_int4wo_linear": ([_p, _i64, _i64, _i64, _p, _p, _i64, _i64, _p, _p, _int, _i64, _p], _int),
+}
+
+_lib = None
+
+
+class AoAmdError(RuntimeError):
+    pass
+
+
+def lib():
+    """The loaded C-ABI library.  Raises if it has not been built (python -m ao_amd._build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: the HIP kernels are not built. Run `python -m ao_amd._build` "
+                "(hipcc, gfx950). ao_amd has no CPU or eager fallback."
+            )
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (argtypes, restype) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes, fn.restype = argtypes, restype
+        _lib = handle
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise AoAmdError(lib().ao_amd_last_error().decode("utf-8", "replace"))
+
+
+def current_stream(device) -> int:
+    """hipStream_t of torch's current stream on `device` (0 = null stream)."""
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_cuda(*tensors) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise AoAmdError(
+                f"ao_amd kernels run on the GPU only; got a tensor on {t.device}. Move it with .cuda() first "
+                "(there is no CPU fallback)."
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise AoAmdError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def packed_shape(N: int, K: int, g: int):
+    """(Np, Kp, packed_bytes, qparam_bytes) of the int4 packed layout."""
+    out = [ctypes.c_int64() for _ in range(4)]
+    check(lib().ao_amd_int4wo_packed_shape(N, K, g, *[ctypes.byref(o) for o in out]))
+    return tuple(o.value for o in out)

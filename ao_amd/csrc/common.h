@@ -1,0 +1,123 @@
+// Shared host/device helpers for the gfx950 weight-only quantized linear kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/ao_amd.h"
+
+namespace ao {
+
+// ---------------------------------------------------------------- error reporting (host)
+char* last_error_buf();  // thread-local, 512 bytes
+
+#define AO_FAIL(code, ...)                                   \
+    do {                                                     \
+        snprintf(ao::last_error_buf(), 512, __VA_ARGS__);    \
+        return (code);                                       \
+    } while (0)
+
+#define AO_REQUIRE(cond, ...)                  \
+    do {                                       \
+        if (!(cond)) AO_FAIL(-1, __VA_ARGS__); \
+    } while (0)
+
+#define AO_LAUNCH_CHECK()                                                               \
+    do {                                                                                \
+        hipError_t e_ = hipGetLastError();                                              \
+        if (e_ != hipSuccess) AO_FAIL(-2, "kernel launch failed: %s", hipGetErrorString(e_)); \
+    } while (0)
+
+inline bool is_float_dtype(int d) { return d == AO_F32 || d == AO_BF16 || d == AO_F16; }
+inline int dtype_size(int d) {
+    switch (d) {
+        case AO_F32: case AO_I32: return 4;
+        case AO_BF16: case AO_F16: return 2;
+        case AO_I64: return 8;
+        default: return 1;
+    }
+}
+inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
+
+// ---------------------------------------------------------------- scalar formats (device)
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// fp32 -> bf16 round-to-nearest-even, NaN -> 0x7FC0: the rounding torch applies when an op writes a
+// bf16 tensor.  Integer arithmetic, so the result does not depend on FP mode registers.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+}
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+    _Float16 v = (_Float16)f;  // v_cvt_f16_f32: RNE, IEEE overflow to inf, subnormals kept
+    uint16_t h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+}
+
+// round an fp32 value through a floating dtype
+__device__ __forceinline__ float rd(int dtype, float v) {
+    if (dtype == AO_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+    if (dtype == AO_F16) return f16_bits_to_f32(f32_to_f16_bits(v));
+    return v;
+}
+__device__ __forceinline__ float rne_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+__device__ __forceinline__ bool is_float_dt(int d) { return d == AO_F32 || d == AO_BF16 || d == AO_F16; }
+__device__ __forceinline__ int promote(int a, int b) {
+    if (!is_float_dt(a)) return b;
+    if (!is_float_dt(b)) return a;
+    return a == b ? a : AO_F32;
+}
+
+__device__ __forceinline__ float load_f(const void* p, int dtype, int64_t i) {
+    switch (dtype) {
+        case AO_F32: return ((const float*)p)[i];
+        case AO_BF16: return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+        case AO_F16: return f16_bits_to_f32(((const uint16_t*)p)[i]);
+        case AO_I32: return (float)((const int32_t*)p)[i];
+        case AO_I64: return (float)((const int64_t*)p)[i];
+        case AO_I8: return (float)((const int8_t*)p)[i];
+        case AO_U8: return (float)((const uint8_t*)p)[i];
+    }
+    return 0.f;
+}
+__device__ __forceinline__ int64_t load_i(const void* p, int dtype, int64_t i) {
+    switch (dtype) {
+        case AO_I32: return ((const int32_t*)p)[i];
+        case AO_I64: return ((const int64_t*)p)[i];
+        case AO_I8: return ((const int8_t*)p)[i];
+        case AO_U8: return ((const uint8_t*)p)[i];
+        default: return (int64_t)load_f(p, dtype, i);
+    }
+}
+__device__ __forceinline__ void store_f(void* p, int dtype, int64_t i, float v) {
+    switch (dtype) {
+        case AO_F32: ((float*)p)[i] = v; break;
+        case AO_BF16: ((uint16_t*)p)[i] = f32_to_bf16_bits(v); break;
+        case AO_F16: ((uint16_t*)p)[i] = f32_to_f16_bits(v); break;
+        case AO_I32: ((int32_t*)p)[i] = (int32_t)v; break;
+        case AO_I64: ((int64_t*)p)[i] = (int64_t)v; break;
+        case AO_I8: ((int8_t*)p)[i] = (int8_t)v; break;
+        case AO_U8: ((uint8_t*)p)[i] = (uint8_t)v; break;
+    }
+}
+
+// ---------------------------------------------------------------- int4 packed layout
+// element e (0..7) of a dword sits in the nibble at bit 4 * nib_pos(e)
+__host__ __device__ __forceinline__ int nib_pos(int e) { return (e >> 1) + 4 * (e & 1); }
+
+constexpr uint32_t kPadQparam = 0x00003586u;  // scale = bf16(1e-6), zero = 0
+constexpr uint32_t kPadCodes = 0x88888888u;   // eight codes of value 8
+
+inline bool valid_group(int64_t g) { return g == 32 || g == 64 || g == 128 || g == 256; }
+
+}  // namespace ao

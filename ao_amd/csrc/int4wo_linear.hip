@@ -1,0 +1,206 @@
+// int4 weight-only linear for gfx950: y[M,N] = x[M,K] @ dequant(W)^T (+ bias).
+//
+// The weight streams once from HBM in the packed layout (see include/ao_amd.h): a wave's 16-byte per
+// lane load brings a 16-row x 128-k tile (1 KiB, contiguous).  Each dword is 8 consecutive k of one
+// row, i.e. exactly the B operand of v_mfma_f32_16x16x32_bf16 for that lane, so the dequantized
+// values never pass through LDS: they are produced in registers and fed straight to the matrix core
+// together with up to 16 activation rows.
+//
+// Dequantization is the reference's dequantize_affine (torchao/quantization/quant_primitives.py:265-274)
+// with both bf16 roundings kept: w = bf16( bf16((q-8)*s) + z ).  Dropping them costs 1.8e-3 relative
+// L2 error on the output, above the 1e-3 tolerance of the path.  Per pair of elements:
+//   P  = (dword >> 4v) & 0x000F000F | 0x43004300      two bf16 values 128+q          (1 v_and_or)
+//   t  = P.lo*s + P.hi*0 - 136*s  /  P.lo*0 + P.hi*s - 136*s   exact (q-8)*s in fp32  (2 v_dot2_f32_bf16)
+//   T  = cvt_pk_bf16(t0, t1)                           first rounding                 (1 v_cvt_pk_bf16_f32)
+//   u  = T.lo*1 + T.hi*0 + z  /  T.lo*0 + T.hi*1 + z   fp32 add of the bf16 operands  (2 v_dot2_f32_bf16)
+//   W  = cvt_pk_bf16(u0, u1)                           second rounding                (1 v_cvt_pk_bf16_f32)
+#include "common.h"
+
+namespace ao {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+struct GroupConst {
+    uint32_t s_lo, s_hi;  // packed bf16 (s, 0) and (0, s)
+    float c136;           // -136 * s (exact in fp32)
+    float z;
+};
+__device__ __forceinline__ GroupConst make_group(uint32_t qp) {
+    GroupConst g;
+    g.s_lo = qp & 0xffffu;
+    g.s_hi = qp << 16;
+    g.c136 = -136.0f * __uint_as_float(qp << 16);
+    g.z = __uint_as_float(qp & 0xffff0000u);
+    return g;
+}
+
+// 8 packed codes -> 8 dequantized bf16 in MFMA B-operand order.
+//
+// One asm block, because the instruction order carries the hardware's dependency rules: a VALU
+// instruction may read the result of a v_dot2 only 3 or more issue slots after it, and the compiler
+// does not look inside inline asm to enforce that.  Every dot2 result below is consumed at least 3
+// instructions later; the trailing s_nop keeps a following consumer of the last v_cvt_pk clear too.
+__device__ __forceinline__ bf16x8_t dequant8(uint32_t w, const GroupConst& g, uint32_t magic, uint32_t one_lo,
+                                             uint32_t one_hi) {
+    union { uint32_t u[4]; bf16x8_t v; } out;
+    uint32_t p0, p1, p2, p3;
+    float a0, a1, a2, a3, a4, a5, a6, a7;
+    asm("v_and_or_b32 %[p0], %[w], %[mask], %[magic]\n\t"
+        "v_lshrrev_b32 %[p1], 4, %[w]\n\t"
+        "v_lshrrev_b32 %[p2], 8, %[w]\n\t"
+        "v_lshrrev_b32 %[p3], 12, %[w]\n\t"
+        "v_and_or_b32 %[p1], %[p1], %[mask], %[magic]\n\t"
+        "v_and_or_b32 %[p2], %[p2], %[mask], %[magic]\n\t"
+        "v_and_or_b32 %[p3], %[p3], %[mask], %[magic]\n\t"
+        "v_dot2_f32_bf16 %[a0], %[p0], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a1], %[p0], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a2], %[p1], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a3], %[p1], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a4], %[p2], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a5], %[p2], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a6], %[p3], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a7], %[p3], %[shi], %[c]\n\t"
+        "v_cvt_pk_bf16_f32 %[p0], %[a0], %[a1]\n\t"
+        "v_cvt_pk_bf16_f32 %[p1], %[a2], %[a3]\n\t"
+        "v_cvt_pk_bf16_f32 %[p2], %[a4], %[a5]\n\t"
+        "v_cvt_pk_bf16_f32 %[p3], %[a6], %[a7]\n\t"
+        "v_dot2_f32_bf16 %[a0], %[p0], %[olo], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a1], %[p0], %[ohi], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a2], %[p1], %[olo], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a3], %[p1], %[ohi], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a4], %[p2], %[olo], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a5], %[p2], %[ohi], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a6], %[p3], %[olo], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a7], %[p3], %[ohi], %[z]\n\t"
+        "v_cvt_pk_bf16_f32 %[o0], %[a0], %[a1]\n\t"
+        "v_cvt_pk_bf16_f32 %[o1], %[a2], %[a3]\n\t"
+        "v_cvt_pk_bf16_f32 %[o2], %[a4], %[a5]\n\t"
+        "v_cvt_pk_bf16_f32 %[o3], %[a6], %[a7]\n\t"
+        "s_nop 1"
+        : [o0] "=&v"(out.u[0]), [o1] "=&v"(out.u[1]), [o2] "=&v"(out.u[2]), [o3] "=&v"(out.u[3]), [p0] "=&v"(p0),
+          [p1] "=&v"(p1), [p2] "=&v"(p2), [p3] "=&v"(p3), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2),
+          [a3] "=&v"(a3), [a4] "=&v"(a4), [a5] "=&v"(a5), [a6] "=&v"(a6), [a7] "=&v"(a7)
+        : [w] "v"(w), [mask] "s"(0x000F000Fu), [magic] "v"(magic), [slo] "v"(g.s_lo), [shi] "v"(g.s_hi),
+          [c] "v"(g.c136), [z] "v"(g.z), [olo] "v"(one_lo), [ohi] "v"(one_hi));
+    return out.v;
+}
+
+// Activation fragment: 8 consecutive bf16 of row m starting at k (zeros outside [0,M) x [0,K)).
+__device__ __forceinline__ bf16x8_t load_x8(const uint16_t* __restrict__ x, int64_t ldx, int64_t m, int64_t M,
+                                            int64_t k, int64_t K, bool vec_ok) {
+    union { uint4 q; uint16_t h[8]; bf16x8_t v; } r;
+    r.q = make_uint4(0, 0, 0, 0);
+    if (m < M) {
+        if (vec_ok && k + 8 <= K) {
+            r.q = *reinterpret_cast<const uint4*>(x + m * ldx + k);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (k + e < K) r.h[e] = x[m * ldx + k + e];
+        }
+    }
+    return r.v;
+}
+
+// One workgroup = one 16-row block of W, WAVES waves splitting K by 128-wide super-slices; blockIdx.y
+// selects a chunk of 16 activation rows.  Partial 16x16 accumulators meet in LDS.
+template <int G, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(
+    const uint16_t* __restrict__ x, int64_t M, int64_t K, int64_t ldx, const uint4* __restrict__ packed,
+    const uint32_t* __restrict__ qparams, int64_t N, int64_t Kp, const uint16_t* __restrict__ bias, void* __restrict__ y,
+    int y_is_f32, int64_t ldy) {
+    __shared__ float red[WAVES][4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, qd = lane >> 4;
+    const int64_t rb = blockIdx.x;
+    const int64_t m0 = (int64_t)blockIdx.y * 16;
+    const int64_t KB = Kp / 128, NG = Kp / G;
+    const bool vec_ok = ((ldx & 7) == 0) && ((((uintptr_t)x) & 15) == 0);
+    const uint32_t magic = 0x43004300u, one_lo = 0x00003F80u, one_hi = 0x3F800000u;
+
+    const uint4* wp = packed + rb * KB * 64 + lane;
+    const uint32_t* qp = qparams + rb * NG * 16 + r;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+
+    for (int64_t kb = wave; kb < KB; kb += WAVES) {
+        const uint4 w4 = wp[kb * 64];
+        const uint32_t ww[4] = {w4.x, w4.y, w4.z, w4.w};
+        GroupConst gc;
+        if (G >= 128) gc = make_group(qp[(kb * 128 / G) * 16]);
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            if (G == 64 && (sl & 1) == 0) gc = make_group(qp[(kb * 2 + (sl >> 1)) * 16]);
+            if (G == 32) gc = make_group(qp[(kb * 4 + sl) * 16]);
+            const bf16x8_t b = dequant8(ww[sl], gc, magic, one_lo, one_hi);
+            const bf16x8_t a = load_x8(x, ldx, m0 + r, M, kb * 128 + sl * 32 + qd * 8, K, vec_ok);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+        }
+    }
+
+    // acc[i] = C[m = 4*qd + i][n = r]
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][i][lane] = acc[i];
+    __syncthreads();
+    if (wave == 0) {
+        const int64_t n = rb * 16 + r;
+        float bv = 0.f;
+        if (bias && n < N) bv = bf16_bits_to_f32(bias[n]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) s += red[w][i][lane];
+            const int64_t m = m0 + 4 * qd + i;
+            if (m < M && n < N) {
+                s += bv;
+                if (y_is_f32) ((float*)y)[m * ldy + n] = s;
+                else ((uint16_t*)y)[m * ldy + n] = f32_to_bf16_bits(s);
+            }
+        }
+    }
+}
+
+template <int WAVES>
+static void launch_linear(int64_t g, dim3 grid, hipStream_t st, const uint16_t* x, int64_t M, int64_t K, int64_t ldx,
+                          const uint4* packed, const uint32_t* qparams, int64_t N, int64_t Kp, const uint16_t* bias,
+                          void* y, int y_is_f32, int64_t ldy) {
+    dim3 block(WAVES * 64);
+    switch (g) {
+        case 32: hipLaunchKernelGGL((int4wo_linear_kernel<32, WAVES>), grid, block, 0, st, x, M, K, ldx, packed, qparams, N, Kp, bias, y, y_is_f32, ldy); break;
+        case 64: hipLaunchKernelGGL((int4wo_linear_kernel<64, WAVES>), grid, block, 0, st, x, M, K, ldx, packed, qparams, N, Kp, bias, y, y_is_f32, ldy); break;
+        case 128: hipLaunchKernelGGL((int4wo_linear_kernel<128, WAVES>), grid, block, 0, st, x, M, K, ldx, packed, qparams, N, Kp, bias, y, y_is_f32, ldy); break;
+        default: hipLaunchKernelGGL((int4wo_linear_kernel<256, WAVES>), grid, block, 0, st, x, M, K, ldx, packed, qparams, N, Kp, bias, y, y_is_f32, ldy); break;
+    }
+}
+
+}  // namespace ao
+
+using namespace ao;
+
+extern "C" int ao_amd_int4wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed,
+                                    const void* qparams, int64_t N, int64_t g, const void* bias_bf16, void* y,
+                                    int y_dtype, int64_t ldy, void* stream) {
+    AO_REQUIRE(x_bf16 && packed && qparams && y, "null pointer argument");
+    AO_REQUIRE(M >= 0, "negative batch");
+    AO_REQUIRE(y_dtype == AO_BF16 || y_dtype == AO_F32, "output dtype must be bf16 or f32, got code %d", y_dtype);
+    int64_t Np, Kp;
+    if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
+    AO_REQUIRE(ldx >= K && ldy >= N, "row strides (ldx=%lld, ldy=%lld) smaller than the rows (K=%lld, N=%lld)",
+               (long long)ldx, (long long)ldy, (long long)K, (long long)N);
+    AO_REQUIRE((((uintptr_t)packed) & 15) == 0, "packed buffer must be 16-byte aligned");
+    if (M == 0) return 0;
+    const int64_t mchunks = (M + 15) / 16;
+    AO_REQUIRE(mchunks <= 65535, "batch too large for one launch: M=%lld", (long long)M);
+    dim3 grid((unsigned)(Np / 16), (unsigned)mchunks);
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t KB = Kp / 128;
+    if (KB >= 8)
+        launch_linear<8>(g, grid, st, (const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams, N, Kp, (const uint16_t*)bias_bf16, y, y_dtype == AO_F32, ldy);
+    else
+        launch_linear<4>(g, grid, st, (const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams, N, Kp, (const uint16_t*)bias_bf16, y, y_dtype == AO_F32, ldy);
+    AO_LAUNCH_CHECK();
+    return 0;
+}

@@ -1,0 +1,530 @@
+// Affine quantization primitives and the int4 weight-only quantize / pack kernels for gfx950.
+//
+// Bit-exactness contract: the reference runs a chain of eager torch ops, each computing in fp32 and
+// rounding its result to the tensor dtype.  Every kernel here reproduces that chain with an explicit
+// round-to-dtype (rd / rb) after each reference op, IEEE fp32 division and rint (half to even).
+#include "common.h"
+
+namespace ao {
+
+char* last_error_buf() {
+    static thread_local char buf[512] = {0};
+    return buf;
+}
+
+__device__ __forceinline__ float dtype_eps_dev(int dtype) {
+    if (dtype == AO_BF16) return 0.0078125f;
+    if (dtype == AO_F16) return 0.0009765625f;
+    return 1.1920928955078125e-07f;
+}
+
+// ---------------------------------------------------------------- choose_qparams_affine (generic 2-D block)
+// torchao/quantization/quant_primitives.py:278-367.  TPB threads cooperate on one (bN x bK) block.
+struct QParamArgs {
+    const void* in;
+    int in_dtype;
+    int64_t N, K, ld, bN, bK;
+    int mapping;
+    int64_t qmin, qmax;
+    float eps;        // < 0: finfo(in_dtype).eps
+    int preserve_zero, zp_domain, scale_dtype, zp_dtype;
+    void* scale;
+    void* zp;
+};
+
+template <int TPB>
+__global__ __launch_bounds__(256) void choose_qparams_kernel(QParamArgs a) {
+    constexpr int BLOCKS_PER_WG = 256 / TPB;
+    __shared__ float red_mn[4], red_mx[4];
+    __shared__ int red_nan[4];
+    const int64_t GK = a.K / a.bK;
+    const int64_t nblocks = (a.N / a.bN) * GK;
+    const int tid = threadIdx.x;
+    const int sub = tid / TPB, t = tid % TPB;
+    const int64_t blk = (int64_t)blockIdx.x * BLOCKS_PER_WG + sub;
+    const bool active = blk < nblocks;
+    const int dt = a.in_dtype;
+
+    float mn = INFINITY, mx = -INFINITY;
+    int has_nan = 0;
+    if (active) {
+        const int64_t gn = blk / GK, gk = blk % GK;
+        const int64_t cnt = a.bN * a.bK;
+        for (int64_t i = t; i < cnt; i += TPB) {
+            int64_t r = gn * a.bN + i / a.bK, c = gk * a.bK + i % a.bK;
+            float v = load_f(a.in, dt, r * a.ld + c);
+            if (v != v) has_nan = 1;
+            mn = fminf(mn, v);
+            mx = fmaxf(mx, v);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        mn = fminf(mn, __shfl_xor(mn, o, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        has_nan |= __shfl_xor(has_nan, o, 64);
+    }
+    if (TPB == 256) {
+        const int w = tid >> 6;
+        if ((tid & 63) == 0) { red_mn[w] = mn; red_mx[w] = mx; red_nan[w] = has_nan; }
+        __syncthreads();
+        mn = fminf(fminf(red_mn[0], red_mn[1]), fminf(red_mn[2], red_mn[3]));
+        mx = fmaxf(fmaxf(red_mx[0], red_mx[1]), fmaxf(red_mx[2], red_mx[3]));
+        has_nan = red_nan[0] | red_nan[1] | red_nan[2] | red_nan[3];
+    }
+    if (!active || t != 0) return;
+    if (has_nan) { mn = NAN; mx = NAN; }   // torch.amin / amax propagate NaN
+
+    const float range = (float)(double)(a.qmax - a.qmin);
+    const float half_range = (float)((double)(a.qmax - a.qmin) / 2.0);
+    const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
+    const float epsv = rd(dt, a.eps < 0.f ? dtype_eps_dev(dt) : a.eps);
+
+    float mn_neg = mn, mx_pos = mx;
+    if (a.preserve_zero) {  // :338-340
+        mn_neg = mn < 0.f ? mn : (mn != mn ? mn : 0.f);
+        mx_pos = mx > 0.f ? mx : (mx != mx ? mx : 0.f);
+    }
+    float scale, zp;
+    if (a.mapping == AO_MAP_SYMMETRIC) {  // :345-353
+        float neg = rd(dt, -mn_neg);
+        mx_pos = neg > mx_pos ? neg : mx_pos;
+        scale = rd(dt, __fdiv_rn(mx_pos, half_range));
+        zp = rd(dt, (float)(int)((double)(a.qmax + a.qmin + 1) / 2.0));
+    } else {
+        float d = rd(dt, mx_pos - mn_neg);  // :355
+        scale = rd(dt, __fdiv_rn(d, range));
+        if (a.preserve_zero) {  // :356-358
+            float q = rd(dt, __fdiv_rn(mn_neg, scale));
+            q = rd(dt, __builtin_rintf(q));
+            zp = rd(dt, (float)a.qmin - q);
+            float lo = rd(dt, (float)a.qmin), hi = rd(dt, (float)a.qmax);
+            zp = zp < lo ? lo : (zp > hi ? hi : zp);
+        } else {  // :360-362
+            float q = rd(dt, scale * mid);
+            zp = rd(dt, mn_neg + q);
+        }
+    }
+    if (!(scale >= epsv) && scale == scale) scale = epsv;  // clamp(min=eps) :365
+    store_f(a.scale, a.scale_dtype, blk, scale);
+    store_f(a.zp, a.zp_dtype, blk, zp);
+}
+
+// ---------------------------------------------------------------- quantize_affine / dequantize_affine (elementwise)
+struct QuantArgs {
+    const void* in;
+    int in_dtype;
+    int64_t N, K, ld, bN, bK;
+    const void* scale;
+    int scale_dtype;
+    const void* zp;
+    int zp_dtype;
+    int64_t qmin, qmax;
+    int zp_domain;
+    void* out;
+    int out_dtype;
+};
+
+// torchao/quantization/quant_primitives.py:134-206
+__global__ __launch_bounds__(256) void quantize_affine_kernel(QuantArgs a) {
+    const int64_t total = a.N * a.K;
+    const int64_t GK = a.K / a.bK;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / a.K, c = i % a.K;
+        const int64_t g = (r / a.bN) * GK + c / a.bK;
+        const float x = load_f(a.in, a.in_dtype, r * a.ld + c);
+        const float s = load_f(a.scale, a.scale_dtype, g);
+        float q;
+        if (a.zp_domain == AO_ZP_INT) {  // :191-194
+            float inv = rd(a.scale_dtype, __fdiv_rn(1.0f, s));
+            int dt1 = promote(a.in_dtype, a.scale_dtype);
+            float t = rd(dt1, x * inv);
+            t = rd(dt1, __builtin_rintf(t));
+            if (a.zp) t = rd(promote(dt1, a.zp_dtype), t + load_f(a.zp, a.zp_dtype, g));
+            q = t;
+        } else {  // :195-203
+            const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
+            const float z = load_f(a.zp, a.zp_dtype, g);
+            int dtm = promote(a.zp_dtype, a.scale_dtype);
+            float sm = rd(a.scale_dtype, s * mid);
+            float mv = rd(dtm, z - sm);
+            int dt1 = promote(a.in_dtype, dtm);
+            float t = rd(dt1, x - mv);
+            t = rd(promote(dt1, a.scale_dtype), __fdiv_rn(t, s));
+            q = __builtin_rintf(t);
+        }
+        if (q < (float)a.qmin) q = (float)a.qmin;
+        if (q > (float)a.qmax) q = (float)a.qmax;
+        if (q != q) q = 0.f;
+        const int64_t qi = (int64_t)q;
+        switch (a.out_dtype) {
+            case AO_I32: ((int32_t*)a.out)[i] = (int32_t)qi; break;
+            case AO_I64: ((int64_t*)a.out)[i] = qi; break;
+            case AO_I8: ((int8_t*)a.out)[i] = (int8_t)qi; break;
+            default: ((uint8_t*)a.out)[i] = (uint8_t)qi; break;
+        }
+    }
+}
+
+// torchao/quantization/quant_primitives.py:208-276
+__global__ __launch_bounds__(256) void dequantize_affine_kernel(QuantArgs a) {
+    const int64_t total = a.N * a.K;
+    const int64_t GK = a.K / a.bK;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / a.K, c = i % a.K;
+        const int64_t g = (r / a.bN) * GK + c / a.bK;
+        const int64_t q = load_i(a.in, a.in_dtype, i);
+        const float s = load_f(a.scale, a.scale_dtype, g);
+        float v;
+        if (a.zp_domain == AO_ZP_INT) {  // :257-264
+            int32_t d = (int32_t)q;
+            if (a.zp) d -= (int32_t)load_i(a.zp, a.zp_dtype, g);
+            v = rd(a.out_dtype, (float)d);
+            v = rd(a.out_dtype, v * s);
+        } else {  // :265-274
+            const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
+            v = rd(a.out_dtype, (float)q - mid);
+            v = rd(a.out_dtype, v * s);
+            if (a.zp) v = rd(a.out_dtype, v + load_f(a.zp, a.zp_dtype, g));
+        }
+        store_f(a.out, a.out_dtype, i, v);
+    }
+}
+
+// ---------------------------------------------------------------- fused int4wo quantize + pack (bf16)
+// One wave handles 16 rows x SPAN = max(128, G) columns.  Lane l = (row r = l%16, quarter qd = l/16)
+// owns, per 32-wide slice, the 8 consecutive k = 32*sl + 8*qd + e -- exactly the 8 values of its packed
+// dword -- so codes never leave registers and the packed tile leaves as one 16-byte store per lane.
+template <int G>
+__global__ __launch_bounds__(256) void int4wo_quantize_pack_kernel(const uint16_t* __restrict__ w, int64_t N, int64_t K,
+                                                                    int64_t ldw, int64_t Kp, uint4* __restrict__ packed,
+                                                                    uint32_t* __restrict__ qparams) {
+    constexpr int SPAN = G > 128 ? G : 128;
+    constexpr int NSL = SPAN / 32;          // slices per lane
+    constexpr int SL_PER_G = G / 32;        // slices per group
+    constexpr int NG = SPAN / G;            // groups per span
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, qd = lane >> 4;
+    const int64_t rb = blockIdx.x;
+    const int64_t span = (int64_t)blockIdx.y * 4 + wave;
+    const int64_t nspans = Kp / SPAN;
+    if (span >= nspans) return;
+    const int64_t row = rb * 16 + r;
+    const int64_t kbase = span * SPAN;
+    const bool vec_ok = ((ldw & 7) == 0) && ((((uintptr_t)w) & 15) == 0);
+
+    float v[NSL][8];
+#pragma unroll
+    for (int sl = 0; sl < NSL; ++sl) {
+        const int64_t k0 = kbase + sl * 32 + qd * 8;
+        if (row < N && k0 + 8 <= K && vec_ok) {
+            uint4 raw = *reinterpret_cast<const uint4*>(w + row * ldw + k0);
+            uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[sl][2 * j] = __uint_as_float(u[j] << 16);
+                v[sl][2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                v[sl][e] = (row < N && k0 + e < K) ? bf16_bits_to_f32(w[row * ldw + k0 + e]) : 0.f;  // F.pad zeros
+        }
+    }
+
+    uint32_t words[NSL];
+#pragma unroll
+    for (int gi = 0; gi < NG; ++gi) {
+        float mn = INFINITY, mx = -INFINITY;
+        int has_nan = 0;
+#pragma unroll
+        for (int s2 = 0; s2 < SL_PER_G; ++s2)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float x = v[gi * SL_PER_G + s2][e];
+                if (x != x) has_nan = 1;
+                mn = fminf(mn, x);
+                mx = fmaxf(mx, x);
+            }
+        // the 4 quarters of a row hold the rest of the group
+        mn = fminf(mn, __shfl_xor(mn, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        has_nan |= __shfl_xor(has_nan, 16, 64);
+        mn = fminf(mn, __shfl_xor(mn, 32, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        has_nan |= __shfl_xor(has_nan, 32, 64);
+        if (has_nan) { mn = NAN; mx = NAN; }
+
+        // choose_qparams_affine, ASYMMETRIC / preserve_zero False / FLOAT (quant_primitives.py:355-365)
+        const float d = rne_bf16(mx - mn);
+        const float s0 = rne_bf16(__fdiv_rn(d, 15.0f));
+        const float zp = rne_bf16(mn + rne_bf16(s0 * 8.0f));         // zero point from the un-clamped scale
+        const float epsv = rne_bf16(1e-6f);
+        const float s = (!(s0 >= epsv) && s0 == s0) ? epsv : s0;
+        // quantize_affine, FLOAT domain (quant_primitives.py:195-203)
+        const float mv = rne_bf16(zp - rne_bf16(s * 8.0f));
+#pragma unroll
+        for (int s2 = 0; s2 < SL_PER_G; ++s2) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float t = rne_bf16(v[gi * SL_PER_G + s2][e] - mv);
+                t = rne_bf16(__fdiv_rn(t, s));
+                float q = __builtin_rintf(t);
+                q = q < 0.f ? 0.f : (q > 15.f ? 15.f : q);
+                if (q != q) q = 0.f;
+                word |= (uint32_t)(int)q << (4 * nib_pos(e));
+            }
+            words[gi * SL_PER_G + s2] = word;
+        }
+        if (qd == (gi & 3)) {
+            const int64_t gidx = kbase / G + gi;
+            qparams[(rb * (Kp / G) + gidx) * 16 + r] =
+                (uint32_t)f32_to_bf16_bits(s) | ((uint32_t)f32_to_bf16_bits(zp) << 16);
+        }
+    }
+#pragma unroll
+    for (int ss = 0; ss < NSL / 4; ++ss) {
+        const int64_t kb = kbase / 128 + ss;
+        packed[(rb * (Kp / 128) + kb) * 64 + lane] =
+            make_uint4(words[4 * ss], words[4 * ss + 1], words[4 * ss + 2], words[4 * ss + 3]);
+    }
+}
+
+// ---------------------------------------------------------------- pack / unpack / dequantize on the packed layout
+__global__ __launch_bounds__(256) void int4wo_pack_kernel(const int32_t* __restrict__ codes, const uint16_t* __restrict__ scale,
+                                                           const uint16_t* __restrict__ zero, int64_t N, int64_t K,
+                                                           int64_t Np, int64_t Kp, int64_t g, uint32_t* __restrict__ packed,
+                                                           uint32_t* __restrict__ qparams) {
+    const int64_t ndw = Np * Kp / 8;
+    const int64_t KB = Kp / 128, G = Kp / g, Gl = K / g;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < ndw) {
+        const int sl = i & 3, l = (i >> 2) & 63;
+        const int64_t tile = i >> 8, kb = tile % KB, rb = tile / KB;
+        const int64_t row = rb * 16 + (l & 15), k0 = kb * 128 + sl * 32 + (l >> 4) * 8;
+        uint32_t word = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            uint32_t c = (row < N && k0 + e < K) ? (uint32_t)codes[row * K + k0 + e] & 15u : 8u;
+            word |= c << (4 * nib_pos(e));
+        }
+        packed[i] = word;
+    }
+    const int64_t nq = (Np / 16) * G * 16;
+    if (i < nq) {
+        const int r = i & 15;
+        const int64_t gi = (i >> 4) % G, rb = (i >> 4) / G;
+        const int64_t row = rb * 16 + r;
+        uint32_t v = kPadQparam;
+        if (row < N && gi < Gl) v = (uint32_t)scale[row * Gl + gi] | ((uint32_t)zero[row * Gl + gi] << 16);
+        qparams[i] = v;
+    }
+}
+
+// mode 0: unpack to int32 codes + bf16 scale/zero (logical region); mode 1: dequantize to bf16 [N,K]
+template <int MODE>
+__global__ __launch_bounds__(256) void int4wo_unpack_kernel(const uint32_t* __restrict__ packed,
+                                                             const uint32_t* __restrict__ qparams, int64_t N, int64_t K,
+                                                             int64_t Np, int64_t Kp, int64_t g, int32_t* __restrict__ codes,
+                                                             uint16_t* __restrict__ scale, uint16_t* __restrict__ zero,
+                                                             uint16_t* __restrict__ out) {
+    const int64_t ndw = Np * Kp / 8;
+    const int64_t KB = Kp / 128, G = Kp / g, Gl = K / g;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < ndw) {
+        const int sl = i & 3, l = (i >> 2) & 63;
+        const int64_t tile = i >> 8, kb = tile % KB, rb = tile / KB;
+        const int64_t row = rb * 16 + (l & 15), k0 = kb * 128 + sl * 32 + (l >> 4) * 8;
+        const uint32_t word = packed[i];
+        if (row < N) {
+            if (MODE == 0) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (k0 + e < K) codes[row * K + k0 + e] = (int32_t)((word >> (4 * nib_pos(e))) & 15u);
+            } else {
+                // dequantize_affine FLOAT domain (quant_primitives.py:265-274): bf16(bf16((q-8)*s) + z)
+                const uint32_t qp = qparams[(rb * G + k0 / g) * 16 + (l & 15)];
+                const float s = __uint_as_float(qp << 16), z = __uint_as_float(qp & 0xffff0000u);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (k0 + e < K) {
+                        float q = (float)(int)((word >> (4 * nib_pos(e))) & 15u) - 8.0f;
+                        out[row * K + k0 + e] = f32_to_bf16_bits(rne_bf16(rne_bf16(q) * s) + z);
+                    }
+            }
+        }
+    }
+    if (MODE == 0) {
+        const int64_t nq = (Np / 16) * G * 16;
+        if (i < nq) {
+            const int r = i & 15;
+            const int64_t gi = (i >> 4) % G, rb = (i >> 4) / G;
+            const int64_t row = rb * 16 + r;
+            if (row < N && gi < Gl) {
+                const uint32_t v = qparams[i];
+                scale[row * Gl + gi] = (uint16_t)(v & 0xffffu);
+                zero[row * Gl + gi] = (uint16_t)(v >> 16);
+            }
+        }
+    }
+}
+
+static int check_block(int64_t N, int64_t K, int64_t bN, int64_t bK) {
+    AO_REQUIRE(N > 0 && K > 0, "empty input: N=%lld K=%lld", (long long)N, (long long)K);
+    AO_REQUIRE(bN > 0 && bK > 0 && N % bN == 0 && K % bK == 0,
+               "Expecting input size (%lld, %lld) to be divisible by block_size (%lld, %lld)", (long long)N,
+               (long long)K, (long long)bN, (long long)bK);
+    return 0;
+}
+
+}  // namespace ao
+
+using namespace ao;
+
+extern "C" int ao_amd_abi_version(void) { return 1; }
+extern "C" const char* ao_amd_last_error(void) { return ao::last_error_buf(); }
+
+extern "C" int ao_amd_choose_qparams_affine(const void* in, int in_dtype, int64_t N, int64_t K, int64_t ld, int64_t bN,
+                                            int64_t bK, int mapping, int64_t qmin, int64_t qmax, double eps,
+                                            int preserve_zero, int zp_domain, int scale_dtype, int zp_dtype, void* scale,
+                                            void* zero_point, void* stream) {
+    AO_REQUIRE(in && scale && zero_point, "null pointer argument");
+    AO_REQUIRE(is_float_dtype(in_dtype), "Unsupported input dtype code: %d", in_dtype);
+    AO_REQUIRE(mapping == AO_MAP_SYMMETRIC || mapping == AO_MAP_ASYMMETRIC, "Unsupported mapping type: %d", mapping);
+    if (int rc = check_block(N, K, bN, bK)) return rc;
+    AO_REQUIRE(ld >= K, "row stride %lld smaller than K=%lld", (long long)ld, (long long)K);
+    AO_REQUIRE(qmax > qmin, "quant_max must exceed quant_min");
+    if (mapping == AO_MAP_SYMMETRIC) {
+        AO_REQUIRE(preserve_zero, "preserve_zero == False is not supported for symmetric quantization");
+        AO_REQUIRE(zp_domain == AO_ZP_INT, "zero_point_domain != ZeroPointDomain.INT is not supported for symmetric quantization");
+    } else if (!preserve_zero) {
+        AO_REQUIRE(zp_domain == AO_ZP_FLOAT, "if not preserve_zero, zero_point must be in FLOAT domain");
+    }
+    QParamArgs a{in, in_dtype, N, K, ld, bN, bK, mapping, qmin, qmax, (float)eps, preserve_zero, zp_domain,
+                 scale_dtype, zp_dtype, scale, zero_point};
+    const int64_t nblocks = (N / bN) * (K / bK);
+    hipStream_t st = (hipStream_t)stream;
+    if (bN * bK <= 2048) {
+        hipLaunchKernelGGL(choose_qparams_kernel<64>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL(choose_qparams_kernel<256>, dim3((unsigned)nblocks), dim3(256), 0, st, a);
+    }
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+static unsigned elementwise_grid(int64_t total) {
+    int64_t b = (total + 255) / 256;
+    return (unsigned)(b > 1048576 ? 1048576 : b);
+}
+
+extern "C" int ao_amd_quantize_affine(const void* in, int in_dtype, int64_t N, int64_t K, int64_t ld, int64_t bN,
+                                      int64_t bK, const void* scale, int scale_dtype, const void* zero_point,
+                                      int zp_dtype, int64_t qmin, int64_t qmax, int zp_domain, void* out, int out_dtype,
+                                      void* stream) {
+    AO_REQUIRE(in && scale && out, "null pointer argument");
+    AO_REQUIRE(is_float_dtype(in_dtype), "Unsupported input dtype code: %d", in_dtype);
+    AO_REQUIRE(is_float_dtype(scale_dtype), "scale must be a floating point tensor");
+    AO_REQUIRE(out_dtype == AO_I32 || out_dtype == AO_I64 || out_dtype == AO_I8 || out_dtype == AO_U8,
+               "Unsupported dtype code: %d", out_dtype);
+    AO_REQUIRE(zp_domain == AO_ZP_INT || zp_domain == AO_ZP_FLOAT, "Unexpected zero point domain: %d", zp_domain);
+    AO_REQUIRE(zero_point || zp_domain == AO_ZP_INT, "zero_point is required in the FLOAT domain");
+    if (int rc = check_block(N, K, bN, bK)) return rc;
+    AO_REQUIRE(ld >= K, "row stride %lld smaller than K=%lld", (long long)ld, (long long)K);
+    QuantArgs a{in, in_dtype, N, K, ld, bN, bK, scale, scale_dtype, zero_point, zp_dtype, qmin, qmax, zp_domain, out, out_dtype};
+    hipLaunchKernelGGL(quantize_affine_kernel, dim3(elementwise_grid(N * K)), dim3(256), 0, (hipStream_t)stream, a);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_dequantize_affine(const void* in, int in_dtype, int64_t N, int64_t K, int64_t bN, int64_t bK,
+                                        const void* scale, int scale_dtype, const void* zero_point, int zp_dtype,
+                                        int64_t qmin, int64_t qmax, int zp_domain, void* out, int out_dtype,
+                                        void* stream) {
+    AO_REQUIRE(in && scale && out, "null pointer argument");
+    AO_REQUIRE(!is_float_dtype(in_dtype), "input must be an integer tensor, got dtype code %d", in_dtype);
+    AO_REQUIRE(is_float_dtype(out_dtype), "Unsupported output dtype code: %d", out_dtype);
+    AO_REQUIRE(zp_domain == AO_ZP_INT || zp_domain == AO_ZP_FLOAT, "Unexpected zero point domain: %d", zp_domain);
+    if (int rc = check_block(N, K, bN, bK)) return rc;
+    QuantArgs a{in, in_dtype, N, K, K, bN, bK, scale, scale_dtype, zero_point, zp_dtype, qmin, qmax, zp_domain, out, out_dtype};
+    hipLaunchKernelGGL(dequantize_affine_kernel, dim3(elementwise_grid(N * K)), dim3(256), 0, (hipStream_t)stream, a);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_int4wo_packed_shape(int64_t N, int64_t K, int64_t g, int64_t* Np, int64_t* Kp,
+                                          int64_t* packed_bytes, int64_t* qparam_bytes) {
+    AO_REQUIRE(N > 0 && K > 0, "empty weight: N=%lld K=%lld", (long long)N, (long long)K);
+    AO_REQUIRE(valid_group(g), "group_size must be one of 32, 64, 128, 256, got %lld", (long long)g);
+    const int64_t np = round_up(N, 16), kp = round_up(K, g > 128 ? g : 128);
+    if (Np) *Np = np;
+    if (Kp) *Kp = kp;
+    if (packed_bytes) *packed_bytes = np * kp / 2;
+    if (qparam_bytes) *qparam_bytes = np * (kp / g) * 4;
+    return 0;
+}
+
+extern "C" int ao_amd_int4wo_quantize_pack(const void* w_bf16, int64_t N, int64_t K, int64_t ldw, int64_t g,
+                                           void* packed, void* qparams, void* stream) {
+    AO_REQUIRE(w_bf16 && packed && qparams, "null pointer argument");
+    int64_t Np, Kp;
+    if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
+    AO_REQUIRE(ldw >= K, "row stride %lld smaller than K=%lld", (long long)ldw, (long long)K);
+    AO_REQUIRE((((uintptr_t)packed) & 15) == 0, "packed buffer must be 16-byte aligned");
+    const int64_t span = g > 128 ? g : 128;
+    const int64_t nspans = Kp / span;
+    AO_REQUIRE(Np / 16 <= 0x7fffffff && (nspans + 3) / 4 <= 65535, "weight too large for one launch");
+    dim3 grid((unsigned)(Np / 16), (unsigned)((nspans + 3) / 4));
+    hipStream_t st = (hipStream_t)stream;
+    const uint16_t* w = (const uint16_t*)w_bf16;
+    switch (g) {
+        case 32: hipLaunchKernelGGL(int4wo_quantize_pack_kernel<32>, grid, dim3(256), 0, st, w, N, K, ldw, Kp, (uint4*)packed, (uint32_t*)qparams); break;
+        case 64: hipLaunchKernelGGL(int4wo_quantize_pack_kernel<64>, grid, dim3(256), 0, st, w, N, K, ldw, Kp, (uint4*)packed, (uint32_t*)qparams); break;
+        case 128: hipLaunchKernelGGL(int4wo_quantize_pack_kernel<128>, grid, dim3(256), 0, st, w, N, K, ldw, Kp, (uint4*)packed, (uint32_t*)qparams); break;
+        default: hipLaunchKernelGGL(int4wo_quantize_pack_kernel<256>, grid, dim3(256), 0, st, w, N, K, ldw, Kp, (uint4*)packed, (uint32_t*)qparams); break;
+    }
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_int4wo_pack(const int32_t* codes, const void* scale_bf16, const void* zero_bf16, int64_t N,
+                                  int64_t K, int64_t g, void* packed, void* qparams, void* stream) {
+    AO_REQUIRE(codes && scale_bf16 && zero_bf16 && packed && qparams, "null pointer argument");
+    int64_t Np, Kp;
+    if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
+    AO_REQUIRE(K % g == 0, "in_features %lld must be divisible by group_size %lld", (long long)K, (long long)g);
+    const int64_t n = Np * Kp / 8;  // >= number of qparam words
+    hipLaunchKernelGGL(int4wo_pack_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, codes,
+                       (const uint16_t*)scale_bf16, (const uint16_t*)zero_bf16, N, K, Np, Kp, g, (uint32_t*)packed,
+                       (uint32_t*)qparams);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_int4wo_unpack(const void* packed, const void* qparams, int64_t N, int64_t K, int64_t g,
+                                    int32_t* codes, void* scale_bf16, void* zero_bf16, void* stream) {
+    AO_REQUIRE(codes && scale_bf16 && zero_bf16 && packed && qparams, "null pointer argument");
+    int64_t Np, Kp;
+    if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
+    AO_REQUIRE(K % g == 0, "in_features %lld must be divisible by group_size %lld", (long long)K, (long long)g);
+    const int64_t n = Np * Kp / 8;
+    hipLaunchKernelGGL(int4wo_unpack_kernel<0>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint32_t*)packed, (const uint32_t*)qparams, N, K, Np, Kp, g, codes, (uint16_t*)scale_bf16,
+                       (uint16_t*)zero_bf16, (uint16_t*)nullptr);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_int4wo_dequantize(const void* packed, const void* qparams, int64_t N, int64_t K, int64_t g,
+                                        void* out_bf16, void* stream) {
+    AO_REQUIRE(packed && qparams && out_bf16, "null pointer argument");
+    int64_t Np, Kp;
+    if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
+    const int64_t n = Np * Kp / 8;
+    hipLaunchKernelGGL(int4wo_unpack_kernel<1>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint32_t*)packed, (const uint32_t*)qparams, N, K, Np, Kp, g, (int32_t*)nullptr,
+                       (uint16_t*)nullptr, (uint16_t*)nullptr, (uint16_t*)out_bf16);
+    AO_LAUNCH_CHECK();
+    return 0;
+}

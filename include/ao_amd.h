@@ -1,0 +1,114 @@
+/*
+ * ao_amd -- C ABI of the MI355X (gfx950) weight-only quantized linear library.
+ *
+ * Plain pointers and sizes only: no torch types cross this boundary.  All device pointers are
+ * HIP device memory on the current device, all kernels are enqueued on `stream` (a hipStream_t
+ * passed as void*; NULL = the null stream) and no entry point synchronises, allocates or frees
+ * device memory, so every call is safe under HIP graph capture.
+ *
+ * Every function returns 0 on success and a negative value on error; ao_amd_last_error() then
+ * returns a thread-local, human readable message (argument-check failures are the counterpart of
+ * the reference's TORCH_CHECK / assert -> RuntimeError / AssertionError paths).
+ *
+ * "Reference" below is pytorch-labs/ao (torchao) 0.3.1; paths are relative to its tree.
+ */
+#ifndef AO_AMD_H
+#define AO_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype codes */
+#define AO_F32 0
+#define AO_BF16 1
+#define AO_F16 2
+#define AO_I32 3
+#define AO_I64 4
+#define AO_I8 5
+#define AO_U8 6
+
+/* mapping_type / zero_point_domain (torchao/quantization/quant_primitives.py:24-47) */
+#define AO_MAP_SYMMETRIC 0
+#define AO_MAP_ASYMMETRIC 1
+#define AO_ZP_INT 0
+#define AO_ZP_FLOAT 1
+
+int ao_amd_abi_version(void);
+const char* ao_amd_last_error(void);
+
+/* ---------------------------------------------------------------- affine primitives (2-D, block (bN,bK))
+ * in: [N,K] with row stride ld (elements).  qparams: contiguous [N/bN, K/bK].
+ * Bit-exact with the reference's eager CPU ops: every reference op rounds to its tensor dtype. */
+
+/* replaces choose_qparams_affine, torchao/quantization/quant_primitives.py:278-367
+ * eps < 0 selects finfo(in_dtype).eps (the reference's eps=None). */
+int ao_amd_choose_qparams_affine(const void* in, int in_dtype, int64_t N, int64_t K, int64_t ld, int64_t bN,
+                                 int64_t bK, int mapping, int64_t qmin, int64_t qmax, double eps, int preserve_zero,
+                                 int zp_domain, int scale_dtype, int zp_dtype, void* scale, void* zero_point,
+                                 void* stream);
+
+/* replaces quantize_affine, torchao/quantization/quant_primitives.py:134-206
+ * zero_point may be NULL in the INT domain.  out: contiguous [N,K] of out_dtype (AO_I32/I64/I8/U8). */
+int ao_amd_quantize_affine(const void* in, int in_dtype, int64_t N, int64_t K, int64_t ld, int64_t bN, int64_t bK,
+                           const void* scale, int scale_dtype, const void* zero_point, int zp_dtype, int64_t qmin,
+                           int64_t qmax, int zp_domain, void* out, int out_dtype, void* stream);
+
+/* replaces dequantize_affine, torchao/quantization/quant_primitives.py:208-276
+ * in: contiguous [N,K] integer codes; out: contiguous [N,K] of out_dtype (AO_F32/BF16/F16). */
+int ao_amd_dequantize_affine(const void* in, int in_dtype, int64_t N, int64_t K, int64_t bN, int64_t bK,
+                             const void* scale, int scale_dtype, const void* zero_point, int zp_dtype, int64_t qmin,
+                             int64_t qmax, int zp_domain, void* out, int out_dtype, void* stream);
+
+/* ---------------------------------------------------------------- int4 weight-only (uint4 groupwise asymmetric)
+ * Packed layout (this library's own; replaces the tensor-core tile order of
+ * aten::_convert_weight_to_int4pack, call site torchao/dtypes/affine_quantized_tensor.py:461, and
+ * pack_tinygemm_scales_and_zeros, torchao/quantization/utils.py:310-322):
+ *   Np = N rounded up to 16, Kp = K rounded up to max(128, g)
+ *   packed : uint32 [Np/16][Kp/128][64 lanes][4]   lane l: row 16*rb + l%16, quarter qd = l/16;
+ *            dword (l, sl) holds k = 128*kb + 32*sl + 8*qd + e (e=0..7) with element e in the nibble at
+ *            bit 4*((e>>1) + 4*(e&1))  -- one wave64 16-byte load per lane = 1 KiB contiguous, and the
+ *            8 values of a dword land in the k-order of a 16x16x32 bf16 MFMA operand.
+ *   qparams: uint32 [Np/16][Kp/g][16] = scale_bf16 | zero_bf16 << 16
+ * Padding holds code 8, scale bf16(1e-6), zero 0, i.e. what quantizing zero padding yields.
+ * group size g must be 32, 64, 128 or 256. */
+int ao_amd_int4wo_packed_shape(int64_t N, int64_t K, int64_t g, int64_t* Np, int64_t* Kp, int64_t* packed_bytes,
+                               int64_t* qparam_bytes);
+
+/* Fused from_float for int4_weight_only: choose_qparams_affine(ASYMMETRIC,(1,g),qmin 0,qmax 15,eps 1e-6,
+ * preserve_zero False, FLOAT zero point, bf16) + quantize_affine + pack in one pass over w.
+ * replaces AffineQuantizedTensor.from_float, torchao/dtypes/affine_quantized_tensor.py:184-229 as called by
+ * torchao/quantization/quant_api.py:372-385.   w: bf16 [N,K], row stride ldw. */
+int ao_amd_int4wo_quantize_pack(const void* w_bf16, int64_t N, int64_t K, int64_t ldw, int64_t g, void* packed,
+                                void* qparams, void* stream);
+
+/* Layout constructor from plain tensors; replaces TensorCoreTiledAQTLayout.from_plain,
+ * torchao/dtypes/affine_quantized_tensor.py:460-465.  codes int32 [N,K] (values 0..15), scale / zero
+ * bf16 [N,K/g], all contiguous, K % g == 0. */
+int ao_amd_int4wo_pack(const int32_t* codes, const void* scale_bf16, const void* zero_bf16, int64_t N, int64_t K,
+                       int64_t g, void* packed, void* qparams, void* stream);
+
+/* Inverse of ao_amd_int4wo_pack; replaces TensorCoreTiledAQTLayout.get_plain,
+ * torchao/dtypes/affine_quantized_tensor.py:509-537 (which recovers codes by multiplying with an identity). */
+int ao_amd_int4wo_unpack(const void* packed, const void* qparams, int64_t N, int64_t K, int64_t g, int32_t* codes,
+                         void* scale_bf16, void* zero_bf16, void* stream);
+
+/* Unpack + dequantize_affine(FLOAT domain) in one pass: out bf16 [N,K] contiguous.
+ * replaces AffineQuantizedTensor.dequantize, torchao/dtypes/affine_quantized_tensor.py:157-161. */
+int ao_amd_int4wo_dequantize(const void* packed, const void* qparams, int64_t N, int64_t K, int64_t g,
+                             void* out_bf16, void* stream);
+
+/* y[M,N] = x[M,K] @ dequant(W)[N,K]^T (+ bias), fp32 accumulation, dequant = bf16(bf16((q-8)*s) + z).
+ * replaces aten::_weight_int4pack_mm as called by _quantized_linear_op,
+ * torchao/dtypes/affine_quantized_tensor.py:600-640.
+ * x: bf16 [M,K] row stride ldx; bias: bf16 [N] or NULL; y: y_dtype (AO_BF16 or AO_F32) row stride ldy. */
+int ao_amd_int4wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed,
+                         const void* qparams, int64_t N, int64_t g, const void* bias_bf16, void* y, int y_dtype,
+                         int64_t ldy, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AO_AMD_H */
