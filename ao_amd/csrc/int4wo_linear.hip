@@ -88,26 +88,34 @@ __device__ __forceinline__ bf16x8_t dequant8(uint32_t w, const GroupConst& g, ui
     return out.v;
 }
 
-// Activation fragment: 8 consecutive bf16 of row m starting at k (zeros outside [0,M) x [0,K)).
-__device__ __forceinline__ bf16x8_t load_x8(const uint16_t* __restrict__ x, int64_t ldx, int64_t m, int64_t M,
-                                            int64_t k, int64_t K, bool vec_ok) {
-    union { uint4 q; uint16_t h[8]; bf16x8_t v; } r;
+// Activation fragment for the slow path: 8 consecutive bf16 of row m starting at k (zeros outside
+// [0,M) x [0,K)), tolerant of any alignment.
+__device__ __forceinline__ uint4 load_x8_checked(const uint16_t* __restrict__ x, int64_t ldx, int64_t m, int64_t M,
+                                                 int64_t k, int64_t K) {
+    union { uint4 q; uint16_t h[8]; } r;
     r.q = make_uint4(0, 0, 0, 0);
     if (m < M) {
-        if (vec_ok && k + 8 <= K) {
-            r.q = *reinterpret_cast<const uint4*>(x + m * ldx + k);
-        } else {
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (k + e < K) r.h[e] = x[m * ldx + k + e];
-        }
+        for (int e = 0; e < 8; ++e)
+            if (k + e < K) r.h[e] = x[m * ldx + k + e];
     }
-    return r.v;
+    return r.q;
 }
 
-// One workgroup = one 16-row block of W, WAVES waves splitting K by 128-wide super-slices; blockIdx.y
-// selects a chunk of 16 activation rows.  Partial 16x16 accumulators meet in LDS.
-template <int G, int WAVES>
+struct TileBuf {
+    uint4 w;      // 32 codes of this lane: k = 128*kb + 32*qd + 0..31
+    uint32_t q;   // (scale, zero) of the lane's group
+    uint4 x[4];   // activations of row m = lane%16 for the same 32 k (zero for rows >= M)
+};
+
+// One workgroup = one 16-row block of W; its WAVES waves take the 128-wide K tiles round-robin, so the
+// workgroup streams its contiguous (K/2 bytes per row) x 16 rows region front to back.  Each lane owns
+// row r = lane%16 and 32 consecutive k per tile; tiles are double-buffered in registers so the next
+// tile's loads are in flight while the current one is dequantized.  blockIdx.y selects a chunk of 16
+// activation rows.  Partial 16x16 accumulators of the waves meet in LDS.
+//
+// FAST: K is a multiple of 128 (no K tail), x rows are 16-byte aligned.
+template <int G, int WAVES, bool FAST>
 __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(
     const uint16_t* __restrict__ x, int64_t M, int64_t K, int64_t ldx, const uint4* __restrict__ packed,
     const uint32_t* __restrict__ qparams, int64_t N, int64_t Kp, const uint16_t* __restrict__ bias, void* __restrict__ y,
@@ -117,27 +125,61 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(
     const int r = lane & 15, qd = lane >> 4;
     const int64_t rb = blockIdx.x;
     const int64_t m0 = (int64_t)blockIdx.y * 16;
-    const int64_t KB = Kp / 128, NG = Kp / G;
-    const bool vec_ok = ((ldx & 7) == 0) && ((((uintptr_t)x) & 15) == 0);
+    const int KB = (int)(Kp / 128);
     const uint32_t magic = 0x43004300u, one_lo = 0x00003F80u, one_hi = 0x3F800000u;
 
     const uint4* wp = packed + rb * KB * 64 + lane;
-    const uint32_t* qp = qparams + rb * NG * 16 + r;
+    const uint32_t* qp = qparams + rb * (Kp / G) * 16 + r;
+    const bool xact = (m0 + r) < M;
+    const uint16_t* xp = x + (xact ? (m0 + r) : 0) * ldx + qd * 32;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 
-    for (int64_t kb = wave; kb < KB; kb += WAVES) {
-        const uint4 w4 = wp[kb * 64];
-        const uint32_t ww[4] = {w4.x, w4.y, w4.z, w4.w};
-        GroupConst gc;
-        if (G >= 128) gc = make_group(qp[(kb * 128 / G) * 16]);
+    auto load_tile = [&](TileBuf& b, int kb) {
+        typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+        const u32x4_t wv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp + (int64_t)kb * 64));
+        b.w = make_uint4(wv.x, wv.y, wv.z, wv.w);
+        b.q = qp[((kb * 128 + qd * 32) / G) * 16];
+        if (FAST) {
+            if (xact) {
+                const uint4* xv = reinterpret_cast<const uint4*>(xp + (int64_t)kb * 128);
+#pragma unroll
+                for (int sl = 0; sl < 4; ++sl) b.x[sl] = xv[sl];
+            }
+        } else {
+#pragma unroll
+            for (int sl = 0; sl < 4; ++sl)
+                b.x[sl] = load_x8_checked(x, ldx, m0 + r, M, (int64_t)kb * 128 + qd * 32 + sl * 8, K);
+        }
+    };
+    auto compute_tile = [&](const TileBuf& b) {
+        const GroupConst gc = make_group(b.q);
+        const uint32_t ww[4] = {b.w.x, b.w.y, b.w.z, b.w.w};
 #pragma unroll
         for (int sl = 0; sl < 4; ++sl) {
-            if (G == 64 && (sl & 1) == 0) gc = make_group(qp[(kb * 2 + (sl >> 1)) * 16]);
-            if (G == 32) gc = make_group(qp[(kb * 4 + sl) * 16]);
-            const bf16x8_t b = dequant8(ww[sl], gc, magic, one_lo, one_hi);
-            const bf16x8_t a = load_x8(x, ldx, m0 + r, M, kb * 128 + sl * 32 + qd * 8, K, vec_ok);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+            union { uint4 q; bf16x8_t v; } a;
+            a.q = b.x[sl];
+            const bf16x8_t bw = dequant8(ww[sl], gc, magic, one_lo, one_hi);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, bw, acc, 0, 0, 0);
         }
+    };
+
+    TileBuf b0, b1;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {  // rows >= M keep these zeros: their loads are masked off
+        b0.x[sl] = make_uint4(0, 0, 0, 0);
+        b1.x[sl] = make_uint4(0, 0, 0, 0);
+    }
+    int kb = wave;
+    if (kb < KB) load_tile(b0, kb);
+    while (kb < KB) {
+        const int kb1 = kb + WAVES, kb2 = kb + 2 * WAVES;
+        if (kb1 < KB) load_tile(b1, kb1);
+        compute_tile(b0);
+        if (kb1 < KB) {
+            if (kb2 < KB) load_tile(b0, kb2);
+            compute_tile(b1);
+        }
+        kb = kb2;
     }
 
     // acc[i] = C[m = 4*qd + i][n = r]
@@ -163,16 +205,35 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(
     }
 }
 
-template <int WAVES>
-static void launch_linear(int64_t g, dim3 grid, hipStream_t st, const uint16_t* x, int64_t M, int64_t K, int64_t ldx,
-                          const uint4* packed, const uint32_t* qparams, int64_t N, int64_t Kp, const uint16_t* bias,
-                          void* y, int y_is_f32, int64_t ldy) {
-    dim3 block(WAVES * 64);
+struct LinearArgs {
+    const uint16_t* x; int64_t M, K, ldx;
+    const uint4* packed; const uint32_t* qparams;
+    int64_t N, Kp;
+    const uint16_t* bias; void* y; int y_is_f32; int64_t ldy;
+};
+
+template <int G, int WAVES, bool FAST>
+static void launch_one(dim3 grid, hipStream_t st, const LinearArgs& a) {
+    hipLaunchKernelGGL((int4wo_linear_kernel<G, WAVES, FAST>), grid, dim3(WAVES * 64), 0, st, a.x, a.M, a.K, a.ldx,
+                       a.packed, a.qparams, a.N, a.Kp, a.bias, a.y, a.y_is_f32, a.ldy);
+}
+template <int G, bool FAST>
+static void launch_waves(int waves, dim3 grid, hipStream_t st, const LinearArgs& a) {
+    switch (waves) {
+        case 1: launch_one<G, 1, FAST>(grid, st, a); break;
+        case 2: launch_one<G, 2, FAST>(grid, st, a); break;
+        case 4: launch_one<G, 4, FAST>(grid, st, a); break;
+        case 8: launch_one<G, 8, FAST>(grid, st, a); break;
+        default: launch_one<G, 16, FAST>(grid, st, a); break;
+    }
+}
+template <bool FAST>
+static void launch_group(int64_t g, int waves, dim3 grid, hipStream_t st, const LinearArgs& a) {
     switch (g) {
-        case 32: hipLaunchKernelGGL((int4wo_linear_kernel<32, WAVES>), grid, block, 0, st, x, M, K, ldx, packed, qparams, N, Kp, bias, y, y_is_f32, ldy); break;
-        case 64: hipLaunchKernelGGL((int4wo_linear_kernel<64, WAVES>), grid, block, 0, st, x, M, K, ldx, packed, qparams, N, Kp, bias, y, y_is_f32, ldy); break;
-        case 128: hipLaunchKernelGGL((int4wo_linear_kernel<128, WAVES>), grid, block, 0, st, x, M, K, ldx, packed, qparams, N, Kp, bias, y, y_is_f32, ldy); break;
-        default: hipLaunchKernelGGL((int4wo_linear_kernel<256, WAVES>), grid, block, 0, st, x, M, K, ldx, packed, qparams, N, Kp, bias, y, y_is_f32, ldy); break;
+        case 32: launch_waves<32, FAST>(waves, grid, st, a); break;
+        case 64: launch_waves<64, FAST>(waves, grid, st, a); break;
+        case 128: launch_waves<128, FAST>(waves, grid, st, a); break;
+        default: launch_waves<256, FAST>(waves, grid, st, a); break;
     }
 }
 
@@ -191,16 +252,20 @@ extern "C" int ao_amd_int4wo_linear(const void* x_bf16, int64_t M, int64_t K, in
     AO_REQUIRE(ldx >= K && ldy >= N, "row strides (ldx=%lld, ldy=%lld) smaller than the rows (K=%lld, N=%lld)",
                (long long)ldx, (long long)ldy, (long long)K, (long long)N);
     AO_REQUIRE((((uintptr_t)packed) & 15) == 0, "packed buffer must be 16-byte aligned");
+    AO_REQUIRE(Kp / 128 < (1 << 23), "in_features too large: K=%lld", (long long)K);
     if (M == 0) return 0;
     const int64_t mchunks = (M + 15) / 16;
     AO_REQUIRE(mchunks <= 65535, "batch too large for one launch: M=%lld", (long long)M);
-    dim3 grid((unsigned)(Np / 16), (unsigned)mchunks);
-    hipStream_t st = (hipStream_t)stream;
-    const int64_t KB = Kp / 128;
-    if (KB >= 8)
-        launch_linear<8>(g, grid, st, (const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams, N, Kp, (const uint16_t*)bias_bf16, y, y_dtype == AO_F32, ldy);
-    else
-        launch_linear<4>(g, grid, st, (const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams, N, Kp, (const uint16_t*)bias_bf16, y, y_dtype == AO_F32, ldy);
+    const int64_t KB = Kp / 128, RB = Np / 16;
+    // enough waves to fill 256 CUs several times over, never more waves than K tiles
+    int waves = 1;
+    while (waves < 16 && RB * mchunks * waves < 6144 && waves * 2 <= KB) waves *= 2;
+    const bool fast = (K == Kp) && ((ldx & 7) == 0) && ((((uintptr_t)x_bf16) & 15) == 0);
+    LinearArgs a{(const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams, N, Kp,
+                 (const uint16_t*)bias_bf16, y, y_dtype == AO_F32, ldy};
+    dim3 grid((unsigned)RB, (unsigned)mchunks);
+    if (fast) launch_group<true>(g, waves, grid, (hipStream_t)stream, a);
+    else launch_group<false>(g, waves, grid, (hipStream_t)stream, a);
     AO_LAUNCH_CHECK();
     return 0;
 }

@@ -193,101 +193,119 @@ __global__ __launch_bounds__(256) void dequantize_affine_kernel(QuantArgs a) {
 
 // ---------------------------------------------------------------- fused int4wo quantize + pack (bf16)
 // One wave handles 16 rows x SPAN = max(128, G) columns.  Lane l = (row r = l%16, quarter qd = l/16)
-// owns, per 32-wide slice, the 8 consecutive k = 32*sl + 8*qd + e -- exactly the 8 values of its packed
-// dword -- so codes never leave registers and the packed tile leaves as one 16-byte store per lane.
+// owns, per 128-wide super-slice, the 32 consecutive k = 32*qd + 8*sl + e -- exactly the values of its
+// four packed dwords -- so codes never leave registers, the weight is read as 64 contiguous bytes per
+// lane and the packed tile leaves as one 16-byte store per lane.  A group of 32 lives in one lane;
+// larger groups are finished with one or two cross-quarter shuffles.
 template <int G>
 __global__ __launch_bounds__(256) void int4wo_quantize_pack_kernel(const uint16_t* __restrict__ w, int64_t N, int64_t K,
                                                                     int64_t ldw, int64_t Kp, uint4* __restrict__ packed,
                                                                     uint32_t* __restrict__ qparams) {
     constexpr int SPAN = G > 128 ? G : 128;
-    constexpr int NSL = SPAN / 32;          // slices per lane
-    constexpr int SL_PER_G = G / 32;        // slices per group
-    constexpr int NG = SPAN / G;            // groups per span
+    constexpr int NSS = SPAN / 128;  // super-slices per wave (2 only for G = 256)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, qd = lane >> 4;
     const int64_t rb = blockIdx.x;
     const int64_t span = (int64_t)blockIdx.y * 4 + wave;
-    const int64_t nspans = Kp / SPAN;
-    if (span >= nspans) return;
+    if (span >= Kp / SPAN) return;
     const int64_t row = rb * 16 + r;
     const int64_t kbase = span * SPAN;
     const bool vec_ok = ((ldw & 7) == 0) && ((((uintptr_t)w) & 15) == 0);
 
-    float v[NSL][8];
+    float v[NSS][4][8];
 #pragma unroll
-    for (int sl = 0; sl < NSL; ++sl) {
-        const int64_t k0 = kbase + sl * 32 + qd * 8;
-        if (row < N && k0 + 8 <= K && vec_ok) {
-            uint4 raw = *reinterpret_cast<const uint4*>(w + row * ldw + k0);
-            uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+    for (int ss = 0; ss < NSS; ++ss)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                v[sl][2 * j] = __uint_as_float(u[j] << 16);
-                v[sl][2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u);
+        for (int sl = 0; sl < 4; ++sl) {
+            const int64_t k0 = kbase + ss * 128 + qd * 32 + sl * 8;
+            if (row < N && k0 + 8 <= K && vec_ok) {
+                uint4 raw = *reinterpret_cast<const uint4*>(w + row * ldw + k0);
+                uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    v[ss][sl][2 * j] = __uint_as_float(u[j] << 16);
+                    v[ss][sl][2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)  // F.pad zeros outside the weight
+                    v[ss][sl][e] = (row < N && k0 + e < K) ? bf16_bits_to_f32(w[row * ldw + k0 + e]) : 0.f;
             }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                v[sl][e] = (row < N && k0 + e < K) ? bf16_bits_to_f32(w[row * ldw + k0 + e]) : 0.f;  // F.pad zeros
         }
-    }
 
-    uint32_t words[NSL];
+    // per-lane partial min/max of each super-slice
+    float mn[NSS], mx[NSS];
+    int has_nan[NSS];
 #pragma unroll
-    for (int gi = 0; gi < NG; ++gi) {
-        float mn = INFINITY, mx = -INFINITY;
-        int has_nan = 0;
+    for (int ss = 0; ss < NSS; ++ss) {
+        mn[ss] = INFINITY; mx[ss] = -INFINITY; has_nan[ss] = 0;
 #pragma unroll
-        for (int s2 = 0; s2 < SL_PER_G; ++s2)
+        for (int sl = 0; sl < 4; ++sl)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                float x = v[gi * SL_PER_G + s2][e];
-                if (x != x) has_nan = 1;
-                mn = fminf(mn, x);
-                mx = fmaxf(mx, x);
+                float x = v[ss][sl][e];
+                if (x != x) has_nan[ss] = 1;
+                mn[ss] = fminf(mn[ss], x);
+                mx[ss] = fmaxf(mx[ss], x);
             }
-        // the 4 quarters of a row hold the rest of the group
-        mn = fminf(mn, __shfl_xor(mn, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        has_nan |= __shfl_xor(has_nan, 16, 64);
-        mn = fminf(mn, __shfl_xor(mn, 32, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        has_nan |= __shfl_xor(has_nan, 32, 64);
-        if (has_nan) { mn = NAN; mx = NAN; }
+    }
+    if (G == 256) {  // both super-slices belong to the one group
+        mn[0] = mn[1] = fminf(mn[0], mn[NSS - 1]);
+        mx[0] = mx[1] = fmaxf(mx[0], mx[NSS - 1]);
+        has_nan[0] = has_nan[1] = has_nan[0] | has_nan[NSS - 1];
+    }
+#pragma unroll
+    for (int ss = 0; ss < NSS; ++ss) {
+        float gmn = mn[ss], gmx = mx[ss];
+        int gnan = has_nan[ss];
+        if (G >= 64) {  // quarters (0,1) and (2,3)
+            gmn = fminf(gmn, __shfl_xor(gmn, 16, 64));
+            gmx = fmaxf(gmx, __shfl_xor(gmx, 16, 64));
+            gnan |= __shfl_xor(gnan, 16, 64);
+        }
+        if (G >= 128) {  // all four quarters
+            gmn = fminf(gmn, __shfl_xor(gmn, 32, 64));
+            gmx = fmaxf(gmx, __shfl_xor(gmx, 32, 64));
+            gnan |= __shfl_xor(gnan, 32, 64);
+        }
+        if (gnan) { gmn = NAN; gmx = NAN; }
 
         // choose_qparams_affine, ASYMMETRIC / preserve_zero False / FLOAT (quant_primitives.py:355-365)
-        const float d = rne_bf16(mx - mn);
+        const float d = rne_bf16(gmx - gmn);
         const float s0 = rne_bf16(__fdiv_rn(d, 15.0f));
-        const float zp = rne_bf16(mn + rne_bf16(s0 * 8.0f));         // zero point from the un-clamped scale
+        const float zp = rne_bf16(gmn + rne_bf16(s0 * 8.0f));  // zero point from the un-clamped scale
         const float epsv = rne_bf16(1e-6f);
         const float s = (!(s0 >= epsv) && s0 == s0) ? epsv : s0;
         // quantize_affine, FLOAT domain (quant_primitives.py:195-203)
         const float mv = rne_bf16(zp - rne_bf16(s * 8.0f));
+        uint32_t words[4];
 #pragma unroll
-        for (int s2 = 0; s2 < SL_PER_G; ++s2) {
+        for (int sl = 0; sl < 4; ++sl) {
             uint32_t word = 0;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                float t = rne_bf16(v[gi * SL_PER_G + s2][e] - mv);
+                float t = rne_bf16(v[ss][sl][e] - mv);
                 t = rne_bf16(__fdiv_rn(t, s));
                 float q = __builtin_rintf(t);
                 q = q < 0.f ? 0.f : (q > 15.f ? 15.f : q);
                 if (q != q) q = 0.f;
                 word |= (uint32_t)(int)q << (4 * nib_pos(e));
             }
-            words[gi * SL_PER_G + s2] = word;
+            words[sl] = word;
         }
-        if (qd == (gi & 3)) {
-            const int64_t gidx = kbase / G + gi;
-            qparams[(rb * (Kp / G) + gidx) * 16 + r] =
-                (uint32_t)f32_to_bf16_bits(s) | ((uint32_t)f32_to_bf16_bits(zp) << 16);
-        }
-    }
-#pragma unroll
-    for (int ss = 0; ss < NSL / 4; ++ss) {
         const int64_t kb = kbase / 128 + ss;
-        packed[(rb * (Kp / 128) + kb) * 64 + lane] =
-            make_uint4(words[4 * ss], words[4 * ss + 1], words[4 * ss + 2], words[4 * ss + 3]);
+        packed[(rb * (Kp / 128) + kb) * 64 + lane] = make_uint4(words[0], words[1], words[2], words[3]);
+
+        // one lane per (row, group) stores the interleaved (scale, zero) word
+        const int64_t k_lane = kbase + ss * 128 + qd * 32;
+        bool writer;
+        if (G == 32) writer = true;
+        else if (G == 64) writer = (qd & 1) == 0;
+        else if (G == 128) writer = qd == 0;
+        else writer = qd == 0 && ss == 0;
+        if (writer)
+            qparams[(rb * (Kp / G) + k_lane / G) * 16 + r] =
+                (uint32_t)f32_to_bf16_bits(s) | ((uint32_t)f32_to_bf16_bits(zp) << 16);
     }
 }
 
@@ -302,7 +320,7 @@ __global__ __launch_bounds__(256) void int4wo_pack_kernel(const int32_t* __restr
     if (i < ndw) {
         const int sl = i & 3, l = (i >> 2) & 63;
         const int64_t tile = i >> 8, kb = tile % KB, rb = tile / KB;
-        const int64_t row = rb * 16 + (l & 15), k0 = kb * 128 + sl * 32 + (l >> 4) * 8;
+        const int64_t row = rb * 16 + (l & 15), k0 = kb * 128 + (l >> 4) * 32 + sl * 8;
         uint32_t word = 0;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -335,7 +353,7 @@ __global__ __launch_bounds__(256) void int4wo_unpack_kernel(const uint32_t* __re
     if (i < ndw) {
         const int sl = i & 3, l = (i >> 2) & 63;
         const int64_t tile = i >> 8, kb = tile % KB, rb = tile / KB;
-        const int64_t row = rb * 16 + (l & 15), k0 = kb * 128 + sl * 32 + (l >> 4) * 8;
+        const int64_t row = rb * 16 + (l & 15), k0 = kb * 128 + (l >> 4) * 32 + sl * 8;
         const uint32_t word = packed[i];
         if (row < N) {
             if (MODE == 0) {

@@ -68,9 +68,10 @@ int ao_amd_dequantize_affine(const void* in, int in_dtype, int64_t N, int64_t K,
  * pack_tinygemm_scales_and_zeros, torchao/quantization/utils.py:310-322):
  *   Np = N rounded up to 16, Kp = K rounded up to max(128, g)
  *   packed : uint32 [Np/16][Kp/128][64 lanes][4]   lane l: row 16*rb + l%16, quarter qd = l/16;
- *            dword (l, sl) holds k = 128*kb + 32*sl + 8*qd + e (e=0..7) with element e in the nibble at
- *            bit 4*((e>>1) + 4*(e&1))  -- one wave64 16-byte load per lane = 1 KiB contiguous, and the
- *            8 values of a dword land in the k-order of a 16x16x32 bf16 MFMA operand.
+ *            dword (l, sl) holds k = 128*kb + 32*qd + 8*sl + e (e=0..7) with element e in the nibble at
+ *            bit 4*((e>>1) + 4*(e&1))  -- one wave64 16-byte load per lane = 1 KiB contiguous; a lane owns
+ *            32 consecutive k (one group's scale/zero for every supported g) and the 8 values of a dword
+ *            are one lane's share of a 16x16x32 bf16 MFMA operand.
  *   qparams: uint32 [Np/16][Kp/g][16] = scale_bf16 | zero_bf16 << 16
  * Padding holds code 8, scale bf16(1e-6), zero 0, i.e. what quantizing zero padding yields.
  * group size g must be 32, 64, 128 or 256. */

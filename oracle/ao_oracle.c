@@ -321,9 +321,9 @@ int ao_oracle_int4wo_quantize(const void* w, int in_dtype, int64_t N, int64_t K,
  * (affine_quantized_tensor.py:460-465, quantization/utils.py:310-322).
  *
  * codes [Np,Kp], Np % 16 == 0, Kp % 128 == 0.
- *   packed: uint32 [Np/16][Kp/128][64 lanes][4 slices]
+ *   packed: uint32 [Np/16][Kp/128][64 lanes][4 dwords]
  *     lane l -> row 16*rb + (l % 16), quarter qd = l / 16
- *     dword (l, sl) covers k = 128*kb + 32*sl + 8*qd + e, e = 0..7
+ *     dword (l, sl) covers k = 128*kb + 32*qd + 8*sl + e, e = 0..7 (a lane owns 32 consecutive k)
  *     element e sits in the nibble at bit 4*((e >> 1) + 4*(e & 1))
  *   qparams: uint32 [Np/16][Kp/g][16 rows] = scale_bf16 | zero_bf16 << 16
  */
@@ -338,7 +338,7 @@ int ao_oracle_int4wo_pack(const int32_t* codes, const uint16_t* scale, const uin
             for (int l = 0; l < 64; ++l)
                 for (int sl = 0; sl < 4; ++sl) {
                     int64_t row = rb * 16 + (l & 15);
-                    int64_t k0 = kb * 128 + sl * 32 + (l >> 4) * 8;
+                    int64_t k0 = kb * 128 + (l >> 4) * 32 + sl * 8;
                     uint32_t w = 0;
                     for (int e = 0; e < 8; ++e) {
                         int32_t c = codes[row * Kp + k0 + e];
@@ -363,7 +363,7 @@ int ao_oracle_int4wo_unpack(const uint32_t* packed, const uint32_t* qparams, int
     for (int64_t row = 0; row < Np; ++row)
         for (int64_t k = 0; k < Kp; ++k) {
             int64_t rb = row / 16, kb = k / 128;
-            int kk = (int)(k % 128), sl = kk / 32, qd = (kk % 32) / 8, e = kk % 8;
+            int kk = (int)(k % 128), qd = kk / 32, sl = (kk % 32) / 8, e = kk % 8;
             int l = qd * 16 + (int)(row % 16);
             uint32_t w = packed[((rb * KB + kb) * 64 + l) * 4 + sl];
             codes[row * Kp + k] = (int32_t)((w >> (4 * nib_pos(e))) & 15u);
