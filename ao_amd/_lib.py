@@ -41,6 +41,7 @@ _SIGNATURES = {
     "ao_amd_int4wo_unpack": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _p], _int),
     "ao_amd_int4wo_dequantize": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
     "ao_amd_int4wo_linear": ([_p, _i64, _i64, _i64, _p, _p, _i64, _i64, _p, _p, _int, _i64, _p], _int),
+    "ao_amd_profile_next_linear": ([_p, _p], _int),
 }
 
 _lib = None

@@ -15,6 +15,7 @@
 //   u  = T.lo*1 + T.hi*0 + z  /  T.lo*0 + T.hi*1 + z   fp32 add of the bf16 operands  (2 v_dot2_f32_bf16)
 //   W  = cvt_pk_bf16(u0, u1)                           second rounding                (1 v_cvt_pk_bf16_f32)
 #include "common.h"
+#include <hip/hip_ext.h>
 
 namespace ao {
 
@@ -212,8 +213,20 @@ struct LinearArgs {
     const uint16_t* bias; void* y; int y_is_f32; int64_t ldy;
 };
 
+// Optional per-kernel timing: when a (start, stop) event pair has been armed on this thread, the next
+// linear launch records the kernel's own begin / end timestamps into it (hipExtLaunchKernelGGL) and
+// disarms.  hipEventElapsedTime(start, stop) is then the kernel's execution time without launch gaps.
+static thread_local hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;
+
 template <int G, int WAVES, bool FAST>
 static void launch_one(dim3 grid, hipStream_t st, const LinearArgs& a) {
+    if (g_prof_start && g_prof_stop) {
+        hipExtLaunchKernelGGL((int4wo_linear_kernel<G, WAVES, FAST>), grid, dim3(WAVES * 64), 0, st, g_prof_start,
+                              g_prof_stop, 0, a.x, a.M, a.K, a.ldx, a.packed, a.qparams, a.N, a.Kp, a.bias, a.y,
+                              a.y_is_f32, a.ldy);
+        g_prof_start = g_prof_stop = nullptr;
+        return;
+    }
     hipLaunchKernelGGL((int4wo_linear_kernel<G, WAVES, FAST>), grid, dim3(WAVES * 64), 0, st, a.x, a.M, a.K, a.ldx,
                        a.packed, a.qparams, a.N, a.Kp, a.bias, a.y, a.y_is_f32, a.ldy);
 }
@@ -240,6 +253,12 @@ static void launch_group(int64_t g, int waves, dim3 grid, hipStream_t st, const 
 }  // namespace ao
 
 using namespace ao;
+
+extern "C" int ao_amd_profile_next_linear(void* start_event, void* stop_event) {
+    g_prof_start = (hipEvent_t)start_event;
+    g_prof_stop = (hipEvent_t)stop_event;
+    return 0;
+}
 
 extern "C" int ao_amd_int4wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed,
                                     const void* qparams, int64_t N, int64_t g, const void* bias_bf16, void* y,

@@ -1,0 +1,258 @@
+#!/usr/bin/env python3
+"""Headline benchmark: batch-1 greedy decode of a random-init Llama-3-8B-architecture model with
+int4 weight-only (group 64) quantization on every nn.Linear, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decoded token (one pass of every quantized linear over one activation row).  The timed
+region is K replays of the HIP graph of the decode step with all weights resident in HBM, bracketed by
+torch.cuda.synchronize().  One JSON line is printed with:
+  value        tokens/s
+  roofline     the int4wo GEMV kernel over the 161 linear launches of one token: algorithmic bytes
+               (N*K*(1/2 + 4/g) + 2*M*K + 2*M*N per launch) / kernel time, kernel time taken from HIP events
+               that carry each kernel's own begin / end timestamps
+  cpu_baseline the C oracle (dequantize_affine + fp32 linear, 1 thread) timed on one transformer layer's
+               linears and scaled to a whole token
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def int4wo_bytes(N, K, g, M=1):
+    return N * K * (0.5 + 4.0 / g) + 2 * M * K + 2 * M * N
+
+
+def _hip():
+    for name in ("libamdhip64.so.7", "libamdhip64.so"):
+        try:
+            return ctypes.CDLL(name)
+        except OSError:
+            continue
+    raise RuntimeError("HIP runtime not found")
+
+
+class KernelTimer:
+    """HIP event pairs armed on the linear launch: elapsed time = the kernel's own duration."""
+
+    def __init__(self, n):
+        self.hip = _hip()
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+        self.pairs = []
+        for _ in range(n):
+            a, b = ctypes.c_void_p(), ctypes.c_void_p()
+            assert self.hip.hipEventCreate(ctypes.byref(a)) == 0
+            assert self.hip.hipEventCreate(ctypes.byref(b)) == 0
+            self.pairs.append((a, b))
+
+    def elapsed_us(self, i):
+        ms = ctypes.c_float()
+        rc = self.hip.hipEventElapsedTime(ctypes.byref(ms), self.pairs[i][0], self.pairs[i][1])
+        assert rc == 0, f"hipEventElapsedTime failed: {rc}"
+        return ms.value * 1e3
+
+    def close(self):
+        for a, b in self.pairs:
+            self.hip.hipEventDestroy(a)
+            self.hip.hipEventDestroy(b)
+
+
+def quantized_linears(model):
+    """(name, AffineQuantizedTensor) of every int4 linear in execution order of one forward pass."""
+    from ao_amd.dtypes import AffineQuantizedTensor
+
+    out = []
+    for layer_idx, layer in enumerate(model.layers):
+        for name, lin in (("wqkv", layer.attention.wqkv), ("wo", layer.attention.wo), ("w1", layer.feed_forward.w1),
+                          ("w3", layer.feed_forward.w3), ("w2", layer.feed_forward.w2)):
+            out.append((f"layers.{layer_idx}.{name}", lin.weight))
+    out.append(("output", model.output.weight))
+    assert all(isinstance(w, AffineQuantizedTensor) for _, w in out)
+    return out
+
+
+def roofline_leg(model, passes=3):
+    """Time the GEMV kernel alone over the linear launches of one token (M=1), `passes` times."""
+    import torch
+
+    from ao_amd import _lib
+
+    L = _lib.lib()
+    lins = quantized_linears(model)
+    dev = torch.device("cuda:0")
+    timer = KernelTimer(len(lins))
+    st = torch.cuda.current_stream().cuda_stream
+    xs = {}
+    total_bytes = 0.0
+    for _, w in lins:
+        lay = w.layout_tensor
+        if lay.K not in xs:
+            xs[lay.K] = torch.randn(1, lay.K, device=dev).bfloat16()
+        total_bytes += int4wo_bytes(lay.N, lay.K, lay.group_size)
+    ys = {n: torch.empty(1, n, dtype=torch.bfloat16, device=dev) for n in {w.layout_tensor.N for _, w in lins}}
+    best = None
+    for _ in range(passes):
+        for i, (_, w) in enumerate(lins):
+            lay = w.layout_tensor
+            x = xs[lay.K]
+            L.ao_amd_profile_next_linear(timer.pairs[i][0], timer.pairs[i][1])
+            _lib.check(L.ao_amd_int4wo_linear(x.data_ptr(), 1, lay.K, lay.K, lay.packed_weight.data_ptr(),
+                                              lay.scale_and_zero.data_ptr(), lay.N, lay.group_size, None,
+                                              ys[lay.N].data_ptr(), _lib.BF16, lay.N, st))
+        torch.cuda.synchronize()
+        durs = [timer.elapsed_us(i) for i in range(len(lins))]
+        if best is None or sum(durs) < sum(best):
+            best = durs
+    timer.close()
+    total_us = sum(best)
+    achieved = total_bytes / total_us / 1e3  # GB/s
+    return {
+        "bound": "hbm",
+        "kernel": "ao::int4wo_linear_kernel (M=1, g=64)",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "launches": len(lins),
+        "bytes_per_launch": round(total_bytes / len(lins)),
+        "avg_launch_us": round(total_us / len(lins), 3),
+        "traffic": _traffic_from_profile(),
+    }
+
+
+def _traffic_from_profile():
+    """HBM bytes per launch from the committed rocprofv3 --pmc summary, if one exists."""
+    path = os.path.join(ROOT, "profiles", "int4wo_gemv_decode_traffic.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            return json.load(f).get("traffic_bytes_per_launch")
+    return None
+
+
+def cpu_baseline_leg(config, group=64, min_seconds=10.0):
+    """C oracle on one layer's linears (M=1): dequantize_affine + fp32 linear, one thread."""
+    import numpy as np
+
+    import oracle as O
+
+    O.lib()
+    rng = np.random.default_rng(1234)
+    dim, ffn = config.dim, config.intermediate_size
+    qkv = (config.n_head + 2 * config.n_local_heads) * config.head_dim
+    shapes = [(qkv, dim), (dim, dim), (ffn, dim), (ffn, dim), (dim, ffn)]  # (N, K)
+    prepared = []
+    for N, K in shapes:
+        w = O.f32_to_bf16_bits((rng.standard_normal((N, K), dtype=np.float32) * 0.02))
+        codes, scale, zero = O.int4wo_quantize(w, O.BF16, group, N, K)
+        x = O.f32_to_bf16_bits(rng.standard_normal((1, K), dtype=np.float32))
+        prepared.append((codes, scale, zero, x))
+    layer_params = sum(n * k for n, k in shapes)
+    t_layer, reps = 0.0, 0
+    while t_layer < min_seconds and reps < 50:
+        t0 = time.perf_counter()
+        for codes, scale, zero, x in prepared:
+            dq = O.dequantize_affine(codes, O.I32, (1, group), scale, O.BF16, zero, O.BF16, 0, 15, 1, O.BF16)
+            O.linear(x, O.BF16, dq, O.BF16)
+        t_layer += time.perf_counter() - t0
+        reps += 1
+    per_layer = t_layer / reps
+    head_params = config.vocab_size * dim
+    per_token = per_layer * config.n_layer + per_layer * head_params / layer_params
+    return {
+        "value": round(1.0 / per_token, 4),
+        "unit": "tokens/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": (f"C oracle dequantize_affine+fp32 linear (M=1, g={group}) on one transformer layer's five linears "
+                   f"({layer_params / 1e6:.0f}M weights), {reps} repetitions, {per_layer:.2f} s per layer; scaled to "
+                   f"{config.n_layer} layers + vocabulary head"),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--model", default="Llama-3-8B")
+    ap.add_argument("--group", type=int, default=64)
+    ap.add_argument("--prompt-len", type=int, default=128)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-roofline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+
+    from ao_amd._models.llama.generate import GraphedDecoder, build_random_model, prefill
+    from ao_amd._models.llama.model import prepare_inputs_for_model
+    from ao_amd.utils import get_model_size_in_bytes
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    quant = f"int4wo-{args.group}"
+    model = build_random_model(args.model, device, quant)
+    cfg = model.config
+    model_size = get_model_size_in_bytes(model, ignore_embeddings=True)
+
+    gen = torch.Generator(device=device).manual_seed(0)
+    prompt = torch.randint(0, cfg.vocab_size, (args.prompt_len,), device=device, dtype=torch.int, generator=gen)
+    total_len = args.prompt_len + args.warmup + args.steps + 8
+    with torch.no_grad():
+        model.setup_caches(max_batch_size=1, max_seq_length=total_len)
+        x, input_pos = prepare_inputs_for_model(prompt)
+        first = prefill(model, x, input_pos, greedy=True).clone()
+        dec = GraphedDecoder(model, device, greedy=True)
+        dec.capture(first, args.prompt_len)
+        for _ in range(args.warmup):
+            dec.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            dec.step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+
+    tok_s = args.steps / elapsed
+    line = {
+        "metric": "tok/s Llama-3-8B-arch int4wo-64 bs=1; int4 GEMV HBM GB/s vs peak",
+        "value": round(tok_s, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": (f"{args.model}-architecture random-init (weights ~N(0,0.02), seed 1234), {quant} on every "
+                         f"nn.Linear, greedy batch-1 decode after a {args.prompt_len}-token uniform-random prompt, "
+                         "HIP-graph replay per token"),
+            "model_size_bytes": model_size,
+            "model_bandwidth_GBs": round(model_size * tok_s / 1e9, 1),
+        },
+    }
+    if not args.no_roofline:
+        line["roofline"] = roofline_leg(model)
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_leg(cfg, args.group)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

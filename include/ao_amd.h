@@ -109,6 +109,12 @@ int ao_amd_int4wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, 
                          const void* qparams, int64_t N, int64_t g, const void* bias_bf16, void* y, int y_dtype,
                          int64_t ldy, void* stream);
 
+/* Measurement aid (no counterpart in the reference): arm a (hipEvent_t start, hipEvent_t stop) pair on the
+ * calling thread; the next ao_amd_int4wo_linear launch records its kernel's own begin / end timestamps into
+ * the pair and disarms, so hipEventElapsedTime(start, stop) is the kernel duration free of launch gaps.
+ * Pass NULLs to disarm. */
+int ao_amd_profile_next_linear(void* start_event, void* stop_event);
+
 #ifdef __cplusplus
 }
 #endif

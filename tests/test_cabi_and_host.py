@@ -1,0 +1,187 @@
+"""CPU-only checks: the C-ABI library exports every symbol the header declares, and the host logic
+(module walk, layout registry, shape helpers, meta-device quantization, error paths) behaves like the
+reference's.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "ao_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ao_amd_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(cabi):
+    names = _declared_functions()
+    assert len(names) >= 10
+    handle = ctypes.CDLL(cabi.LIB_PATH)
+    for n in names:
+        assert hasattr(handle, n), f"{n} declared in include/ao_amd.h but not exported"
+    assert cabi.lib().ao_amd_abi_version() == 1
+    assert set(cabi._SIGNATURES) == set(names)
+
+
+def test_packed_shape_host_entry(cabi):
+    from ao_amd.ops import int4wo_packed_shapes
+
+    for (N, K, g) in [(4096, 4096, 64), (17, 64, 32), (128256, 4096, 64), (48, 192, 256), (4096, 14336, 128)]:
+        Np, Kp, pb, qb = cabi.packed_shape(N, K, g)
+        assert Np % 16 == 0 and Np >= N and Kp % max(128, g) == 0 and Kp >= K
+        assert pb == Np * Kp // 2 and qb == Np * (Kp // g) * 4
+        ps, qs = int4wo_packed_shapes(N, K, g)
+        assert ps == (Np // 16, Kp // 128, 64, 4) and qs == (Np // 16, Kp // g, 16)
+    L = cabi.lib()
+    assert L.ao_amd_int4wo_packed_shape(16, 128, 48, None, None, None, None) != 0
+    assert b"group_size" in L.ao_amd_last_error()
+
+
+def test_argument_errors_without_launch(cabi):
+    L = cabi.lib()
+    assert L.ao_amd_int4wo_linear(None, 1, 128, 128, None, None, 16, 64, None, None, cabi.BF16, 16, None) != 0
+    assert b"null" in L.ao_amd_last_error()
+    assert L.ao_amd_choose_qparams_affine(None, 0, 4, 4, 4, 1, 4, 1, 0, 15, -1.0, 1, 0, 0, 0, None, None, None) != 0
+
+
+def test_cpu_tensors_are_rejected():
+    """There is no CPU fallback: a CPU tensor raises instead of silently computing somewhere else."""
+    import ao_amd
+    from ao_amd import ops
+    from ao_amd.quantization import MappingType, choose_qparams_affine
+
+    w = torch.randn(32, 128).bfloat16()
+    with pytest.raises(RuntimeError):
+        ops.int4wo_quantize_pack(w, 64)
+    with pytest.raises(RuntimeError):
+        choose_qparams_affine(w, MappingType.ASYMMETRIC, (1, 64), torch.int32, 0, 15)
+    lin = torch.nn.Linear(128, 32, bias=False).bfloat16()
+    with pytest.raises(RuntimeError):
+        ao_amd.quantize_(lin, ao_amd.int4_weight_only(64))
+
+
+def test_quantize_walks_modules_and_respects_filter():
+    import ao_amd
+    from ao_amd.dtypes import AffineQuantizedTensor
+
+    class Toy(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = torch.nn.Linear(256, 64, bias=False)
+            self.inner = torch.nn.Sequential(torch.nn.Linear(64, 128), torch.nn.ReLU(), torch.nn.Linear(128, 32))
+            self.emb = torch.nn.Embedding(10, 256)
+
+    m = Toy().to(device="meta", dtype=torch.bfloat16)
+    out = ao_amd.quantize(m, ao_amd.int4_weight_only(group_size=32))
+    assert out is m
+    assert isinstance(m.a.weight, AffineQuantizedTensor)
+    assert isinstance(m.inner[0].weight, AffineQuantizedTensor) and isinstance(m.inner[2].weight, AffineQuantizedTensor)
+    assert not isinstance(m.emb.weight, AffineQuantizedTensor)
+    assert m.a.weight.shape == (64, 256) and m.a.weight.dtype is torch.bfloat16
+    assert m.a.weight.extended_layout == "gfx950_wave_tiled" and m.a.weight.block_size == (1, 32)
+    assert not m.a.weight.requires_grad
+    lay = m.inner[2].weight.layout_tensor
+    assert lay.packed_weight.shape == (2, 1, 64, 4) and lay.scale_and_zero.shape == (2, 4, 16)
+    # second call: already-quantized weights are skipped
+    before = m.a.weight
+    ao_amd.quantize_(m, ao_amd.int4_weight_only(group_size=32))
+    assert m.a.weight is before
+
+    m2 = Toy().to(device="meta", dtype=torch.bfloat16)
+    ao_amd.quantize_(m2, ao_amd.int4_weight_only(64), filter_fn=lambda mod, fqn: isinstance(mod, torch.nn.Linear) and fqn == "inner.0")
+    assert isinstance(m2.inner[0].weight, AffineQuantizedTensor) and not isinstance(m2.a.weight, AffineQuantizedTensor)
+
+
+def test_subclass_protocol_on_meta():
+    from ao_amd import int4_weight_only
+    from ao_amd.dtypes import AffineQuantizedTensor
+
+    w = torch.empty(64, 256, dtype=torch.bfloat16, device="meta")
+    q = int4_weight_only(64)(w)
+    names, attrs = q.__tensor_flatten__()
+    assert names == ["layout_tensor"]
+    inner_names, inner_attrs = q.layout_tensor.__tensor_flatten__()
+    assert inner_names == ["packed_weight", "scale_and_zero"] and inner_attrs == [64, 256, 64, False]
+    rebuilt_layout = type(q.layout_tensor).__tensor_unflatten__(
+        {n: getattr(q.layout_tensor, n) for n in inner_names}, inner_attrs, None, None)
+    rebuilt = AffineQuantizedTensor.__tensor_unflatten__({"layout_tensor": rebuilt_layout}, attrs, None, None)
+    assert rebuilt.shape == q.shape and rebuilt.block_size == q.block_size
+    # repeated transposes keep the shape bookkeeping right (test/dtypes/test_affine_quantized.py:11-26)
+    t = q.t()
+    assert t.shape == (256, 64) and t.layout_tensor.transposed and t.block_size == (64, 1)
+    tt = t.t()
+    assert tt.shape == (64, 256) and not tt.layout_tensor.transposed
+    d = q.detach()
+    assert isinstance(d, AffineQuantizedTensor) and d.shape == q.shape
+
+
+def test_layout_registry_and_errors():
+    from ao_amd.dtypes.affine_quantized_tensor import (Gfx950WaveTiledAQTLayout, PlainAQTLayout,
+                                                       get_layout_tensor_constructor)
+
+    assert get_layout_tensor_constructor("plain") == PlainAQTLayout.from_plain
+    assert get_layout_tensor_constructor("gfx950_wave_tiled") == Gfx950WaveTiledAQTLayout.from_plain
+    assert get_layout_tensor_constructor("tensor_core_tiled") == Gfx950WaveTiledAQTLayout.from_plain
+    with pytest.raises(ValueError, match="is not supported yet"):
+        get_layout_tensor_constructor("no_such_layout")
+    import ao_amd
+
+    with pytest.raises(ValueError):
+        ao_amd.int4_weight_only(group_size=48)
+
+
+def test_primitive_argument_checks():
+    """Error behaviour of the primitives (test_quant_primitives.py:405-448)."""
+    from ao_amd.quantization import MappingType, ZeroPointDomain, choose_qparams_affine, quantize_affine
+
+    x = torch.empty(10, 256, device="meta")
+    with pytest.raises(ValueError, match="preserve_zero == False is not supported for symmetric quantization"):
+        choose_qparams_affine(x, MappingType.SYMMETRIC, (1, 128), torch.int8, 0, 15, 1e-6, scale_dtype=torch.bfloat16,
+                              zero_point_dtype=torch.bfloat16, preserve_zero=False)
+    s, z = choose_qparams_affine(x, MappingType.ASYMMETRIC, (1, 128), torch.int8)
+    assert s.shape == (10, 2) and z.shape == (10, 2)
+    with pytest.raises(AssertionError, match="Unsupported input dtype:"):
+        quantize_affine(x.to(torch.int32), (1, 128), s, z, torch.int8)
+    with pytest.raises(RuntimeError, match="is invalid for input of size 20"):
+        quantize_affine(x, (1, 1), s, z, torch.int8)
+    with pytest.raises(ValueError, match="Unsupported dtype"):
+        choose_qparams_affine(x, MappingType.ASYMMETRIC, (1, 128), torch.float64)
+    with pytest.raises(AssertionError, match="quant_max out of bound"):
+        choose_qparams_affine(x, MappingType.ASYMMETRIC, (1, 128), torch.int8, 0, 1000)
+    q = quantize_affine(x, (1, 128), s, z, torch.int8, zero_point_domain=ZeroPointDomain.INT)
+    assert q.shape == x.shape and q.dtype is torch.int8
+
+
+def test_block_mapping_and_helpers():
+    from ao_amd.quantization.quant_primitives import _as_2d_blocks, _get_reduction_params, _qparam_shape
+    from ao_amd.utils import find_multiple, get_model_size_in_bytes
+
+    assert _get_reduction_params((3, 3, 2, 10), (3, 3, 10, 10)) == ([3, 3, 5, 2, 10], [0, 1, 3, 4])
+    assert _qparam_shape((1, 64), (8, 256)) == [8, 4]
+    assert _as_2d_blocks((1, 64), (8, 256)) == (8, 256, 1, 64)
+    assert _as_2d_blocks((8, 256), (8, 256)) == (8, 256, 8, 256)
+    assert _as_2d_blocks((1, 1, 32), (2, 4, 64)) == (16, 32, 1, 32)
+    assert _as_2d_blocks((1, 4, 64), (2, 4, 64)) == (2, 256, 1, 256)
+    assert _as_2d_blocks((2, 4, 64), (2, 4, 64)) == (1, 512, 1, 512)
+    with pytest.raises(NotImplementedError):
+        _as_2d_blocks((2, 1, 64), (2, 4, 64))
+    assert find_multiple(4096, 1024) == 4096 and find_multiple(100, 8) == 104 and find_multiple(3, 2, 5) == 10
+    m = torch.nn.Sequential(torch.nn.Embedding(10, 8), torch.nn.Linear(8, 4, bias=False))
+    assert get_model_size_in_bytes(m) == (80 + 32) * 4 and get_model_size_in_bytes(m, ignore_embeddings=True) == 32 * 4
+
+
+def test_llama_model_shapes_on_meta():
+    from ao_amd._models.llama.model import ModelArgs, Transformer
+
+    cfg = ModelArgs.from_name("Llama-3-8B")
+    assert (cfg.n_layer, cfg.dim, cfg.n_head, cfg.n_local_heads, cfg.intermediate_size, cfg.vocab_size,
+            cfg.head_dim) == (32, 4096, 32, 8, 14336, 128256, 128)
+    with torch.device("meta"):
+        m = Transformer(cfg)
+    n_lin = sum(p.numel() for name, p in m.named_parameters() if p.dim() == 2 and "tok_embeddings" not in name)
+    assert n_lin == 7_504_658_432  # linear weights per decoded token
+    assert m.layers[0].attention.wqkv.weight.shape == (6144, 4096)
