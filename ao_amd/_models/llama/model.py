@@ -29,6 +29,9 @@ transformer_configs = {
     # two-layer model of Llama-3-8B width for smoke tests
     "Llama-3-8B-2L": dict(block_size=8192, n_layer=2, n_head=32, n_local_heads=8, dim=4096, intermediate_size=14336,
                           vocab_size=128256),
+    # small model with the head size of the fused decode kernels
+    "tiny128": dict(block_size=512, n_layer=2, n_head=4, n_local_heads=2, dim=512, intermediate_size=1024,
+                    vocab_size=1024),
     "tiny": dict(block_size=256, n_layer=2, n_head=4, n_local_heads=2, dim=256, intermediate_size=512, vocab_size=512),
 }
 
@@ -183,6 +186,8 @@ class Transformer(nn.Module):
         self.causal_mask: Optional[Tensor] = None
         self.max_batch_size = -1
         self.max_seq_length = -1
+        # single-token batch-1 steps go through the fused HIP decode path whenever the model qualifies
+        self.use_fused_decode = True
 
     @classmethod
     def from_name(cls, name: str):
@@ -202,8 +207,62 @@ class Transformer(nn.Module):
                                               dtype, device)
         self.causal_mask = torch.tril(torch.ones(max_seq_length, max_seq_length, dtype=torch.bool, device=device))
 
+    def fused_decode_ready(self) -> bool:
+        """True when a batch-1 single-token step can run on the fused HIP path: every linear is an int4
+        weight in the gfx950 layout with one group size, bf16 everywhere, head_dim 128, caches set up."""
+        from ...dtypes.affine_quantized_tensor import AffineQuantizedTensor, Gfx950WaveTiledAQTLayout
+
+        if self.freqs_cis is None or self.max_batch_size != 1 or self.config.head_dim != 128 \
+                or self.max_seq_length > 8192:
+            return False
+        lins = [self.output] + [m for b in self.layers for m in (b.attention.wqkv, b.attention.wo, b.feed_forward.w1,
+                                                                  b.feed_forward.w3, b.feed_forward.w2)]
+        groups = set()
+        for lin in lins:
+            w = lin.weight
+            if lin.bias is not None or not isinstance(w, AffineQuantizedTensor) or w.dtype is not torch.bfloat16:
+                return False
+            lay = w.layout_tensor
+            if not isinstance(lay, Gfx950WaveTiledAQTLayout) or lay.transposed or not w.is_cuda:
+                return False
+            groups.add(lay.group_size)
+        return len(groups) == 1 and self.tok_embeddings.weight.dtype is torch.bfloat16
+
+    def _fused_decode(self, idx: Tensor, input_pos: Tensor) -> Tensor:
+        """One token, batch 1: seven launches per layer (norm, qkv, attention, wo + residual, norm,
+        gate/up + SwiGLU, down + residual).  Same roundings as the module-by-module path."""
+        from ... import ops
+
+        cfg = self.config
+
+        def lin(x, layer, residual=None):
+            lay = layer.weight.layout_tensor
+            if residual is None:
+                return ops.int4wo_linear(x, lay.packed_weight, lay.scale_and_zero, lay.group_size, lay.N)
+            return ops.int4wo_linear_residual(x, lay.packed_weight, lay.scale_and_zero, lay.group_size, lay.N, residual)
+
+        x = self.tok_embeddings(idx).view(1, cfg.dim)
+        pos = input_pos.to(torch.int32) if input_pos.dtype is not torch.int32 else input_pos
+        for b in self.layers:
+            att = b.attention
+            xn = ops.rmsnorm(x, b.attention_norm.weight, b.attention_norm.eps)
+            qkv = lin(xn, att.wqkv)
+            y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
+                                           cfg.n_head, cfg.n_local_heads)
+            h = lin(y, att.wo, residual=x)
+            hn = ops.rmsnorm(h, b.ffn_norm.weight, b.ffn_norm.eps)
+            g, u = b.feed_forward.w1.weight.layout_tensor, b.feed_forward.w3.weight.layout_tensor
+            ff = ops.int4wo_swiglu(hn, g.packed_weight, g.scale_and_zero, u.packed_weight, u.scale_and_zero,
+                                   g.group_size, g.N)
+            x = lin(ff, b.feed_forward.w2, residual=h)
+        xn = ops.rmsnorm(x, self.norm.weight, self.norm.eps)
+        return lin(xn, self.output).view(1, 1, cfg.vocab_size)
+
     def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None) -> Tensor:
         assert self.freqs_cis is not None, "Caches must be initialized first"
+        if self.use_fused_decode and idx.numel() == 1 and input_pos is not None and input_pos.numel() == 1 \
+                and self.fused_decode_ready():
+            return self._fused_decode(idx, input_pos)
         mask = self.causal_mask[None, None, input_pos]
         freqs_cis = self.freqs_cis[input_pos]
         x = self.tok_embeddings(idx)

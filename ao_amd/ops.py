@@ -12,6 +12,10 @@ from . import _lib
 from ._lib import BF16, DTYPE_CODE, F32, check, current_stream, lib, require_cuda
 
 __all__ = [
+    "int4wo_linear_residual",
+    "int4wo_swiglu",
+    "rmsnorm",
+    "llama_decode_attention",
     "int4wo_quantize_pack",
     "int4wo_pack",
     "int4wo_unpack",
@@ -26,6 +30,10 @@ _LIB.define("int4wo_pack(Tensor codes, Tensor scale, Tensor zero_point, int grou
 _LIB.define("int4wo_unpack(Tensor packed, Tensor qparams, int N, int K, int group_size) -> (Tensor, Tensor, Tensor)")
 _LIB.define("int4wo_dequantize(Tensor packed, Tensor qparams, int N, int K, int group_size) -> Tensor")
 _LIB.define("int4wo_linear(Tensor x, Tensor packed, Tensor qparams, int group_size, int N, Tensor? bias, bool fp32_out) -> Tensor")
+_LIB.define("int4wo_linear_residual(Tensor x, Tensor packed, Tensor qparams, int group_size, int N, Tensor? bias, Tensor residual) -> Tensor")
+_LIB.define("int4wo_swiglu(Tensor x, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
+_LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
+_LIB.define("llama_decode_attention(Tensor qkv, Tensor freqs_cis, Tensor input_pos, Tensor(a!) k_cache, Tensor(b!) v_cache, int n_head, int n_kv) -> Tensor")
 
 
 def int4wo_packed_shapes(N: int, K: int, group_size: int):
@@ -122,6 +130,76 @@ def _linear_cuda(x: Tensor, packed: Tensor, qparams: Tensor, group_size: int, N:
     return y
 
 
+def _linear_residual_cuda(x, packed, qparams, group_size, N, bias, residual):
+    require_cuda(x, packed, qparams, bias, residual)
+    torch._check(x.dim() == 2 and x.dtype is torch.bfloat16, lambda: "input must be a 2d bfloat16 tensor")
+    M, K = x.shape
+    _check_packed(packed, qparams, N, K, group_size)
+    torch._check(residual.dtype is torch.bfloat16 and tuple(residual.shape) == (M, N) and residual.stride(1) == 1,
+                 lambda: f"residual must be bfloat16 [{M}, {N}] with unit inner stride")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    if bias is not None:
+        torch._check(bias.dtype is torch.bfloat16 and bias.numel() == N, lambda: "bias must be bfloat16 of size N")
+        bias = bias.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    check(lib().ao_amd_int4wo_linear_residual(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, packed.data_ptr(),
+                                              qparams.data_ptr(), N, group_size,
+                                              None if bias is None else bias.data_ptr(), residual.data_ptr(),
+                                              residual.stride(0), y.data_ptr(), N, current_stream(x.device)))
+    return y
+
+
+def _swiglu_cuda(x, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
+    require_cuda(x, packed_gate, qparams_gate, packed_up, qparams_up)
+    torch._check(x.dim() == 2 and x.dtype is torch.bfloat16, lambda: "input must be a 2d bfloat16 tensor")
+    M, K = x.shape
+    _check_packed(packed_gate, qparams_gate, N, K, group_size)
+    _check_packed(packed_up, qparams_up, N, K, group_size)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    check(lib().ao_amd_int4wo_swiglu(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, packed_gate.data_ptr(),
+                                     qparams_gate.data_ptr(), packed_up.data_ptr(), qparams_up.data_ptr(), N, group_size,
+                                     y.data_ptr(), N, current_stream(x.device)))
+    return y
+
+
+def _rmsnorm_cuda(x, weight, eps):
+    require_cuda(x, weight)
+    torch._check(x.dtype is torch.bfloat16 and weight.dtype is torch.bfloat16, lambda: "rmsnorm needs bfloat16 tensors")
+    dim = x.shape[-1]
+    torch._check(weight.numel() == dim, lambda: "weight size does not match the last dimension")
+    xc = x.contiguous()
+    out = torch.empty_like(xc)
+    check(lib().ao_amd_rmsnorm_bf16(xc.data_ptr(), weight.contiguous().data_ptr(), xc.numel() // dim, dim, float(eps),
+                                    out.data_ptr(), current_stream(x.device)))
+    return out
+
+
+def _decode_attention_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv):
+    require_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache)
+    torch._check(qkv.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16 and v_cache.dtype is torch.bfloat16
+                 and freqs_cis.dtype is torch.bfloat16, lambda: "decode attention needs bfloat16 tensors")
+    torch._check(input_pos.dtype is torch.int32 and input_pos.numel() == 1, lambda: "input_pos must be one int32")
+    torch._check(k_cache.dim() == 4 and k_cache.shape[0] == 1 and k_cache.shape[1] == n_kv and k_cache.is_contiguous()
+                 and v_cache.shape == k_cache.shape and v_cache.is_contiguous(),
+                 lambda: "caches must be contiguous [1, n_kv, max_seq, head_dim]")
+    head_dim, max_seq = k_cache.shape[3], k_cache.shape[2]
+    torch._check(qkv.numel() == (n_head + 2 * n_kv) * head_dim and qkv.is_contiguous(),
+                 lambda: "qkv must be the contiguous fused projection of one token")
+    torch._check(freqs_cis.is_contiguous() and freqs_cis.shape[-2:] == (head_dim // 2, 2), lambda: "bad freqs_cis shape")
+    out = torch.empty((1, n_head * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    check(lib().ao_amd_llama_decode_attention(qkv.data_ptr(), freqs_cis.data_ptr(), input_pos.data_ptr(),
+                                              k_cache.data_ptr(), v_cache.data_ptr(), n_head, n_kv, head_dim, max_seq,
+                                              out.data_ptr(), current_stream(qkv.device)))
+    return out
+
+
+_LIB.impl("int4wo_linear_residual", _linear_residual_cuda, "CUDA")
+_LIB.impl("int4wo_swiglu", _swiglu_cuda, "CUDA")
+_LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
+_LIB.impl("llama_decode_attention", _decode_attention_cuda, "CUDA")
 _LIB.impl("int4wo_quantize_pack", _quantize_pack_cuda, "CUDA")
 _LIB.impl("int4wo_pack", _pack_cuda, "CUDA")
 _LIB.impl("int4wo_unpack", _unpack_cuda, "CUDA")
@@ -135,7 +213,8 @@ def _no_cpu(name):
     return impl
 
 
-for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear"):
+for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
+              "int4wo_linear_residual", "int4wo_swiglu", "rmsnorm", "llama_decode_attention"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
 
@@ -175,7 +254,47 @@ def _(x, packed, qparams, group_size, N, bias, fp32_out):
     return x.new_empty((x.shape[0], N), dtype=torch.float32 if fp32_out else torch.bfloat16)
 
 
+@torch.library.register_fake("torchao::int4wo_linear_residual")
+def _(x, packed, qparams, group_size, N, bias, residual):
+    return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::int4wo_swiglu")
+def _(x, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
+    return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::rmsnorm")
+def _(x, weight, eps):
+    return torch.empty_like(x)
+
+
+@torch.library.register_fake("torchao::llama_decode_attention")
+def _(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv):
+    return qkv.new_empty((1, n_head * k_cache.shape[3]))
+
+
 # ------------------------------------------------------------------------------------ python wrappers
+
+def int4wo_linear_residual(x, packed, qparams, group_size, N, residual, bias=None):
+    """bf16( bf16(x W^T + bias) + residual ) in one launch."""
+    return torch.ops.torchao.int4wo_linear_residual.default(x, packed, qparams, group_size, N, bias, residual)
+
+
+def int4wo_swiglu(x, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
+    """silu(x W_gate^T) * (x W_up^T) in one launch (both weights [N,K], same group size)."""
+    return torch.ops.torchao.int4wo_swiglu.default(x, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N)
+
+
+def rmsnorm(x, weight, eps: float):
+    """RMSNorm over the last dimension of a bf16 tensor."""
+    return torch.ops.torchao.rmsnorm.default(x, weight, eps)
+
+
+def llama_decode_attention(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head: int, n_kv: int):
+    """RoPE + KV-cache update + attention of one new token (batch 1).  Writes the caches in place."""
+    return torch.ops.torchao.llama_decode_attention.default(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv)
+
 
 def int4wo_quantize_pack(w: Tensor, group_size: int):
     """Fused choose_qparams + quantize + pack of a bf16 weight [N,K] -> (packed int32, qparams int32)."""

@@ -109,6 +109,33 @@ int ao_amd_int4wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, 
                          const void* qparams, int64_t N, int64_t g, const void* bias_bf16, void* y, int y_dtype,
                          int64_t ldy, void* stream);
 
+/* Same product with fused epilogues, used by the decode loop so that a token costs few launches.
+ * y = bf16( bf16(x W^T + bias) + residual ): F.linear followed by the residual add of TransformerBlock.forward,
+ * torchao/_models/llama/model.py:160-163. */
+int ao_amd_int4wo_linear_residual(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed,
+                                  const void* qparams, int64_t N, int64_t g, const void* bias_bf16,
+                                  const void* residual_bf16, int64_t ldres, void* y_bf16, int64_t ldy, void* stream);
+
+/* y = silu(x W_gate^T) * (x W_up^T) with the bf16 roundings of the module chain: FeedForward.forward,
+ * torchao/_models/llama/model.py:221-222 (w1 = gate, w3 = up).  Both weights [N,K], same group size. */
+int ao_amd_int4wo_swiglu(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed_gate,
+                         const void* qparams_gate, const void* packed_up, const void* qparams_up, int64_t N, int64_t g,
+                         void* y_bf16, int64_t ldy, void* stream);
+
+/* ---------------------------------------------------------------- Llama decode harness kernels (bf16)
+ * out[rows,dim] = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * weight ): RMSNorm.forward,
+ * torchao/_models/llama/model.py:232-244. */
+int ao_amd_rmsnorm_bf16(const void* x, const void* weight, int64_t rows, int64_t dim, float eps, void* out,
+                        void* stream);
+
+/* One new token, batch 1: rotary embedding of q and k, KV-cache update at *pos_dev, grouped-query attention over
+ * positions 0..*pos_dev.  Attention.forward, torchao/_models/llama/model.py:190-211 with apply_rotary_emb :250-266
+ * and KVCache.update :85-98.  qkv: [(n_head + 2 n_kv) * head_dim] (fused wqkv output); freqs_cis: [*, head_dim/2, 2]
+ * (cos, sin); caches: [n_kv, max_seq, head_dim]; out: [n_head * head_dim].  head_dim must be 128, max_seq <= 8192. */
+int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* freqs_cis_bf16, const int32_t* pos_dev,
+                                  void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim, int64_t max_seq,
+                                  void* out_bf16, void* stream);
+
 /* Measurement aid (no counterpart in the reference): arm a (hipEvent_t start, hipEvent_t stop) pair on the
  * calling thread; the next ao_amd_int4wo_linear launch records its kernel's own begin / end timestamps into
  * the pair and disarms, so hipEventElapsedTime(start, stop) is the kernel duration free of launch gaps.

@@ -1,0 +1,139 @@
+"""GPU tests of the decode-loop kernels: fused epilogues of the int4 linear (bit-exact against the
+plain kernel + the module's rounding chain), RMSNorm and decode attention (floating point: compared with a
+plain PyTorch fp32 restatement of the module, tolerances stated per test), and the fused decode step
+against the module-by-module forward."""
+import numpy as np
+import pytest
+import torch
+
+from _util import bits16, make_act, make_weight, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    assert torch.cuda.is_available()
+    return torch.device("cuda:0")
+
+
+def _rb(a):
+    """numpy fp32 -> bf16 (round to nearest even) -> fp32."""
+    import oracle as O
+
+    return O.bf16_bits_to_f32(O.f32_to_bf16_bits(a))
+
+
+@pytest.mark.parametrize("M", [1, 3])
+def test_linear_residual_epilogue(M):
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K, g = 256, 1024, 64
+    w = make_weight(N, K, seed=21).to(dev)
+    x = make_act(M, K, seed=22).to(dev)
+    res = make_act(M, N, seed=23).to(dev)
+    bias = (torch.randn(N) * 0.1).bfloat16().to(dev)
+    packed, qp = ops.int4wo_quantize_pack(w, g)
+    y32 = ops.int4wo_linear(x, packed, qp, g, N, bias, True).cpu().numpy()
+    y = ops.int4wo_linear_residual(x, packed, qp, g, N, res, bias)
+    expect = _rb(_rb(y32) + res.float().cpu().numpy())
+    assert np.array_equal(y.float().cpu().numpy(), expect)
+
+
+@pytest.mark.parametrize("M", [1, 5])
+def test_swiglu_epilogue(M):
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K, g = 512, 1024, 64
+    wg = make_weight(N, K, seed=31).to(dev)
+    wu = make_weight(N, K, seed=32).to(dev)
+    x = make_act(M, K, seed=33).to(dev)
+    pg, qg = ops.int4wo_quantize_pack(wg, g)
+    pu, qu = ops.int4wo_quantize_pack(wu, g)
+    a = ops.int4wo_linear(x, pg, qg, g, N, None, False)   # bf16, as the module chain produces
+    b = ops.int4wo_linear(x, pu, qu, g, N, None, False)
+    expect = (torch.nn.functional.silu(a) * b).float().cpu().numpy()
+    y = ops.int4wo_swiglu(x, pg, qg, pu, qu, g, N).float().cpu().numpy()
+    # same roundings as the chain; expf on the device may differ from torch's by an ulp on rare elements
+    mism = np.count_nonzero(y != expect)
+    assert mism <= 0.002 * y.size, f"{mism} of {y.size} elements differ"
+    assert rel_l2(y, expect) <= 1e-3
+
+
+def test_rmsnorm_matches_module():
+    from ao_amd import ops
+    from ao_amd._models.llama.model import RMSNorm
+
+    dev = _dev()
+    torch.manual_seed(3)
+    x = (torch.randn(3, 4096) * 2).bfloat16().to(dev)
+    norm = RMSNorm(4096, 1e-5).to(dev).bfloat16()
+    norm.weight.data = (1 + 0.1 * torch.randn(4096)).bfloat16().to(dev)
+    with torch.no_grad():
+        ref = norm(x).float().cpu().numpy()
+        out = ops.rmsnorm(x, norm.weight, norm.eps).float().cpu().numpy()
+    # fp32 statistics summed in a different order: at most one bf16 ulp on a few elements
+    assert rel_l2(out, ref) <= 2e-3
+    assert np.count_nonzero(out != ref) <= 0.02 * out.size
+
+
+@pytest.mark.parametrize("pos", [0, 5, 130])
+def test_decode_attention_matches_module_math(pos):
+    """fp32 restatement of Attention.forward for one token (RoPE on interleaved pairs, cache update,
+    GQA softmax attention); tolerance 1e-2 relative L2 (bf16 inputs and output)."""
+    from ao_amd import ops
+    from ao_amd._models.llama.model import apply_rotary_emb, precompute_freqs_cis
+
+    dev = _dev()
+    torch.manual_seed(pos)
+    n_head, n_kv, hd, S = 8, 2, 128, 256
+    qkv = torch.randn(1, (n_head + 2 * n_kv) * hd).bfloat16().to(dev)
+    freqs = precompute_freqs_cis(512, hd, 10000, torch.bfloat16, dev)
+    k_cache = torch.randn(1, n_kv, S, hd).bfloat16().to(dev)
+    v_cache = torch.randn(1, n_kv, S, hd).bfloat16().to(dev)
+    kc, vc = k_cache.clone(), v_cache.clone()
+    p = torch.tensor([pos], dtype=torch.int32, device=dev)
+    out = ops.llama_decode_attention(qkv, freqs, p, kc, vc, n_head, n_kv)
+
+    q, k, v = qkv.view(1, 1, -1).split([n_head * hd, n_kv * hd, n_kv * hd], dim=-1)
+    fc = freqs[p.long()]
+    q = apply_rotary_emb(q.view(1, 1, n_head, hd), fc).transpose(1, 2)
+    k = apply_rotary_emb(k.view(1, 1, n_kv, hd), fc).transpose(1, 2)
+    v = v.view(1, 1, n_kv, hd).transpose(1, 2)
+    k_ref, v_ref = k_cache.clone(), v_cache.clone()
+    k_ref[:, :, pos] = k[:, :, 0]
+    v_ref[:, :, pos] = v[:, :, 0]
+    assert torch.equal(kc, k_ref) and torch.equal(vc, v_ref), "cache rows written by the kernel differ"
+    kk = k_ref[:, :, : pos + 1].repeat_interleave(n_head // n_kv, dim=1).float()
+    vv = v_ref[:, :, : pos + 1].repeat_interleave(n_head // n_kv, dim=1).float()
+    att = torch.softmax((q.float() @ kk.transpose(-1, -2)) / hd**0.5, dim=-1) @ vv
+    ref = att.transpose(1, 2).reshape(1, n_head * hd).cpu().numpy()
+    assert rel_l2(out.float().cpu().numpy(), ref) <= 1e-2
+
+
+def test_fused_decode_step_matches_module_path():
+    """One decode step of a small quantized model: fused HIP path vs module-by-module forward, same cache
+    state.  bf16 model, different summation orders: logits agree to 3e-2 relative L2 and pick the same token."""
+    from ao_amd._models.llama.generate import build_random_model, generate
+
+    dev = _dev()
+    model = build_random_model("tiny128", dev, "int4wo-64")
+    prompt = torch.randint(0, model.config.vocab_size, (12,), device=dev, dtype=torch.int)
+    with torch.no_grad():
+        model.setup_caches(1, 64)
+        assert model.fused_decode_ready()
+        pos = torch.arange(12, device=dev)
+        model(prompt.view(1, -1), pos)  # prefill fills the caches
+        tok = torch.tensor([[7]], device=dev, dtype=torch.int)
+        p = torch.tensor([12], device=dev, dtype=torch.int)
+        model.use_fused_decode = False
+        ref = model(tok, p).float()
+        model.use_fused_decode = True
+        out = model(tok, p).float()
+    assert out.shape == ref.shape == (1, 1, model.config.vocab_size)
+    assert rel_l2(out.cpu().numpy(), ref.cpu().numpy()) <= 3e-2
+    # whole generation: graph replay of the fused path vs eager fused path
+    a = generate(model, prompt, 10, use_graph=True, greedy=True)
+    b = generate(model, prompt, 10, use_graph=False, greedy=True)
+    assert torch.equal(a, b)
