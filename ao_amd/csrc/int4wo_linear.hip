@@ -19,6 +19,10 @@
 
 namespace ao {
 
+#ifndef AO_MFMA_ADD
+#define AO_MFMA_ADD 1
+#endif
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
@@ -89,6 +93,81 @@ __device__ __forceinline__ bf16x8_t dequant8(uint32_t w, const GroupConst& g, ui
     return out.v;
 }
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// The dequantization of a dword (8 codes) runs as a three-stage software pipeline so that the VALU and the
+// matrix core overlap; each stage is one asm volatile block (volatile blocks keep their program order, which
+// is what carries the dependency distances the hardware needs):
+//
+//   stage 1  first_half   VALU: 8 codes -> T = bf16((q-8)*s) as 4 packed pairs       (19 instructions)
+//   stage 2  add_zero     MFMA x2: u = T + z for the lane's own 8 values, in fp32.  With B = T (lane (row, qd)
+//                         holds kk = 8*qd + e) and the 0/1 selection matrices sel_a[i][kk] = (kk == 8*(i/4) + i%4),
+//                         sel_b = the same + 4, the 16x16 results C[i][row] = T[row][8*(i/4) + i%4 (+4)] + z land
+//                         back in the lane they came from (the C layout gives lane (row, qd') the rows
+//                         i = 4*qd' + r): the matrix core does the bf16 -> fp32 unpack and the add.
+//   stage 3  round_pack   VALU: W = bf16(u) as 4 packed pairs = the MFMA B operand     (4 instructions)
+//
+// A 4-pass MFMA result may be read by the VALU 7 issue slots later at the earliest; the caller puts stage 1
+// of the NEXT dword between stage 2 and stage 3 of the current one, which fills those slots with useful work.
+__device__ __forceinline__ u32x4_t first_half(uint32_t w, const GroupConst& g, uint32_t magic) {
+    uint32_t p0, p1, p2, p3;
+    float a0, a1, a2, a3, a4, a5, a6, a7;
+    asm volatile(
+        "v_and_or_b32 %[p0], %[w], %[mask], %[magic]\n\t"
+        "v_lshrrev_b32 %[p1], 4, %[w]\n\t"
+        "v_lshrrev_b32 %[p2], 8, %[w]\n\t"
+        "v_lshrrev_b32 %[p3], 12, %[w]\n\t"
+        "v_and_or_b32 %[p1], %[p1], %[mask], %[magic]\n\t"
+        "v_and_or_b32 %[p2], %[p2], %[mask], %[magic]\n\t"
+        "v_and_or_b32 %[p3], %[p3], %[mask], %[magic]\n\t"
+        "v_dot2_f32_bf16 %[a0], %[p0], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a1], %[p0], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a2], %[p1], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a3], %[p1], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a4], %[p2], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a5], %[p2], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a6], %[p3], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a7], %[p3], %[shi], %[c]\n\t"
+        "v_cvt_pk_bf16_f32 %[p0], %[a0], %[a1]\n\t"
+        "v_cvt_pk_bf16_f32 %[p1], %[a2], %[a3]\n\t"
+        "v_cvt_pk_bf16_f32 %[p2], %[a4], %[a5]\n\t"
+        "v_cvt_pk_bf16_f32 %[p3], %[a6], %[a7]\n\t"
+        "s_nop 1"
+        : [p0] "=&v"(p0), [p1] "=&v"(p1), [p2] "=&v"(p2), [p3] "=&v"(p3), [a0] "=&v"(a0), [a1] "=&v"(a1),
+          [a2] "=&v"(a2), [a3] "=&v"(a3), [a4] "=&v"(a4), [a5] "=&v"(a5), [a6] "=&v"(a6), [a7] "=&v"(a7)
+        : [w] "v"(w), [mask] "s"(0x000F000Fu), [magic] "v"(magic), [slo] "v"(g.s_lo), [shi] "v"(g.s_hi),
+          [c] "v"(g.c136));
+    const u32x4_t t = {p0, p1, p2, p3};
+    return t;
+}
+
+__device__ __forceinline__ void add_zero(u32x4_t t, const f32x4_t& zz, u32x4_t sel_a, u32x4_t sel_b, f32x4_t& ua,
+                                         f32x4_t& ub) {
+    // s_nop: a VGPR written by the VALU (the compiler may have just built zz) needs 2 idle slots before an MFMA reads it
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_mfma_f32_16x16x32_bf16 %[ua], %[sa], %[t], %[zz]\n\t"
+        "v_mfma_f32_16x16x32_bf16 %[ub], %[sb], %[t], %[zz]"
+        : [ua] "=&v"(ua), [ub] "=&v"(ub)
+        : [sa] "v"(sel_a), [sb] "v"(sel_b), [t] "v"(t), [zz] "v"(zz));
+}
+
+template <bool WAIT>
+__device__ __forceinline__ bf16x8_t round_pack(const f32x4_t& ua, const f32x4_t& ub) {
+    union { uint32_t u[4]; bf16x8_t v; } out;
+    if (WAIT) asm volatile("s_nop 7");  // nothing was overlapped: sit out the MFMA result latency
+    asm volatile(
+        "v_cvt_pk_bf16_f32 %[o0], %[a0], %[a1]\n\t"
+        "v_cvt_pk_bf16_f32 %[o1], %[a2], %[a3]\n\t"
+        "v_cvt_pk_bf16_f32 %[o2], %[b0], %[b1]\n\t"
+        "v_cvt_pk_bf16_f32 %[o3], %[b2], %[b3]\n\t"
+        "s_nop 1"
+        : [o0] "=&v"(out.u[0]), [o1] "=&v"(out.u[1]), [o2] "=&v"(out.u[2]), [o3] "=&v"(out.u[3])
+        : [a0] "v"(ua[0]), [a1] "v"(ua[1]), [a2] "v"(ua[2]), [a3] "v"(ua[3]), [b0] "v"(ub[0]), [b1] "v"(ub[1]),
+          [b2] "v"(ub[2]), [b3] "v"(ub[3]));
+    return out.v;
+}
+
 // Activation fragment for the slow path: 8 consecutive bf16 of row m starting at k (zeros outside
 // [0,M) x [0,K)), tolerant of any alignment.
 __device__ __forceinline__ uint4 load_x8_checked(const uint16_t* __restrict__ x, int64_t ldx, int64_t m, int64_t M,
@@ -102,14 +181,6 @@ __device__ __forceinline__ uint4 load_x8_checked(const uint16_t* __restrict__ x,
     }
     return r.q;
 }
-
-struct TileBuf {
-    uint4 w;      // 32 codes of this lane: k = 128*kb + 32*qd + 0..31
-    uint32_t q;   // (scale, zero) of the lane's group
-    uint4 w2;     // same for the second weight (SwiGLU pair) when DUAL
-    uint32_t q2;
-    uint4 x[4];   // activations of row m = lane%16 for the same 32 k (zero for rows >= M)
-};
 
 struct LinearArgs {
     const uint16_t* x; int64_t M, K, ldx;
@@ -126,25 +197,101 @@ __device__ __forceinline__ float silu_bf16(float a) {
     return rne_bf16(a / (1.0f + expf(-a)));
 }
 
+// How a wave gets its activation fragments (MFMA A operand: row m = lane%16, 8 consecutive k):
+constexpr int X_GLOBAL = 0;   // 16-byte global loads, prefetched with the weight tile (K % 128 == 0, aligned rows)
+constexpr int X_CHECKED = 1;  // element-wise global loads with bounds checks (any K, any alignment)
+constexpr int X_LDS = 2;      // the workgroup stages its <= 16 activation rows in LDS once (small M x K)
+
+template <int XMODE, bool DUAL>
+struct TileBuf {
+    u32x4_t w;    // 32 codes of this lane: k = 128*kb + 32*qd + 0..31
+    uint32_t q;   // (scale, zero) of the lane's group
+    u32x4_t w2;   // same for the second weight (SwiGLU pair) when DUAL
+    uint32_t q2;
+    uint4 x[4];   // activations for the same 32 k (zero for rows >= M)
+};
+
+// Weight-stream loads of the X_LDS path are issued from inline asm and waited for with explicit vmcnt counts.
+// The compiler cannot keep a precise count across the conditional loads of the register ring and falls back to
+// vmcnt(0), i.e. it would drain every prefetch before each tile.  The wait block takes the loaded registers as
+// in/out operands, so no consumer of them can be scheduled above the wait.
+// scalar base (SGPR pair) + 32-bit per-lane byte offset: the per-tile address update is one scalar add
+__device__ __forceinline__ u32x4_t asm_load_b128_nt(const void* sbase, uint32_t voff) {
+    u32x4_t v;
+    asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    return v;
+}
+__device__ __forceinline__ uint32_t asm_load_b32(const void* sbase, uint32_t voff) {
+    uint32_t v;
+    asm volatile("global_load_dword %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    return v;
+}
+// Wait until at most `younger_tiles` tiles' worth of loads are outstanding (loads return in order, so the
+// tile requested before them has arrived).  The block has no register operands: every consumer of loaded
+// registers is itself an asm volatile block (make_group_asm, first_half), and volatile blocks stay in order.
+template <int LPT>
+__device__ __forceinline__ void wait_tiles(int younger_tiles) {
+    if (younger_tiles >= 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LPT) : "memory");
+    else if (younger_tiles == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPT) : "memory");
+    else if (younger_tiles == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// Group constants + the broadcast zero point (stage-2 C operand) from a loaded (scale, zero) word, as an asm
+// volatile block so that it cannot move above the wait for that word.
+struct GroupRegs {
+    GroupConst g;
+    f32x4_t zz;
+};
+__device__ __forceinline__ GroupRegs make_group_asm(uint32_t qp) {
+    GroupRegs r;
+    float z0, z1, z2, z3;
+    asm volatile(
+        "v_and_b32 %[slo], 0xffff, %[q]\n\t"
+        "v_lshlrev_b32 %[shi], 16, %[q]\n\t"
+        "v_and_b32 %[z0], 0xffff0000, %[q]\n\t"
+        "v_mul_f32 %[c], 0xc3080000, %[shi]\n\t"
+        "v_mov_b32 %[z1], %[z0]\n\t"
+        "v_mov_b32 %[z2], %[z0]\n\t"
+        "v_mov_b32 %[z3], %[z0]"
+        : [slo] "=&v"(r.g.s_lo), [shi] "=&v"(r.g.s_hi), [c] "=&v"(r.g.c136), [z0] "=&v"(z0), [z1] "=&v"(z1),
+          [z2] "=&v"(z2), [z3] "=&v"(z3)
+        : [q] "v"(qp));
+    r.g.z = z0;
+    r.zz = f32x4_t{z0, z1, z2, z3};
+    return r;
+}
+
 // One workgroup = one 16-row block of W; its WAVES waves take the 128-wide K tiles round-robin, so the
 // workgroup streams its contiguous (K/2 bytes per row) x 16 rows region front to back.  Each lane owns
-// row r = lane%16 and 32 consecutive k per tile; tiles are double-buffered in registers so the next
-// tile's loads are in flight while the current one is dequantized.  blockIdx.y selects a chunk of 16
-// activation rows.  Partial 16x16 accumulators of the waves meet in LDS.
+// row r = lane%16 and 32 consecutive k per tile.  Weight tiles go through a register ring of depth D so
+// that D-1 tiles (1 KiB each per wave) are in flight while one is dequantized.  blockIdx.y selects a
+// chunk of 16 activation rows.  Partial 16x16 accumulators of the waves meet in LDS.
 //
-// FAST: K is a multiple of 128 (no K tail), x rows are 16-byte aligned.
 // DUAL: two weights of the same shape share the activation; the output is silu(x W1^T) * (x W2^T) with
 //       the bf16 roundings of the unfused module chain (linear -> silu -> mul).
 // Epilogue order for the single-weight form: y = bf16(acc + bias), then y = bf16(y + residual).
-template <int G, int WAVES, bool FAST, bool DUAL>
+template <int G, int WAVES, int XMODE, bool DUAL>
 __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(const LinearArgs a) {
-    __shared__ float red[DUAL ? 2 : 1][WAVES][4][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    static_assert(XMODE == X_GLOBAL || XMODE == X_CHECKED, "the LDS-staged path is int4wo_gemv_kernel");
+    constexpr int D = 2;
+    constexpr int NRED = DUAL ? 2 : 1;
+    __shared__ float red[NRED][WAVES][4][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, qd = lane >> 4;
     const int64_t rb = blockIdx.x;
     const int64_t m0 = (int64_t)blockIdx.y * 16;
     const int KB = (int)(a.Kp / 128);
     const uint32_t magic = 0x43004300u, one_lo = 0x00003F80u, one_hi = 0x3F800000u;
+    // selection matrices of stage 2 as A operands: lane (i = lane%16, qd) holds kk = 8*qd + e; the single 1.0 of
+    // row i sits at kk = 8*(i/4) + i%4 (sel_a) or + 4 (sel_b), i.e. only in the lanes with qd == i/4
+    const bool sel_lane = qd == (r >> 2);
+    const uint32_t one_bits = (r & 1) ? 0x3F800000u : 0x00003F80u;
+    const uint32_t s_even = (sel_lane && ((r & 3) >> 1) == 0) ? one_bits : 0u;
+    const uint32_t s_odd = (sel_lane && ((r & 3) >> 1) == 1) ? one_bits : 0u;
+    const u32x4_t sel_a = {s_even, s_odd, 0u, 0u};
+    const u32x4_t sel_b = {0u, 0u, s_even, s_odd};
 
     const int64_t woff = rb * KB * 64 + lane;
     const int64_t qoff = rb * (a.Kp / G) * 16 + r;
@@ -153,78 +300,103 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(const LinearA
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     f32x4_t acc2 = {0.f, 0.f, 0.f, 0.f};
 
-    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-    auto load_w = [&](const uint4* base, int kb) {
-        const u32x4_t wv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(base + woff + (int64_t)kb * 64));
-        return make_uint4(wv.x, wv.y, wv.z, wv.w);
+    typedef TileBuf<XMODE, DUAL> Buf;
+    auto load_w = [&](const uint4* base, int kb) -> u32x4_t {
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(base + woff + (int64_t)kb * 64));
     };
-    auto load_tile = [&](TileBuf& b, int kb) {
+    auto load_q = [&](const uint32_t* base, int gidx) -> uint32_t { return base[qoff + gidx]; };
+    auto load_tile = [&](Buf& b, int kb) {
         const int gidx = ((kb * 128 + qd * 32) / G) * 16;
         b.w = load_w(a.packed, kb);
-        b.q = a.qparams[qoff + gidx];
+        b.q = load_q(a.qparams, gidx);
         if (DUAL) {
             b.w2 = load_w(a.packed2, kb);
-            b.q2 = a.qparams2[qoff + gidx];
+            b.q2 = load_q(a.qparams2, gidx);
         }
-        if (FAST) {
+        if (XMODE == X_GLOBAL) {
             if (xact) {
                 const uint4* xv = reinterpret_cast<const uint4*>(xp + (int64_t)kb * 128);
 #pragma unroll
                 for (int sl = 0; sl < 4; ++sl) b.x[sl] = xv[sl];
             }
-        } else {
+        } else if (XMODE == X_CHECKED) {
 #pragma unroll
             for (int sl = 0; sl < 4; ++sl)
                 b.x[sl] = load_x8_checked(a.x, a.ldx, m0 + r, a.M, (int64_t)kb * 128 + qd * 32 + sl * 8, a.K);
         }
     };
-    auto compute_tile = [&](const TileBuf& b) {
+    u32x4_t tcur = {0, 0, 0, 0};  // stage-1 result of the dword that enters stage 2 next
+
+    // One tile = 4 dwords per lane (8 when DUAL).  `nb` is the wave's next tile (its stage 1 of dword 0 is
+    // overlapped with the last dword of this tile); has_next is wave-uniform.
+    auto compute_tile = [&](const Buf& b, const Buf& nb, bool has_next) {
         const GroupConst gc = make_group(b.q);
-        const uint32_t ww[4] = {b.w.x, b.w.y, b.w.z, b.w.w};
+        const GroupConst gc2 = make_group(DUAL ? b.q2 : b.q);
+        const uint32_t ww[8] = {b.w.x, b.w.y, b.w.z, b.w.w, b.w2.x, b.w2.y, b.w2.z, b.w2.w};
+        constexpr int NE = DUAL ? 8 : 4;
 #pragma unroll
-        for (int sl = 0; sl < 4; ++sl) {
+        for (int e = 0; e < NE; ++e) {
+            const GroupConst& ge = e < 4 ? gc : gc2;
             union { uint4 q; bf16x8_t v; } xa;
-            xa.q = b.x[sl];
-            const bf16x8_t bw = dequant8(ww[sl], gc, magic, one_lo, one_hi);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw, acc, 0, 0, 0);
-        }
-        if (DUAL) {
-            const GroupConst gc2 = make_group(b.q2);
-            const uint32_t w2[4] = {b.w2.x, b.w2.y, b.w2.z, b.w2.w};
-#pragma unroll
-            for (int sl = 0; sl < 4; ++sl) {
-                union { uint4 q; bf16x8_t v; } xa;
-                xa.q = b.x[sl];
-                const bf16x8_t bw = dequant8(w2[sl], gc2, magic, one_lo, one_hi);
-                acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw, acc2, 0, 0, 0);
+            xa.q = b.x[e & 3];
+            bf16x8_t bw;
+            if (AO_MFMA_ADD) {
+                f32x4_t ua, ub;
+                const f32x4_t zz = {ge.z, ge.z, ge.z, ge.z};
+                add_zero(tcur, zz, sel_a, sel_b, ua, ub);
+                if (e + 1 < NE) {
+                    tcur = first_half(ww[e + 1], (e + 1) < 4 ? gc : gc2, magic);
+                    bw = round_pack<false>(ua, ub);
+                } else if (has_next) {
+                    tcur = first_half(nb.w.x, make_group(nb.q), magic);
+                    bw = round_pack<false>(ua, ub);
+                } else {
+                    bw = round_pack<true>(ua, ub);
+                }
+            } else {
+                bw = dequant8(ww[e], ge, magic, one_lo, one_hi);
             }
+            if (e < 4) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw, acc, 0, 0, 0);
+            else acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw, acc2, 0, 0, 0);
         }
     };
 
-    TileBuf b0, b1;
+    Buf buf[D];
 #pragma unroll
-    for (int sl = 0; sl < 4; ++sl) {  // rows >= M keep these zeros: their loads are masked off
-        b0.x[sl] = make_uint4(0, 0, 0, 0);
-        b1.x[sl] = make_uint4(0, 0, 0, 0);
+    for (int j = 0; j < D; ++j) {
+        buf[j].w = u32x4_t{0, 0, 0, 0};
+        buf[j].w2 = u32x4_t{0, 0, 0, 0};
+        buf[j].q = 0;
+        buf[j].q2 = 0;
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl)  // rows >= M keep these zeros: their loads are masked off
+            buf[j].x[sl] = make_uint4(0, 0, 0, 0);
     }
-    int kb = wave;
-    if (kb < KB) load_tile(b0, kb);
-    while (kb < KB) {
-        const int kb1 = kb + WAVES, kb2 = kb + 2 * WAVES;
-        if (kb1 < KB) load_tile(b1, kb1);
-        compute_tile(b0);
-        if (kb1 < KB) {
-            if (kb2 < KB) load_tile(b0, kb2);
-            compute_tile(b1);
+    // prologue: D-1 weight tiles in flight before anything else
+#pragma unroll
+    for (int j = 0; j < D - 1; ++j) {
+        const int kbj = wave + j * WAVES;
+        if (kbj < KB) load_tile(buf[j], kbj);
+    }
+    // tiles of this wave: kb = wave + i*WAVES, i = 0..nt-1; tile i lives in buf[i % 2]
+    const int nt = wave < KB ? (KB - wave + WAVES - 1) / WAVES : 0;
+    if (nt > 0 && AO_MFMA_ADD) tcur = first_half(buf[0].w.x, make_group(buf[0].q), magic);
+    for (int i0 = 0; i0 < nt; i0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            const int i = i0 + j;
+            if (i < nt) {
+                if (i + 1 < nt) load_tile(buf[(j + 1) % D], wave + (i + 1) * WAVES);
+                compute_tile(buf[j], buf[(j + 1) % D], i + 1 < nt);
+            }
         }
-        kb = kb2;
     }
 
     // acc[i] = C[m = 4*qd + i][n = r]
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         red[0][wave][i][lane] = acc[i];
-        if (DUAL) red[DUAL ? 1 : 0][wave][i][lane] = acc2[i];
+        if (DUAL) red[NRED - 1][wave][i][lane] = acc2[i];
     }
     __syncthreads();
     if (wave == 0) {
@@ -237,7 +409,185 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(const LinearA
 #pragma unroll
             for (int w = 0; w < WAVES; ++w) {
                 s += red[0][w][i][lane];
-                if (DUAL) s2 += red[DUAL ? 1 : 0][w][i][lane];
+                if (DUAL) s2 += red[NRED - 1][w][i][lane];
+            }
+            const int64_t m = m0 + 4 * qd + i;
+            if (m < a.M && n < a.N) {
+                if (DUAL) {
+                    s = rne_bf16(silu_bf16(rne_bf16(s)) * rne_bf16(s2));
+                } else {
+                    s += bv;
+                    if (a.residual) s = rne_bf16(s) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
+                }
+                if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = s;
+                else ((uint16_t*)a.y)[m * a.ldy + n] = f32_to_bf16_bits(s);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- skinny path (M <= 16 rows staged in LDS)
+// The decode kernel.  Same tiling as int4wo_linear_kernel, tuned for instruction count: the wave index is
+// made scalar so that every tile-loop branch is a scalar branch, the weight / qparam streams are addressed as
+// scalar base + constant per-lane offset (no vector address arithmetic per tile), loads are issued from asm
+// with exact vmcnt waits, and the three dequantization stages are software-pipelined across dwords and tiles.
+struct GemvTile {
+    u32x4_t w; uint32_t q;
+    u32x4_t w2; uint32_t q2;
+};
+
+template <int G, int WAVES, bool DUAL>
+__global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArgs a) {
+    constexpr int D = 4;
+    constexpr int NRED = DUAL ? 2 : 1;
+    __shared__ float red[NRED][WAVES][4][64];
+    extern __shared__ __align__(16) uint16_t xs[];  // [rows][Kp] bf16
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, qd = lane >> 4;
+    const int64_t rb = blockIdx.x;
+    const int64_t m0 = (int64_t)blockIdx.y * 16;
+    const int KB = (int)(a.Kp / 128);
+    const uint32_t magic = 0x43004300u;
+    const bool sel_lane = qd == (r >> 2);
+    const uint32_t one_bits = (r & 1) ? 0x3F800000u : 0x00003F80u;
+    const uint32_t s_even = (sel_lane && ((r & 3) >> 1) == 0) ? one_bits : 0u;
+    const uint32_t s_odd = (sel_lane && ((r & 3) >> 1) == 1) ? one_bits : 0u;
+    const u32x4_t sel_a = {s_even, s_odd, 0u, 0u};
+    const u32x4_t sel_b = {0u, 0u, s_even, s_odd};
+
+    // scalar bases of this row block's streams; per-lane offsets never change
+    const char* wbase = reinterpret_cast<const char*>(a.packed) + rb * KB * 1024;
+    const char* wbase2 = reinterpret_cast<const char*>(DUAL ? a.packed2 : a.packed) + rb * KB * 1024;
+    const char* qbase = reinterpret_cast<const char*>(a.qparams) + rb * (a.Kp / G) * 64;
+    const char* qbase2 = reinterpret_cast<const char*>(DUAL ? a.qparams2 : a.qparams) + rb * (a.Kp / G) * 64;
+    const uint32_t woff = lane * 16;
+    // group of (tile kb, quarter qd) = (kb*128 + qd*32) / G = tile part + lane part for every G in {32..256}
+    const uint32_t qoff = (uint32_t)(r + (G < 128 ? (qd * 32 / G) * 16 : 0)) * 4;
+    auto tile_group_bytes = [&](int kb) -> int { return (G <= 128 ? kb * (128 / G) : kb / (G / 128)) * 64; };
+
+    const bool xact = (m0 + r) < a.M;
+    const uint16_t* xs_lane = xs + (int64_t)r * a.Kp + qd * 32;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4_t acc2 = {0.f, 0.f, 0.f, 0.f};
+
+    auto load_tile = [&](GemvTile& b, int kb) {
+        b.w = asm_load_b128_nt(wbase + (int64_t)kb * 1024, woff);
+        b.q = asm_load_b32(qbase + tile_group_bytes(kb), qoff);
+        if (DUAL) {
+            b.w2 = asm_load_b128_nt(wbase2 + (int64_t)kb * 1024, woff);
+            b.q2 = asm_load_b32(qbase2 + tile_group_bytes(kb), qoff);
+        }
+    };
+
+    uint4 xl[4];
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) xl[sl] = make_uint4(0, 0, 0, 0);  // rows >= M stay zero
+    constexpr int LPT = DUAL ? 4 : 2;  // loads per tile
+    u32x4_t tcur = {0, 0, 0, 0};  // stage-1 result of the dword that enters stage 2 next
+    GroupRegs gnext;              // group constants of the tile whose dword 0 is in tcur
+    gnext.g.s_lo = gnext.g.s_hi = 0; gnext.g.c136 = 0.f; gnext.g.z = 0.f;
+    gnext.zz = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    auto compute_tile = [&](const GemvTile& b, int kb, const GemvTile& nb, bool has_next, int younger_of_next) {
+        if (xact) {
+            const uint4* xv = reinterpret_cast<const uint4*>(xs_lane + kb * 128);
+#pragma unroll
+            for (int sl = 0; sl < 4; ++sl) xl[sl] = xv[sl];
+        }
+        const GroupRegs g1 = gnext;
+        const GroupRegs g2 = DUAL ? make_group_asm(b.q2) : gnext;
+        const GroupConst& gc = g1.g;
+        const GroupConst& gc2 = g2.g;
+        const f32x4_t& zz = g1.zz;
+        const f32x4_t& zz2 = g2.zz;
+        const uint32_t ww[8] = {b.w.x, b.w.y, b.w.z, b.w.w, b.w2.x, b.w2.y, b.w2.z, b.w2.w};
+        constexpr int NE = DUAL ? 8 : 4;
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            union { uint4 q; bf16x8_t v; } xa;
+            xa.q = xl[e & 3];
+            f32x4_t ua, ub;
+            add_zero(tcur, e < 4 ? zz : zz2, sel_a, sel_b, ua, ub);
+            bf16x8_t bw;
+            if (e + 1 < NE) {
+                tcur = first_half(ww[e + 1], (e + 1) < 4 ? gc : gc2, magic);
+                bw = round_pack<false>(ua, ub);
+            } else if (has_next) {
+                wait_tiles<LPT>(younger_of_next);
+                gnext = make_group_asm(nb.q);
+                tcur = first_half(nb.w.x, gnext.g, magic);
+                bw = round_pack<false>(ua, ub);
+            } else {
+                bw = round_pack<true>(ua, ub);
+            }
+            if (e < 4) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw, acc, 0, 0, 0);
+            else acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw, acc2, 0, 0, 0);
+        }
+    };
+
+    GemvTile buf[D];
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+        buf[j].w = u32x4_t{0, 0, 0, 0};
+        buf[j].w2 = u32x4_t{0, 0, 0, 0};
+        buf[j].q = 0;
+        buf[j].q2 = 0;
+    }
+    // tiles of this wave: kb = wave + i*WAVES, i = 0..nt-1; tile i lives in buf[i % D]
+    const int nt = wave < KB ? (KB - wave + WAVES - 1) / WAVES : 0;
+#pragma unroll
+    for (int j = 0; j < D - 1; ++j)
+        if (j < nt) load_tile(buf[j], wave + j * WAVES);
+    {
+        // stage the activation rows of this chunk: rows x Kp bf16, 16 bytes per thread per step
+        const int rows = (int)((a.M - m0) < 16 ? (a.M - m0) : 16);
+        const int chunks_per_row = (int)(a.Kp / 8);
+        for (int i = threadIdx.x; i < rows * chunks_per_row; i += WAVES * 64) {
+            const int rr = i / chunks_per_row, c = i - rr * chunks_per_row;
+            reinterpret_cast<uint4*>(xs)[i] = reinterpret_cast<const uint4*>(a.x + (m0 + rr) * a.ldx)[c];
+        }
+        __syncthreads();
+    }
+    // number of tiles requested after tile i that can still be outstanding when tile i is waited for: at the
+    // top of iteration i tiles up to i+D-1 have been requested; one fewer when tile i is waited for early
+    auto younger = [&](int i, int ahead) { return (nt - 1 - i) < ahead ? (nt - 1 - i) : ahead; };
+    if (nt > 0) {
+        wait_tiles<LPT>(younger(0, D - 2));
+        gnext = make_group_asm(buf[0].q);
+        tcur = first_half(buf[0].w.x, gnext.g, magic);
+    }
+    for (int i0 = 0; i0 < nt; i0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            const int i = i0 + j;
+            if (i < nt) {
+                const int nxt = i + (D - 1);
+                if (nxt < nt) load_tile(buf[(j + D - 1) % D], wave + nxt * WAVES);
+                wait_tiles<LPT>(younger(i, D - 1));
+                compute_tile(buf[j], wave + i * WAVES, buf[(j + 1) % D], i + 1 < nt, younger(i + 1, D - 2));
+            }
+        }
+    }
+
+    // acc[i] = C[m = 4*qd + i][n = r]
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        red[0][wave][i][lane] = acc[i];
+        if (DUAL) red[NRED - 1][wave][i][lane] = acc2[i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int64_t n = rb * 16 + r;
+        float bv = 0.f;
+        if (a.bias && n < a.N) bv = bf16_bits_to_f32(a.bias[n]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float s = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                s += red[0][w][i][lane];
+                if (DUAL) s2 += red[NRED - 1][w][i][lane];
             }
             const int64_t m = m0 + 4 * qd + i;
             if (m < a.M && n < a.N) {
@@ -259,33 +609,63 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(const LinearA
 // disarms.  hipEventElapsedTime(start, stop) is then the kernel's execution time without launch gaps.
 static thread_local hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;
 
-template <int G, int WAVES, bool FAST, bool DUAL>
-static void launch_one(dim3 grid, hipStream_t st, const LinearArgs& a) {
+template <int G, int WAVES, int XMODE, bool DUAL>
+static void launch_one(dim3 grid, size_t smem, hipStream_t st, const LinearArgs& a) {
     if (g_prof_start && g_prof_stop) {
-        hipExtLaunchKernelGGL((int4wo_linear_kernel<G, WAVES, FAST, DUAL>), grid, dim3(WAVES * 64), 0, st, g_prof_start,
+        hipExtLaunchKernelGGL((int4wo_linear_kernel<G, WAVES, XMODE, DUAL>), grid, dim3(WAVES * 64), smem, st,
+                              g_prof_start, g_prof_stop, 0, a);
+        g_prof_start = g_prof_stop = nullptr;
+        return;
+    }
+    hipLaunchKernelGGL((int4wo_linear_kernel<G, WAVES, XMODE, DUAL>), grid, dim3(WAVES * 64), smem, st, a);
+}
+template <int G, int XMODE, bool DUAL>
+static void launch_waves(int waves, dim3 grid, size_t smem, hipStream_t st, const LinearArgs& a) {
+    switch (waves) {
+        case 1: launch_one<G, 1, XMODE, DUAL>(grid, smem, st, a); break;
+        case 2: launch_one<G, 2, XMODE, DUAL>(grid, smem, st, a); break;
+        case 4: launch_one<G, 4, XMODE, DUAL>(grid, smem, st, a); break;
+        case 8: launch_one<G, 8, XMODE, DUAL>(grid, smem, st, a); break;
+        default: launch_one<G, 16, XMODE, DUAL>(grid, smem, st, a); break;
+    }
+}
+template <int G, int WAVES, bool DUAL>
+static void launch_gemv_one(dim3 grid, size_t smem, hipStream_t st, const LinearArgs& a) {
+    if (g_prof_start && g_prof_stop) {
+        hipExtLaunchKernelGGL((int4wo_gemv_kernel<G, WAVES, DUAL>), grid, dim3(WAVES * 64), smem, st, g_prof_start,
                               g_prof_stop, 0, a);
         g_prof_start = g_prof_stop = nullptr;
         return;
     }
-    hipLaunchKernelGGL((int4wo_linear_kernel<G, WAVES, FAST, DUAL>), grid, dim3(WAVES * 64), 0, st, a);
+    hipLaunchKernelGGL((int4wo_gemv_kernel<G, WAVES, DUAL>), grid, dim3(WAVES * 64), smem, st, a);
 }
-template <int G, bool FAST, bool DUAL>
-static void launch_waves(int waves, dim3 grid, hipStream_t st, const LinearArgs& a) {
+template <int G, bool DUAL>
+static void launch_gemv_waves(int waves, dim3 grid, size_t smem, hipStream_t st, const LinearArgs& a) {
     switch (waves) {
-        case 1: launch_one<G, 1, FAST, DUAL>(grid, st, a); break;
-        case 2: launch_one<G, 2, FAST, DUAL>(grid, st, a); break;
-        case 4: launch_one<G, 4, FAST, DUAL>(grid, st, a); break;
-        case 8: launch_one<G, 8, FAST, DUAL>(grid, st, a); break;
-        default: launch_one<G, 16, FAST, DUAL>(grid, st, a); break;
+        case 1: launch_gemv_one<G, 1, DUAL>(grid, smem, st, a); break;
+        case 2: launch_gemv_one<G, 2, DUAL>(grid, smem, st, a); break;
+        case 4: launch_gemv_one<G, 4, DUAL>(grid, smem, st, a); break;
+        case 8: launch_gemv_one<G, 8, DUAL>(grid, smem, st, a); break;
+        default: launch_gemv_one<G, 16, DUAL>(grid, smem, st, a); break;
     }
 }
-template <bool FAST, bool DUAL>
-static void launch_group(int64_t g, int waves, dim3 grid, hipStream_t st, const LinearArgs& a) {
+template <bool DUAL>
+static void launch_gemv(int64_t g, int waves, dim3 grid, size_t smem, hipStream_t st, const LinearArgs& a) {
     switch (g) {
-        case 32: launch_waves<32, FAST, DUAL>(waves, grid, st, a); break;
-        case 64: launch_waves<64, FAST, DUAL>(waves, grid, st, a); break;
-        case 128: launch_waves<128, FAST, DUAL>(waves, grid, st, a); break;
-        default: launch_waves<256, FAST, DUAL>(waves, grid, st, a); break;
+        case 32: launch_gemv_waves<32, DUAL>(waves, grid, smem, st, a); break;
+        case 64: launch_gemv_waves<64, DUAL>(waves, grid, smem, st, a); break;
+        case 128: launch_gemv_waves<128, DUAL>(waves, grid, smem, st, a); break;
+        default: launch_gemv_waves<256, DUAL>(waves, grid, smem, st, a); break;
+    }
+}
+
+template <int XMODE, bool DUAL>
+static void launch_group(int64_t g, int waves, dim3 grid, size_t smem, hipStream_t st, const LinearArgs& a) {
+    switch (g) {
+        case 32: launch_waves<32, XMODE, DUAL>(waves, grid, smem, st, a); break;
+        case 64: launch_waves<64, XMODE, DUAL>(waves, grid, smem, st, a); break;
+        case 128: launch_waves<128, XMODE, DUAL>(waves, grid, smem, st, a); break;
+        default: launch_waves<256, XMODE, DUAL>(waves, grid, smem, st, a); break;
     }
 }
 
@@ -308,21 +688,28 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     const int64_t mchunks = (M + 15) / 16;
     AO_REQUIRE(mchunks <= 65535, "batch too large for one launch: M=%lld", (long long)M);
     const int64_t KB = Kp / 128, RB = Np / 16;
-    // enough waves to fill 256 CUs several times over, never more waves than K tiles
+    // about 16 waves per CU over 256 CUs, each with as many K tiles as the shape allows
     int waves = 1;
-    while (waves < 16 && RB * mchunks * waves < 6144 && waves * 2 <= KB) waves *= 2;
-    const bool fast = (K == Kp) && ((ldx & 7) == 0) && ((((uintptr_t)x_bf16) & 15) == 0);
+    while (waves < 16 && RB * mchunks * waves * 2 <= 4096 + RB * mchunks && waves * 2 <= KB) waves *= 2;
+    const bool aligned = (K == Kp) && ((ldx & 7) == 0) && ((((uintptr_t)x_bf16) & 15) == 0);
+    const int64_t rows = M < 16 ? M : 16;
+    const size_t xbytes = (size_t)rows * (size_t)Kp * 2;
+    // LDS staging only while it leaves room for about 16 waves per CU (160 KB of LDS per CU)
+    int xmode = aligned ? (xbytes <= (size_t)waves * 10 * 1024 ? X_LDS : X_GLOBAL) : X_CHECKED;
     LinearArgs a{(const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams,
                  (const uint4*)packed2, (const uint32_t*)qparams2, N, Kp, (const uint16_t*)bias_bf16,
                  (const uint16_t*)residual_bf16, ldres, y, y_dtype == AO_F32, ldy};
     dim3 grid((unsigned)RB, (unsigned)mchunks);
     hipStream_t st = (hipStream_t)stream;
+    const size_t smem = xmode == X_LDS ? xbytes : 0;
     if (dual) {
-        if (fast) launch_group<true, true>(g, waves, grid, st, a);
-        else launch_group<false, true>(g, waves, grid, st, a);
+        if (xmode == X_LDS) launch_gemv<true>(g, waves, grid, smem, st, a);
+        else if (xmode == X_GLOBAL) launch_group<X_GLOBAL, true>(g, waves, grid, smem, st, a);
+        else launch_group<X_CHECKED, true>(g, waves, grid, smem, st, a);
     } else {
-        if (fast) launch_group<true, false>(g, waves, grid, st, a);
-        else launch_group<false, false>(g, waves, grid, st, a);
+        if (xmode == X_LDS) launch_gemv<false>(g, waves, grid, smem, st, a);
+        else if (xmode == X_GLOBAL) launch_group<X_GLOBAL, false>(g, waves, grid, smem, st, a);
+        else launch_group<X_CHECKED, false>(g, waves, grid, smem, st, a);
     }
     AO_LAUNCH_CHECK();
     return 0;

@@ -21,12 +21,60 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 // out = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * w ), statistics in fp32.  One workgroup per row.
+// VEC: dim is a multiple of 8 and the rows are 16-byte aligned; every thread then issues all of its
+// 16-byte loads (up to 4 chunks, dim <= 8192) before the first use so the row is read in one round trip.
+template <bool VEC>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                        int64_t dim, float eps, uint16_t* __restrict__ out) {
     __shared__ float part[4];
     const int64_t row = blockIdx.x;
     const uint16_t* xr = x + row * dim;
     float ss = 0.f;
+    if (VEC) {
+        constexpr int MAXC = 4;
+        const int nchunk = (int)(dim / 8);
+        uint4 xv[MAXC], wv[MAXC];
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c) {
+            const int idx = threadIdx.x + c * 256;
+            xv[c] = make_uint4(0, 0, 0, 0);
+            wv[c] = make_uint4(0, 0, 0, 0);
+            if (idx < nchunk) {
+                xv[c] = reinterpret_cast<const uint4*>(xr)[idx];
+                wv[c] = reinterpret_cast<const uint4*>(w)[idx];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c) {
+            const uint32_t u[4] = {xv[c].x, xv[c].y, xv[c].z, xv[c].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float lo = __uint_as_float(u[j] << 16), hi = __uint_as_float(u[j] & 0xffff0000u);
+                ss += lo * lo + hi * hi;
+            }
+        }
+        ss = wave_sum(ss);
+        if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        const float r = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)dim + eps);
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c) {
+            const int idx = threadIdx.x + c * 256;
+            if (idx < nchunk) {
+                const uint32_t u[4] = {xv[c].x, xv[c].y, xv[c].z, xv[c].w};
+                const uint32_t g[4] = {wv[c].x, wv[c].y, wv[c].z, wv[c].w};
+                uint32_t o[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float lo = rne_bf16(__uint_as_float(u[j] << 16) * r) * __uint_as_float(g[j] << 16);
+                    const float hi = rne_bf16(__uint_as_float(u[j] & 0xffff0000u) * r) * __uint_as_float(g[j] & 0xffff0000u);
+                    o[j] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+                }
+                reinterpret_cast<uint4*>(out + row * dim)[idx] = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+        }
+        return;
+    }
     for (int64_t i = threadIdx.x; i < dim; i += 256) {
         float v = bf16_bits_to_f32(xr[i]);
         ss += v * v;
@@ -97,36 +145,48 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t* _
     }
     __syncthreads();
 
-    // scores: 16 lanes x 8 elements per position, 16 positions per pass over the workgroup
+    // scores: 16 lanes x 8 elements per position, 16 positions per pass over the workgroup, 4 passes in
+    // flight (all loads of a batch are issued before the first use: the loop is latency bound otherwise)
     const int sub = lane >> 4, l16 = lane & 15;
-    float qreg[8];
+    float qreg[8], knew[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) qreg[e] = q_s[l16 * 8 + e];
+    for (int e = 0; e < 8; ++e) {
+        qreg[e] = q_s[l16 * 8 + e];
+        knew[e] = knew_s[l16 * 8 + e];
+    }
     const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
     float lmax = -INFINITY;
-    for (int t0 = 0; t0 < T; t0 += 16) {
-        const int t = t0 + wave * 4 + sub;
-        float d = 0.f;
-        if (t < T) {
-            if (t == pos) {
+    constexpr int U = 4;
+    for (int t0 = 0; t0 < T; t0 += 16 * U) {
+        uint4 raw[U];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) d += qreg[e] * knew_s[l16 * 8 + e];
-            } else {
-                const uint4 raw = *reinterpret_cast<const uint4*>(kc + (int64_t)t * HD + l16 * 8);
-                const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    d += qreg[2 * j] * __uint_as_float(u[j] << 16);
-                    d += qreg[2 * j + 1] * __uint_as_float(u[j] & 0xffff0000u);
-                }
-            }
+        for (int u = 0; u < U; ++u) {
+            const int t = t0 + u * 16 + wave * 4 + sub;
+            raw[u] = make_uint4(0, 0, 0, 0);
+            if (t < pos) raw[u] = *reinterpret_cast<const uint4*>(kc + (int64_t)t * HD + l16 * 8);
         }
 #pragma unroll
-        for (int o = 8; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);
-        d *= scale;
-        if (t < T) {
-            if (l16 == 0) sc[t] = d;
-            lmax = fmaxf(lmax, d);
+        for (int u = 0; u < U; ++u) {
+            const int t = t0 + u * 16 + wave * 4 + sub;
+            const uint32_t w4[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+            float d = 0.f;
+            if (t == pos) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) d += qreg[e] * knew[e];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    d += qreg[2 * j] * __uint_as_float(w4[j] << 16);
+                    d += qreg[2 * j + 1] * __uint_as_float(w4[j] & 0xffff0000u);
+                }
+            }
+#pragma unroll
+            for (int o = 8; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);
+            d *= scale;
+            if (t < T) {
+                if (l16 == 0) sc[t] = d;
+                lmax = fmaxf(lmax, d);
+            }
         }
     }
     lmax = wave_max(lmax);
@@ -145,25 +205,48 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t* _
     __syncthreads();
     const float inv = 1.0f / (red[4] + red[5] + red[6] + red[7]);
 
-    // out[d] = sum_t p_t * V[t][d]: lane owns the pair d = 2*lane, 2*lane+1; the 4 waves split t
-    float o0 = 0.f, o1 = 0.f;
-    for (int t = wave; t < T; t += 4) {
-        const float p = sc[t];
-        float v0, v1;
-        if (t == pos) {
-            v0 = vnew_s[2 * lane];
-            v1 = vnew_s[2 * lane + 1];
-        } else {
-            const uint32_t u = *reinterpret_cast<const uint32_t*>(vc + (int64_t)t * HD + 2 * lane);
-            v0 = __uint_as_float(u << 16);
-            v1 = __uint_as_float(u & 0xffff0000u);
+    // out[d] = sum_t p_t * V[t][d]: same thread mapping (position = wave*4 + sub, 8 values of d per lane)
+    float oacc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) oacc[e] = 0.f;
+    for (int t0 = 0; t0 < T; t0 += 16 * U) {
+        uint4 raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int t = t0 + u * 16 + wave * 4 + sub;
+            raw[u] = make_uint4(0, 0, 0, 0);
+            if (t < pos) raw[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)t * HD + l16 * 8);
         }
-        o0 += p * v0;
-        o1 += p * v1;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int t = t0 + u * 16 + wave * 4 + sub;
+            if (t < T) {
+                const float p = sc[t];
+                if (t == pos) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) oacc[e] += p * vnew_s[l16 * 8 + e];
+                } else {
+                    const uint32_t w4[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        oacc[2 * j] += p * __uint_as_float(w4[j] << 16);
+                        oacc[2 * j + 1] += p * __uint_as_float(w4[j] & 0xffff0000u);
+                    }
+                }
+            }
+        }
+    }
+    // fold the 4 position slots of a wave, then the 4 waves
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        oacc[e] += __shfl_xor(oacc[e], 16, 64);
+        oacc[e] += __shfl_xor(oacc[e], 32, 64);
     }
     float* po = red + 8;  // [4][128]
-    po[wave * HD + 2 * lane] = o0;
-    po[wave * HD + 2 * lane + 1] = o1;
+    if (sub == 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) po[wave * HD + l16 * 8 + e] = oacc[e];
+    }
     __syncthreads();
     if (tid < HD) {
         const float o = (po[tid] + po[HD + tid] + po[2 * HD + tid] + po[3 * HD + tid]) * inv;
@@ -180,8 +263,14 @@ extern "C" int ao_amd_rmsnorm_bf16(const void* x, const void* weight, int64_t ro
     AO_REQUIRE(x && weight && out, "null pointer argument");
     AO_REQUIRE(rows >= 0 && dim > 0, "bad shape rows=%lld dim=%lld", (long long)rows, (long long)dim);
     if (rows == 0) return 0;
-    hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x,
-                       (const uint16_t*)weight, dim, eps, (uint16_t*)out);
+    const bool vec = (dim % 8 == 0) && dim <= 8192 &&
+                     (((uintptr_t)x | (uintptr_t)weight | (uintptr_t)out) & 15) == 0;
+    if (vec)
+        hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream,
+                           (const uint16_t*)x, (const uint16_t*)weight, dim, eps, (uint16_t*)out);
+    else
+        hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream,
+                           (const uint16_t*)x, (const uint16_t*)weight, dim, eps, (uint16_t*)out);
     AO_LAUNCH_CHECK();
     return 0;
 }
