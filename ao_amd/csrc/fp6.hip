@@ -1,0 +1,384 @@
+// FP6-LLM (Quant-LLM) weight-only path for gfx950: 6-bit floating point weights (e3m2 or e2m3) with one fp16
+// scale per output row.
+//
+// Interchange format = the reference's TC-FPx bytes (torchao/prototype/quant_llm/quant_llm.py:90-106): all
+// bytes of the 2-bit plane (code >> 4) followed by all bytes of the 4-bit plane (code & 15), ordered for
+// NVIDIA mma.m16n8k16 fragments.  The quantize / dequantize kernels here read and write exactly those bytes.
+//
+// Kernel format ("native"): the same codes rearranged once for wave64: per 16-row x 128-k tile, lane
+// l = (row l%16, quarter l/16) owns the 32 consecutive k = 128*kb + 32*(l/16) + i, stored as 32 x 6 bits in
+// natural order (value i at bit 6*i of a 192-bit string = 6 dwords).  A tile is 1536 bytes:
+// [64 lanes][dwords 0..3] then [64 lanes][dwords 4..5], so a wave reads it with one 16-byte and one 8-byte
+// load per lane, both fully coalesced.  v_cvt_scalef32_pk32_f16_bf6 / _fp6 turns a lane's 6 dwords into its
+// 32 fp16 values in one instruction, already in the k-order of four 16x16x32 f16 MFMA B operands.
+#include "common.h"
+
+namespace ao {
+
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x32_t __attribute__((ext_vector_type(32)));
+typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------- scalar casts
+// fp32 -> FPx code in the low 1+ebits+mbits bits: round to nearest even, saturate to the largest normal, no
+// inf / nan codes.  Bit-for-bit torchao/prototype/custom_fp_utils.py:27-140.
+__device__ __forceinline__ uint32_t f32_to_fpx(float xf, int ebits, int mbits) {
+    const int MB = 23, EB = 8, F32_BIAS = 127;
+    const int exp_bias = (1 << (ebits - 1)) - 1;
+    const uint32_t max_int = (1u << (ebits + mbits)) - 1u;
+    const uint32_t sign_mask = 1u << (ebits + mbits);
+    const uint32_t magic_adder = (1u << (MB - mbits - 1)) - 1u;
+    const float max_normal = __uint_as_float((uint32_t)(((1 << ebits) - 1) - exp_bias + F32_BIAS) << MB) *
+                             ((float)((1 << (mbits + 1)) - 1) / (float)(1 << mbits));
+    const float min_normal = __uint_as_float((uint32_t)(1 - exp_bias + F32_BIAS) << MB);
+    const uint32_t denorm_mask_int = (uint32_t)((F32_BIAS - exp_bias) + (MB - mbits) + 1) << MB;
+    const float denorm_mask_float = __uint_as_float(denorm_mask_int);
+
+    uint32_t xi = __float_as_uint(xf);
+    const uint32_t sign = xi & 0x80000000u;
+    xi ^= sign;
+    const float x = __uint_as_float(xi);
+    uint32_t res;
+    if (x >= max_normal) {
+        res = max_int;
+    } else if (x < min_normal) {
+        // adding 2^(denorm exponent) makes the fp32 adder do the round-to-nearest-even to the subnormal grid
+        res = (__float_as_uint(__fadd_rn(x, denorm_mask_float)) - denorm_mask_int) & 0xffu;
+    } else if (x != x) {
+        res = max_int;
+    } else {
+        uint32_t n = xi;
+        const uint32_t mant_odd = (n >> (MB - mbits)) & 1u;
+        n += ((uint32_t)(exp_bias - F32_BIAS) << MB) + magic_adder;
+        n += mant_odd;
+        res = (n >> (MB - mbits)) & 0xffu;
+    }
+    return res | ((sign >> (MB + EB - mbits - ebits)) & sign_mask);
+}
+
+// FPx code -> fp32 (torchao/prototype/custom_fp_utils.py:145-229)
+__device__ __forceinline__ float fpx_to_f32(uint32_t code, int ebits, int mbits) {
+    const int exp_bias = (1 << (ebits - 1)) - 1;
+    const uint32_t sign = (code >> (ebits + mbits)) & 1u;
+    const uint32_t e = (code >> mbits) & ((1u << ebits) - 1u);
+    const uint32_t m = code & ((1u << mbits) - 1u);
+    float v;
+    if (e == 0) v = (float)m * __uint_as_float((uint32_t)(1 - exp_bias - mbits + 127) << 23);
+    else v = (float)((1u << mbits) | m) * __uint_as_float((uint32_t)((int)e - exp_bias - mbits + 127) << 23);
+    return sign ? -v : v;
+}
+
+// ---------------------------------------------------------------- TC-FP6 byte positions
+// code of element (row, col) of a [R, C] weight: 2 high bits at (byte B2, shift sh2) of plane 2, 4 low bits at
+// (byte B4, shift sh4) of plane 4 (plane 4 starts at byte R*C/4).  Index form of _pack_tc_fp6.
+struct TcPos { int64_t b2; int sh2; int64_t b4; int sh4; };
+__device__ __forceinline__ TcPos tc_fp6_pos(int64_t row, int64_t col, int64_t C) {
+    const int64_t a = row >> 6, e = col >> 4, E = C >> 4;
+    const int rr = (int)(row & 63), i1 = rr >> 5, i2 = (rr >> 4) & 1, i3 = (rr >> 3) & 1, d = rr & 7;
+    const int f = (int)((col >> 3) & 1), g = (int)(col & 7), p = 1 - i3;
+    TcPos t;
+    t.b2 = ((((a * E + e) * 2 + i1) * 8 + d) * 8 + g) * 2 + p;
+    t.sh2 = 6 - 2 * (i2 * 2 + f);
+    t.b4 = (((((a * E + e) * 2 + i1) * 2 + i2) * 8 + d) * 8 + g) * 2 + p;
+    t.sh4 = 4 - 4 * f;
+    return t;
+}
+
+// ---------------------------------------------------------------- quantize + pack (to_scaled_tc_fpx)
+// One workgroup per 64-row block.  Pass 1: row amax -> fp32 scale (amax clamped at 1e-12, divided by the largest
+// normal).  Pass 2, per 16-column slice: 1024 codes into LDS, then every thread assembles one byte of the 2-bit
+// plane and two bytes of the 4-bit plane of that slice.
+__global__ __launch_bounds__(256) void fp6_quantize_pack_kernel(const void* __restrict__ w, int w_dtype, int64_t N,
+                                                                 int64_t K, int ebits, int mbits,
+                                                                 uint8_t* __restrict__ out, uint16_t* __restrict__ scale_out) {
+    __shared__ float scale_s[64];
+    __shared__ uint8_t codes_s[64][17];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t a = blockIdx.x;
+    const int exp_bias = (1 << (ebits - 1)) - 1;
+    const float max_normal = __uint_as_float((uint32_t)(((1 << ebits) - 1) - exp_bias + 127) << 23) *
+                             ((float)((1 << (mbits + 1)) - 1) / (float)(1 << mbits));
+    for (int rr = wave * 16; rr < wave * 16 + 16; ++rr) {
+        const int64_t row = a * 64 + rr;
+        float amax = 0.f;
+        bool has_nan = false;
+        for (int64_t c = lane; c < K; c += 64) {
+            const float v = fabsf(load_f(w, w_dtype, row * K + c));
+            if (v != v) has_nan = true;
+            amax = fmaxf(amax, v);
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) {
+            amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            has_nan |= (bool)__shfl_xor((int)has_nan, o, 64);
+        }
+        if (lane == 0) {
+            float s = has_nan ? NAN : (amax < 1e-12f ? 1e-12f : amax);
+            s = __fdiv_rn(s, max_normal);
+            scale_s[rr] = s;
+            scale_out[row] = f32_to_f16_bits(s);
+        }
+    }
+    __syncthreads();
+    uint8_t* p2 = out;
+    uint8_t* p4 = out + N * K / 4;
+    const int64_t E = K >> 4;
+    for (int64_t e = 0; e < E; ++e) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int idx = tid + j * 256, rr = idx >> 4, cc = idx & 15;
+            const float v = load_f(w, w_dtype, (a * 64 + rr) * K + e * 16 + cc);
+            codes_s[rr][cc] = (uint8_t)f32_to_fpx(__fdiv_rn(v, scale_s[rr]), ebits, mbits);
+        }
+        __syncthreads();
+        {
+            const int i1 = tid >> 7, d = (tid >> 4) & 7, g = (tid >> 1) & 7, p = tid & 1, i3 = 1 - p;
+            uint32_t b2 = 0;
+#pragma unroll
+            for (int i2 = 0; i2 < 2; ++i2)
+#pragma unroll
+                for (int f = 0; f < 2; ++f)
+                    b2 = (b2 << 2) | ((codes_s[32 * i1 + 16 * i2 + 8 * i3 + d][8 * f + g] >> 4) & 3u);
+            p2[(a * E + e) * 256 + tid] = (uint8_t)b2;
+#pragma unroll
+            for (int i2 = 0; i2 < 2; ++i2) {
+                const int rr = 32 * i1 + 16 * i2 + 8 * i3 + d;
+                const uint32_t b4 = ((codes_s[rr][g] & 15u) << 4) | (codes_s[rr][8 + g] & 15u);
+                p4[(a * E + e) * 512 + (((i1 * 2 + i2) * 8 + d) * 8 + g) * 2 + p] = (uint8_t)b4;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// from_scaled_tc_fpx: fp32 [N,K] = fpx_to_f32(code) * float(scale)
+__global__ __launch_bounds__(256) void fp6_dequantize_kernel(const uint8_t* __restrict__ tc, const uint16_t* __restrict__ scale,
+                                                              int64_t N, int64_t K, int ebits, int mbits, float* __restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N * K) return;
+    const int64_t row = i / K, col = i % K;
+    const TcPos t = tc_fp6_pos(row, col, K);
+    const uint32_t code = (((tc[t.b2] >> t.sh2) & 3u) << 4) | ((tc[N * K / 4 + t.b4] >> t.sh4) & 15u);
+    float v = fpx_to_f32(code, ebits, mbits);
+    if (scale) v *= f16_bits_to_f32(scale[row]);
+    out[i] = v;
+}
+
+// TC-FP6 bytes -> native tiles.  One thread per (lane, tile): gathers its 32 codes and writes 6 dwords.
+__global__ __launch_bounds__(256) void fp6_repack_kernel(const uint8_t* __restrict__ tc, int64_t N, int64_t K, int64_t Kp,
+                                                          uint32_t* __restrict__ native) {
+    const int64_t KB = Kp / 128;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (N / 16) * KB * 64) return;
+    const int l = (int)(i & 63);
+    const int64_t tile = i >> 6, kb = tile % KB, rb = tile / KB;
+    const int64_t row = rb * 16 + (l & 15), k0 = kb * 128 + (l >> 4) * 32;
+    uint32_t words[6] = {0, 0, 0, 0, 0, 0};
+    for (int j = 0; j < 32; ++j) {
+        uint32_t code = 0;
+        if (k0 + j < K) {
+            const TcPos t = tc_fp6_pos(row, k0 + j, K);
+            code = (((tc[t.b2] >> t.sh2) & 3u) << 4) | ((tc[N * K / 4 + t.b4] >> t.sh4) & 15u);
+        }
+        const int bit = 6 * j;
+        words[bit >> 5] |= code << (bit & 31);
+        if ((bit & 31) > 26) words[(bit >> 5) + 1] |= code >> (32 - (bit & 31));
+    }
+    uint32_t* base = native + tile * 384;  // 1536 bytes per tile
+#pragma unroll
+    for (int j = 0; j < 4; ++j) base[l * 4 + j] = words[j];
+    base[256 + l * 2] = words[4];
+    base[256 + l * 2 + 1] = words[5];
+}
+
+// ---------------------------------------------------------------- linear
+// out[M,N] fp16 = x[M,K] fp16 @ W^T, W = fp16(fp6 * scale), fp32 accumulation (quant_llm_linear,
+// torchao/csrc/cuda/fp6_llm/fp6_linear.cu:139-196 with the dequantization of utils_parallel_dequant.cuh:47-59).
+// One workgroup per 16-row block; WAVES waves take the 128-wide K tiles round-robin, double-buffered;
+// blockIdx.y selects a chunk of 16 activation rows.  E3M2: e3m2 codes, otherwise e2m3.
+template <int WAVES, bool E3M2>
+__global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
+                                                                 const uint32_t* __restrict__ native,
+                                                                 const uint16_t* __restrict__ scale, int64_t N, int64_t Kp,
+                                                                 uint16_t* __restrict__ out) {
+    __shared__ float red[WAVES][4][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, qd = lane >> 4;
+    const int64_t rb = blockIdx.x, m0 = (int64_t)blockIdx.y * 16;
+    const int KB = (int)(Kp / 128);
+    const uint32_t* tiles = native + rb * KB * 384;
+    const bool xact = (m0 + r) < M;
+    const uint16_t* xp = x + (xact ? (m0 + r) : 0) * K + qd * 32;
+    union { uint16_t h; _Float16 f; } sc;
+    sc.h = scale[rb * 16 + r];
+    const f16x2_t sc2 = {sc.f, sc.f};
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+
+    struct Buf { uint4 lo; uint2 hi; uint4 x[4]; };
+    auto load_tile = [&](Buf& b, int kb) {
+        const uint32_t* t = tiles + (int64_t)kb * 384;
+        b.lo = reinterpret_cast<const uint4*>(t)[lane];
+        b.hi = reinterpret_cast<const uint2*>(t + 256)[lane];
+        if (xact) {
+            const int64_t k0 = (int64_t)kb * 128 + qd * 32;
+            if (k0 + 32 <= K) {
+                const uint4* xv = reinterpret_cast<const uint4*>(xp + (int64_t)kb * 128);
+#pragma unroll
+                for (int sl = 0; sl < 4; ++sl) b.x[sl] = xv[sl];
+            } else {
+#pragma unroll
+                for (int sl = 0; sl < 4; ++sl) {
+                    union { uint4 q; uint16_t h[8]; } u;
+                    u.q = make_uint4(0, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (k0 + sl * 8 + e < K) u.h[e] = xp[(int64_t)kb * 128 + sl * 8 + e];
+                    b.x[sl] = u.q;
+                }
+            }
+        }
+    };
+    auto compute_tile = [&](const Buf& b) {
+        const u32x6_t packed = {b.lo.x, b.lo.y, b.lo.z, b.lo.w, b.hi.x, b.hi.y};
+        f16x32_t v;
+        if (E3M2) v = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(packed, 1.0f);
+        else v = __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(packed, 1.0f);
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            union { f16x2_t p[4]; f16x8_t v; } w;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f16x2_t pr = {v[sl * 8 + 2 * j], v[sl * 8 + 2 * j + 1]};
+                w.p[j] = pr * sc2;  // v_pk_mul_f16: fp16(fp6 * scale), the one rounding of the reference kernel
+            }
+            union { uint4 q; f16x8_t v; } xa;
+            xa.q = b.x[sl];
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa.v, w.v, acc, 0, 0, 0);
+        }
+    };
+
+    Buf b0, b1;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+        b0.x[sl] = make_uint4(0, 0, 0, 0);
+        b1.x[sl] = make_uint4(0, 0, 0, 0);
+    }
+    int kb = wave;
+    if (kb < KB) load_tile(b0, kb);
+    while (kb < KB) {
+        const int kb1 = kb + WAVES, kb2 = kb + 2 * WAVES;
+        if (kb1 < KB) load_tile(b1, kb1);
+        compute_tile(b0);
+        if (kb1 < KB) {
+            if (kb2 < KB) load_tile(b0, kb2);
+            compute_tile(b1);
+        }
+        kb = kb2;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][i][lane] = acc[i];
+    __syncthreads();
+    if (wave == 0) {
+        const int64_t n = rb * 16 + r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) s += red[w][i][lane];
+            const int64_t m = m0 + 4 * qd + i;
+            if (m < M && n < N) out[m * N + n] = f32_to_f16_bits(s);
+        }
+    }
+}
+
+static int check_fp6_format(int ebits, int mbits) {
+    AO_REQUIRE((ebits == 3 && mbits == 2) || (ebits == 2 && mbits == 3),
+               "FP%d E%dM%d is not supported (6-bit formats e3m2 and e2m3 only)", 1 + ebits + mbits, ebits, mbits);
+    return 0;
+}
+
+}  // namespace ao
+
+using namespace ao;
+
+extern "C" int ao_amd_fp6_quantize_pack(const void* w, int w_dtype, int64_t N, int64_t K, int ebits, int mbits,
+                                        void* out_tc, void* out_scale_f16, void* stream) {
+    AO_REQUIRE(w && out_tc && out_scale_f16, "null pointer argument");
+    AO_REQUIRE(is_float_dtype(w_dtype), "Unsupported input dtype code: %d", w_dtype);
+    if (int rc = check_fp6_format(ebits, mbits)) return rc;
+    AO_REQUIRE(N > 0 && K > 0 && N % 64 == 0 && K % 64 == 0,
+               "TC-FPx packing needs out_features and in_features to be multiples of 64, got (%lld, %lld)", (long long)N,
+               (long long)K);
+    hipLaunchKernelGGL(fp6_quantize_pack_kernel, dim3((unsigned)(N / 64)), dim3(256), 0, (hipStream_t)stream, w, w_dtype, N,
+                       K, ebits, mbits, (uint8_t*)out_tc, (uint16_t*)out_scale_f16);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_fp6_dequantize(const void* tc, const void* scale_f16, int64_t N, int64_t K, int ebits, int mbits,
+                                     float* out, void* stream) {
+    AO_REQUIRE(tc && out, "null pointer argument");
+    if (int rc = check_fp6_format(ebits, mbits)) return rc;
+    AO_REQUIRE(N > 0 && K > 0 && N % 64 == 0 && K % 64 == 0, "TC-FPx shapes must be multiples of 64, got (%lld, %lld)",
+               (long long)N, (long long)K);
+    const int64_t n = N * K;
+    hipLaunchKernelGGL(fp6_dequantize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint8_t*)tc, (const uint16_t*)scale_f16, N, K, ebits, mbits, out);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_fp6_native_bytes(int64_t N, int64_t K, int64_t* bytes) {
+    AO_REQUIRE(N > 0 && K > 0 && N % 16 == 0, "out_features must be a positive multiple of 16, got %lld", (long long)N);
+    if (bytes) *bytes = (N / 16) * (round_up(K, 128) / 128) * 1536;
+    return 0;
+}
+
+extern "C" int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, void* native, void* stream) {
+    AO_REQUIRE(tc && native, "null pointer argument");
+    AO_REQUIRE(N > 0 && K > 0 && N % 64 == 0 && K % 64 == 0, "TC-FPx shapes must be multiples of 64, got (%lld, %lld)",
+               (long long)N, (long long)K);
+    const int64_t Kp = round_up(K, 128);
+    const int64_t n = (N / 16) * (Kp / 128) * 64;
+    hipLaunchKernelGGL(fp6_repack_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint8_t*)tc, N, K, Kp, (uint32_t*)native);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native,
+                                 const void* scale_f16, int64_t N, int ebits, int mbits, void* out_f16, void* stream) {
+    AO_REQUIRE(x_f16 && weights_native && scale_f16 && out_f16, "null pointer argument");
+    if (int rc = check_fp6_format(ebits, mbits)) return rc;
+    AO_REQUIRE(K % 64 == 0, "Expected in_features to be a multiple of 64, but received %lld", (long long)K);
+    AO_REQUIRE(N > 0 && N % 16 == 0, "out_features must be a positive multiple of 16, got %lld", (long long)N);
+    AO_REQUIRE(M >= 0, "negative batch");
+    AO_REQUIRE((((uintptr_t)x_f16) & 15) == 0 && (((uintptr_t)weights_native) & 15) == 0, "buffers must be 16-byte aligned");
+    if (M == 0) return 0;
+    const int64_t Kp = round_up(K, 128), KB = Kp / 128, RB = N / 16, mchunks = (M + 15) / 16;
+    AO_REQUIRE(mchunks <= 65535, "batch too large for one launch: M=%lld", (long long)M);
+    int waves = 1;
+    while (waves < 16 && RB * mchunks * waves * 2 <= 4096 + RB * mchunks && waves * 2 <= KB) waves *= 2;
+    dim3 grid((unsigned)RB, (unsigned)mchunks);
+    hipStream_t st = (hipStream_t)stream;
+    const uint16_t* xx = (const uint16_t*)x_f16;
+    const uint32_t* nat = (const uint32_t*)weights_native;
+    const uint16_t* sc = (const uint16_t*)scale_f16;
+    uint16_t* o = (uint16_t*)out_f16;
+#define AO_FP6_LAUNCH(W)                                                                                             \
+    if (ebits == 3) hipLaunchKernelGGL((fp6_linear_kernel<W, true>), grid, dim3(W * 64), 0, st, xx, M, K, nat, sc, N, Kp, o); \
+    else hipLaunchKernelGGL((fp6_linear_kernel<W, false>), grid, dim3(W * 64), 0, st, xx, M, K, nat, sc, N, Kp, o)
+    switch (waves) {
+        case 1: AO_FP6_LAUNCH(1); break;
+        case 2: AO_FP6_LAUNCH(2); break;
+        case 4: AO_FP6_LAUNCH(4); break;
+        case 8: AO_FP6_LAUNCH(8); break;
+        default: AO_FP6_LAUNCH(16); break;
+    }
+#undef AO_FP6_LAUNCH
+    AO_LAUNCH_CHECK();
+    return 0;
+}

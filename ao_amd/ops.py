@@ -5,6 +5,8 @@ registration of torchao/csrc/fp6_llm.cpp:5-8.  The device implementations call t
 include/ao_amd.h with raw pointers on torch's current stream; there is no CPU implementation:
 a CPU tensor raises.
 """
+import weakref
+
 import torch
 from torch import Tensor
 
@@ -12,6 +14,11 @@ from . import _lib
 from ._lib import BF16, DTYPE_CODE, F32, check, current_stream, lib, require_cuda
 
 __all__ = [
+    "quant_llm_linear",
+    "fp6_quantize_pack",
+    "fp6_dequantize",
+    "fp6_repack",
+    "fp6_linear_native",
     "int4wo_linear_residual",
     "int4wo_swiglu",
     "rmsnorm",
@@ -34,6 +41,12 @@ _LIB.define("int4wo_linear_residual(Tensor x, Tensor packed, Tensor qparams, int
 _LIB.define("int4wo_swiglu(Tensor x, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
 _LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
 _LIB.define("llama_decode_attention(Tensor qkv, Tensor freqs_cis, Tensor input_pos, Tensor(a!) k_cache, Tensor(b!) v_cache, int n_head, int n_kv) -> Tensor")
+# schema of the reference op, verbatim (torchao/csrc/fp6_llm.cpp:7)
+_LIB.define("quant_llm_linear(int EXPONENT, int MANTISSA, Tensor _in_feats, Tensor _weights, Tensor _scales, int splitK) -> Tensor")
+_LIB.define("fp6_quantize_pack(Tensor w, int ebits, int mbits) -> (Tensor, Tensor)")
+_LIB.define("fp6_dequantize(Tensor fpx_data, Tensor? scale, int ebits, int mbits) -> Tensor")
+_LIB.define("fp6_repack(Tensor fpx_data) -> Tensor")
+_LIB.define("fp6_linear_native(int ebits, int mbits, Tensor x, Tensor native, Tensor scale) -> Tensor")
 
 
 def int4wo_packed_shapes(N: int, K: int, group_size: int):
@@ -196,6 +209,101 @@ def _decode_attention_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, 
     return out
 
 
+# ------------------------------------------------------------------------------------ FP6-LLM
+
+def _fp6_native_numel(N: int, K: int) -> int:
+    return (N // 16) * ((K + 127) // 128) * 384  # int32 words: 1536 bytes per 16-row x 128-k tile
+
+
+def _check_fp6_format(ebits, mbits):
+    torch._check((ebits, mbits) in ((3, 2), (2, 3)),
+                 lambda: f"FP{1 + ebits + mbits} E{ebits}M{mbits} is not supported (6-bit formats e3m2 and e2m3 only)")
+
+
+def _fp6_quantize_pack_cuda(w, ebits, mbits):
+    require_cuda(w)
+    _check_fp6_format(ebits, mbits)
+    torch._check(w.dim() == 2, lambda: f"weight should be a 2d tensor, got {w.dim()}D")
+    torch._check(w.dtype in (torch.float32, torch.bfloat16, torch.float16), lambda: f"unsupported weight dtype {w.dtype}")
+    N, K = w.shape
+    torch._check(N % 64 == 0 and K % 64 == 0, lambda: f"TC-FPx packing needs multiples of 64, got ({N}, {K})")
+    w = w.contiguous()
+    data = torch.empty((N, K // 8 * 6), dtype=torch.uint8, device=w.device)
+    scale = torch.empty((N,), dtype=torch.float16, device=w.device)
+    check(lib().ao_amd_fp6_quantize_pack(w.data_ptr(), DTYPE_CODE[w.dtype], N, K, ebits, mbits, data.data_ptr(),
+                                         scale.data_ptr(), current_stream(w.device)))
+    return data, scale
+
+
+def _fp6_dequantize_cuda(fpx_data, scale, ebits, mbits):
+    require_cuda(fpx_data, scale)
+    _check_fp6_format(ebits, mbits)
+    torch._check(fpx_data.dim() == 2 and fpx_data.dtype is torch.uint8, lambda: "fpx_data must be a 2d uint8 tensor")
+    N, K = fpx_data.shape[0], fpx_data.shape[1] // 6 * 8
+    if scale is not None:
+        torch._check(scale.dtype is torch.float16 and scale.numel() == N, lambda: "scale must be float16 of size N")
+        scale = scale.contiguous()
+    out = torch.empty((N, K), dtype=torch.float32, device=fpx_data.device)
+    check(lib().ao_amd_fp6_dequantize(fpx_data.contiguous().data_ptr(), None if scale is None else scale.data_ptr(), N, K,
+                                      ebits, mbits, out.data_ptr(), current_stream(fpx_data.device)))
+    return out
+
+
+def _fp6_repack_cuda(fpx_data):
+    require_cuda(fpx_data)
+    torch._check(fpx_data.dim() == 2 and fpx_data.dtype is torch.uint8, lambda: "fpx_data must be a 2d uint8 tensor")
+    N, K = fpx_data.shape[0], fpx_data.shape[1] // 6 * 8
+    native = torch.empty((_fp6_native_numel(N, K),), dtype=torch.int32, device=fpx_data.device)
+    check(lib().ao_amd_fp6_repack(fpx_data.contiguous().data_ptr(), N, K, native.data_ptr(),
+                                  current_stream(fpx_data.device)))
+    return native
+
+
+def _fp6_linear_native_cuda(ebits, mbits, x, native, scale):
+    require_cuda(x, native, scale)
+    _check_fp6_format(ebits, mbits)
+    torch._check(x.dim() == 2, lambda: f"input should be a 2d tensor, got {x.dim()}D")
+    torch._check(x.dtype is torch.float16, lambda: f"weight must be FP16, got {x.dtype}")
+    torch._check(scale.dim() == 1 and scale.dtype is torch.float16, lambda: "scale must be a 1d FP16 tensor")
+    M, K = x.shape
+    N = scale.shape[0]
+    torch._check(native.dtype is torch.int32 and native.numel() == _fp6_native_numel(N, K), lambda: "Dimensions mismatched")
+    out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    check(lib().ao_amd_fp6_linear(x.contiguous().data_ptr(), M, K, native.data_ptr(), scale.contiguous().data_ptr(), N,
+                                  ebits, mbits, out.data_ptr(), current_stream(x.device)))
+    return out
+
+
+# quant_llm_linear takes the TC-FPx bytes on every call (torchao/ops.py:15-37); the kernel wants the native
+# order, so the repack is cached per weight tensor object (weak reference) and version counter.  A new tensor
+# object, even one that reuses a freed address, never hits a stale entry.
+_REPACK_CACHE = {}
+
+
+def _quant_llm_linear_cuda(EXPONENT, MANTISSA, _in_feats, _weights, _scales, splitK):
+    # splitK is a tuning hint for the reference's NVIDIA kernel; this kernel sizes its own K split
+    torch._check(_weights.dim() == 2 and _weights.dtype is torch.uint8, lambda: f"weight must be UINT8, got {_weights.dtype}")
+    torch._check(_in_feats.dim() == 2 and _in_feats.shape[1] // 8 * (1 + EXPONENT + MANTISSA) == _weights.shape[1],
+                 lambda: "Dimensions mismatched")
+    torch._check(_weights.shape[0] == _scales.shape[0], lambda: "Dimensions mismatched")
+    key = id(_weights)
+    entry = _REPACK_CACHE.get(key)
+    if entry is not None and entry[0]() is _weights and entry[1] == (_weights._version, _weights.data_ptr()):
+        native = entry[2]
+    else:
+        if len(_REPACK_CACHE) >= 256:
+            _REPACK_CACHE.clear()
+        native = _fp6_repack_cuda(_weights)
+        _REPACK_CACHE[key] = (weakref.ref(_weights, lambda _, k=key: _REPACK_CACHE.pop(k, None)),
+                              (_weights._version, _weights.data_ptr()), native)
+    return _fp6_linear_native_cuda(EXPONENT, MANTISSA, _in_feats, native, _scales)
+
+
+_LIB.impl("fp6_quantize_pack", _fp6_quantize_pack_cuda, "CUDA")
+_LIB.impl("fp6_dequantize", _fp6_dequantize_cuda, "CUDA")
+_LIB.impl("fp6_repack", _fp6_repack_cuda, "CUDA")
+_LIB.impl("fp6_linear_native", _fp6_linear_native_cuda, "CUDA")
+_LIB.impl("quant_llm_linear", _quant_llm_linear_cuda, "CUDA")
 _LIB.impl("int4wo_linear_residual", _linear_residual_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu", _swiglu_cuda, "CUDA")
 _LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
@@ -214,7 +322,8 @@ def _no_cpu(name):
 
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
-              "int4wo_linear_residual", "int4wo_swiglu", "rmsnorm", "llama_decode_attention"):
+              "int4wo_linear_residual", "int4wo_swiglu", "rmsnorm", "llama_decode_attention", "quant_llm_linear",
+              "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
 
@@ -274,7 +383,73 @@ def _(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv):
     return qkv.new_empty((1, n_head * k_cache.shape[3]))
 
 
+@torch.library.register_fake("torchao::quant_llm_linear")
+def _(EXPONENT, MANTISSA, _in_feats, _weights, _scales, splitK=1):
+    # same checks as the reference's fake impl (torchao/ops.py:40-55)
+    torch._check(_in_feats.dim() == 2, lambda: f"input should be a 2d tensor, got {_in_feats.dim()}D")
+    torch._check(_in_feats.dtype is torch.float16, lambda: f"weight must be FP16, got {_in_feats.dtype}")
+    torch._check(_weights.dim() == 2, lambda: f"weight should be a 2d tensor, got {_weights.dim()}D")
+    torch._check(_weights.dtype is torch.uint8, lambda: f"weight must be UINT8, got {_weights.dtype}")
+    torch._check(_scales.dim() == 1, lambda: f"scale should be a 2d tensor, got {_scales.dim()}D")
+    torch._check(_scales.dtype is torch.float16, lambda: f"scale must be FP16, got {_scales.dtype}")
+    BS, IC = _in_feats.shape
+    OC, _ = _weights.shape
+    torch._check(IC // 8 * (1 + EXPONENT + MANTISSA) == _weights.shape[1], lambda: "Dimensions mismatched")
+    torch._check(OC == _scales.shape[0], lambda: "Dimensions mismatched")
+    return _in_feats.new_empty((BS, OC))
+
+
+@torch.library.register_fake("torchao::fp6_quantize_pack")
+def _(w, ebits, mbits):
+    return (w.new_empty((w.shape[0], w.shape[1] // 8 * 6), dtype=torch.uint8),
+            w.new_empty((w.shape[0],), dtype=torch.float16))
+
+
+@torch.library.register_fake("torchao::fp6_dequantize")
+def _(fpx_data, scale, ebits, mbits):
+    return fpx_data.new_empty((fpx_data.shape[0], fpx_data.shape[1] // 6 * 8), dtype=torch.float32)
+
+
+@torch.library.register_fake("torchao::fp6_repack")
+def _(fpx_data):
+    return fpx_data.new_empty((_fp6_native_numel(fpx_data.shape[0], fpx_data.shape[1] // 6 * 8),), dtype=torch.int32)
+
+
+@torch.library.register_fake("torchao::fp6_linear_native")
+def _(ebits, mbits, x, native, scale):
+    return x.new_empty((x.shape[0], scale.shape[0]))
+
+
 # ------------------------------------------------------------------------------------ python wrappers
+
+def quant_llm_linear(EXPONENT: int, MANTISSA: int, _in_feats: Tensor, _weights: Tensor, _scales: Tensor,
+                     splitK: int = 1) -> Tensor:
+    """Quant-LLM linear layer A @ W.T (https://arxiv.org/abs/2401.14112), same signature as torchao/ops.py:15-37.
+
+    _in_feats: FP16 activations [B, IC]; _weights: packed FPx weights in the TC-FPx layout [OC, IC/8*nbits];
+    _scales: FP16 [OC]; splitK is accepted for compatibility and not used."""
+    return torch.ops.torchao.quant_llm_linear.default(EXPONENT, MANTISSA, _in_feats, _weights, _scales, splitK)
+
+
+def fp6_quantize_pack(w: Tensor, ebits: int, mbits: int):
+    """float [N,K] -> (TC-FPx bytes uint8 [N, K*6/8], fp16 row scales [N])."""
+    return torch.ops.torchao.fp6_quantize_pack.default(w, ebits, mbits)
+
+
+def fp6_dequantize(fpx_data: Tensor, scale, ebits: int, mbits: int) -> Tensor:
+    """TC-FPx bytes (+ optional fp16 row scales) -> fp32 [N,K]."""
+    return torch.ops.torchao.fp6_dequantize.default(fpx_data, scale, ebits, mbits)
+
+
+def fp6_repack(fpx_data: Tensor) -> Tensor:
+    """TC-FPx bytes -> the kernel's wave64 tile order (int32 words)."""
+    return torch.ops.torchao.fp6_repack.default(fpx_data)
+
+
+def fp6_linear_native(ebits: int, mbits: int, x: Tensor, native: Tensor, scale: Tensor) -> Tensor:
+    """x fp16 [M,K] @ W^T with W given in the native tile order -> fp16 [M,N]."""
+    return torch.ops.torchao.fp6_linear_native.default(ebits, mbits, x, native, scale)
+
 
 def int4wo_linear_residual(x, packed, qparams, group_size, N, residual, bias=None):
     """bf16( bf16(x W^T + bias) + residual ) in one launch."""

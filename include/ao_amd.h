@@ -136,6 +136,36 @@ int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* freqs_cis_bf
                                   void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim, int64_t max_seq,
                                   void* out_bf16, void* stream);
 
+/* ---------------------------------------------------------------- FP6-LLM (Quant-LLM FPx, e3m2 / e2m2 ...)
+ * Interchange format = the reference's TC-FPx bytes, bit for bit. */
+
+/* replaces to_scaled_tc_fpx, torchao/prototype/quant_llm/quant_llm.py:116-130 for 6-bit formats
+ * (ebits + mbits == 5): per-row scale = amax|w| / max_normal (fp32) stored as fp16, codes =
+ * _f32_to_fpx_unpacked(w / scale) (torchao/prototype/custom_fp_utils.py:27-140), bytes = _pack_tc_fp6
+ * (quant_llm.py:90-106).  w: [N,K] of w_dtype (AO_F32/BF16/F16) contiguous; N % 64 == 0, K % 64 == 0.
+ * out_tc: uint8 [N, K*6/8]; out_scale: fp16 [N]. */
+int ao_amd_fp6_quantize_pack(const void* w, int w_dtype, int64_t N, int64_t K, int ebits, int mbits, void* out_tc,
+                             void* out_scale_f16, void* stream);
+
+/* replaces from_scaled_tc_fpx, torchao/prototype/quant_llm/quant_llm.py:203-208 (6-bit formats):
+ * out fp32 [N,K] = fpx_to_f32(unpack(tc)) * float(scale) (scale may be NULL). */
+int ao_amd_fp6_dequantize(const void* tc, const void* scale_f16, int64_t N, int64_t K, int ebits, int mbits,
+                          float* out, void* stream);
+
+/* One-time device repack of the TC-FP6 bytes into the kernel's wave64 order (no counterpart in the reference, whose
+ * kernel reads the TC bytes directly with 32-lane fragment loads):
+ *   native: per 16-row x 128-k tile 1536 bytes = [64 lanes][4 dwords] then [64 lanes][2 dwords]; lane l owns row
+ *   16*rb + l%16 and the 32 consecutive k = 128*kb + 32*(l/16) + i, value i at bit 6*i of its 6 dwords; K is padded
+ *   with zero codes to a multiple of 128.  ao_amd_fp6_native_bytes gives the buffer size. */
+int ao_amd_fp6_native_bytes(int64_t N, int64_t K, int64_t* bytes);
+int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, void* native, void* stream);
+
+/* out[M,N] fp16 = x[M,K] fp16 @ W^T with W = fp16(fp6 value * scale), fp32 accumulation.
+ * replaces torchao::quant_llm_linear, schema torchao/csrc/fp6_llm.cpp:7, CUDA implementation
+ * torchao/csrc/cuda/fp6_llm/fp6_linear.cu:139-196.  `weights_native` is the output of ao_amd_fp6_repack. */
+int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
+                      int64_t N, int ebits, int mbits, void* out_f16, void* stream);
+
 /* Measurement aid (no counterpart in the reference): arm a (hipEvent_t start, hipEvent_t stop) pair on the
  * calling thread; the next ao_amd_int4wo_linear launch records its kernel's own begin / end timestamps into
  * the pair and disarms, so hipEventElapsedTime(start, stop) is the kernel duration free of launch gaps.

@@ -1,0 +1,128 @@
+"""GPU parity tests of the FP6-LLM path through the C ABI / ops: quantize+pack bit-exact against the oracle
+(which is pinned to the reference's packer and cast tables), dequantize bit-exact, linear within the reference
+test's tolerance (mean relative error < 1e-3, test/test_ops.py:47-62) and the north star's 1e-3 relative L2."""
+import numpy as np
+import pytest
+import torch
+
+from _util import bits16, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    assert torch.cuda.is_available()
+    return torch.device("cuda:0")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(64, 64), (256, 128), (512, 1024)])
+def test_quantize_pack_bit_exact(oracle, shape, dtype):
+    from ao_amd import ops
+
+    N, K = shape
+    print(f"case fp6 quantize_pack N={N} K={K} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(N + K)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(dtype)
+    w[1, :] = 0          # all-zero row: scale clamps at 1e-12 / 28
+    w[2, 5] = 3.0        # outlier
+    data, scale = ops.fp6_quantize_pack(w.to(_dev()), 3, 2)
+    code = {torch.float32: oracle.F32, torch.bfloat16: oracle.BF16, torch.float16: oracle.F16}[dtype]
+    wn = w.numpy() if dtype is torch.float32 else bits16(w)
+    codes_ref, scale_ref = oracle.fpx_quantize(wn, code, 3, 2)
+    packed_ref = oracle.pack_tc_fp6(codes_ref)
+    assert np.array_equal(bits16(scale), scale_ref)
+    assert np.array_equal(data.cpu().numpy(), packed_ref)
+
+
+def test_dequantize_and_repack_round_trip(oracle):
+    from ao_amd import ops
+
+    dev = _dev()
+    rng = np.random.default_rng(3)
+    N, K = 128, 192
+    codes = rng.integers(0, 64, (N, K), dtype=np.uint8)
+    scale = (rng.random(N) * 0.01 + 1e-3).astype(np.float16)
+    packed = oracle.pack_tc_fp6(codes)
+    pd = torch.from_numpy(packed).to(dev)
+    sd = torch.from_numpy(scale).to(dev)
+    out = ops.fp6_dequantize(pd, sd, 3, 2).cpu().numpy()
+    ref = oracle.fpx_to_f32(codes, 3, 2) * scale.astype(np.float32)[:, None]
+    assert np.array_equal(out, ref)
+    out_noscale = ops.fp6_dequantize(pd, None, 3, 2).cpu().numpy()
+    assert np.array_equal(out_noscale, oracle.fpx_to_f32(codes, 3, 2))
+    # native order: value i of lane (row%16, k%128/32) at bit 6*i, K padded to 256 with zero codes
+    native = ops.fp6_repack(pd).cpu().numpy().view(np.uint32).reshape(N // 16, 2, 384)
+    for (row, k) in [(0, 0), (5, 7), (17, 33), (127, 191), (64, 100), (31, 127), (40, 128)]:
+        tile = native[row // 16, k // 128]
+        lane = (row % 16) + 16 * ((k % 128) // 32)
+        words = np.concatenate([tile[lane * 4: lane * 4 + 4], tile[256 + lane * 2: 256 + lane * 2 + 2]])
+        big = sum(int(wd) << (32 * j) for j, wd in enumerate(words))
+        assert (big >> (6 * (k % 32))) & 63 == codes[row, k]
+    assert np.all(native[:, 1, :].reshape(-1, 384)[:, :0] == 0)
+
+
+@pytest.mark.parametrize("M", [1, 2, 16, 40])
+@pytest.mark.parametrize("shape", [(256, 1024), (2048, 4096), (512, 192)])
+def test_linear_matches_oracle(oracle, shape, M):
+    """Shapes include the reference op test's (BS, OC, IC) = (1, 2048, 4096) (test/test_ops.py:49-51); inputs as there:
+    activations rand + 0.5, random bytes as weights, scales rand + 0.5."""
+    from ao_amd import ops
+
+    N, K = shape
+    print(f"case fp6 linear N={N} K={K} M={M}", flush=True)
+    dev = _dev()
+    g = torch.Generator().manual_seed(N * 3 + K + M)
+    x = (torch.rand(M, K, generator=g) + 0.5).half()
+    packed = torch.randint(0, 256, (N, K // 8 * 6), dtype=torch.uint8, generator=g)
+    scale = (torch.rand(N, generator=g) + 0.5).half()
+    y = ops.quant_llm_linear(3, 2, x.to(dev), packed.to(dev), scale.to(dev), 1).float().cpu().numpy()
+    codes = oracle.unpack_tc_fp6(packed.numpy(), N, K)
+    y_ref = oracle.fpx_linear(bits16(x), codes, bits16(scale), 3, 2)
+    y_ref16 = y_ref.astype(np.float16).astype(np.float32)
+    assert rel_l2(y, y_ref16) <= 1e-3
+    rel = np.abs(y - y_ref16) / np.maximum(np.abs(y_ref16), 1e-6)
+    assert rel.mean() < 1e-3
+
+
+def test_e2m3_format(oracle):
+    from ao_amd import ops
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(11)
+    N, K = 256, 256
+    w = (torch.randn(N, K, generator=g) * 0.05)
+    data, scale = ops.fp6_quantize_pack(w.to(dev), 2, 3)
+    codes_ref, scale_ref = oracle.fpx_quantize(w.numpy(), oracle.F32, 2, 3)
+    assert np.array_equal(data.cpu().numpy(), oracle.pack_tc_fp6(codes_ref))
+    assert np.array_equal(bits16(scale), scale_ref)
+    x = torch.randn(3, K, generator=g).half()
+    y = ops.quant_llm_linear(2, 3, x.to(dev), data, scale, 1).float().cpu().numpy()
+    y_ref = oracle.fpx_linear(bits16(x), codes_ref, scale_ref, 2, 3).astype(np.float16).astype(np.float32)
+    assert rel_l2(y, y_ref) <= 1e-3
+
+
+def test_weight_subclass_and_api(oracle):
+    """quantize(model, fp6_llm_weight_only()): shapes the kernel cannot take stay float; forward matches the oracle;
+    leading dims and bias work (test/prototype/test_quant_llm.py:68-99)."""
+    import ao_amd
+    from ao_amd.prototype.quant_llm import QuantLlmLinearWeight
+
+    dev = _dev()
+    torch.manual_seed(0)
+    m = torch.nn.Sequential(torch.nn.Linear(256, 512, bias=True), torch.nn.Linear(512, 100, bias=False)).half().to(dev)
+    w0 = m[0].weight.detach().clone()
+    ao_amd.quantize(m, ao_amd.fp6_llm_weight_only())
+    assert isinstance(m[0].weight, QuantLlmLinearWeight) and m[0].weight.shape == (512, 256)
+    assert not isinstance(m[1].weight, QuantLlmLinearWeight)  # 100 outputs: not a multiple of 256
+    x = torch.randn(2, 3, 256, device=dev).half()
+    with torch.no_grad():
+        y = m[0](x)
+    assert y.shape == (2, 3, 512) and y.dtype is torch.float16
+    codes, scale = oracle.fpx_quantize(bits16(w0), oracle.F16, 3, 2)
+    y_ref = oracle.fpx_linear(bits16(x.reshape(-1, 256)), codes, scale, 3, 2).astype(np.float16).astype(np.float32)
+    y_ref = (torch.from_numpy(y_ref).half() + m[0].bias.detach().cpu()).float().numpy()
+    assert rel_l2(y.float().cpu().numpy().reshape(-1, 512), y_ref) <= 2e-3
+    dq = m[0].weight.dequantize(torch.float32).cpu().numpy()
+    ref = oracle.fpx_to_f32(codes, 3, 2) * scale.view(np.float16).astype(np.float32)[:, None]
+    assert np.array_equal(dq, ref)
