@@ -1,6 +1,7 @@
 // Shared host/device helpers for the gfx950 weight-only quantized linear kernels.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
@@ -28,6 +29,12 @@ char* last_error_buf();  // thread-local, 512 bytes
         hipError_t e_ = hipGetLastError();                                              \
         if (e_ != hipSuccess) AO_FAIL(-2, "kernel launch failed: %s", hipGetErrorString(e_)); \
     } while (0)
+
+// Optional per-kernel timing shared by the linear launchers: when a (start, stop) event pair has been armed on
+// this thread (ao_amd_profile_next_linear), the next linear launch records the kernel's own begin / end
+// timestamps into it (hipExtLaunchKernelGGL) and disarms; hipEventElapsedTime(start, stop) is then the
+// kernel's execution time without launch gaps.
+extern thread_local hipEvent_t g_prof_start, g_prof_stop;
 
 inline bool is_float_dtype(int d) { return d == AO_F32 || d == AO_BF16 || d == AO_F16; }
 inline int dtype_size(int d) {

@@ -368,9 +368,13 @@ extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const 
     const uint32_t* nat = (const uint32_t*)weights_native;
     const uint16_t* sc = (const uint16_t*)scale_f16;
     uint16_t* o = (uint16_t*)out_f16;
-#define AO_FP6_LAUNCH(W)                                                                                             \
-    if (ebits == 3) hipLaunchKernelGGL((fp6_linear_kernel<W, true>), grid, dim3(W * 64), 0, st, xx, M, K, nat, sc, N, Kp, o); \
-    else hipLaunchKernelGGL((fp6_linear_kernel<W, false>), grid, dim3(W * 64), 0, st, xx, M, K, nat, sc, N, Kp, o)
+    hipEvent_t ev0 = g_prof_start, ev1 = g_prof_stop;  // optional per-kernel timing, see common.h
+    g_prof_start = g_prof_stop = nullptr;
+#define AO_FP6_LAUNCH(W)                                                                                                 \
+    if (ebits == 3)                                                                                                      \
+        hipExtLaunchKernelGGL((fp6_linear_kernel<W, true>), grid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o); \
+    else                                                                                                                 \
+        hipExtLaunchKernelGGL((fp6_linear_kernel<W, false>), grid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o)
     switch (waves) {
         case 1: AO_FP6_LAUNCH(1); break;
         case 2: AO_FP6_LAUNCH(2); break;

@@ -15,7 +15,6 @@
 //   u  = T.lo*1 + T.hi*0 + z  /  T.lo*0 + T.hi*1 + z   fp32 add of the bf16 operands  (2 v_dot2_f32_bf16)
 //   W  = cvt_pk_bf16(u0, u1)                           second rounding                (1 v_cvt_pk_bf16_f32)
 #include "common.h"
-#include <hip/hip_ext.h>
 
 namespace ao {
 
@@ -604,10 +603,129 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     }
 }
 
-// Optional per-kernel timing: when a (start, stop) event pair has been armed on this thread, the next
-// linear launch records the kernel's own begin / end timestamps into it (hipExtLaunchKernelGGL) and
-// disarms.  hipEventElapsedTime(start, stop) is then the kernel's execution time without launch gaps.
-static thread_local hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;
+// ---------------------------------------------------------------- GEMM path (M > 16)
+// Workgroup tile: 128 activation rows x 128 weight rows, K walked in 128-wide tiles.  Each of the 4 waves owns
+// two 16-row weight blocks: it loads their packed tiles straight into registers, dequantizes every dword once
+// and multiplies it against all eight 16-row activation blocks (16 MFMAs per pair of dequantized dwords), so
+// the dequantization cost is spread over 128 activation rows.  The activation tile goes through LDS (row
+// stride 272 bytes: the 16-byte fragment reads of 8 consecutive lanes fall on distinct banks) and is fetched
+// one K tile ahead into registers.
+template <int G>
+__global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a) {
+    constexpr int BM = 128, XSTRIDE = 136;  // bf16 elements per LDS row
+    __shared__ __align__(16) uint16_t xs[BM * XSTRIDE];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, qd = lane >> 4;
+    const int KB = (int)(a.Kp / 128);
+    const int64_t nblocks = (a.N + 15) / 16;
+    const int64_t nb0 = (int64_t)blockIdx.x * 8 + 2 * wave;
+    const bool has0 = nb0 < nblocks, has1 = nb0 + 1 < nblocks;
+    const int64_t m0 = (int64_t)blockIdx.y * BM;
+    const uint32_t magic = 0x43004300u, one_lo = 0x00003F80u, one_hi = 0x3F800000u;
+
+    // activation tile loader: thread t covers rows (t>>4) + 16*j, 16-byte chunk t&15 of the 256-byte row slice
+    const int xrow = tid >> 4, xchunk = tid & 15;
+    uint4 xr[8];
+    auto load_x = [&](int kb) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int64_t m = m0 + xrow + 16 * j;
+            xr[j] = make_uint4(0, 0, 0, 0);
+            if (m < a.M) xr[j] = *reinterpret_cast<const uint4*>(a.x + m * a.ldx + (int64_t)kb * 128 + xchunk * 8);
+        }
+    };
+    auto store_x = [&]() {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            *reinterpret_cast<uint4*>(xs + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
+    };
+
+    struct WBuf { u32x4_t w0, w1; uint32_t q0, q1; };
+    const uint4* wp0 = a.packed + (has0 ? nb0 : 0) * KB * 64 + lane;
+    const uint4* wp1 = a.packed + (has1 ? nb0 + 1 : 0) * KB * 64 + lane;
+    const uint32_t* qp0 = a.qparams + (has0 ? nb0 : 0) * (a.Kp / G) * 16 + r;
+    const uint32_t* qp1 = a.qparams + (has1 ? nb0 + 1 : 0) * (a.Kp / G) * 16 + r;
+    auto load_w = [&](WBuf& b, int kb) {
+        const int gidx = ((kb * 128 + qd * 32) / G) * 16;
+        b.w0 = *reinterpret_cast<const u32x4_t*>(wp0 + (int64_t)kb * 64);
+        b.w1 = *reinterpret_cast<const u32x4_t*>(wp1 + (int64_t)kb * 64);
+        b.q0 = qp0[gidx];
+        b.q1 = qp1[gidx];
+    };
+
+    f32x4_t acc0[8], acc1[8];
+#pragma unroll
+    for (int mb = 0; mb < 8; ++mb) {
+        acc0[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        acc1[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    auto compute = [&](const WBuf& b) {
+        const GroupConst g0 = make_group(b.q0), g1 = make_group(b.q1);
+        const uint32_t w0[4] = {b.w0.x, b.w0.y, b.w0.z, b.w0.w};
+        const uint32_t w1[4] = {b.w1.x, b.w1.y, b.w1.z, b.w1.w};
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            const bf16x8_t bw0 = dequant8(w0[sl], g0, magic, one_lo, one_hi);
+            const bf16x8_t bw1 = dequant8(w1[sl], g1, magic, one_lo, one_hi);
+#pragma unroll
+            for (int mb = 0; mb < 8; ++mb) {
+                union { uint4 q; bf16x8_t v; } xa;
+                xa.q = *reinterpret_cast<const uint4*>(xs + (mb * 16 + r) * XSTRIDE + qd * 32 + sl * 8);
+                acc0[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw0, acc0[mb], 0, 0, 0);
+                acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw1, acc1[mb], 0, 0, 0);
+            }
+        }
+    };
+
+    WBuf b0, b1;
+    load_x(0);
+    load_w(b0, 0);
+    for (int kb = 0; kb < KB; kb += 2) {
+        __syncthreads();
+        store_x();
+        __syncthreads();
+        if (kb + 1 < KB) { load_x(kb + 1); load_w(b1, kb + 1); }
+        compute(b0);
+        if (kb + 1 < KB) {
+            __syncthreads();
+            store_x();
+            __syncthreads();
+            if (kb + 2 < KB) { load_x(kb + 2); load_w(b0, kb + 2); }
+            compute(b1);
+        }
+    }
+
+    // acc[mb][i] = C[m = m0 + 16*mb + 4*qd + i][n = 16*nb + r]
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        if (!(h == 0 ? has0 : has1)) continue;
+        const int64_t n = (nb0 + h) * 16 + r;
+        if (n >= a.N) continue;
+        const float bv = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.f;
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t m = m0 + mb * 16 + 4 * qd + i;
+                if (m < a.M) {
+                    const float v = (h == 0 ? acc0[mb][i] : acc1[mb][i]) + bv;
+                    if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = v;
+                    else ((uint16_t*)a.y)[m * a.ldy + n] = f32_to_bf16_bits(v);
+                }
+            }
+    }
+}
+
+template <typename Kernel>
+static void launch_timed(Kernel kernel, dim3 grid, dim3 block, size_t smem, hipStream_t st, const LinearArgs& a) {
+    if (g_prof_start && g_prof_stop) {
+        hipExtLaunchKernelGGL(kernel, grid, block, smem, st, g_prof_start, g_prof_stop, 0, a);
+        g_prof_start = g_prof_stop = nullptr;
+        return;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, smem, st, a);
+}
 
 template <int G, int WAVES, int XMODE, bool DUAL>
 static void launch_one(dim3 grid, size_t smem, hipStream_t st, const LinearArgs& a) {
@@ -699,8 +817,20 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     LinearArgs a{(const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams,
                  (const uint4*)packed2, (const uint32_t*)qparams2, N, Kp, (const uint16_t*)bias_bf16,
                  (const uint16_t*)residual_bf16, ldres, y, y_dtype == AO_F32, ldy};
-    dim3 grid((unsigned)RB, (unsigned)mchunks);
     hipStream_t st = (hipStream_t)stream;
+    if (M > 16 && aligned && !dual && !residual_bf16) {
+        dim3 ggrid((unsigned)((RB + 7) / 8), (unsigned)((M + 127) / 128));
+        AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
+        switch (g) {
+            case 32: launch_timed(int4wo_gemm_kernel<32>, ggrid, dim3(256), 0, st, a); break;
+            case 64: launch_timed(int4wo_gemm_kernel<64>, ggrid, dim3(256), 0, st, a); break;
+            case 128: launch_timed(int4wo_gemm_kernel<128>, ggrid, dim3(256), 0, st, a); break;
+            default: launch_timed(int4wo_gemm_kernel<256>, ggrid, dim3(256), 0, st, a); break;
+        }
+        AO_LAUNCH_CHECK();
+        return 0;
+    }
+    dim3 grid((unsigned)RB, (unsigned)mchunks);
     const size_t smem = xmode == X_LDS ? xbytes : 0;
     if (dual) {
         if (xmode == X_LDS) launch_gemv<true>(g, waves, grid, smem, st, a);

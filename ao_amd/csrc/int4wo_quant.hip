@@ -7,6 +7,8 @@
 
 namespace ao {
 
+thread_local hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;
+
 char* last_error_buf() {
     static thread_local char buf[512] = {0};
     return buf;

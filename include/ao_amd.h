@@ -167,7 +167,7 @@ int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weigh
                       int64_t N, int ebits, int mbits, void* out_f16, void* stream);
 
 /* Measurement aid (no counterpart in the reference): arm a (hipEvent_t start, hipEvent_t stop) pair on the
- * calling thread; the next ao_amd_int4wo_linear launch records its kernel's own begin / end timestamps into
+ * calling thread; the next linear launch (int4wo or fp6) records its kernel's own begin / end timestamps into
  * the pair and disarms, so hipEventElapsedTime(start, stop) is the kernel duration free of launch gaps.
  * Pass NULLs to disarm. */
 int ao_amd_profile_next_linear(void* start_event, void* stop_event);

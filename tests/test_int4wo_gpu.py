@@ -196,6 +196,27 @@ def test_linear_matches_oracle(cabi, oracle, shape, g, M):
     assert err16 <= REL_L2_TOL
 
 
+@pytest.mark.parametrize("g", [32, 64, 128, 256])
+@pytest.mark.parametrize("case", [(272, 1024, 200), (128, 512, 128), (1040, 2048, 333), (100, 256, 17)])
+def test_linear_gemm_path(cabi, oracle, case, g):
+    """M > 16 goes through the LDS-tiled GEMM kernel: ragged N (not a multiple of 128 or 16), ragged M, bias."""
+    N, K, M = case
+    print(f"case gemm N={N} K={K} M={M} g={g}", flush=True)
+    w = make_weight(N, K, seed=77 + N + g)
+    x = make_act(M, K, seed=M + K + 1)
+    bias = (torch.randn(N) * 0.1).bfloat16()
+    dev = _dev()
+    packed, qparams, _, _ = _quantize_pack(cabi, w.to(dev), g)
+    _, y_ref = _oracle_linear(oracle, w, x, g, bias)
+    y32 = _linear(cabi, x.to(dev), packed, qparams, N, g, bias=bias.to(dev), fp32=True).cpu().numpy()
+    err = rel_l2(y32, y_ref)
+    print(f"  rel_l2 fp32-out = {err:.3e}", flush=True)
+    assert err <= REL_L2_TOL
+    y16 = _linear(cabi, x.to(dev), packed, qparams, N, g, bias=bias.to(dev), fp32=False)
+    y_ref16 = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(y_ref))
+    assert rel_l2(y16.float().cpu().numpy(), y_ref16) <= REL_L2_TOL
+
+
 def test_linear_rejects_bad_arguments(cabi):
     dev = _dev()
     x = torch.zeros(1, 128, dtype=torch.bfloat16, device=dev)
