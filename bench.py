@@ -118,7 +118,7 @@ def roofline_leg(model, passes=3):
     achieved = total_bytes / total_us / 1e3  # GB/s
     return {
         "bound": "hbm",
-        "kernel": "ao::int4wo_linear_kernel (M=1, g=64)",
+        "kernel": "ao::int4wo_gemv_kernel (M=1, g=64)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
@@ -131,12 +131,27 @@ def roofline_leg(model, passes=3):
 
 
 def _traffic_from_profile():
-    """HBM bytes per launch from the committed rocprofv3 --pmc summary, if one exists."""
-    path = os.path.join(ROOT, "profiles", "int4wo_gemv_decode_traffic.json")
+    """HBM bytes per launch of the GEMV kernel from the committed rocprofv3 --pmc summary (its
+    'traffic_bytes_per_launch:' line), if one exists."""
+    path = os.path.join(ROOT, "profiles", "int4wo_gemv_llama3_8b_decode_pmc.txt")
     if os.path.exists(path):
         with open(path) as f:
-            return json.load(f).get("traffic_bytes_per_launch")
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return int(float(line.split(":", 1)[1]))
     return None
+
+
+def copy_calibration(mib=256):
+    """One elementwise copy kernel of known size (reads and writes `mib` MiB) for scaling the FETCH_SIZE /
+    WRITE_SIZE counters of a rocprofv3 --pmc run of this script."""
+    import torch
+
+    src = torch.ones(mib << 18, dtype=torch.float32, device="cuda:0")
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    torch.add(src, 1.0, out=dst)
+    torch.cuda.synchronize()
 
 
 def cpu_baseline_leg(config, group=64, min_seconds=10.0):
@@ -179,6 +194,90 @@ def cpu_baseline_leg(config, group=64, min_seconds=10.0):
     }
 
 
+MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 MFMA, published
+
+SWEEP_ROTATE_BYTES = 640 << 20  # the sweeps rotate over weight copies totalling at least this much
+LLAMA3_8B_SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)]  # (N, K)
+
+
+def _time_linear(L, launch, iters):
+    """Median of the kernel's own duration (us) over `iters` armed launches; launch(i) is given the iteration
+    number so that it can rotate over copies of the weight (each launch then reads HBM, not the last-level cache)."""
+    import torch
+
+    timer = KernelTimer(iters)
+    for i in range(3):
+        launch(i)
+    for i in range(iters):
+        L.ao_amd_profile_next_linear(timer.pairs[i][0], timer.pairs[i][1])
+        launch(i + 3)
+    torch.cuda.synchronize()
+    durs = sorted(timer.elapsed_us(i) for i in range(iters))
+    timer.close()
+    return durs[len(durs) // 2]
+
+
+def sweep(kind, iters=15):
+    """Per-kernel lines for the shapes of the other benchmark configurations: int4 GEMV (M in 1, 4; g in 64, 128),
+    int4 GEMM (M in 16 .. 2048, g=64) and the FP6 e3m2 linear (M in 1, 16, 128); one JSON line per case."""
+    import torch
+
+    from ao_amd import _lib
+
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device=dev).manual_seed(0)
+    if kind in ("gemv", "gemm"):
+        cases = ([(N, K, M, g) for (N, K) in LLAMA3_8B_SHAPES for g in (64, 128) for M in (1, 4)] if kind == "gemv" else
+                 [(N, K, M, 64) for (N, K) in LLAMA3_8B_SHAPES for M in (16, 128, 512, 2048) if N * M < 1 << 28])
+        for N, K, M, g in cases:
+            _, _, pb, qb = _lib.packed_shape(N, K, g)
+            w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).bfloat16()
+            copies = max(2, -(-SWEEP_ROTATE_BYTES // pb))
+            packed = torch.empty(copies, pb // 4, dtype=torch.int32, device=dev)
+            qp = torch.empty(copies, qb // 4, dtype=torch.int32, device=dev)
+            _lib.check(L.ao_amd_int4wo_quantize_pack(w.data_ptr(), N, K, K, g, packed.data_ptr(), qp.data_ptr(), st))
+            packed[1:] = packed[0]
+            qp[1:] = qp[0]
+            x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
+            y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+            us = _time_linear(L, lambda i: _lib.check(L.ao_amd_int4wo_linear(
+                x.data_ptr(), M, K, K, packed[i % copies].data_ptr(), qp[i % copies].data_ptr(), N, g, None,
+                y.data_ptr(), _lib.BF16, N, st)), iters)
+            gbs = int4wo_bytes(N, K, g, M) / us / 1e3
+            tfs = 2.0 * M * N * K / us / 1e6
+            print(json.dumps({"kernel": "int4wo_linear", "N": N, "K": K, "M": M, "group": g, "us": round(us, 2),
+                              "GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+                              "TFLOPs": round(tfs, 2), "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
+            del w, packed, qp, x, y
+    elif kind == "fp6":
+        for N, K in [(4096, 4096), (14336, 4096), (4096, 14336)]:
+            w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).half()
+            tc = torch.empty(N * K * 3 // 4, dtype=torch.uint8, device=dev)
+            sc = torch.empty(N, dtype=torch.float16, device=dev)
+            _lib.check(L.ao_amd_fp6_quantize_pack(w.data_ptr(), _lib.F16, N, K, 3, 2, tc.data_ptr(), sc.data_ptr(), st))
+            nbytes = ctypes.c_int64()
+            _lib.check(L.ao_amd_fp6_native_bytes(N, K, ctypes.byref(nbytes)))
+            copies = max(2, -(-SWEEP_ROTATE_BYTES // nbytes.value))
+            native = torch.empty(copies, nbytes.value, dtype=torch.uint8, device=dev)
+            _lib.check(L.ao_amd_fp6_repack(tc.data_ptr(), N, K, native.data_ptr(), st))
+            native[1:] = native[0]
+            for M in (1, 16, 128):
+                x = torch.randn(M, K, device=dev, generator=gen).half()
+                y = torch.empty(M, N, dtype=torch.float16, device=dev)
+                us = _time_linear(L, lambda i: _lib.check(L.ao_amd_fp6_linear(
+                    x.data_ptr(), M, K, native[i % copies].data_ptr(), sc.data_ptr(), N, 3, 2, y.data_ptr(), st)), iters)
+                gbs = (N * K * 0.75 + 2 * N + 2 * M * K + 2 * M * N) / us / 1e3
+                tfs = 2.0 * M * N * K / us / 1e6
+                print(json.dumps({"kernel": "fp6_linear_e3m2", "N": N, "K": K, "M": M, "us": round(us, 2),
+                                  "GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+                                  "TFLOPs": round(tfs, 2), "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
+            del w, tc, native
+    else:
+        sys.exit(f"unknown sweep {kind}")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -189,9 +288,21 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=128)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="build the model, run one pass of the roofline leg and a copy kernel of known size, no decode "
+                         "loop: the command to put under rocprofv3 --pmc")
+    ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6"), default=None,
+                    help="instead of the decode benchmark, print one line per kernel case of the named sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.sweep:
+        import torch
+
+        assert torch.cuda.is_available(), "bench.py needs the GPU"
+        torch.cuda.set_device(0)
+        sweep(args.sweep)
+        return
 
     import torch
 
@@ -206,6 +317,11 @@ def main():
     model = build_random_model(args.model, device, quant)
     cfg = model.config
     model_size = get_model_size_in_bytes(model, ignore_embeddings=True)
+
+    if args.roofline_only:
+        copy_calibration()
+        print(json.dumps({"roofline": roofline_leg(model, passes=1)}), flush=True)
+        return
 
     gen = torch.Generator(device=device).manual_seed(0)
     prompt = torch.randint(0, cfg.vocab_size, (args.prompt_len,), device=device, dtype=torch.int, generator=gen)
