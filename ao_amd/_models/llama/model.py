@@ -229,8 +229,8 @@ class Transformer(nn.Module):
         return len(groups) == 1 and self.tok_embeddings.weight.dtype is torch.bfloat16
 
     def _fused_decode(self, idx: Tensor, input_pos: Tensor) -> Tensor:
-        """One token, batch 1: seven launches per layer (norm, qkv, attention, wo + residual, norm,
-        gate/up + SwiGLU, down + residual).  Same roundings as the module-by-module path."""
+        """One token, batch 1: five launches per layer (norm + qkv, attention, wo + residual, norm + gate/up +
+        SwiGLU, down + residual).  Same roundings as the module-by-module path."""
         from ... import ops
 
         cfg = self.config
@@ -245,15 +245,15 @@ class Transformer(nn.Module):
         pos = input_pos.to(torch.int32) if input_pos.dtype is not torch.int32 else input_pos
         for b in self.layers:
             att = b.attention
-            xn = ops.rmsnorm(x, b.attention_norm.weight, b.attention_norm.eps)
-            qkv = lin(xn, att.wqkv)
+            qw = att.wqkv.weight.layout_tensor
+            qkv = ops.int4wo_rmsnorm_linear(x, b.attention_norm.weight, b.attention_norm.eps, qw.packed_weight,
+                                            qw.scale_and_zero, qw.group_size, qw.N)
             y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
                                            cfg.n_head, cfg.n_local_heads)
             h = lin(y, att.wo, residual=x)
-            hn = ops.rmsnorm(h, b.ffn_norm.weight, b.ffn_norm.eps)
             g, u = b.feed_forward.w1.weight.layout_tensor, b.feed_forward.w3.weight.layout_tensor
-            ff = ops.int4wo_swiglu(hn, g.packed_weight, g.scale_and_zero, u.packed_weight, u.scale_and_zero,
-                                   g.group_size, g.N)
+            ff = ops.int4wo_rmsnorm_swiglu(h, b.ffn_norm.weight, b.ffn_norm.eps, g.packed_weight, g.scale_and_zero,
+                                           u.packed_weight, u.scale_and_zero, g.group_size, g.N)
             x = lin(ff, b.feed_forward.w2, residual=h)
         xn = ops.rmsnorm(x, self.norm.weight, self.norm.eps)
         return lin(xn, self.output).view(1, 1, cfg.vocab_size)

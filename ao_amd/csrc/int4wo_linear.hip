@@ -189,6 +189,7 @@ struct LinearArgs {
     const uint16_t* bias;                              // [N] or null
     const uint16_t* residual; int64_t ldres;           // [M,N] or null
     void* y; int y_is_f32; int64_t ldy;
+    const uint16_t* norm_w; float norm_eps;            // GEMV only: RMSNorm weight [K] applied to x while staging, or null
 };
 
 __device__ __forceinline__ float silu_bf16(float a) {
@@ -542,9 +543,63 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
         // stage the activation rows of this chunk: rows x Kp bf16, 16 bytes per thread per step
         const int rows = (int)((a.M - m0) < 16 ? (a.M - m0) : 16);
         const int chunks_per_row = (int)(a.Kp / 8);
-        for (int i = threadIdx.x; i < rows * chunks_per_row; i += WAVES * 64) {
-            const int rr = i / chunks_per_row, c = i - rr * chunks_per_row;
-            reinterpret_cast<uint4*>(xs)[i] = reinterpret_cast<const uint4*>(a.x + (m0 + rr) * a.ldx)[c];
+        if (a.norm_w == nullptr) {
+            for (int i = threadIdx.x; i < rows * chunks_per_row; i += WAVES * 64) {
+                const int rr = i / chunks_per_row, c = i - rr * chunks_per_row;
+                reinterpret_cast<uint4*>(xs)[i] = reinterpret_cast<const uint4*>(a.x + (m0 + rr) * a.ldx)[c];
+            }
+        } else {
+            // RMSNorm fused into the staging (torchao/_models/llama/model.py:232-244): the row's mean square in fp32,
+            // then bf16(bf16(x * rsqrt(ms + eps)) * w).  The first two chunks of a thread stay in registers
+            // between the two passes; a longer row is read again (cache hits).
+            __shared__ float norm_part[WAVES];
+            constexpr int T = WAVES * 64;
+            const int tid = threadIdx.x;
+            const uint4* wrow = reinterpret_cast<const uint4*>(a.norm_w);
+            auto sumsq = [](const uint4& v) {
+                const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+                float t = 0.f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float lo = __uint_as_float(u[j] << 16), hi = __uint_as_float(u[j] & 0xffff0000u);
+                    t += lo * lo + hi * hi;
+                }
+                return t;
+            };
+            auto scaled = [](const uint4& v, const uint4& g, float rs) {
+                const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+                const uint32_t gw[4] = {g.x, g.y, g.z, g.w};
+                uint32_t o[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float lo = rne_bf16(__uint_as_float(u[j] << 16) * rs) * __uint_as_float(gw[j] << 16);
+                    const float hi = rne_bf16(__uint_as_float(u[j] & 0xffff0000u) * rs) * __uint_as_float(gw[j] & 0xffff0000u);
+                    o[j] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+                }
+                return make_uint4(o[0], o[1], o[2], o[3]);
+            };
+            for (int rr = 0; rr < rows; ++rr) {
+                const uint4* xrow = reinterpret_cast<const uint4*>(a.x + (m0 + rr) * a.ldx);
+                uint4* orow = reinterpret_cast<uint4*>(xs) + rr * chunks_per_row;
+                const bool h0 = tid < chunks_per_row, h1 = tid + T < chunks_per_row;
+                uint4 v0 = make_uint4(0, 0, 0, 0), v1 = v0, g0 = v0, g1 = v0;
+                if (h0) { v0 = xrow[tid]; g0 = wrow[tid]; }
+                if (h1) { v1 = xrow[tid + T]; g1 = wrow[tid + T]; }
+                float ss = sumsq(v0) + sumsq(v1);
+                for (int c = tid + 2 * T; c < chunks_per_row; c += T) ss += sumsq(xrow[c]);
+#pragma unroll
+                for (int o = 32; o >= 1; o >>= 1) ss += __shfl_xor(ss, o, 64);
+                if (lane == 0) norm_part[wave] = ss;
+                __syncthreads();
+                float tot = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) tot += norm_part[w];
+                const float rs = rsqrtf(tot / (float)a.K + a.norm_eps);
+                if (h0) orow[tid] = scaled(v0, g0, rs);
+                if (h1) orow[tid + T] = scaled(v1, g1, rs);
+                for (int c = tid + 2 * T; c < chunks_per_row; c += T) orow[c] = scaled(xrow[c], wrow[c], rs);
+                if (rr + 1 < rows) __syncthreads();  // norm_part is rewritten for the next row
+            }
         }
         __syncthreads();
     }
@@ -789,7 +844,8 @@ static void launch_group(int64_t g, int waves, dim3 grid, size_t smem, hipStream
 
 static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed, const void* qparams,
                            const void* packed2, const void* qparams2, int64_t N, int64_t g, const void* bias_bf16,
-                           const void* residual_bf16, int64_t ldres, void* y, int y_dtype, int64_t ldy, void* stream) {
+                           const void* residual_bf16, int64_t ldres, void* y, int y_dtype, int64_t ldy, void* stream,
+                           const void* norm_weight_bf16 = nullptr, float norm_eps = 0.f) {
     AO_REQUIRE(x_bf16 && packed && qparams && y, "null pointer argument");
     AO_REQUIRE(M >= 0, "negative batch");
     AO_REQUIRE(y_dtype == AO_BF16 || y_dtype == AO_F32, "output dtype must be bf16 or f32, got code %d", y_dtype);
@@ -816,9 +872,14 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     int xmode = aligned ? (xbytes <= (size_t)waves * 10 * 1024 ? X_LDS : X_GLOBAL) : X_CHECKED;
     LinearArgs a{(const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams,
                  (const uint4*)packed2, (const uint32_t*)qparams2, N, Kp, (const uint16_t*)bias_bf16,
-                 (const uint16_t*)residual_bf16, ldres, y, y_dtype == AO_F32, ldy};
+                 (const uint16_t*)residual_bf16, ldres, y, y_dtype == AO_F32, ldy,
+                 (const uint16_t*)norm_weight_bf16, norm_eps};
     hipStream_t st = (hipStream_t)stream;
-    if (M > 16 && aligned && !dual && !residual_bf16) {
+    // the fused RMSNorm lives in the activation staging of the GEMV kernel only
+    AO_REQUIRE(!norm_weight_bf16 || (xmode == X_LDS && M <= 16 && (((uintptr_t)norm_weight_bf16) & 15) == 0),
+               "fused rmsnorm needs M <= 16, K a multiple of max(128, group), 16-byte aligned rows and norm weight, and "
+               "activations that fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);
+    if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16) {
         dim3 ggrid((unsigned)((RB + 7) / 8), (unsigned)((M + 127) / 128));
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
         switch (g) {
@@ -877,4 +938,22 @@ extern "C" int ao_amd_int4wo_swiglu(const void* x_bf16, int64_t M, int64_t K, in
     AO_REQUIRE(packed_up && qparams_up, "null pointer argument");
     return linear_dispatch(x_bf16, M, K, ldx, packed_gate, qparams_gate, packed_up, qparams_up, N, g, nullptr, nullptr, 0,
                            y_bf16, AO_BF16, ldy, stream);
+}
+
+extern "C" int ao_amd_int4wo_rmsnorm_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx,
+                                            const void* norm_weight_bf16, float eps, const void* packed,
+                                            const void* qparams, int64_t N, int64_t g, const void* bias_bf16, void* y,
+                                            int y_dtype, int64_t ldy, void* stream) {
+    AO_REQUIRE(norm_weight_bf16, "null pointer argument");
+    return linear_dispatch(x_bf16, M, K, ldx, packed, qparams, nullptr, nullptr, N, g, bias_bf16, nullptr, 0, y, y_dtype,
+                           ldy, stream, norm_weight_bf16, eps);
+}
+
+extern "C" int ao_amd_int4wo_rmsnorm_swiglu(const void* x_bf16, int64_t M, int64_t K, int64_t ldx,
+                                            const void* norm_weight_bf16, float eps, const void* packed_gate,
+                                            const void* qparams_gate, const void* packed_up, const void* qparams_up,
+                                            int64_t N, int64_t g, void* y_bf16, int64_t ldy, void* stream) {
+    AO_REQUIRE(norm_weight_bf16 && packed_up && qparams_up, "null pointer argument");
+    return linear_dispatch(x_bf16, M, K, ldx, packed_gate, qparams_gate, packed_up, qparams_up, N, g, nullptr, nullptr, 0,
+                           y_bf16, AO_BF16, ldy, stream, norm_weight_bf16, eps);
 }

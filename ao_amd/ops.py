@@ -21,6 +21,8 @@ __all__ = [
     "fp6_linear_native",
     "int4wo_linear_residual",
     "int4wo_swiglu",
+    "int4wo_rmsnorm_linear",
+    "int4wo_rmsnorm_swiglu",
     "rmsnorm",
     "llama_decode_attention",
     "int4wo_quantize_pack",
@@ -39,6 +41,8 @@ _LIB.define("int4wo_dequantize(Tensor packed, Tensor qparams, int N, int K, int 
 _LIB.define("int4wo_linear(Tensor x, Tensor packed, Tensor qparams, int group_size, int N, Tensor? bias, bool fp32_out) -> Tensor")
 _LIB.define("int4wo_linear_residual(Tensor x, Tensor packed, Tensor qparams, int group_size, int N, Tensor? bias, Tensor residual) -> Tensor")
 _LIB.define("int4wo_swiglu(Tensor x, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
+_LIB.define("int4wo_rmsnorm_linear(Tensor x, Tensor norm_weight, float eps, Tensor packed, Tensor qparams, int group_size, int N, Tensor? bias) -> Tensor")
+_LIB.define("int4wo_rmsnorm_swiglu(Tensor x, Tensor norm_weight, float eps, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
 _LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
 _LIB.define("llama_decode_attention(Tensor qkv, Tensor freqs_cis, Tensor input_pos, Tensor(a!) k_cache, Tensor(b!) v_cache, int n_head, int n_kv) -> Tensor")
 # schema of the reference op, verbatim (torchao/csrc/fp6_llm.cpp:7)
@@ -178,6 +182,47 @@ def _swiglu_cuda(x, packed_gate, qparams_gate, packed_up, qparams_up, group_size
     return y
 
 
+def _check_norm(x, norm_weight):
+    torch._check(x.dim() == 2 and x.dtype is torch.bfloat16, lambda: "input must be a 2d bfloat16 tensor")
+    torch._check(norm_weight.dtype is torch.bfloat16 and norm_weight.numel() == x.shape[1] and norm_weight.is_contiguous(),
+                 lambda: "norm weight must be a contiguous bfloat16 vector of the input's row length")
+
+
+def _rmsnorm_linear_cuda(x, norm_weight, eps, packed, qparams, group_size, N, bias):
+    """linear(rmsnorm(x)) in one launch; decode shapes only (the library rejects the others)."""
+    require_cuda(x, norm_weight, packed, qparams, bias)
+    _check_norm(x, norm_weight)
+    M, K = x.shape
+    _check_packed(packed, qparams, N, K, group_size)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    if bias is not None:
+        torch._check(bias.dtype is torch.bfloat16 and bias.numel() == N, lambda: "bias must be bfloat16 of size N")
+        bias = bias.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    check(lib().ao_amd_int4wo_rmsnorm_linear(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, norm_weight.data_ptr(),
+                                             float(eps), packed.data_ptr(), qparams.data_ptr(), N, group_size,
+                                             None if bias is None else bias.data_ptr(), y.data_ptr(), BF16, N,
+                                             current_stream(x.device)))
+    return y
+
+
+def _rmsnorm_swiglu_cuda(x, norm_weight, eps, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
+    require_cuda(x, norm_weight, packed_gate, qparams_gate, packed_up, qparams_up)
+    _check_norm(x, norm_weight)
+    M, K = x.shape
+    _check_packed(packed_gate, qparams_gate, N, K, group_size)
+    _check_packed(packed_up, qparams_up, N, K, group_size)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    check(lib().ao_amd_int4wo_rmsnorm_swiglu(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, norm_weight.data_ptr(),
+                                             float(eps), packed_gate.data_ptr(), qparams_gate.data_ptr(),
+                                             packed_up.data_ptr(), qparams_up.data_ptr(), N, group_size, y.data_ptr(), N,
+                                             current_stream(x.device)))
+    return y
+
+
 def _rmsnorm_cuda(x, weight, eps):
     require_cuda(x, weight)
     torch._check(x.dtype is torch.bfloat16 and weight.dtype is torch.bfloat16, lambda: "rmsnorm needs bfloat16 tensors")
@@ -306,6 +351,8 @@ _LIB.impl("fp6_linear_native", _fp6_linear_native_cuda, "CUDA")
 _LIB.impl("quant_llm_linear", _quant_llm_linear_cuda, "CUDA")
 _LIB.impl("int4wo_linear_residual", _linear_residual_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu", _swiglu_cuda, "CUDA")
+_LIB.impl("int4wo_rmsnorm_linear", _rmsnorm_linear_cuda, "CUDA")
+_LIB.impl("int4wo_rmsnorm_swiglu", _rmsnorm_swiglu_cuda, "CUDA")
 _LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
 _LIB.impl("llama_decode_attention", _decode_attention_cuda, "CUDA")
 _LIB.impl("int4wo_quantize_pack", _quantize_pack_cuda, "CUDA")
@@ -322,7 +369,7 @@ def _no_cpu(name):
 
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
-              "int4wo_linear_residual", "int4wo_swiglu", "rmsnorm", "llama_decode_attention", "quant_llm_linear",
+              "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "rmsnorm", "llama_decode_attention", "quant_llm_linear",
               "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
@@ -370,6 +417,16 @@ def _(x, packed, qparams, group_size, N, bias, residual):
 
 @torch.library.register_fake("torchao::int4wo_swiglu")
 def _(x, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
+    return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::int4wo_rmsnorm_linear")
+def _(x, norm_weight, eps, packed, qparams, group_size, N, bias):
+    return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::int4wo_rmsnorm_swiglu")
+def _(x, norm_weight, eps, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
     return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
 
 
@@ -459,6 +516,17 @@ def int4wo_linear_residual(x, packed, qparams, group_size, N, residual, bias=Non
 def int4wo_swiglu(x, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
     """silu(x W_gate^T) * (x W_up^T) in one launch (both weights [N,K], same group size)."""
     return torch.ops.torchao.int4wo_swiglu.default(x, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N)
+
+
+def int4wo_rmsnorm_linear(x, norm_weight, eps: float, packed, qparams, group_size, N, bias=None):
+    """linear(rmsnorm(x, norm_weight, eps)) in one launch, for M <= 16 rows (decode)."""
+    return torch.ops.torchao.int4wo_rmsnorm_linear.default(x, norm_weight, eps, packed, qparams, group_size, N, bias)
+
+
+def int4wo_rmsnorm_swiglu(x, norm_weight, eps: float, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
+    """swiglu(rmsnorm(x, norm_weight, eps)) in one launch, for M <= 16 rows (decode)."""
+    return torch.ops.torchao.int4wo_rmsnorm_swiglu.default(x, norm_weight, eps, packed_gate, qparams_gate, packed_up,
+                                                           qparams_up, group_size, N)
 
 
 def rmsnorm(x, weight, eps: float):

@@ -122,6 +122,19 @@ int ao_amd_int4wo_swiglu(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, 
                          const void* qparams_gate, const void* packed_up, const void* qparams_up, int64_t N, int64_t g,
                          void* y_bf16, int64_t ldy, void* stream);
 
+/* The same two products with RMSNorm applied to the activation rows while they are staged:
+ * x' = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * norm_weight ) (RMSNorm.forward, torchao/_models/llama/model.py:232-244),
+ * then linear / SwiGLU of x' as above: `self.attention(self.attention_norm(x), ...)` and
+ * `self.feed_forward(self.ffn_norm(h))` of TransformerBlock.forward, model.py:160-163, in one launch each.
+ * Decode shapes only: M <= 16, K a multiple of max(128, group), 16-byte aligned rows and norm weight, M*K*2 bytes
+ * within the kernel's LDS staging (40 KB at K = 4096 .. 160 KB); anything else is rejected with an error. */
+int ao_amd_int4wo_rmsnorm_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* norm_weight_bf16,
+                                 float eps, const void* packed, const void* qparams, int64_t N, int64_t g,
+                                 const void* bias_bf16, void* y, int y_dtype, int64_t ldy, void* stream);
+int ao_amd_int4wo_rmsnorm_swiglu(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* norm_weight_bf16,
+                                 float eps, const void* packed_gate, const void* qparams_gate, const void* packed_up,
+                                 const void* qparams_up, int64_t N, int64_t g, void* y_bf16, int64_t ldy, void* stream);
+
 /* ---------------------------------------------------------------- Llama decode harness kernels (bf16)
  * out[rows,dim] = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * weight ): RMSNorm.forward,
  * torchao/_models/llama/model.py:232-244. */

@@ -78,6 +78,55 @@ def test_rmsnorm_matches_module():
     assert np.count_nonzero(out != ref) <= 0.02 * out.size
 
 
+@pytest.mark.parametrize("M,N,K,g", [(1, 6144, 4096, 64), (1, 512, 1024, 128), (3, 256, 2048, 32), (16, 64, 512, 256)])
+def test_rmsnorm_linear_fused(M, N, K, g):
+    """linear(rmsnorm(x)) in one launch against the two separate launches.  The statistics are summed in a
+    different order, which can move the normalised activation by one bf16 ulp on rare elements: the outputs agree
+    to 1e-3 relative L2 (fp32 comparison of bf16 results) and most are identical."""
+    from ao_amd import ops
+
+    dev = _dev()
+    w = make_weight(N, K, seed=41).to(dev)
+    x = (make_act(M, K, seed=42) * 3).to(dev)
+    nw = (1 + 0.1 * torch.randn(K, generator=torch.Generator().manual_seed(43))).bfloat16().to(dev)
+    packed, qp = ops.int4wo_quantize_pack(w, g)
+    xn = ops.rmsnorm(x, nw, 1e-5)
+    ref = ops.int4wo_linear(xn, packed, qp, g, N).float().cpu().numpy()
+    out = ops.int4wo_rmsnorm_linear(x, nw, 1e-5, packed, qp, g, N).float().cpu().numpy()
+    assert rel_l2(out, ref) <= 1e-3
+    assert np.count_nonzero(out != ref) <= 0.05 * out.size
+
+
+@pytest.mark.parametrize("M", [1, 4])
+def test_rmsnorm_swiglu_fused(M):
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K, g = 1024, 4096, 64
+    wg = make_weight(N, K, seed=51).to(dev)
+    wu = make_weight(N, K, seed=52).to(dev)
+    x = (make_act(M, K, seed=53) * 0.5).to(dev)
+    nw = (1 + 0.1 * torch.randn(K, generator=torch.Generator().manual_seed(54))).bfloat16().to(dev)
+    pg, qg = ops.int4wo_quantize_pack(wg, g)
+    pu, qu = ops.int4wo_quantize_pack(wu, g)
+    xn = ops.rmsnorm(x, nw, 1e-5)
+    ref = ops.int4wo_swiglu(xn, pg, qg, pu, qu, g, N).float().cpu().numpy()
+    out = ops.int4wo_rmsnorm_swiglu(x, nw, 1e-5, pg, qg, pu, qu, g, N).float().cpu().numpy()
+    assert rel_l2(out, ref) <= 1e-3
+    assert np.count_nonzero(out != ref) <= 0.05 * out.size
+
+
+def test_rmsnorm_linear_rejects_prefill_shapes():
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K, g = 64, 512, 64
+    packed, qp = ops.int4wo_quantize_pack(make_weight(N, K, seed=61).to(dev), g)
+    nw = torch.ones(K, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="fused rmsnorm"):
+        ops.int4wo_rmsnorm_linear(make_act(17, K, seed=62).to(dev), nw, 1e-5, packed, qp, g, N)
+
+
 @pytest.mark.parametrize("pos", [0, 5, 130])
 def test_decode_attention_matches_module_math(pos):
     """fp32 restatement of Attention.forward for one token (RoPE on interleaved pairs, cache update,
