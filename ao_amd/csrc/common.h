@@ -78,6 +78,24 @@ __device__ __forceinline__ float rd(int dtype, float v) {
 }
 __device__ __forceinline__ float rne_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
+// The same rounding by the hardware converter (v_cvt_pk_bf16_f32, one instruction): identical for every
+// finite value and infinity; a NaN stays a NaN but keeps its sign and payload bits instead of becoming 0x7FC0.
+// Used on the hot paths, where a NaN input is already a NaN output.
+__device__ __forceinline__ uint16_t hw_bf16_bits(float f) {
+    const __bf16 b = (__bf16)f;
+    uint16_t u;
+    __builtin_memcpy(&u, &b, 2);
+    return u;
+}
+__device__ __forceinline__ float hw_rne_bf16(float v) { return bf16_bits_to_f32(hw_bf16_bits(v)); }
+__device__ __forceinline__ uint32_t hw_bf16_pack(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 p = {(__bf16)lo, (__bf16)hi};
+    uint32_t u;
+    __builtin_memcpy(&u, &p, 4);
+    return u;
+}
+
 __device__ __forceinline__ bool is_float_dt(int d) { return d == AO_F32 || d == AO_BF16 || d == AO_F16; }
 __device__ __forceinline__ int promote(int a, int b) {
     if (!is_float_dt(a)) return b;

@@ -194,7 +194,7 @@ struct LinearArgs {
 
 __device__ __forceinline__ float silu_bf16(float a) {
     // F.silu on a bf16 tensor: computed in fp32, result rounded to bf16
-    return rne_bf16(a / (1.0f + expf(-a)));
+    return hw_rne_bf16(a / (1.0f + expf(-a)));
 }
 
 // How a wave gets its activation fragments (MFMA A operand: row m = lane%16, 8 consecutive k):
@@ -219,6 +219,11 @@ struct TileBuf {
 __device__ __forceinline__ u32x4_t asm_load_b128_nt(const void* sbase, uint32_t voff) {
     u32x4_t v;
     asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    return v;
+}
+__device__ __forceinline__ u32x4_t asm_load_b128(const void* sbase, uint32_t voff) {
+    u32x4_t v;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
     return v;
 }
 __device__ __forceinline__ uint32_t asm_load_b32(const void* sbase, uint32_t voff) {
@@ -536,69 +541,92 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     }
     // tiles of this wave: kb = wave + i*WAVES, i = 0..nt-1; tile i lives in buf[i % D]
     const int nt = wave < KB ? (KB - wave + WAVES - 1) / WAVES : 0;
+
+    // ---- activations -> LDS.  Decode shape (one row that fits two 16-byte chunks per thread): the row is
+    // requested BEFORE the weight prefetch, so it does not queue behind megabytes of weight traffic, and is
+    // waited for with a count that leaves the weight tiles in flight.  Other shapes: plain loads afterwards.
+    constexpr int T = WAVES * 64;
+    const int tid = threadIdx.x;
+    const int rows = (int)((a.M - m0) < 16 ? (a.M - m0) : 16);
+    const int chunks_per_row = (int)(a.Kp / 8);
+    const bool fast_stage = rows == 1 && chunks_per_row <= 2 * T;
+    // The early loads are unconditional (indices clamped into the row, the norm weight replaced by the row itself
+    // when there is none) and so is the wait below: a register that an asm load is still filling must reach its
+    // wait without the compiler merging or copying it on the way, which branches around the loads would invite.
+    const char* xrow0 = reinterpret_cast<const char*>(a.x + m0 * a.ldx);
+    const char* nrow0 = a.norm_w ? reinterpret_cast<const char*>(a.norm_w) : xrow0;
+    const uint32_t ci0 = (uint32_t)(tid < chunks_per_row ? tid : chunks_per_row - 1) * 16;
+    const uint32_t ci1 = (uint32_t)(tid + T < chunks_per_row ? tid + T : chunks_per_row - 1) * 16;
+    u32x4_t xv0 = asm_load_b128(xrow0, ci0);
+    u32x4_t xv1 = asm_load_b128(xrow0, ci1);
+    u32x4_t nv0 = asm_load_b128(nrow0, ci0);
+    u32x4_t nv1 = asm_load_b128(nrow0, ci1);
+    // always D-1 tiles' worth of weight loads (a wave with fewer tiles requests its last one again), so that the
+    // count below is a constant; later waits only ever wait for more than they need because of it
 #pragma unroll
-    for (int j = 0; j < D - 1; ++j)
-        if (j < nt) load_tile(buf[j], wave + j * WAVES);
+    for (int j = 0; j < D - 1; ++j) load_tile(buf[j], wave + (j < nt ? j : (nt > 0 ? nt - 1 : 0)) * WAVES);
+    asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(xv0), "+v"(xv1), "+v"(nv0), "+v"(nv1) : [n] "n"((D - 1) * LPT) : "memory");
     {
-        // stage the activation rows of this chunk: rows x Kp bf16, 16 bytes per thread per step
-        const int rows = (int)((a.M - m0) < 16 ? (a.M - m0) : 16);
-        const int chunks_per_row = (int)(a.Kp / 8);
-        if (a.norm_w == nullptr) {
-            for (int i = threadIdx.x; i < rows * chunks_per_row; i += WAVES * 64) {
-                const int rr = i / chunks_per_row, c = i - rr * chunks_per_row;
-                reinterpret_cast<uint4*>(xs)[i] = reinterpret_cast<const uint4*>(a.x + (m0 + rr) * a.ldx)[c];
+        __shared__ float norm_part[WAVES];
+        auto sumsq = [](const uint4& v) {
+            const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+            float t = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float lo = __uint_as_float(u[j] << 16), hi = __uint_as_float(u[j] & 0xffff0000u);
+                t += lo * lo + hi * hi;
             }
+            return t;
+        };
+        // RMSNorm of one chunk (torchao/_models/llama/model.py:232-244): bf16(bf16(x * rs) * w)
+        auto scaled = [](const uint4& v, const uint4& g, float rs) {
+            const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+            const uint32_t gw[4] = {g.x, g.y, g.z, g.w};
+            uint32_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float lo = hw_rne_bf16(__uint_as_float(u[j] << 16) * rs) * __uint_as_float(gw[j] << 16);
+                const float hi = hw_rne_bf16(__uint_as_float(u[j] & 0xffff0000u) * rs) * __uint_as_float(gw[j] & 0xffff0000u);
+                o[j] = hw_bf16_pack(lo, hi);
+            }
+            return make_uint4(o[0], o[1], o[2], o[3]);
+        };
+        auto block_sum = [&](float ss) {  // the same total in every thread; one barrier
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            if (lane == 0) norm_part[wave] = ss;
+            __syncthreads();
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) tot += norm_part[w];
+            return tot;
+        };
+        if (fast_stage) {
+            uint4 c0 = make_uint4(xv0.x, xv0.y, xv0.z, xv0.w), c1 = make_uint4(xv1.x, xv1.y, xv1.z, xv1.w);
+            if (a.norm_w) {
+                // clamped (duplicate) chunks do not count
+                const float tot = block_sum((tid < chunks_per_row ? sumsq(c0) : 0.f) +
+                                            (tid + T < chunks_per_row ? sumsq(c1) : 0.f));
+                const float rs = rsqrtf(tot / (float)a.K + a.norm_eps);
+                c0 = scaled(c0, make_uint4(nv0.x, nv0.y, nv0.z, nv0.w), rs);
+                c1 = scaled(c1, make_uint4(nv1.x, nv1.y, nv1.z, nv1.w), rs);
+            }
+            if (tid < chunks_per_row) reinterpret_cast<uint4*>(xs)[tid] = c0;
+            if (tid + T < chunks_per_row) reinterpret_cast<uint4*>(xs)[tid + T] = c1;
         } else {
-            // RMSNorm fused into the staging (torchao/_models/llama/model.py:232-244): the row's mean square in fp32,
-            // then bf16(bf16(x * rsqrt(ms + eps)) * w).  The first two chunks of a thread stay in registers
-            // between the two passes; a longer row is read again (cache hits).
-            __shared__ float norm_part[WAVES];
-            constexpr int T = WAVES * 64;
-            const int tid = threadIdx.x;
             const uint4* wrow = reinterpret_cast<const uint4*>(a.norm_w);
-            auto sumsq = [](const uint4& v) {
-                const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-                float t = 0.f;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float lo = __uint_as_float(u[j] << 16), hi = __uint_as_float(u[j] & 0xffff0000u);
-                    t += lo * lo + hi * hi;
-                }
-                return t;
-            };
-            auto scaled = [](const uint4& v, const uint4& g, float rs) {
-                const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-                const uint32_t gw[4] = {g.x, g.y, g.z, g.w};
-                uint32_t o[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float lo = rne_bf16(__uint_as_float(u[j] << 16) * rs) * __uint_as_float(gw[j] << 16);
-                    const float hi = rne_bf16(__uint_as_float(u[j] & 0xffff0000u) * rs) * __uint_as_float(gw[j] & 0xffff0000u);
-                    o[j] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
-                }
-                return make_uint4(o[0], o[1], o[2], o[3]);
-            };
             for (int rr = 0; rr < rows; ++rr) {
                 const uint4* xrow = reinterpret_cast<const uint4*>(a.x + (m0 + rr) * a.ldx);
                 uint4* orow = reinterpret_cast<uint4*>(xs) + rr * chunks_per_row;
-                const bool h0 = tid < chunks_per_row, h1 = tid + T < chunks_per_row;
-                uint4 v0 = make_uint4(0, 0, 0, 0), v1 = v0, g0 = v0, g1 = v0;
-                if (h0) { v0 = xrow[tid]; g0 = wrow[tid]; }
-                if (h1) { v1 = xrow[tid + T]; g1 = wrow[tid + T]; }
-                float ss = sumsq(v0) + sumsq(v1);
-                for (int c = tid + 2 * T; c < chunks_per_row; c += T) ss += sumsq(xrow[c]);
-#pragma unroll
-                for (int o = 32; o >= 1; o >>= 1) ss += __shfl_xor(ss, o, 64);
-                if (lane == 0) norm_part[wave] = ss;
-                __syncthreads();
-                float tot = 0.f;
-#pragma unroll
-                for (int w = 0; w < WAVES; ++w) tot += norm_part[w];
-                const float rs = rsqrtf(tot / (float)a.K + a.norm_eps);
-                if (h0) orow[tid] = scaled(v0, g0, rs);
-                if (h1) orow[tid + T] = scaled(v1, g1, rs);
-                for (int c = tid + 2 * T; c < chunks_per_row; c += T) orow[c] = scaled(xrow[c], wrow[c], rs);
-                if (rr + 1 < rows) __syncthreads();  // norm_part is rewritten for the next row
+                if (a.norm_w == nullptr) {
+                    for (int c = tid; c < chunks_per_row; c += T) orow[c] = xrow[c];
+                } else {
+                    float ss = 0.f;
+                    for (int c = tid; c < chunks_per_row; c += T) ss += sumsq(xrow[c]);
+                    const float rs = rsqrtf(block_sum(ss) / (float)a.K + a.norm_eps);
+                    for (int c = tid; c < chunks_per_row; c += T) orow[c] = scaled(xrow[c], wrow[c], rs);
+                    if (rr + 1 < rows) __syncthreads();  // norm_part is rewritten for the next row
+                }
             }
         }
         __syncthreads();
@@ -646,13 +674,13 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
             const int64_t m = m0 + 4 * qd + i;
             if (m < a.M && n < a.N) {
                 if (DUAL) {
-                    s = rne_bf16(silu_bf16(rne_bf16(s)) * rne_bf16(s2));
+                    s = hw_rne_bf16(silu_bf16(hw_rne_bf16(s)) * hw_rne_bf16(s2));
                 } else {
                     s += bv;
-                    if (a.residual) s = rne_bf16(s) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
+                    if (a.residual) s = hw_rne_bf16(s) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
                 }
                 if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = s;
-                else ((uint16_t*)a.y)[m * a.ldy + n] = f32_to_bf16_bits(s);
+                else ((uint16_t*)a.y)[m * a.ldy + n] = hw_bf16_bits(s);
             }
         }
     }
