@@ -90,29 +90,41 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
     }
 }
 
-// One workgroup (256 threads) per query head; head_dim = 128.
+// One workgroup (1024 threads = 16 waves) per query head; head_dim = 128.
 //   qkv      [ (n_head + 2*n_kv) * 128 ] bf16 : q heads, then k heads, then v heads (the fused wqkv output)
 //   freqs    [max_pos][64][2] bf16 (cos, sin)
 //   k_cache, v_cache [n_kv][S][128] bf16; the new k (rotated) and v are written at row *pos
 //   out      [ n_head * 128 ] bf16
 // Scores, softmax and the weighted sum run in fp32 on the bf16 cache contents.
-__global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t* __restrict__ qkv,
-                                                                const uint16_t* __restrict__ freqs,
-                                                                const int32_t* __restrict__ pos_ptr,
-                                                                uint16_t* __restrict__ k_cache,
-                                                                uint16_t* __restrict__ v_cache, int n_head, int n_kv,
-                                                                int64_t S, uint16_t* __restrict__ out) {
-    constexpr int HD = 128;
+//
+// The step is latency bound (a few hundred KB per head at most), so the kernel is shaped to pay one memory round
+// trip: a group of 16 lanes owns one cache row (16 bytes per lane), the 64 groups of the workgroup cover 64
+// positions per pass, and the K AND V rows of the first 8 passes (512 positions) are all requested at the very
+// start, before the rotary embedding of the new token; longer contexts continue in further chunks of 512.
+constexpr int ATT_THREADS = 1024;
+constexpr int ATT_U = 8;                 // passes per chunk
+constexpr int ATT_CHUNK = 64 * ATT_U;    // positions per chunk
+
+__global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uint16_t* __restrict__ qkv,
+                                                                        const uint16_t* __restrict__ freqs,
+                                                                        const int32_t* __restrict__ pos_ptr,
+                                                                        uint16_t* __restrict__ k_cache,
+                                                                        uint16_t* __restrict__ v_cache, int n_head,
+                                                                        int n_kv, int64_t S, uint16_t* __restrict__ out) {
+    constexpr int HD = 128, U = ATT_U;
     extern __shared__ float smem[];
     float* q_s = smem;             // [128] rotated q (bf16-rounded values)
     float* knew_s = smem + HD;     // [128] rotated new k
     float* vnew_s = smem + 2 * HD; // [128] new v
-    float* red = smem + 3 * HD;    // [8] reductions, then [4][128] partial outputs
-    float* sc = smem + 3 * HD + 8 + 4 * HD;  // [pos + 1] scores
+    float* red = smem + 3 * HD;    // [32] reductions
+    float* po = red + 32;          // [16][128] per-wave partial outputs
+    float* sc = po + 16 * HD;      // [pos + 1] scores, then probabilities
     const int h = blockIdx.x;
     const int rep = n_head / n_kv;
     const int hk = h / rep;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane >> 4, l16 = lane & 15;
+    const int rg = wave * 4 + sub;  // row group 0..63
     const int pos = pos_ptr[0];
     const int T = pos + 1;
 
@@ -121,6 +133,20 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t* _
     const uint16_t* vp = qkv + (int64_t)(n_head + n_kv + hk) * HD;
     uint16_t* kc = k_cache + (int64_t)hk * S * HD;
     uint16_t* vc = v_cache + (int64_t)hk * S * HD;
+
+    // chunk 0 of both caches, requested before anything else (row pos itself comes from qkv, not from the cache:
+    // another workgroup of the same KV head may be writing it right now)
+    uint4 rawk[U], rawv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int t = u * 64 + rg;
+        rawk[u] = make_uint4(0, 0, 0, 0);
+        rawv[u] = make_uint4(0, 0, 0, 0);
+        if (t < pos) {
+            rawk[u] = *reinterpret_cast<const uint4*>(kc + (int64_t)t * HD + l16 * 8);
+            rawv[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)t * HD + l16 * 8);
+        }
+    }
 
     // rotary embedding on pairs (2i, 2i+1), fp32 math, result rounded to bf16 like the module does
     if (tid < 128) {
@@ -137,7 +163,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t* _
             kc[(int64_t)pos * HD + 2 * i] = f32_to_bf16_bits(o0);
             kc[(int64_t)pos * HD + 2 * i + 1] = f32_to_bf16_bits(o1);
         }
-    } else {
+    } else if (tid < 256) {
         const int i = tid - 128;
         const uint16_t v = vp[i];
         vnew_s[i] = bf16_bits_to_f32(v);
@@ -145,9 +171,6 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t* _
     }
     __syncthreads();
 
-    // scores: 16 lanes x 8 elements per position, 16 positions per pass over the workgroup, 4 passes in
-    // flight (all loads of a batch are issued before the first use: the loop is latency bound otherwise)
-    const int sub = lane >> 4, l16 = lane & 15;
     float qreg[8], knew[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -156,19 +179,19 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t* _
     }
     const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
     float lmax = -INFINITY;
-    constexpr int U = 4;
-    for (int t0 = 0; t0 < T; t0 += 16 * U) {
-        uint4 raw[U];
+    for (int t0 = 0; t0 < T; t0 += ATT_CHUNK) {
+        if (t0 > 0) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int t = t0 + u * 16 + wave * 4 + sub;
-            raw[u] = make_uint4(0, 0, 0, 0);
-            if (t < pos) raw[u] = *reinterpret_cast<const uint4*>(kc + (int64_t)t * HD + l16 * 8);
+            for (int u = 0; u < U; ++u) {
+                const int t = t0 + u * 64 + rg;
+                rawk[u] = make_uint4(0, 0, 0, 0);
+                if (t < pos) rawk[u] = *reinterpret_cast<const uint4*>(kc + (int64_t)t * HD + l16 * 8);
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int t = t0 + u * 16 + wave * 4 + sub;
-            const uint32_t w4[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+            const int t = t0 + u * 64 + rg;
+            const uint32_t w4[4] = {rawk[u].x, rawk[u].y, rawk[u].z, rawk[u].w};
             float d = 0.f;
             if (t == pos) {
 #pragma unroll
@@ -192,41 +215,46 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t* _
     lmax = wave_max(lmax);
     if (lane == 0) red[wave] = lmax;
     __syncthreads();
-    const float gmax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float gmax = red[0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) gmax = fmaxf(gmax, red[w]);
     float lsum = 0.f;
-    for (int t = tid; t < T; t += 256) {
+    for (int t = tid; t < T; t += ATT_THREADS) {
         const float p = expf(sc[t] - gmax);
         sc[t] = p;
         lsum += p;
     }
     lsum = wave_sum(lsum);
-    __syncthreads();  // everyone has read red[0..3] and written its p values
-    if (lane == 0) red[4 + wave] = lsum;
-    __syncthreads();
-    const float inv = 1.0f / (red[4] + red[5] + red[6] + red[7]);
+    if (lane == 0) red[16 + wave] = lsum;
+    __syncthreads();  // probabilities and the partial sums are visible
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) tot += red[16 + w];
+    const float inv = 1.0f / tot;
 
-    // out[d] = sum_t p_t * V[t][d]: same thread mapping (position = wave*4 + sub, 8 values of d per lane)
+    // out[d] = sum_t p_t * V[t][d]: same thread mapping (one position per 16-lane group, 8 values of d per lane)
     float oacc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) oacc[e] = 0.f;
-    for (int t0 = 0; t0 < T; t0 += 16 * U) {
-        uint4 raw[U];
+    for (int t0 = 0; t0 < T; t0 += ATT_CHUNK) {
+        if (t0 > 0) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int t = t0 + u * 16 + wave * 4 + sub;
-            raw[u] = make_uint4(0, 0, 0, 0);
-            if (t < pos) raw[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)t * HD + l16 * 8);
+            for (int u = 0; u < U; ++u) {
+                const int t = t0 + u * 64 + rg;
+                rawv[u] = make_uint4(0, 0, 0, 0);
+                if (t < pos) rawv[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)t * HD + l16 * 8);
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int t = t0 + u * 16 + wave * 4 + sub;
+            const int t = t0 + u * 64 + rg;
             if (t < T) {
                 const float p = sc[t];
                 if (t == pos) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) oacc[e] += p * vnew_s[l16 * 8 + e];
                 } else {
-                    const uint32_t w4[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+                    const uint32_t w4[4] = {rawv[u].x, rawv[u].y, rawv[u].z, rawv[u].w};
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         oacc[2 * j] += p * __uint_as_float(w4[j] << 16);
@@ -236,21 +264,22 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t* _
             }
         }
     }
-    // fold the 4 position slots of a wave, then the 4 waves
+    // fold the 4 position slots of a wave, then the 16 waves
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         oacc[e] += __shfl_xor(oacc[e], 16, 64);
         oacc[e] += __shfl_xor(oacc[e], 32, 64);
     }
-    float* po = red + 8;  // [4][128]
     if (sub == 0) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) po[wave * HD + l16 * 8 + e] = oacc[e];
     }
     __syncthreads();
     if (tid < HD) {
-        const float o = (po[tid] + po[HD + tid] + po[2 * HD + tid] + po[3 * HD + tid]) * inv;
-        out[(int64_t)h * HD + tid] = f32_to_bf16_bits(o);
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) o += po[w * HD + tid];
+        out[(int64_t)h * HD + tid] = f32_to_bf16_bits(o * inv);
     }
 }
 
@@ -282,8 +311,8 @@ extern "C" int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* f
     AO_REQUIRE(head_dim == 128, "decode attention kernel is built for head_dim 128, got %d", head_dim);
     AO_REQUIRE(n_kv > 0 && n_head % n_kv == 0, "n_head=%d must be a multiple of n_kv=%d", n_head, n_kv);
     AO_REQUIRE(max_seq > 0 && max_seq <= 8192, "max_seq=%lld outside (0, 8192]", (long long)max_seq);
-    const size_t smem = (size_t)(3 * 128 + 8 + 4 * 128 + max_seq + 8) * sizeof(float);
-    hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head), dim3(256), smem, (hipStream_t)stream,
+    const size_t smem = (size_t)(3 * 128 + 32 + 16 * 128 + max_seq + 8) * sizeof(float);
+    hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head), dim3(ATT_THREADS), smem, (hipStream_t)stream,
                        (const uint16_t*)qkv_bf16, (const uint16_t*)freqs_cis_bf16, pos_dev, (uint16_t*)k_cache,
                        (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16);
     AO_LAUNCH_CHECK();

@@ -127,7 +127,7 @@ def test_rmsnorm_linear_rejects_prefill_shapes():
         ops.int4wo_rmsnorm_linear(make_act(17, K, seed=62).to(dev), nw, 1e-5, packed, qp, g, N)
 
 
-@pytest.mark.parametrize("pos", [0, 5, 130])
+@pytest.mark.parametrize("pos", [0, 5, 130, 511, 512, 700, 1500])
 def test_decode_attention_matches_module_math(pos):
     """fp32 restatement of Attention.forward for one token (RoPE on interleaved pairs, cache update,
     GQA softmax attention); tolerance 1e-2 relative L2 (bf16 inputs and output)."""
@@ -136,9 +136,9 @@ def test_decode_attention_matches_module_math(pos):
 
     dev = _dev()
     torch.manual_seed(pos)
-    n_head, n_kv, hd, S = 8, 2, 128, 256
+    n_head, n_kv, hd, S = 8, 2, 128, (256 if pos < 256 else 2048)   # the kernel walks the cache in chunks of 512
     qkv = torch.randn(1, (n_head + 2 * n_kv) * hd).bfloat16().to(dev)
-    freqs = precompute_freqs_cis(512, hd, 10000, torch.bfloat16, dev)
+    freqs = precompute_freqs_cis(2048, hd, 10000, torch.bfloat16, dev)
     k_cache = torch.randn(1, n_kv, S, hd).bfloat16().to(dev)
     v_cache = torch.randn(1, n_kv, S, hd).bfloat16().to(dev)
     kc, vc = k_cache.clone(), v_cache.clone()
