@@ -37,6 +37,10 @@ def sample(logits, temperature: float = 1.0, top_k: Optional[int] = None, greedy
     """Next token from the last position's logits.  greedy=True is argmax (no random numbers)."""
     if greedy:
         last = logits[0, -1]
+        if last.is_cuda and last.dtype is torch.bfloat16 and last.is_contiguous():
+            from ... import ops
+
+            return ops.argmax_bf16(last), None
         return torch.argmax(last, dim=-1, keepdim=True).to(dtype=torch.int), None
     probs = logits_to_probs(logits[0, -1], temperature, top_k)
     return multinomial_sample_one_no_sync(probs), probs

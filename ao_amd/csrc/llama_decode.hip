@@ -283,6 +283,68 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     }
 }
 
+// Index of the largest of n bf16 values (the lowest such index; a NaN counts as larger than any number), for
+// greedy sampling of one token: torch.argmax on the logits row, generate.py `sample`.  One workgroup; every
+// thread requests all of its 16-byte chunks (up to 16: n <= 131072 elements in one round trip) before the first
+// comparison.
+__global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __restrict__ x, int64_t n,
+                                                            int32_t* __restrict__ out) {
+    __shared__ float bv_s[16];
+    __shared__ int32_t bi_s[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float best = -INFINITY;
+    int32_t besti = 0x7fffffff;
+    auto consider = [&](float v, int32_t i) {
+        const bool vnan = v != v, bnan = best != best;
+        if ((vnan && !bnan) || (!bnan && v > best) || (v == best && i < besti) || (vnan && bnan && i < besti)) {
+            best = v;
+            besti = i;
+        }
+    };
+    const int64_t nchunk = n / 8;
+    const bool vec = (((uintptr_t)x) & 15) == 0;
+    constexpr int MAXC = 16;
+    if (vec) {
+        for (int64_t c0 = 0; c0 < nchunk; c0 += (int64_t)MAXC * 1024) {
+            uint4 raw[MAXC];
+#pragma unroll
+            for (int j = 0; j < MAXC; ++j) {
+                const int64_t c = c0 + (int64_t)j * 1024 + tid;
+                raw[j] = make_uint4(0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u);  // -inf
+                if (c < nchunk) raw[j] = reinterpret_cast<const uint4*>(x)[c];
+            }
+#pragma unroll
+            for (int j = 0; j < MAXC; ++j) {
+                const int64_t c = c0 + (int64_t)j * 1024 + tid;
+                if (c < nchunk) {
+                    const uint32_t u[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        consider(__uint_as_float(u[e] << 16), (int32_t)(c * 8 + 2 * e));
+                        consider(__uint_as_float(u[e] & 0xffff0000u), (int32_t)(c * 8 + 2 * e + 1));
+                    }
+                }
+            }
+        }
+    }
+    for (int64_t i = (vec ? nchunk * 8 : 0) + tid; i < n; i += 1024) consider(bf16_bits_to_f32(x[i]), (int32_t)i);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int32_t oi = __shfl_xor(besti, o, 64);
+        consider(ov, oi);
+    }
+    if (lane == 0) {
+        bv_s[wave] = best;
+        bi_s[wave] = besti;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 16; ++w) consider(bv_s[w], bi_s[w]);
+        out[0] = besti;
+    }
+}
+
 }  // namespace ao
 
 using namespace ao;
@@ -315,6 +377,15 @@ extern "C" int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* f
     hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head), dim3(ATT_THREADS), smem, (hipStream_t)stream,
                        (const uint16_t*)qkv_bf16, (const uint16_t*)freqs_cis_bf16, pos_dev, (uint16_t*)k_cache,
                        (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_argmax_bf16(const void* x_bf16, int64_t n, int32_t* out_index, void* stream) {
+    AO_REQUIRE(x_bf16 && out_index, "null pointer argument");
+    AO_REQUIRE(n > 0 && n < (int64_t)1 << 31, "argmax over n=%lld elements is outside (0, 2^31)", (long long)n);
+    hipLaunchKernelGGL(argmax_bf16_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint16_t*)x_bf16, n,
+                       out_index);
     AO_LAUNCH_CHECK();
     return 0;
 }

@@ -25,6 +25,7 @@ __all__ = [
     "int4wo_rmsnorm_swiglu",
     "rmsnorm",
     "llama_decode_attention",
+    "argmax_bf16",
     "int4wo_quantize_pack",
     "int4wo_pack",
     "int4wo_unpack",
@@ -44,6 +45,7 @@ _LIB.define("int4wo_swiglu(Tensor x, Tensor packed_gate, Tensor qparams_gate, Te
 _LIB.define("int4wo_rmsnorm_linear(Tensor x, Tensor norm_weight, float eps, Tensor packed, Tensor qparams, int group_size, int N, Tensor? bias) -> Tensor")
 _LIB.define("int4wo_rmsnorm_swiglu(Tensor x, Tensor norm_weight, float eps, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
 _LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
+_LIB.define("argmax_bf16(Tensor x) -> Tensor")
 _LIB.define("llama_decode_attention(Tensor qkv, Tensor freqs_cis, Tensor input_pos, Tensor(a!) k_cache, Tensor(b!) v_cache, int n_head, int n_kv) -> Tensor")
 # schema of the reference op, verbatim (torchao/csrc/fp6_llm.cpp:7)
 _LIB.define("quant_llm_linear(int EXPONENT, int MANTISSA, Tensor _in_feats, Tensor _weights, Tensor _scales, int splitK) -> Tensor")
@@ -235,6 +237,15 @@ def _rmsnorm_cuda(x, weight, eps):
     return out
 
 
+def _argmax_bf16_cuda(x):
+    require_cuda(x)
+    torch._check(x.dtype is torch.bfloat16 and x.dim() == 1 and x.is_contiguous() and x.numel() > 0,
+                 lambda: "argmax_bf16 needs a non-empty contiguous 1d bfloat16 tensor")
+    out = torch.empty(1, dtype=torch.int32, device=x.device)
+    check(lib().ao_amd_argmax_bf16(x.data_ptr(), x.numel(), out.data_ptr(), current_stream(x.device)))
+    return out
+
+
 def _decode_attention_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv):
     require_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache)
     torch._check(qkv.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16 and v_cache.dtype is torch.bfloat16
@@ -355,6 +366,7 @@ _LIB.impl("int4wo_rmsnorm_linear", _rmsnorm_linear_cuda, "CUDA")
 _LIB.impl("int4wo_rmsnorm_swiglu", _rmsnorm_swiglu_cuda, "CUDA")
 _LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
 _LIB.impl("llama_decode_attention", _decode_attention_cuda, "CUDA")
+_LIB.impl("argmax_bf16", _argmax_bf16_cuda, "CUDA")
 _LIB.impl("int4wo_quantize_pack", _quantize_pack_cuda, "CUDA")
 _LIB.impl("int4wo_pack", _pack_cuda, "CUDA")
 _LIB.impl("int4wo_unpack", _unpack_cuda, "CUDA")
@@ -369,7 +381,7 @@ def _no_cpu(name):
 
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
-              "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "rmsnorm", "llama_decode_attention", "quant_llm_linear",
+              "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
               "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
@@ -428,6 +440,11 @@ def _(x, norm_weight, eps, packed, qparams, group_size, N, bias):
 @torch.library.register_fake("torchao::int4wo_rmsnorm_swiglu")
 def _(x, norm_weight, eps, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
     return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::argmax_bf16")
+def _(x):
+    return x.new_empty((1,), dtype=torch.int32)
 
 
 @torch.library.register_fake("torchao::rmsnorm")
@@ -532,6 +549,11 @@ def int4wo_rmsnorm_swiglu(x, norm_weight, eps: float, packed_gate, qparams_gate,
 def rmsnorm(x, weight, eps: float):
     """RMSNorm over the last dimension of a bf16 tensor."""
     return torch.ops.torchao.rmsnorm.default(x, weight, eps)
+
+
+def argmax_bf16(x: Tensor) -> Tensor:
+    """int32 [1]: index of the largest element of a 1d bf16 tensor (lowest index among equals)."""
+    return torch.ops.torchao.argmax_bf16.default(x)
 
 
 def llama_decode_attention(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head: int, n_kv: int):

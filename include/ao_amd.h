@@ -149,6 +149,11 @@ int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* freqs_cis_bf
                                   void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim, int64_t max_seq,
                                   void* out_bf16, void* stream);
 
+/* out_index[0] = index of the largest of n bf16 values (lowest index among equals; NaN counts as largest): the greedy
+ * branch of `sample` in the decode harness, torch.argmax over the last position's logits
+ * (torchao/_models/llama/generate.py:34-53 samples from the same logits row). */
+int ao_amd_argmax_bf16(const void* x_bf16, int64_t n, int32_t* out_index, void* stream);
+
 /* ---------------------------------------------------------------- FP6-LLM (Quant-LLM FPx, e3m2 / e2m2 ...)
  * Interchange format = the reference's TC-FPx bytes, bit for bit. */
 

@@ -161,6 +161,22 @@ def test_decode_attention_matches_module_math(pos):
     assert rel_l2(out.float().cpu().numpy(), ref) <= 1e-2
 
 
+@pytest.mark.parametrize("n", [1, 7, 8, 1000, 128256])
+def test_argmax_bf16(n):
+    from ao_amd import ops
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(n, generator=g).bfloat16()
+    if n >= 1000:
+        x[n // 3] = x[n - 5] = x.max() + 1   # a tie: the lower index wins
+    out = ops.argmax_bf16(x.to(dev))
+    assert out.dtype is torch.int32 and out.shape == (1,)
+    xf = x.float()
+    expect = int((xf == xf.max()).nonzero()[0, 0])
+    assert int(out.item()) == expect
+
+
 def test_fused_decode_step_matches_module_path():
     """One decode step of a small quantized model: fused HIP path vs module-by-module forward, same cache
     state.  bf16 model, different summation orders: logits agree to 3e-2 relative L2 and pick the same token."""
