@@ -1,0 +1,139 @@
+"""GPU tests at the full Llama-3-8B sizes, where the scalar CPU oracle would take minutes: size-independent
+properties of the path instead of element-by-element comparison with the oracle.
+
+  * codes stay in [0, 15]; pack / unpack round-trip bit for bit
+  * quantize_affine(dequantized weight, same scale / zero) returns the same codes (the idempotence the reference
+    checks with `check_idempotent`, test/quantization/test_quant_primitives.py:42-47)
+  * the linear with a one-hot activation row returns a column of the dequantized weight, bit for bit
+  * linearity of the fp32-output linear: y(x1) + y(x2) vs y(x1 + x2) with exactly representable sums
+  * the M = 1 kernel, the M <= 16 kernel and the M > 16 kernel agree on the same activation row
+  * FP6: quantize(dequantize(codes)) returns the same bytes; one-hot rows of the linear return weight columns
+"""
+import numpy as np
+import pytest
+import torch
+
+from _util import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(14336, 4096), (4096, 14336), (128256, 4096)]   # (N, K) of w1/w3, w2 and the vocabulary head
+
+
+def _dev():
+    assert torch.cuda.is_available()
+    return torch.device("cuda:0")
+
+
+def _weight(N, K, seed):
+    g = torch.Generator(device=_dev()).manual_seed(seed)
+    return (torch.randn(N, K, device=_dev(), generator=g) * 0.02).bfloat16()
+
+
+@pytest.mark.parametrize("g", [64, 128])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_int4_quantize_properties(shape, g):
+    from ao_amd import ops
+
+    N, K = shape
+    print(f"case int4 full-size N={N} K={K} g={g}", flush=True)
+    w = _weight(N, K, seed=N + g)
+    packed, qp = ops.int4wo_quantize_pack(w, g)
+    codes, scale, zero = ops.int4wo_unpack(packed, qp, N, K, g)
+    assert codes.shape == (N, K) and scale.shape == (N, K // g)
+    assert int(codes.min()) >= 0 and int(codes.max()) <= 15
+    # every group reaches both ends of the range on random data (group min -> 0, group max -> 15)
+    cg = codes.view(N, K // g, g)
+    assert bool((cg.amin(dim=2) == 0).all()) and bool((cg.amax(dim=2) == 15).all())
+    # pack(unpack(.)) reproduces the packed words
+    packed2, qp2 = ops.int4wo_pack(codes, scale, zero, g)
+    assert torch.equal(packed2, packed) and torch.equal(qp2, qp)
+    del packed2, qp2, cg
+    # reconstruction error within half a step (+ bf16 rounding of the result)
+    dq = ops.int4wo_dequantize(packed, qp, N, K, g)
+    step = scale.float().repeat_interleave(g, dim=1)
+    err = (dq.float() - w.float()).abs()
+    assert bool((err <= 0.75 * step + w.float().abs() * 2.0 ** -6 + 1e-6).all())
+    del err, step
+    # dequantized values quantize back to their own codes under the same (scale, zero), and the generic
+    # dequantize_affine primitive agrees with the fused kernel
+    from ao_amd.quantization.quant_primitives import ZeroPointDomain, dequantize_affine, quantize_affine
+
+    codes2 = quantize_affine(dq, (1, g), scale, zero, torch.int32, 0, 15, ZeroPointDomain.FLOAT)
+    assert torch.equal(codes2, codes)
+    del codes2
+    dq2 = dequantize_affine(codes, (1, g), scale, zero, torch.int32, 0, 15, ZeroPointDomain.FLOAT,
+                            output_dtype=torch.bfloat16)
+    assert torch.equal(dq2, dq)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_int4_linear_properties(shape):
+    from ao_amd import ops
+
+    N, K = shape
+    g = 64
+    print(f"case int4 linear full-size N={N} K={K}", flush=True)
+    dev = _dev()
+    w = _weight(N, K, seed=7 + N)
+    packed, qp = ops.int4wo_quantize_pack(w, g)
+    dq = ops.int4wo_dequantize(packed, qp, N, K, g)
+    del w
+    # one-hot rows: M = 1 (GEMV), M = 5 (GEMV, several rows), M = 20 (GEMM kernel)
+    ks = [0, 1, 63, 64, 127, 128, K // 2 + 3, K - 129, K - 2, K - 1, 1000, 2049, 77, 4000, 31, 32, 33, 500, 900, 1300]
+    for M in (1, 5, 20):
+        x = torch.zeros(M, K, dtype=torch.bfloat16, device=dev)
+        for m in range(M):
+            x[m, ks[m]] = 1.0
+        y = ops.int4wo_linear(x, packed, qp, g, N, None, True)
+        for m in range(M):
+            assert torch.equal(y[m], dq[:, ks[m]].float()), (M, m, ks[m])
+    # linearity on values whose sums and products are exact in the kernel's arithmetic: small integers
+    gen = torch.Generator(device=dev).manual_seed(11)
+    x1 = torch.randint(-4, 5, (1, K), device=dev, generator=gen).bfloat16()
+    x2 = torch.randint(-4, 5, (1, K), device=dev, generator=gen).bfloat16()
+    y1 = ops.int4wo_linear(x1, packed, qp, g, N, None, True)
+    y2 = ops.int4wo_linear(x2, packed, qp, g, N, None, True)
+    y12 = ops.int4wo_linear(x1 + x2, packed, qp, g, N, None, True)
+    assert rel_l2((y1 + y2).cpu().numpy(), y12.cpu().numpy()) <= 1e-5
+    # the three kernels on the same row: fp32 outputs agree to accumulation-order noise
+    xr = torch.randn(1, K, device=dev, generator=gen).bfloat16()
+    ya = ops.int4wo_linear(xr, packed, qp, g, N, None, True)
+    yb = ops.int4wo_linear(xr.repeat(4, 1), packed, qp, g, N, None, True)
+    yc = ops.int4wo_linear(xr.repeat(40, 1), packed, qp, g, N, None, True)
+    assert rel_l2(yb[3:4].cpu().numpy(), ya.cpu().numpy()) <= 1e-5
+    assert rel_l2(yc[39:40].cpu().numpy(), ya.cpu().numpy()) <= 1e-5
+    # and against torch's fp32 matmul on the dequantized weight (tolerance of the path: 1e-3)
+    ref = xr.float() @ dq.float().t()
+    assert rel_l2(ya.cpu().numpy(), ref.cpu().numpy()) <= 1e-3
+
+
+@pytest.mark.parametrize("shape", [(14336, 4096), (4096, 14336)])
+def test_fp6_properties(shape):
+    from ao_amd import ops
+
+    N, K = shape
+    print(f"case fp6 full-size N={N} K={K}", flush=True)
+    dev = _dev()
+    gen = torch.Generator(device=dev).manual_seed(N)
+    w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).half()
+    tc, scale = ops.fp6_quantize_pack(w, 3, 2)
+    assert tc.shape == (N, K * 6 // 8) and scale.shape == (N,)
+    # row scale = amax / 28 (largest e3m2 normal), computed in fp32 and rounded to fp16
+    expect = (w.float().abs().amax(dim=1).clamp(min=1e-12) / 28.0).half()
+    assert torch.equal(scale, expect)
+    # codes -> values -> codes is the identity (unit scale: every e3m2 value is exactly representable)
+    vals = ops.fp6_dequantize(tc, None, 3, 2)
+    assert bool((vals.abs().amax(dim=1) == 28.0).all())   # the row maximum lands on the largest normal
+    tc2, scale2 = ops.fp6_quantize_pack(vals, 3, 2)
+    assert torch.equal(tc2, tc) and bool((scale2 == 1.0).all())
+    # one-hot activation rows return columns of the scaled dequantized weight, rounded once to fp16
+    dq = ops.fp6_dequantize(tc, scale, 3, 2)
+    ks = [0, 1, 31, 32, 127, 128, K - 1, K // 2, 777, 4001, 15, 16, 17, 2048, 63, 64, 65, 300]
+    for M in (1, 18):
+        x = torch.zeros(M, K, dtype=torch.float16, device=dev)
+        for m in range(M):
+            x[m, ks[m]] = 1.0
+        y = ops.quant_llm_linear(3, 2, x, tc, scale)
+        for m in range(M):
+            assert rel_l2(y[m].float().cpu().numpy(), dq[:, ks[m]].cpu().numpy()) <= 1e-3, (M, m)
