@@ -696,7 +696,7 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
 template <int G>
 __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a) {
     constexpr int BM = 128, XSTRIDE = 136;  // bf16 elements per LDS row
-    __shared__ __align__(16) uint16_t xs[BM * XSTRIDE];
+    __shared__ __align__(16) uint16_t xs_all[2][BM * XSTRIDE];  // two K tiles: one being read, one being filled
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, qd = lane >> 4;
@@ -718,10 +718,10 @@ __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a)
             if (m < a.M) xr[j] = *reinterpret_cast<const uint4*>(a.x + m * a.ldx + (int64_t)kb * 128 + xchunk * 8);
         }
     };
-    auto store_x = [&]() {
+    auto store_x = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            *reinterpret_cast<uint4*>(xs + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
+            *reinterpret_cast<uint4*>(xs_all[buf] + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
     };
 
     struct WBuf { u32x4_t w0, w1; uint32_t q0, q1; };
@@ -743,39 +743,58 @@ __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a)
         acc0[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         acc1[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
-    auto compute = [&](const WBuf& b) {
+    auto compute = [&](const WBuf& b, int buf) {
+        const uint16_t* xs = xs_all[buf];
         const GroupConst g0 = make_group(b.q0), g1 = make_group(b.q1);
         const uint32_t w0[4] = {b.w0.x, b.w0.y, b.w0.z, b.w0.w};
         const uint32_t w1[4] = {b.w1.x, b.w1.y, b.w1.z, b.w1.w};
+        // The eight activation fragments of a k slice are read from LDS one slice ahead, before the dequantization of
+        // that slice, so that the LDS latency hides behind the VALU work; the scheduling barriers keep the compiler
+        // from sinking the reads back down to their first use.
+        union XFrag { uint4 q; bf16x8_t v; };
+        XFrag xa[2][8];
+        auto read_frags = [&](int sl, XFrag* dst) {
+#pragma unroll
+            for (int mb = 0; mb < 8; ++mb)
+                dst[mb].q = *reinterpret_cast<const uint4*>(xs + (mb * 16 + r) * XSTRIDE + qd * 32 + sl * 8);
+        };
+        read_frags(0, xa[0]);
 #pragma unroll
         for (int sl = 0; sl < 4; ++sl) {
+            if (sl + 1 < 4) read_frags(sl + 1, xa[(sl + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
             const bf16x8_t bw0 = dequant8(w0[sl], g0, magic, one_lo, one_hi);
             const bf16x8_t bw1 = dequant8(w1[sl], g1, magic, one_lo, one_hi);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int mb = 0; mb < 8; ++mb) {
-                union { uint4 q; bf16x8_t v; } xa;
-                xa.q = *reinterpret_cast<const uint4*>(xs + (mb * 16 + r) * XSTRIDE + qd * 32 + sl * 8);
-                acc0[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw0, acc0[mb], 0, 0, 0);
-                acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw1, acc1[mb], 0, 0, 0);
+                acc0[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[sl & 1][mb].v, bw0, acc0[mb], 0, 0, 0);
+                acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[sl & 1][mb].v, bw1, acc1[mb], 0, 0, 0);
             }
         }
     };
 
+    // Per K tile: one barrier.  Registers hold tile kb+1 of x (requested one iteration earlier); it is written to the
+    // idle LDS buffer, the global request for tile kb+2 goes out, then tile kb is multiplied out of the other buffer.
+    // The barrier at the end of the iteration separates these reads from the next iteration's writes to the buffer.
     WBuf b0, b1;
     load_x(0);
     load_w(b0, 0);
+    store_x(0);
+    if (KB > 1) { load_x(1); load_w(b1, 1); }
+    __syncthreads();
     for (int kb = 0; kb < KB; kb += 2) {
+        if (kb + 1 < KB) store_x(1);
+        if (kb + 2 < KB) load_x(kb + 2);
+        compute(b0, 0);
+        if (kb + 2 < KB) load_w(b0, kb + 2);
         __syncthreads();
-        store_x();
-        __syncthreads();
-        if (kb + 1 < KB) { load_x(kb + 1); load_w(b1, kb + 1); }
-        compute(b0);
         if (kb + 1 < KB) {
+            if (kb + 2 < KB) store_x(0);
+            if (kb + 3 < KB) load_x(kb + 3);
+            compute(b1, 1);
+            if (kb + 3 < KB) load_w(b1, kb + 3);
             __syncthreads();
-            store_x();
-            __syncthreads();
-            if (kb + 2 < KB) { load_x(kb + 2); load_w(b0, kb + 2); }
-            compute(b1);
         }
     }
 
