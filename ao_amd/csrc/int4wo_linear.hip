@@ -709,19 +709,23 @@ __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a)
 
     // activation tile loader: thread t covers rows (t>>4) + 16*j, 16-byte chunk t&15 of the 256-byte row slice
     const int xrow = tid >> 4, xchunk = tid & 15;
-    uint4 xr[8];
+    u32x4_t xr[8];
+    // rows past M alias the last row: their products land in output rows that are never stored, and a loader
+    // without branches lets the compiler keep exact counts of the loads in flight
+    const uint16_t* xrow_ptr[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int64_t m = m0 + xrow + 16 * j;
+        xrow_ptr[j] = a.x + (m < a.M ? m : a.M - 1) * a.ldx + xchunk * 8;
+    }
     auto load_x = [&](int kb) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int64_t m = m0 + xrow + 16 * j;
-            xr[j] = make_uint4(0, 0, 0, 0);
-            if (m < a.M) xr[j] = *reinterpret_cast<const uint4*>(a.x + m * a.ldx + (int64_t)kb * 128 + xchunk * 8);
-        }
+        for (int j = 0; j < 8; ++j) xr[j] = *reinterpret_cast<const u32x4_t*>(xrow_ptr[j] + (int64_t)kb * 128);
     };
     auto store_x = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            *reinterpret_cast<uint4*>(xs_all[buf] + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
+            *reinterpret_cast<u32x4_t*>(xs_all[buf] + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
     };
 
     struct WBuf { u32x4_t w0, w1; uint32_t q0, q1; };
@@ -774,29 +778,29 @@ __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a)
         }
     };
 
-    // Per K tile: one barrier.  Registers hold tile kb+1 of x (requested one iteration earlier); it is written to the
-    // idle LDS buffer, the global request for tile kb+2 goes out, then tile kb is multiplied out of the other buffer.
-    // The barrier at the end of the iteration separates these reads from the next iteration's writes to the buffer.
     WBuf b0, b1;
+    const int last = KB - 1;
     load_x(0);
     load_w(b0, 0);
     store_x(0);
-    if (KB > 1) { load_x(1); load_w(b1, 1); }
+    load_x(1 < last ? 1 : last);
+    load_w(b1, 1 < last ? 1 : last);
     __syncthreads();
-    for (int kb = 0; kb < KB; kb += 2) {
-        if (kb + 1 < KB) store_x(1);
-        if (kb + 2 < KB) load_x(kb + 2);
+    // Tiles in pairs, every load unconditional (tile indices past the end repeat the last tile and are never used):
+    // straight-line code keeps the compiler's vmcnt waits exact, so a wait for one tile does not drain the next.
+    for (int kb = 0; kb + 1 < KB; kb += 2) {
+        store_x(1);
+        load_x(kb + 2 < last ? kb + 2 : last);
         compute(b0, 0);
-        if (kb + 2 < KB) load_w(b0, kb + 2);
+        load_w(b0, kb + 2 < last ? kb + 2 : last);
         __syncthreads();
-        if (kb + 1 < KB) {
-            if (kb + 2 < KB) store_x(0);
-            if (kb + 3 < KB) load_x(kb + 3);
-            compute(b1, 1);
-            if (kb + 3 < KB) load_w(b1, kb + 3);
-            __syncthreads();
-        }
+        store_x(0);
+        load_x(kb + 3 < last ? kb + 3 : last);
+        compute(b1, 1);
+        load_w(b1, kb + 3 < last ? kb + 3 : last);
+        __syncthreads();
     }
+    if (KB & 1) compute(b0, 0);
 
     // acc[mb][i] = C[m = m0 + 16*mb + 4*qd + i][n = 16*nb + r]
 #pragma unroll
