@@ -294,6 +294,142 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* 
     }
 }
 
+// ---------------------------------------------------------------- GEMM path (M > 16)
+// Workgroup tile: 128 activation rows x 128 weight rows, K walked in 128-wide tiles; the same skeleton as the int4
+// GEMM.  Each of the 4 waves owns two 16-row weight blocks: it loads their native tiles (24 bytes per lane) straight
+// into registers, converts them once (one v_cvt_scalef32_pk32 + 16 v_pk_mul_f16 per block and tile) and multiplies
+// them against the eight 16-row activation blocks of the tile (64 MFMAs per wave and tile).  The activation tile is
+// double-buffered in LDS (row stride 272 bytes), fetched two tiles ahead into registers; every load is
+// unconditional (rows past M alias the last row, tiles past the end repeat the last tile) so that the compiler's
+// vmcnt waits stay exact.
+template <bool E3M2>
+__global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
+                                                           const uint32_t* __restrict__ native,
+                                                           const uint16_t* __restrict__ scale, int64_t N,
+                                                           uint16_t* __restrict__ out) {
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    constexpr int BM = 128, XSTRIDE = 136;  // fp16 elements per LDS row
+    __shared__ __align__(16) uint16_t xs_all[2][BM * XSTRIDE];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, qd = lane >> 4;
+    const int KB = (int)(K / 128);
+    const int64_t nblocks = N / 16;
+    const int64_t nb0 = (int64_t)blockIdx.x * 8 + 2 * wave;
+    const bool has0 = nb0 < nblocks, has1 = nb0 + 1 < nblocks;
+    const int64_t m0 = (int64_t)blockIdx.y * BM;
+
+    const int xrow = tid >> 4, xchunk = tid & 15;
+    const uint16_t* xrow_ptr[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int64_t m = m0 + xrow + 16 * j;
+        xrow_ptr[j] = x + (m < M ? m : M - 1) * K + xchunk * 8;
+    }
+    u32x4_t xr[8];
+    auto load_x = [&](int kb) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xr[j] = *reinterpret_cast<const u32x4_t*>(xrow_ptr[j] + (int64_t)kb * 128);
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            *reinterpret_cast<u32x4_t*>(xs_all[buf] + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
+    };
+
+    struct WBuf { u32x4_t lo0, lo1; u32x2_t hi0, hi1; };
+    const uint32_t* t0 = native + (has0 ? nb0 : 0) * KB * 384;
+    const uint32_t* t1 = native + (has1 ? nb0 + 1 : 0) * KB * 384;
+    auto load_w = [&](WBuf& b, int kb) {
+        b.lo0 = reinterpret_cast<const u32x4_t*>(t0 + (int64_t)kb * 384)[lane];
+        b.hi0 = reinterpret_cast<const u32x2_t*>(t0 + (int64_t)kb * 384 + 256)[lane];
+        b.lo1 = reinterpret_cast<const u32x4_t*>(t1 + (int64_t)kb * 384)[lane];
+        b.hi1 = reinterpret_cast<const u32x2_t*>(t1 + (int64_t)kb * 384 + 256)[lane];
+    };
+    union { uint16_t h; _Float16 f; } s0, s1;
+    s0.h = scale[(has0 ? nb0 : 0) * 16 + r];
+    s1.h = scale[(has1 ? nb0 + 1 : 0) * 16 + r];
+    const f16x2_t sc0 = {s0.f, s0.f}, sc1 = {s1.f, s1.f};
+
+    f32x4_t acc0[8], acc1[8];
+#pragma unroll
+    for (int mb = 0; mb < 8; ++mb) {
+        acc0[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        acc1[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    auto convert = [&](const u32x4_t& lo, const u32x2_t& hi) {
+        const u32x6_t packed = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y};
+        if (E3M2) return __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(packed, 1.0f);
+        return __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(packed, 1.0f);
+    };
+    auto compute = [&](const WBuf& b, int buf) {
+        const uint16_t* xs = xs_all[buf];
+        const f16x32_t v0 = convert(b.lo0, b.hi0), v1 = convert(b.lo1, b.hi1);
+        union XFrag { uint4 q; f16x8_t v; };
+        XFrag xa[2][8];
+        auto read_frags = [&](int sl, XFrag* dst) {
+#pragma unroll
+            for (int mb = 0; mb < 8; ++mb)
+                dst[mb].q = *reinterpret_cast<const uint4*>(xs + (mb * 16 + r) * XSTRIDE + qd * 32 + sl * 8);
+        };
+        read_frags(0, xa[0]);
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            if (sl + 1 < 4) read_frags(sl + 1, xa[(sl + 1) & 1]);
+            union { f16x2_t p[4]; f16x8_t v; } w0, w1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f16x2_t p0 = {v0[sl * 8 + 2 * j], v0[sl * 8 + 2 * j + 1]};
+                const f16x2_t p1 = {v1[sl * 8 + 2 * j], v1[sl * 8 + 2 * j + 1]};
+                w0.p[j] = p0 * sc0;  // v_pk_mul_f16: fp16(fp6 * scale), the one rounding of the reference kernel
+                w1.p[j] = p1 * sc1;
+            }
+#pragma unroll
+            for (int mb = 0; mb < 8; ++mb) {
+                acc0[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[sl & 1][mb].v, w0.v, acc0[mb], 0, 0, 0);
+                acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[sl & 1][mb].v, w1.v, acc1[mb], 0, 0, 0);
+            }
+        }
+    };
+
+    WBuf b0, b1;
+    const int last = KB - 1;
+    load_x(0);
+    load_w(b0, 0);
+    store_x(0);
+    load_x(1 < last ? 1 : last);
+    load_w(b1, 1 < last ? 1 : last);
+    __syncthreads();
+    for (int kb = 0; kb + 1 < KB; kb += 2) {
+        store_x(1);
+        load_x(kb + 2 < last ? kb + 2 : last);
+        compute(b0, 0);
+        load_w(b0, kb + 2 < last ? kb + 2 : last);
+        __syncthreads();
+        store_x(0);
+        load_x(kb + 3 < last ? kb + 3 : last);
+        compute(b1, 1);
+        load_w(b1, kb + 3 < last ? kb + 3 : last);
+        __syncthreads();
+    }
+    if (KB & 1) compute(b0, 0);
+
+    // acc[mb][i] = C[m = m0 + 16*mb + 4*qd + i][n = 16*nb + r]
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        if (!(h == 0 ? has0 : has1)) continue;
+        const int64_t n = (nb0 + h) * 16 + r;
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t m = m0 + mb * 16 + 4 * qd + i;
+                if (m < M) out[m * N + n] = f32_to_f16_bits(h == 0 ? acc0[mb][i] : acc1[mb][i]);
+            }
+    }
+}
+
 static int check_fp6_format(int ebits, int mbits) {
     AO_REQUIRE((ebits == 3 && mbits == 2) || (ebits == 2 && mbits == 3),
                "FP%d E%dM%d is not supported (6-bit formats e3m2 and e2m3 only)", 1 + ebits + mbits, ebits, mbits);
@@ -370,6 +506,19 @@ extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const 
     uint16_t* o = (uint16_t*)out_f16;
     hipEvent_t ev0 = g_prof_start, ev1 = g_prof_stop;  // optional per-kernel timing, see common.h
     g_prof_start = g_prof_stop = nullptr;
+    // the tiled kernel pays off once its grid can occupy a good part of the 256 CUs; below that the skinny kernel
+    // (one workgroup per 16 x 16 output block, K split over waves) has more parallelism
+    const int64_t gemm_wgs = ((RB + 7) / 8) * ((M + 127) / 128);
+    if (M > 16 && K % 128 == 0 && (gemm_wgs >= 96 || M >= 256)) {
+        dim3 ggrid((unsigned)((RB + 7) / 8), (unsigned)((M + 127) / 128));
+        AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
+        if (ebits == 3)
+            hipExtLaunchKernelGGL((fp6_gemm_kernel<true>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+        else
+            hipExtLaunchKernelGGL((fp6_gemm_kernel<false>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+        AO_LAUNCH_CHECK();
+        return 0;
+    }
 #define AO_FP6_LAUNCH(W)                                                                                                 \
     if (ebits == 3)                                                                                                      \
         hipExtLaunchKernelGGL((fp6_linear_kernel<W, true>), grid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o); \

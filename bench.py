@@ -219,7 +219,7 @@ def _time_linear(L, launch, iters):
 
 def sweep(kind, iters=15):
     """Per-kernel lines for the shapes of the other benchmark configurations: int4 GEMV (M in 1, 4; g in 64, 128),
-    int4 GEMM (M in 16 .. 2048, g=64) and the FP6 e3m2 linear (M in 1, 16, 128); one JSON line per case."""
+    int4 GEMM (M in 16 .. 2048, g=64) and the FP6 e3m2 linear (M in 1, 16, 128, 512); one JSON line per case."""
     import torch
 
     from ao_amd import _lib
@@ -263,7 +263,7 @@ def sweep(kind, iters=15):
             native = torch.empty(copies, nbytes.value, dtype=torch.uint8, device=dev)
             _lib.check(L.ao_amd_fp6_repack(tc.data_ptr(), N, K, native.data_ptr(), st))
             native[1:] = native[0]
-            for M in (1, 16, 128):
+            for M in (1, 16, 128, 512):
                 x = torch.randn(M, K, device=dev, generator=gen).half()
                 y = torch.empty(M, N, dtype=torch.float16, device=dev)
                 us = _time_linear(L, lambda i: _lib.check(L.ao_amd_fp6_linear(
