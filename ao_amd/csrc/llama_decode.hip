@@ -286,21 +286,18 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
 // Index of the largest of n bf16 values (the lowest such index; a NaN counts as larger than any number), for
 // greedy sampling of one token: torch.argmax on the logits row, generate.py `sample`.  One workgroup; every
 // thread requests all of its 16-byte chunks (up to 16: n <= 131072 elements in one round trip) before the first
-// comparison.
+// comparison.  A thread meets its elements in increasing index order, so "strictly greater" keeps the lowest
+// index; NaNs only raise a flag in the hot loop and are located by a second pass in the rare case that one exists.
 __global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __restrict__ x, int64_t n,
                                                             int32_t* __restrict__ out) {
     __shared__ float bv_s[16];
     __shared__ int32_t bi_s[16];
+    __shared__ int nan_s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) nan_s = 0x7fffffff;
     float best = -INFINITY;
     int32_t besti = 0x7fffffff;
-    auto consider = [&](float v, int32_t i) {
-        const bool vnan = v != v, bnan = best != best;
-        if ((vnan && !bnan) || (!bnan && v > best) || (v == best && i < besti) || (vnan && bnan && i < besti)) {
-            best = v;
-            besti = i;
-        }
-    };
+    bool any_nan = false;
     const int64_t nchunk = n / 8;
     const bool vec = (((uintptr_t)x) & 15) == 0;
     constexpr int MAXC = 16;
@@ -315,33 +312,51 @@ __global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __res
             }
 #pragma unroll
             for (int j = 0; j < MAXC; ++j) {
-                const int64_t c = c0 + (int64_t)j * 1024 + tid;
-                if (c < nchunk) {
-                    const uint32_t u[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+                const int32_t base = (int32_t)((c0 + (int64_t)j * 1024 + tid) * 8);
+                const uint32_t u[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        consider(__uint_as_float(u[e] << 16), (int32_t)(c * 8 + 2 * e));
-                        consider(__uint_as_float(u[e] & 0xffff0000u), (int32_t)(c * 8 + 2 * e + 1));
-                    }
+                for (int e = 0; e < 4; ++e) {
+                    const float lo = __uint_as_float(u[e] << 16), hi = __uint_as_float(u[e] & 0xffff0000u);
+                    any_nan |= (lo != lo) | (hi != hi);
+                    if (lo > best) { best = lo; besti = base + 2 * e; }
+                    if (hi > best) { best = hi; besti = base + 2 * e + 1; }
                 }
             }
         }
     }
-    for (int64_t i = (vec ? nchunk * 8 : 0) + tid; i < n; i += 1024) consider(bf16_bits_to_f32(x[i]), (int32_t)i);
+    for (int64_t i = (vec ? nchunk * 8 : 0) + tid; i < n; i += 1024) {
+        const float v = bf16_bits_to_f32(x[i]);
+        any_nan |= v != v;
+        if (v > best) { best = v; besti = (int32_t)i; }
+    }
+    // an all -inf input leaves besti unset in every thread: index 0 is the answer then
+    auto merge = [&](float ov, int32_t oi) {
+        if (ov > best || (ov == best && oi < besti)) { best = ov; besti = oi; }
+    };
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) {
         const float ov = __shfl_xor(best, o, 64);
         const int32_t oi = __shfl_xor(besti, o, 64);
-        consider(ov, oi);
+        merge(ov, oi);
     }
     if (lane == 0) {
         bv_s[wave] = best;
         bi_s[wave] = besti;
     }
     __syncthreads();
+    if (__syncthreads_or(any_nan)) {
+        // rare path: the answer is the first NaN
+        for (int64_t i = tid; i < n; i += 1024) {
+            const float v = bf16_bits_to_f32(x[i]);
+            if (v != v) { atomicMin(&nan_s, (int)i); break; }
+        }
+        __syncthreads();
+        if (tid == 0) out[0] = nan_s;
+        return;
+    }
     if (tid == 0) {
-        for (int w = 1; w < 16; ++w) consider(bv_s[w], bi_s[w]);
-        out[0] = besti;
+        for (int w = 1; w < 16; ++w) merge(bv_s[w], bi_s[w]);
+        out[0] = besti == 0x7fffffff ? 0 : besti;
     }
 }
 

@@ -175,6 +175,11 @@ def test_argmax_bf16(n):
     xf = x.float()
     expect = int((xf == xf.max()).nonzero()[0, 0])
     assert int(out.item()) == expect
+    if n >= 8:
+        x[n - 2] = float("nan")   # a NaN counts as the largest value, like torch.argmax
+        x[n // 2] = float("nan")
+        assert int(ops.argmax_bf16(x.to(dev)).item()) == n // 2
+        assert int(ops.argmax_bf16(torch.full((n,), float("-inf")).bfloat16().to(dev)).item()) == 0
 
 
 def test_fused_decode_step_matches_module_path():
