@@ -63,7 +63,7 @@ def test_dequantize_and_repack_round_trip(oracle):
 
 
 @pytest.mark.parametrize("M", [1, 2, 16, 40, 130, 257])
-@pytest.mark.parametrize("shape", [(256, 1024), (2048, 4096), (512, 192)])
+@pytest.mark.parametrize("shape", [(256, 1024), (2048, 4096), (512, 192), (320, 256)])
 def test_linear_matches_oracle(oracle, shape, M):
     """Shapes include the reference op test's (BS, OC, IC) = (1, 2048, 4096) (test/test_ops.py:49-51); inputs as there:
     activations rand + 0.5, random bytes as weights, scales rand + 0.5."""
