@@ -13,10 +13,11 @@ from . import dtypes, ops, quantization  # noqa: F401
 from .quantization import (  # noqa: F401
     fp6_llm_weight_only,
     int4_weight_only,
+    int8_weight_only,
     quant_llm_fpx_weight_only,
     quantize,
     quantize_,
 )
 
-__all__ = ["dtypes", "ops", "quantization", "quantize", "quantize_", "int4_weight_only", "fp6_llm_weight_only",
+__all__ = ["dtypes", "ops", "quantization", "quantize", "quantize_", "int4_weight_only", "int8_weight_only", "fp6_llm_weight_only",
            "quant_llm_fpx_weight_only"]

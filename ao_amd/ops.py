@@ -32,6 +32,7 @@ __all__ = [
     "int4wo_dequantize",
     "int4wo_linear",
     "int4wo_packed_shapes",
+    "int8wo_linear",
 ]
 
 _LIB = torch.library.Library("torchao", "FRAGMENT")
@@ -44,6 +45,7 @@ _LIB.define("int4wo_linear_residual(Tensor x, Tensor packed, Tensor qparams, int
 _LIB.define("int4wo_swiglu(Tensor x, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
 _LIB.define("int4wo_rmsnorm_linear(Tensor x, Tensor norm_weight, float eps, Tensor packed, Tensor qparams, int group_size, int N, Tensor? bias) -> Tensor")
 _LIB.define("int4wo_rmsnorm_swiglu(Tensor x, Tensor norm_weight, float eps, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
+_LIB.define("int8wo_linear(Tensor x, Tensor w_int8, Tensor scale, Tensor? bias, bool fp32_out) -> Tensor")
 _LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
 _LIB.define("argmax_bf16(Tensor x) -> Tensor")
 _LIB.define("llama_decode_attention(Tensor qkv, Tensor freqs_cis, Tensor input_pos, Tensor(a!) k_cache, Tensor(b!) v_cache, int n_head, int n_kv) -> Tensor")
@@ -181,6 +183,28 @@ def _swiglu_cuda(x, packed_gate, qparams_gate, packed_up, qparams_up, group_size
     check(lib().ao_amd_int4wo_swiglu(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, packed_gate.data_ptr(),
                                      qparams_gate.data_ptr(), packed_up.data_ptr(), qparams_up.data_ptr(), N, group_size,
                                      y.data_ptr(), N, current_stream(x.device)))
+    return y
+
+
+def _int8wo_linear_cuda(x, w_int8, scale, bias, fp32_out):
+    require_cuda(x, w_int8, scale, bias)
+    torch._check(x.dim() == 2 and x.dtype is torch.bfloat16, lambda: "input must be a 2d bfloat16 tensor")
+    torch._check(w_int8.dim() == 2 and w_int8.dtype is torch.int8 and w_int8.stride(1) == 1,
+                 lambda: "weight must be a 2d int8 tensor with unit inner stride")
+    M, K = x.shape
+    N = w_int8.shape[0]
+    torch._check(w_int8.shape[1] == K, lambda: f"weight in_features {w_int8.shape[1]} != input features {K}")
+    torch._check(scale.dtype is torch.bfloat16 and scale.numel() == N, lambda: "scale must be bfloat16 of size N")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    scale = scale.contiguous()
+    if bias is not None:
+        torch._check(bias.dtype is torch.bfloat16 and bias.numel() == N, lambda: "bias must be bfloat16 of size N")
+        bias = bias.contiguous()
+    y = torch.empty((M, N), dtype=torch.float32 if fp32_out else torch.bfloat16, device=x.device)
+    check(lib().ao_amd_int8wo_linear(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, w_int8.data_ptr(),
+                                     w_int8.stride(0), scale.data_ptr(), N, None if bias is None else bias.data_ptr(),
+                                     y.data_ptr(), F32 if fp32_out else BF16, N, current_stream(x.device)))
     return y
 
 
@@ -364,6 +388,7 @@ _LIB.impl("int4wo_linear_residual", _linear_residual_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu", _swiglu_cuda, "CUDA")
 _LIB.impl("int4wo_rmsnorm_linear", _rmsnorm_linear_cuda, "CUDA")
 _LIB.impl("int4wo_rmsnorm_swiglu", _rmsnorm_swiglu_cuda, "CUDA")
+_LIB.impl("int8wo_linear", _int8wo_linear_cuda, "CUDA")
 _LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
 _LIB.impl("llama_decode_attention", _decode_attention_cuda, "CUDA")
 _LIB.impl("argmax_bf16", _argmax_bf16_cuda, "CUDA")
@@ -381,7 +406,7 @@ def _no_cpu(name):
 
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
-              "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
+              "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int8wo_linear", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
               "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
@@ -440,6 +465,11 @@ def _(x, norm_weight, eps, packed, qparams, group_size, N, bias):
 @torch.library.register_fake("torchao::int4wo_rmsnorm_swiglu")
 def _(x, norm_weight, eps, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
     return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::int8wo_linear")
+def _(x, w_int8, scale, bias, fp32_out):
+    return x.new_empty((x.shape[0], w_int8.shape[0]), dtype=torch.float32 if fp32_out else torch.bfloat16)
 
 
 @torch.library.register_fake("torchao::argmax_bf16")
@@ -544,6 +574,11 @@ def int4wo_rmsnorm_swiglu(x, norm_weight, eps: float, packed_gate, qparams_gate,
     """swiglu(rmsnorm(x, norm_weight, eps)) in one launch, for M <= 16 rows (decode)."""
     return torch.ops.torchao.int4wo_rmsnorm_swiglu.default(x, norm_weight, eps, packed_gate, qparams_gate, packed_up,
                                                            qparams_up, group_size, N)
+
+
+def int8wo_linear(x: Tensor, w_int8: Tensor, scale: Tensor, bias=None, fp32_out: bool = False) -> Tensor:
+    """bf16(bf16(x @ w_int8^T) * scale) (+ bias): x bf16 [M,K], w_int8 int8 [N,K] (plain layout), scale bf16 [N]."""
+    return torch.ops.torchao.int8wo_linear.default(x, w_int8, scale, bias, fp32_out)
 
 
 def rmsnorm(x, weight, eps: float):

@@ -1,4 +1,11 @@
-from .quant_api import fp6_llm_weight_only, int4_weight_only, quant_llm_fpx_weight_only, quantize, quantize_
+from .quant_api import (
+    fp6_llm_weight_only,
+    int4_weight_only,
+    int8_weight_only,
+    quant_llm_fpx_weight_only,
+    quantize,
+    quantize_,
+)
 from .quant_primitives import (
     MappingType,
     ZeroPointDomain,

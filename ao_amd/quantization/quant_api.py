@@ -11,7 +11,8 @@ import torch
 
 from .quant_primitives import MappingType, ZeroPointDomain
 
-__all__ = ["quantize", "quantize_", "int4_weight_only", "fp6_llm_weight_only", "quant_llm_fpx_weight_only"]
+__all__ = ["quantize", "quantize_", "int4_weight_only", "int8_weight_only", "fp6_llm_weight_only",
+           "quant_llm_fpx_weight_only"]
 
 
 def _replace_with_custom_fn_if_matches_filter(model, replacement_fn, filter_fn, cur_fqn=""):
@@ -84,6 +85,19 @@ def int4_weight_only(group_size=128, inner_k_tiles=8):
             extended_layout="gfx950_wave_tiled", inner_k_tiles=inner_k_tiles)
 
     return apply_int4_weight_only_quant
+
+
+def int8_weight_only():
+    """int8 weight-only symmetric per-channel quantization (reference :390-405): one bf16 scale per output row,
+    zero point 0, codes kept in the plain [N, K] layout, which the gfx950 kernel reads in place."""
+
+    def apply_int8wo_quant(weight):
+        from ..dtypes import to_affine_quantized
+
+        return to_affine_quantized(weight, MappingType.SYMMETRIC, (1, weight.shape[1]), torch.int8,
+                                   eps=torch.finfo(torch.float32).eps, zero_point_dtype=torch.int64)
+
+    return apply_int8wo_quant
 
 
 def quant_llm_fpx_weight_only(ebits: int, mbits: int):

@@ -219,7 +219,8 @@ def _time_linear(L, launch, iters):
 
 def sweep(kind, iters=15):
     """Per-kernel lines for the shapes of the other benchmark configurations: int4 GEMV (M in 1, 4; g in 64, 128),
-    int4 GEMM (M in 16 .. 2048, g=64) and the FP6 e3m2 linear (M in 1, 16, 128, 512); one JSON line per case."""
+    int4 GEMM (M in 16 .. 2048, g=64), the FP6 e3m2 linear (M in 1, 16, 128, 512) and the int8 weight-only linear
+    (M in 1, 4, 16); one JSON line per case."""
     import torch
 
     from ao_amd import _lib
@@ -274,6 +275,23 @@ def sweep(kind, iters=15):
                                   "GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
                                   "TFLOPs": round(tfs, 2), "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
             del w, tc, native
+    elif kind == "int8":
+        for N, K in LLAMA3_8B_SHAPES:
+            copies = max(2, -(-SWEEP_ROTATE_BYTES // (N * K)))
+            wq = torch.randint(-127, 128, (copies, N, K), device=dev, dtype=torch.int8, generator=gen)
+            sc = (torch.rand(N, device=dev, generator=gen) * 1e-3 + 1e-4).bfloat16()
+            for M in (1, 4, 16):
+                x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
+                y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+                us = _time_linear(L, lambda i: _lib.check(L.ao_amd_int8wo_linear(
+                    x.data_ptr(), M, K, K, wq[i % copies].data_ptr(), K, sc.data_ptr(), N, None, y.data_ptr(), _lib.BF16,
+                    N, st)), iters)
+                gbs = (N * K + 2 * N + 2 * M * K + 2 * M * N) / us / 1e3
+                tfs = 2.0 * M * N * K / us / 1e6
+                print(json.dumps({"kernel": "int8wo_linear", "N": N, "K": K, "M": M, "us": round(us, 2),
+                                  "GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+                                  "TFLOPs": round(tfs, 2), "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
+            del wq
     else:
         sys.exit(f"unknown sweep {kind}")
 
@@ -291,7 +309,7 @@ def main():
     ap.add_argument("--roofline-only", action="store_true",
                     help="build the model, run one pass of the roofline leg and a copy kernel of known size, no decode "
                          "loop: the command to put under rocprofv3 --pmc")
-    ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6"), default=None,
+    ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6", "int8"), default=None,
                     help="instead of the decode benchmark, print one line per kernel case of the named sweep")
     args = ap.parse_args()
     if args.gpus != 1:

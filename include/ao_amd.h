@@ -135,6 +135,18 @@ int ao_amd_int4wo_rmsnorm_swiglu(const void* x_bf16, int64_t M, int64_t K, int64
                                  float eps, const void* packed_gate, const void* qparams_gate, const void* packed_up,
                                  const void* qparams_up, int64_t N, int64_t g, void* y_bf16, int64_t ldy, void* stream);
 
+/* ---------------------------------------------------------------- int8 weight-only linear
+ * y[M,N] = bf16( bf16(x[M,K] @ bf16(w)^T) * scale[N] ) (+ bias, rounded to bf16 again): the per-channel int8
+ * weight-only branch of _quantized_linear_op, torchao/dtypes/affine_quantized_tensor.py:641-665
+ * (`torch.mm(x, w_int8.t().to(x.dtype)) * scale`), for the weight that int8_weight_only() produces
+ * (torchao/quantization/quant_api.py:390-405: symmetric, block (1, K), plain layout).
+ *   w_int8 : int8 [N, K] row-major with row stride ldw (the reference's plain layout, read in place);
+ *   K % 128 == 0; x, w 16-byte aligned with 16-byte aligned rows; y_dtype AO_BF16 or AO_F32 (AO_F32 stores the value
+ *   before the last rounding). */
+int ao_amd_int8wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* w_int8, int64_t ldw,
+                         const void* scale_bf16, int64_t N, const void* bias_bf16, void* y, int y_dtype, int64_t ldy,
+                         void* stream);
+
 /* ---------------------------------------------------------------- Llama decode harness kernels (bf16)
  * out[rows,dim] = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * weight ): RMSNorm.forward,
  * torchao/_models/llama/model.py:232-244. */

@@ -1,0 +1,130 @@
+"""GPU parity tests of the int8 weight-only path (symmetric per-channel, plain layout): quantization through the
+generic primitives bit-exact against the CPU oracle; the linear against the oracle's fp32-accumulated product with
+the reference's rounding chain bf16(bf16(x @ q^T) * scale) (+ bias) applied on top
+(torchao/dtypes/affine_quantized_tensor.py:641-665)."""
+import numpy as np
+import pytest
+import torch
+
+from _util import bits16, make_act, make_weight, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    assert torch.cuda.is_available()
+    return torch.device("cuda:0")
+
+
+def _rb(oracle, a):
+    return oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(np.asarray(a, np.float32)))
+
+
+def _oracle_quant(oracle, w):
+    eps = float(torch.finfo(torch.float32).eps)
+    N, K = w.shape
+    s, z = oracle.choose_qparams_affine(bits16(w), oracle.BF16, (1, K), 0, -128, 127, eps=eps, zp_dtype=oracle.I64)
+    q = oracle.quantize_affine(bits16(w), oracle.BF16, (1, K), s, oracle.BF16, z, oracle.I64, -128, 127, zp_domain=0,
+                               out_dtype=oracle.I8)
+    return q, s, z
+
+
+@pytest.mark.parametrize("shape", [(64, 256), (48, 192), (17, 64), (256, 1024)])
+def test_quantize_bit_exact(oracle, shape):
+    from ao_amd.dtypes import AffineQuantizedTensor
+    from ao_amd.quantization import int8_weight_only
+
+    N, K = shape
+    print(f"case int8 quantize N={N} K={K}", flush=True)
+    w = make_weight(N, K, seed=3 * N + K)
+    qw = int8_weight_only()(w.to(_dev()))
+    assert isinstance(qw, AffineQuantizedTensor) and qw.shape == (N, K) and qw.dtype is torch.bfloat16
+    int_data, scale, zero = qw.layout_tensor.get_plain()
+    q, s, z = _oracle_quant(oracle, w)
+    assert int_data.dtype is torch.int8 and scale.dtype is torch.bfloat16 and zero.dtype is torch.int64
+    assert np.array_equal(int_data.cpu().numpy(), q)
+    assert np.array_equal(bits16(scale).reshape(-1), s.reshape(-1))
+    assert np.array_equal(zero.cpu().numpy().reshape(-1), z.reshape(-1))
+
+
+@pytest.mark.parametrize("M", [1, 4, 16, 33])
+@pytest.mark.parametrize("shape", [(256, 1024), (48, 256), (1000, 4096)])
+def test_linear_matches_oracle(oracle, shape, M):
+    from ao_amd import ops
+
+    N, K = shape
+    print(f"case int8 linear N={N} K={K} M={M}", flush=True)
+    dev = _dev()
+    w = make_weight(N, K, seed=5 + N)
+    x = make_act(M, K, seed=M + K)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(9)) * 0.1).bfloat16() if M == 4 else None
+    q, s, _ = _oracle_quant(oracle, w)
+    acc = oracle.linear(bits16(x), oracle.BF16, q, oracle.I8)            # fp32-accumulated x @ q^T
+    sf = oracle.bf16_bits_to_f32(s.reshape(1, -1))
+    pre = _rb(oracle, acc) * sf                                          # value before the last rounding
+    if bias is not None:
+        pre = _rb(oracle, pre) + bias.float().numpy().reshape(1, -1)
+    expect = _rb(oracle, pre)
+    qd = torch.from_numpy(q).to(dev)
+    sd = torch.from_numpy(s.reshape(-1).view(np.int16)).view(torch.bfloat16).to(dev)
+    bd = None if bias is None else bias.to(dev)
+    y32 = ops.int8wo_linear(x.to(dev), qd, sd, bd, True).cpu().numpy()
+    y16 = ops.int8wo_linear(x.to(dev), qd, sd, bd, False).float().cpu().numpy()
+    # the accumulation order differs from the oracle's: an element whose sum sits on a bf16 rounding boundary may
+    # move by one bf16 ulp, everything else is identical
+    assert rel_l2(y32, pre) <= 1e-3
+    assert rel_l2(y16, expect) <= 1e-3
+    assert np.count_nonzero(y16 != expect) <= 0.02 * y16.size + 1
+
+
+def test_one_hot_rows_return_scaled_codes(oracle):
+    """x = e_k: the product is the code itself, so the output must be exactly bf16(q[n,k] * scale[n])."""
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K = 80, 512
+    w = make_weight(N, K, seed=123)
+    q, s, _ = _oracle_quant(oracle, w)
+    ks = [0, 1, 3, 4, 7, 8, 31, 32, 33, 127, 128, 255, 256, 300, 510, 511]
+    x = torch.zeros(len(ks), K, dtype=torch.bfloat16)
+    for m, k in enumerate(ks):
+        x[m, k] = 1.0
+    sd = torch.from_numpy(s.reshape(-1).view(np.int16)).view(torch.bfloat16)
+    y = ops.int8wo_linear(x.to(dev), torch.from_numpy(q).to(dev), sd.to(dev), None, False).float().cpu().numpy()
+    sf = oracle.bf16_bits_to_f32(s.reshape(-1))
+    for m, k in enumerate(ks):
+        assert np.array_equal(y[m], _rb(oracle, q[:, k].astype(np.float32) * sf)), (m, k)
+
+
+def test_module_api_and_fallback():
+    """quantize_(model, int8_weight_only()) swaps nn.Linear weights; F.linear runs the HIP kernel when
+    in_features is a multiple of 128 and the dequantize path (reference :683-690) otherwise."""
+    from ao_amd import int8_weight_only, quantize_
+    from ao_amd.dtypes import AffineQuantizedTensor
+
+    dev = _dev()
+    torch.manual_seed(0)
+    for K in (256, 192):
+        lin = torch.nn.Linear(K, 96, bias=True).to(dev).bfloat16()
+        ref_w = lin.weight.detach().clone()
+        x = torch.randn(5, K, device=dev).bfloat16()
+        quantize_(lin, int8_weight_only())
+        assert isinstance(lin.weight, AffineQuantizedTensor)
+        with torch.no_grad():
+            y = lin(x)
+            y_ref = torch.nn.functional.linear(x, lin.weight.dequantize(), lin.bias)
+            y_fp = torch.nn.functional.linear(x, ref_w, lin.bias)
+        assert y.shape == (5, 96) and y.dtype is torch.bfloat16
+        assert rel_l2(y.float().cpu().numpy(), y_ref.float().cpu().numpy()) <= 1e-2   # two bf16 rounding chains
+        assert rel_l2(y.float().cpu().numpy(), y_fp.float().cpu().numpy()) <= 3e-2    # 8-bit quantization error
+
+
+def test_rejects_bad_arguments(cabi):
+    dev = _dev()
+    x = torch.zeros(1, 192, dtype=torch.bfloat16, device=dev)
+    w = torch.zeros(16, 192, dtype=torch.int8, device=dev)
+    s = torch.ones(16, dtype=torch.bfloat16, device=dev)
+    y = torch.zeros(1, 16, dtype=torch.bfloat16, device=dev)
+    rc = cabi.lib().ao_amd_int8wo_linear(x.data_ptr(), 1, 192, 192, w.data_ptr(), 192, s.data_ptr(), 16, None, y.data_ptr(),
+                                         cabi.BF16, 16, None)
+    assert rc != 0 and b"multiple of 128" in cabi.lib().ao_amd_last_error()

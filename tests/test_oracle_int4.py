@@ -229,3 +229,29 @@ def test_linear_against_float64(oracle):
     y = oracle.linear(bits16(x), oracle.BF16, bits16(w), oracle.BF16, bits16(bias), oracle.BF16)
     ref = x.double().numpy() @ w.double().numpy().T + bias.double().numpy()
     assert np.max(np.abs(y - ref)) <= 1e-5 * np.max(np.abs(ref))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_int8_symmetric_per_channel_stepwise(oracle, dtype):
+    """The int8 weight-only recipe (symmetric, block (1, K), eps = finfo(float32).eps, zero point int64;
+    torchao/quantization/quant_api.py:390-405) against torch's own CPU kernels run op by op in the weight's dtype:
+    quant_primitives.py:335-367 for the parameters, :191-194 for the codes.  For bf16 tensors torch rounds after
+    every op by itself, which is the behaviour the oracle has to restate."""
+    w = make_weight(48, 256, seed=77, dtype=dtype)
+    eps = torch.finfo(torch.float32).eps
+    mn, mx = w.amin(dim=1), w.amax(dim=1)
+    mn_neg, mx_pos = torch.min(mn, torch.zeros_like(mn)), torch.max(mx, torch.zeros_like(mx))
+    scale_ref = torch.clamp(torch.max(-mn_neg, mx_pos) / (float(127 - (-128)) / 2), min=eps)
+    q_ref = torch.clamp(torch.round(w * (1.0 / scale_ref.reshape(-1, 1))) + torch.zeros(48, 1, dtype=torch.int64),
+                        -128, 127).to(torch.int8)
+    code = oracle.BF16 if dtype is torch.bfloat16 else oracle.F32
+    wn = bits16(w) if dtype is torch.bfloat16 else _np(w)
+    s, z = oracle.choose_qparams_affine(wn, code, (1, 256), 0, -128, 127, eps=eps, zp_dtype=oracle.I64)
+    if dtype is torch.bfloat16:
+        assert np.array_equal(s[:, 0], bits16(scale_ref))
+    else:
+        assert np.array_equal(s[:, 0], _np(scale_ref))
+    assert np.all(z == 0)
+    q = oracle.quantize_affine(wn, code, (1, 256), s, code, z, oracle.I64, -128, 127, zp_domain=0, out_dtype=oracle.I8)
+    assert np.array_equal(q, q_ref.numpy())
+    assert q.min() >= -128 and q.max() <= 127 and np.abs(q).max() >= 127   # the row maximum maps to +-127 or -128
