@@ -687,44 +687,46 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
 }
 
 // ---------------------------------------------------------------- GEMM path (M > 16)
-// Workgroup tile: 128 activation rows x 128 weight rows, K walked in 128-wide tiles.  Each of the 4 waves owns
-// two 16-row weight blocks: it loads their packed tiles straight into registers, dequantizes every dword once
-// and multiplies it against all eight 16-row activation blocks (16 MFMAs per pair of dequantized dwords), so
-// the dequantization cost is spread over 128 activation rows.  The activation tile goes through LDS (row
-// stride 272 bytes: the 16-byte fragment reads of 8 consecutive lanes fall on distinct banks) and is fetched
-// one K tile ahead into registers.
-template <int G>
+// Workgroup tile: BM = 16 * MBLK activation rows x 64 * NBW weight rows, K walked in 128-wide tiles (128 x 128 when
+// such tiles give at least one workgroup per CU, 64 x 64 otherwise).  Each of the 4 waves owns NBW 16-row weight
+// blocks: it loads their packed tiles straight into registers, dequantizes every dword once and multiplies it
+// against all MBLK 16-row activation blocks, so the dequantization cost is spread over BM activation rows.  The
+// activation tile is double-buffered in LDS (row stride 272 bytes: the 16-byte fragment reads of 8 consecutive
+// lanes fall on distinct banks), fetched two K tiles ahead into registers.
+template <int G, int NBW, int MBLK>
 __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a) {
-    constexpr int BM = 128, XSTRIDE = 136;  // bf16 elements per LDS row
+    // NBW 16-row weight blocks per wave (workgroup: 64 * NBW weight rows), MBLK 16-row activation blocks per tile
+    constexpr int BM = 16 * MBLK, XSTRIDE = 136;  // bf16 elements per LDS row
+    constexpr int XCH = BM / 16;                  // 16-byte activation chunks per thread and K tile
     __shared__ __align__(16) uint16_t xs_all[2][BM * XSTRIDE];  // two K tiles: one being read, one being filled
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, qd = lane >> 4;
     const int KB = (int)(a.Kp / 128);
     const int64_t nblocks = (a.N + 15) / 16;
-    const int64_t nb0 = (int64_t)blockIdx.x * 8 + 2 * wave;
-    const bool has0 = nb0 < nblocks, has1 = nb0 + 1 < nblocks;
+    const int64_t nb0 = (int64_t)blockIdx.x * (4 * NBW) + NBW * wave;
+    const bool has0 = nb0 < nblocks, has1 = NBW > 1 && nb0 + 1 < nblocks;
     const int64_t m0 = (int64_t)blockIdx.y * BM;
     const uint32_t magic = 0x43004300u, one_lo = 0x00003F80u, one_hi = 0x3F800000u;
 
     // activation tile loader: thread t covers rows (t>>4) + 16*j, 16-byte chunk t&15 of the 256-byte row slice
     const int xrow = tid >> 4, xchunk = tid & 15;
-    u32x4_t xr[8];
+    u32x4_t xr[XCH];
     // rows past M alias the last row: their products land in output rows that are never stored, and a loader
     // without branches lets the compiler keep exact counts of the loads in flight
-    const uint16_t* xrow_ptr[8];
+    const uint16_t* xrow_ptr[XCH];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < XCH; ++j) {
         const int64_t m = m0 + xrow + 16 * j;
         xrow_ptr[j] = a.x + (m < a.M ? m : a.M - 1) * a.ldx + xchunk * 8;
     }
     auto load_x = [&](int kb) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) xr[j] = *reinterpret_cast<const u32x4_t*>(xrow_ptr[j] + (int64_t)kb * 128);
+        for (int j = 0; j < XCH; ++j) xr[j] = *reinterpret_cast<const u32x4_t*>(xrow_ptr[j] + (int64_t)kb * 128);
     };
     auto store_x = [&](int buf) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < XCH; ++j)
             *reinterpret_cast<u32x4_t*>(xs_all[buf] + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
     };
 
@@ -736,14 +738,16 @@ __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a)
     auto load_w = [&](WBuf& b, int kb) {
         const int gidx = ((kb * 128 + qd * 32) / G) * 16;
         b.w0 = *reinterpret_cast<const u32x4_t*>(wp0 + (int64_t)kb * 64);
-        b.w1 = *reinterpret_cast<const u32x4_t*>(wp1 + (int64_t)kb * 64);
         b.q0 = qp0[gidx];
-        b.q1 = qp1[gidx];
+        if (NBW > 1) {
+            b.w1 = *reinterpret_cast<const u32x4_t*>(wp1 + (int64_t)kb * 64);
+            b.q1 = qp1[gidx];
+        }
     };
 
-    f32x4_t acc0[8], acc1[8];
+    f32x4_t acc0[MBLK], acc1[MBLK];
 #pragma unroll
-    for (int mb = 0; mb < 8; ++mb) {
+    for (int mb = 0; mb < MBLK; ++mb) {
         acc0[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         acc1[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
@@ -756,10 +760,10 @@ __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a)
         // that slice, so that the LDS latency hides behind the VALU work; the scheduling barriers keep the compiler
         // from sinking the reads back down to their first use.
         union XFrag { uint4 q; bf16x8_t v; };
-        XFrag xa[2][8];
+        XFrag xa[2][MBLK];
         auto read_frags = [&](int sl, XFrag* dst) {
 #pragma unroll
-            for (int mb = 0; mb < 8; ++mb)
+            for (int mb = 0; mb < MBLK; ++mb)
                 dst[mb].q = *reinterpret_cast<const uint4*>(xs + (mb * 16 + r) * XSTRIDE + qd * 32 + sl * 8);
         };
         read_frags(0, xa[0]);
@@ -768,12 +772,14 @@ __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a)
             if (sl + 1 < 4) read_frags(sl + 1, xa[(sl + 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
             const bf16x8_t bw0 = dequant8(w0[sl], g0, magic, one_lo, one_hi);
-            const bf16x8_t bw1 = dequant8(w1[sl], g1, magic, one_lo, one_hi);
+            bf16x8_t bw1 = bw0;
+            if (NBW > 1) bw1 = dequant8(w1[sl], g1, magic, one_lo, one_hi);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mb = 0; mb < 8; ++mb) {
+            for (int mb = 0; mb < MBLK; ++mb) {
                 acc0[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[sl & 1][mb].v, bw0, acc0[mb], 0, 0, 0);
-                acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[sl & 1][mb].v, bw1, acc1[mb], 0, 0, 0);
+                if (NBW > 1)
+                    acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[sl & 1][mb].v, bw1, acc1[mb], 0, 0, 0);
             }
         }
     };
@@ -804,13 +810,13 @@ __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a)
 
     // acc[mb][i] = C[m = m0 + 16*mb + 4*qd + i][n = 16*nb + r]
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < NBW; ++h) {
         if (!(h == 0 ? has0 : has1)) continue;
         const int64_t n = (nb0 + h) * 16 + r;
         if (n >= a.N) continue;
         const float bv = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.f;
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb)
+        for (int mb = 0; mb < MBLK; ++mb)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int64_t m = m0 + mb * 16 + 4 * qd + i;
@@ -934,14 +940,22 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
                "fused rmsnorm needs M <= 16, K a multiple of max(128, group), 16-byte aligned rows and norm weight, and "
                "activations that fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);
     if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16) {
-        dim3 ggrid((unsigned)((RB + 7) / 8), (unsigned)((M + 127) / 128));
+        // 128 x 128 workgroup tiles when they fill a good part of the 256 CUs, else 64 x 64 tiles: four times
+        // the workgroups, each dequantizing for 64 activation rows only
+        const bool big = ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
+        dim3 ggrid(big ? (unsigned)((RB + 7) / 8) : (unsigned)((RB + 3) / 4),
+                   big ? (unsigned)((M + 127) / 128) : (unsigned)((M + 63) / 64));
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
+#define AO_GEMM_LAUNCH(GG)                                                                        \
+    if (big) launch_timed(int4wo_gemm_kernel<GG, 2, 8>, ggrid, dim3(256), 0, st, a);              \
+    else launch_timed(int4wo_gemm_kernel<GG, 1, 4>, ggrid, dim3(256), 0, st, a)
         switch (g) {
-            case 32: launch_timed(int4wo_gemm_kernel<32>, ggrid, dim3(256), 0, st, a); break;
-            case 64: launch_timed(int4wo_gemm_kernel<64>, ggrid, dim3(256), 0, st, a); break;
-            case 128: launch_timed(int4wo_gemm_kernel<128>, ggrid, dim3(256), 0, st, a); break;
-            default: launch_timed(int4wo_gemm_kernel<256>, ggrid, dim3(256), 0, st, a); break;
+            case 32: AO_GEMM_LAUNCH(32); break;
+            case 64: AO_GEMM_LAUNCH(64); break;
+            case 128: AO_GEMM_LAUNCH(128); break;
+            default: AO_GEMM_LAUNCH(256); break;
         }
+#undef AO_GEMM_LAUNCH
         AO_LAUNCH_CHECK();
         return 0;
     }

@@ -164,11 +164,13 @@ def test_linear_one_hot_is_exact_dequant(cabi, oracle, g):
     x = torch.zeros(len(ks), K, dtype=torch.bfloat16)
     for m, k in enumerate(ks):
         x[m, k] = 1.0
-    y = _linear(cabi, x.to(_dev()), packed, qparams, N, g, fp32=True).cpu().numpy()
     dq, _ = _oracle_linear(oracle, w, x, g)
     dqf = oracle.bf16_bits_to_f32(dq)
-    for m, k in enumerate(ks):
-        assert np.array_equal(y[m], dqf[:, k]), (m, k)
+    # 18 rows run on the tiled kernel (M > 16), 16 and 1 on the decode kernel: each has its own dequantization code
+    for rows in (len(ks), 16, 1):
+        y = _linear(cabi, x[:rows].contiguous().to(_dev()), packed, qparams, N, g, fp32=True).cpu().numpy()
+        for m, k in enumerate(ks[:rows]):
+            assert np.array_equal(y[m], dqf[:, k]), (rows, m, k)
 
 
 @pytest.mark.parametrize("M", [1, 4, 16, 33])
