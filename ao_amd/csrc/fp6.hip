@@ -302,39 +302,40 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* 
 // double-buffered in LDS (row stride 272 bytes), fetched two tiles ahead into registers; every load is
 // unconditional (rows past M alias the last row, tiles past the end repeat the last tile) so that the compiler's
 // vmcnt waits stay exact.
-template <bool E3M2>
+template <bool E3M2, int NBW, int MBLK>
 __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
                                                            const uint32_t* __restrict__ native,
                                                            const uint16_t* __restrict__ scale, int64_t N,
                                                            uint16_t* __restrict__ out) {
     typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
     typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-    constexpr int BM = 128, XSTRIDE = 136;  // fp16 elements per LDS row
+    constexpr int BM = 16 * MBLK, XSTRIDE = 136;  // fp16 elements per LDS row
+    constexpr int XCH = BM / 16;                  // 16-byte activation chunks per thread and K tile
     __shared__ __align__(16) uint16_t xs_all[2][BM * XSTRIDE];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, qd = lane >> 4;
     const int KB = (int)(K / 128);
     const int64_t nblocks = N / 16;
-    const int64_t nb0 = (int64_t)blockIdx.x * 8 + 2 * wave;
-    const bool has0 = nb0 < nblocks, has1 = nb0 + 1 < nblocks;
+    const int64_t nb0 = (int64_t)blockIdx.x * (4 * NBW) + NBW * wave;
+    const bool has0 = nb0 < nblocks, has1 = NBW > 1 && nb0 + 1 < nblocks;
     const int64_t m0 = (int64_t)blockIdx.y * BM;
 
     const int xrow = tid >> 4, xchunk = tid & 15;
-    const uint16_t* xrow_ptr[8];
+    const uint16_t* xrow_ptr[XCH];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < XCH; ++j) {
         const int64_t m = m0 + xrow + 16 * j;
         xrow_ptr[j] = x + (m < M ? m : M - 1) * K + xchunk * 8;
     }
-    u32x4_t xr[8];
+    u32x4_t xr[XCH];
     auto load_x = [&](int kb) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) xr[j] = *reinterpret_cast<const u32x4_t*>(xrow_ptr[j] + (int64_t)kb * 128);
+        for (int j = 0; j < XCH; ++j) xr[j] = *reinterpret_cast<const u32x4_t*>(xrow_ptr[j] + (int64_t)kb * 128);
     };
     auto store_x = [&](int buf) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < XCH; ++j)
             *reinterpret_cast<u32x4_t*>(xs_all[buf] + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
     };
 
@@ -344,17 +345,19 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
     auto load_w = [&](WBuf& b, int kb) {
         b.lo0 = reinterpret_cast<const u32x4_t*>(t0 + (int64_t)kb * 384)[lane];
         b.hi0 = reinterpret_cast<const u32x2_t*>(t0 + (int64_t)kb * 384 + 256)[lane];
-        b.lo1 = reinterpret_cast<const u32x4_t*>(t1 + (int64_t)kb * 384)[lane];
-        b.hi1 = reinterpret_cast<const u32x2_t*>(t1 + (int64_t)kb * 384 + 256)[lane];
+        if (NBW > 1) {
+            b.lo1 = reinterpret_cast<const u32x4_t*>(t1 + (int64_t)kb * 384)[lane];
+            b.hi1 = reinterpret_cast<const u32x2_t*>(t1 + (int64_t)kb * 384 + 256)[lane];
+        }
     };
     union { uint16_t h; _Float16 f; } s0, s1;
     s0.h = scale[(has0 ? nb0 : 0) * 16 + r];
     s1.h = scale[(has1 ? nb0 + 1 : 0) * 16 + r];
     const f16x2_t sc0 = {s0.f, s0.f}, sc1 = {s1.f, s1.f};
 
-    f32x4_t acc0[8], acc1[8];
+    f32x4_t acc0[MBLK], acc1[MBLK];
 #pragma unroll
-    for (int mb = 0; mb < 8; ++mb) {
+    for (int mb = 0; mb < MBLK; ++mb) {
         acc0[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         acc1[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
@@ -365,12 +368,12 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
     };
     auto compute = [&](const WBuf& b, int buf) {
         const uint16_t* xs = xs_all[buf];
-        const f16x32_t v0 = convert(b.lo0, b.hi0), v1 = convert(b.lo1, b.hi1);
+        const f16x32_t v0 = convert(b.lo0, b.hi0), v1 = NBW > 1 ? convert(b.lo1, b.hi1) : v0;
         union XFrag { uint4 q; f16x8_t v; };
-        XFrag xa[2][8];
+        XFrag xa[2][MBLK];
         auto read_frags = [&](int sl, XFrag* dst) {
 #pragma unroll
-            for (int mb = 0; mb < 8; ++mb)
+            for (int mb = 0; mb < MBLK; ++mb)
                 dst[mb].q = *reinterpret_cast<const uint4*>(xs + (mb * 16 + r) * XSTRIDE + qd * 32 + sl * 8);
         };
         read_frags(0, xa[0]);
@@ -386,9 +389,10 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
                 w1.p[j] = p1 * sc1;
             }
 #pragma unroll
-            for (int mb = 0; mb < 8; ++mb) {
+            for (int mb = 0; mb < MBLK; ++mb) {
                 acc0[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[sl & 1][mb].v, w0.v, acc0[mb], 0, 0, 0);
-                acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[sl & 1][mb].v, w1.v, acc1[mb], 0, 0, 0);
+                if (NBW > 1)
+                    acc1[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[sl & 1][mb].v, w1.v, acc1[mb], 0, 0, 0);
             }
         }
     };
@@ -417,11 +421,11 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
 
     // acc[mb][i] = C[m = m0 + 16*mb + 4*qd + i][n = 16*nb + r]
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < NBW; ++h) {
         if (!(h == 0 ? has0 : has1)) continue;
         const int64_t n = (nb0 + h) * 16 + r;
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb)
+        for (int mb = 0; mb < MBLK; ++mb)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int64_t m = m0 + mb * 16 + 4 * qd + i;
@@ -506,16 +510,19 @@ extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const 
     uint16_t* o = (uint16_t*)out_f16;
     hipEvent_t ev0 = g_prof_start, ev1 = g_prof_stop;  // optional per-kernel timing, see common.h
     g_prof_start = g_prof_stop = nullptr;
-    // the tiled kernel pays off once its grid can occupy a good part of the 256 CUs; below that the skinny kernel
-    // (one workgroup per 16 x 16 output block, K split over waves) has more parallelism
-    const int64_t gemm_wgs = ((RB + 7) / 8) * ((M + 127) / 128);
-    if (M > 16 && K % 128 == 0 && (gemm_wgs >= 96 || M >= 256)) {
-        dim3 ggrid((unsigned)((RB + 7) / 8), (unsigned)((M + 127) / 128));
+    // tiled kernel: 128 x 128 workgroup tiles when they give at least one workgroup per CU, else 64 x 64
+    if (M > 16 && K % 128 == 0) {
+        const bool big = ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
+        dim3 ggrid(big ? (unsigned)((RB + 7) / 8) : (unsigned)((RB + 3) / 4),
+                   big ? (unsigned)((M + 127) / 128) : (unsigned)((M + 63) / 64));
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
-        if (ebits == 3)
-            hipExtLaunchKernelGGL((fp6_gemm_kernel<true>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
-        else
-            hipExtLaunchKernelGGL((fp6_gemm_kernel<false>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+        if (ebits == 3) {
+            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 2, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            else hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+        } else {
+            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 2, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            else hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+        }
         AO_LAUNCH_CHECK();
         return 0;
     }
