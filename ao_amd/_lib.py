@@ -45,7 +45,7 @@ _SIGNATURES = {
     "ao_amd_fp6_quantize_pack": ([_p, _int, _i64, _i64, _int, _int, _p, _p, _p], _int),
     "ao_amd_fp6_dequantize": ([_p, _p, _i64, _i64, _int, _int, _p, _p], _int),
     "ao_amd_fp6_native_bytes": ([_i64, _i64, _i64p], _int),
-    "ao_amd_fp6_repack": ([_p, _i64, _i64, _p, _p], _int),
+    "ao_amd_fp6_repack": ([_p, _i64, _i64, _int, _p, _p], _int),
     "ao_amd_fp6_linear": ([_p, _i64, _i64, _p, _p, _i64, _int, _int, _p, _p], _int),
     "ao_amd_int4wo_linear_residual": ([_p, _i64, _i64, _i64, _p, _p, _i64, _i64, _p, _p, _i64, _p, _i64, _p], _int),
     "ao_amd_int4wo_swiglu": ([_p, _i64, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p], _int),

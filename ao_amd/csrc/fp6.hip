@@ -86,10 +86,31 @@ __device__ __forceinline__ TcPos tc_fp6_pos(int64_t row, int64_t col, int64_t C)
     return t;
 }
 
+// FP5 (e2m2, e3m1): planes are 1 bit (code >> 4) then 4 bits (quant_llm.py:60-86 with nbits = 5).  The 4-bit plane
+// is laid out exactly as for FP6; the top bit of element (row, col) sits at (byte B1, shift sh1) of plane 1.
+__device__ __forceinline__ void tc_fp5_hi_pos(int64_t row, int64_t col, int64_t C, int64_t& b1, int& sh1) {
+    const int64_t a = row >> 6, e = col >> 4, E = C >> 4;
+    const int rr = (int)(row & 63), i1 = rr >> 5, i2 = (rr >> 4) & 1, i3 = (rr >> 3) & 1, d = rr & 7;
+    const int f = (int)((col >> 3) & 1), g = (int)(col & 7), p = 1 - i3;
+    b1 = (((a * E + e) * 8 + d) * 8 + g) * 2 + p;
+    sh1 = 7 - (f + 2 * i2 + 4 * i1);
+}
+// code of element (row, col) from the TC-FPx bytes of a [N, K] weight, nbits in {5, 6}
+__device__ __forceinline__ uint32_t tc_fpx_code(const uint8_t* __restrict__ tc, int64_t N, int64_t K, int64_t row,
+                                                int64_t col, int nbits) {
+    const TcPos t = tc_fp6_pos(row, col, K);
+    if (nbits == 6) return (((tc[t.b2] >> t.sh2) & 3u) << 4) | ((tc[N * K / 4 + t.b4] >> t.sh4) & 15u);
+    int64_t b1;
+    int sh1;
+    tc_fp5_hi_pos(row, col, K, b1, sh1);
+    return (((tc[b1] >> sh1) & 1u) << 4) | ((tc[N * K / 8 + t.b4] >> t.sh4) & 15u);
+}
+
 // ---------------------------------------------------------------- quantize + pack (to_scaled_tc_fpx)
 // One workgroup per 64-row block.  Pass 1: row amax -> fp32 scale (amax clamped at 1e-12, divided by the largest
-// normal).  Pass 2, per 16-column slice: 1024 codes into LDS, then every thread assembles one byte of the 2-bit
-// plane and two bytes of the 4-bit plane of that slice.
+// normal).  Pass 2, per 16-column slice: 1024 codes into LDS, then the threads assemble the bytes of the high
+// plane (FP6: one byte of the 2-bit plane per thread; FP5: one byte of the 1-bit plane per thread of the first
+// two waves) and two bytes of the 4-bit plane of that slice.
 __global__ __launch_bounds__(256) void fp6_quantize_pack_kernel(const void* __restrict__ w, int w_dtype, int64_t N,
                                                                  int64_t K, int ebits, int mbits,
                                                                  uint8_t* __restrict__ out, uint16_t* __restrict__ scale_out) {
@@ -122,8 +143,9 @@ __global__ __launch_bounds__(256) void fp6_quantize_pack_kernel(const void* __re
         }
     }
     __syncthreads();
+    const int nbits = 1 + ebits + mbits;
     uint8_t* p2 = out;
-    uint8_t* p4 = out + N * K / 4;
+    uint8_t* p4 = out + (nbits == 6 ? N * K / 4 : N * K / 8);
     const int64_t E = K >> 4;
     for (int64_t e = 0; e < E; ++e) {
 #pragma unroll
@@ -135,13 +157,27 @@ __global__ __launch_bounds__(256) void fp6_quantize_pack_kernel(const void* __re
         __syncthreads();
         {
             const int i1 = tid >> 7, d = (tid >> 4) & 7, g = (tid >> 1) & 7, p = tid & 1, i3 = 1 - p;
-            uint32_t b2 = 0;
+            if (nbits == 6) {
+                uint32_t b2 = 0;
 #pragma unroll
-            for (int i2 = 0; i2 < 2; ++i2)
+                for (int i2 = 0; i2 < 2; ++i2)
 #pragma unroll
-                for (int f = 0; f < 2; ++f)
-                    b2 = (b2 << 2) | ((codes_s[32 * i1 + 16 * i2 + 8 * i3 + d][8 * f + g] >> 4) & 3u);
-            p2[(a * E + e) * 256 + tid] = (uint8_t)b2;
+                    for (int f = 0; f < 2; ++f)
+                        b2 = (b2 << 2) | ((codes_s[32 * i1 + 16 * i2 + 8 * i3 + d][8 * f + g] >> 4) & 3u);
+                p2[(a * E + e) * 256 + tid] = (uint8_t)b2;
+            } else if (tid < 128) {
+                // byte (d, g, p) of the 1-bit plane: bits, MSB first, in the order (j1, j2, f) = 4*j1 + 2*j2 + f
+                const int dd = tid >> 4, gg = (tid >> 1) & 7, pp = tid & 1, j3 = 1 - pp;
+                uint32_t b1 = 0;
+#pragma unroll
+                for (int j1 = 0; j1 < 2; ++j1)
+#pragma unroll
+                    for (int j2 = 0; j2 < 2; ++j2)
+#pragma unroll
+                        for (int f = 0; f < 2; ++f)
+                            b1 = (b1 << 1) | ((codes_s[32 * j1 + 16 * j2 + 8 * j3 + dd][8 * f + gg] >> 4) & 1u);
+                p2[(a * E + e) * 128 + tid] = (uint8_t)b1;
+            }
 #pragma unroll
             for (int i2 = 0; i2 < 2; ++i2) {
                 const int rr = 32 * i1 + 16 * i2 + 8 * i3 + d;
@@ -159,16 +195,17 @@ __global__ __launch_bounds__(256) void fp6_dequantize_kernel(const uint8_t* __re
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= N * K) return;
     const int64_t row = i / K, col = i % K;
-    const TcPos t = tc_fp6_pos(row, col, K);
-    const uint32_t code = (((tc[t.b2] >> t.sh2) & 3u) << 4) | ((tc[N * K / 4 + t.b4] >> t.sh4) & 15u);
+    const uint32_t code = tc_fpx_code(tc, N, K, row, col, 1 + ebits + mbits);
     float v = fpx_to_f32(code, ebits, mbits);
     if (scale) v *= f16_bits_to_f32(scale[row]);
     out[i] = v;
 }
 
-// TC-FP6 bytes -> native tiles.  One thread per (lane, tile): gathers its 32 codes and writes 6 dwords.
+// TC-FPx bytes -> native tiles.  One thread per (lane, tile): gathers its 32 codes and writes 6 dwords.  A 5-bit
+// code becomes the 6-bit code of the same value (one more mantissa bit, zero): e2m2 -> e2m3, e3m1 -> e3m2, so the
+// linear kernels only ever see the two 6-bit formats the hardware converts.
 __global__ __launch_bounds__(256) void fp6_repack_kernel(const uint8_t* __restrict__ tc, int64_t N, int64_t K, int64_t Kp,
-                                                          uint32_t* __restrict__ native) {
+                                                          int nbits, uint32_t* __restrict__ native) {
     const int64_t KB = Kp / 128;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (N / 16) * KB * 64) return;
@@ -178,10 +215,7 @@ __global__ __launch_bounds__(256) void fp6_repack_kernel(const uint8_t* __restri
     uint32_t words[6] = {0, 0, 0, 0, 0, 0};
     for (int j = 0; j < 32; ++j) {
         uint32_t code = 0;
-        if (k0 + j < K) {
-            const TcPos t = tc_fp6_pos(row, k0 + j, K);
-            code = (((tc[t.b2] >> t.sh2) & 3u) << 4) | ((tc[N * K / 4 + t.b4] >> t.sh4) & 15u);
-        }
+        if (k0 + j < K) code = tc_fpx_code(tc, N, K, row, k0 + j, nbits) << (6 - nbits);
         const int bit = 6 * j;
         words[bit >> 5] |= code << (bit & 31);
         if ((bit & 31) > 26) words[(bit >> 5) + 1] |= code >> (32 - (bit & 31));
@@ -435,8 +469,9 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
 }
 
 static int check_fp6_format(int ebits, int mbits) {
-    AO_REQUIRE((ebits == 3 && mbits == 2) || (ebits == 2 && mbits == 3),
-               "FP%d E%dM%d is not supported (6-bit formats e3m2 and e2m3 only)", 1 + ebits + mbits, ebits, mbits);
+    AO_REQUIRE((ebits == 3 && mbits == 2) || (ebits == 2 && mbits == 3) || (ebits == 2 && mbits == 2) ||
+                   (ebits == 3 && mbits == 1),
+               "FP%d E%dM%d is not supported (e3m2, e2m3, e2m2 and e3m1 only)", 1 + ebits + mbits, ebits, mbits);
     return 0;
 }
 
@@ -477,14 +512,15 @@ extern "C" int ao_amd_fp6_native_bytes(int64_t N, int64_t K, int64_t* bytes) {
     return 0;
 }
 
-extern "C" int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, void* native, void* stream) {
+extern "C" int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, int nbits, void* native, void* stream) {
     AO_REQUIRE(tc && native, "null pointer argument");
+    AO_REQUIRE(nbits == 5 || nbits == 6, "TC-FPx codes of %d bits are not supported (5 or 6)", nbits);
     AO_REQUIRE(N > 0 && K > 0 && N % 64 == 0 && K % 64 == 0, "TC-FPx shapes must be multiples of 64, got (%lld, %lld)",
                (long long)N, (long long)K);
     const int64_t Kp = round_up(K, 128);
     const int64_t n = (N / 16) * (Kp / 128) * 64;
     hipLaunchKernelGGL(fp6_repack_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       (const uint8_t*)tc, N, K, Kp, (uint32_t*)native);
+                       (const uint8_t*)tc, N, K, Kp, nbits, (uint32_t*)native);
     AO_LAUNCH_CHECK();
     return 0;
 }

@@ -53,7 +53,7 @@ _LIB.define("llama_decode_attention(Tensor qkv, Tensor freqs_cis, Tensor input_p
 _LIB.define("quant_llm_linear(int EXPONENT, int MANTISSA, Tensor _in_feats, Tensor _weights, Tensor _scales, int splitK) -> Tensor")
 _LIB.define("fp6_quantize_pack(Tensor w, int ebits, int mbits) -> (Tensor, Tensor)")
 _LIB.define("fp6_dequantize(Tensor fpx_data, Tensor? scale, int ebits, int mbits) -> Tensor")
-_LIB.define("fp6_repack(Tensor fpx_data) -> Tensor")
+_LIB.define("fp6_repack(Tensor fpx_data, int nbits=6) -> Tensor")
 _LIB.define("fp6_linear_native(int ebits, int mbits, Tensor x, Tensor native, Tensor scale) -> Tensor")
 
 
@@ -296,8 +296,8 @@ def _fp6_native_numel(N: int, K: int) -> int:
 
 
 def _check_fp6_format(ebits, mbits):
-    torch._check((ebits, mbits) in ((3, 2), (2, 3)),
-                 lambda: f"FP{1 + ebits + mbits} E{ebits}M{mbits} is not supported (6-bit formats e3m2 and e2m3 only)")
+    torch._check((ebits, mbits) in ((3, 2), (2, 3), (2, 2), (3, 1)),
+                 lambda: f"FP{1 + ebits + mbits} E{ebits}M{mbits} is not supported (e3m2, e2m3, e2m2 and e3m1 only)")
 
 
 def _fp6_quantize_pack_cuda(w, ebits, mbits):
@@ -308,7 +308,7 @@ def _fp6_quantize_pack_cuda(w, ebits, mbits):
     N, K = w.shape
     torch._check(N % 64 == 0 and K % 64 == 0, lambda: f"TC-FPx packing needs multiples of 64, got ({N}, {K})")
     w = w.contiguous()
-    data = torch.empty((N, K // 8 * 6), dtype=torch.uint8, device=w.device)
+    data = torch.empty((N, K // 8 * (1 + ebits + mbits)), dtype=torch.uint8, device=w.device)
     scale = torch.empty((N,), dtype=torch.float16, device=w.device)
     check(lib().ao_amd_fp6_quantize_pack(w.data_ptr(), DTYPE_CODE[w.dtype], N, K, ebits, mbits, data.data_ptr(),
                                          scale.data_ptr(), current_stream(w.device)))
@@ -319,7 +319,7 @@ def _fp6_dequantize_cuda(fpx_data, scale, ebits, mbits):
     require_cuda(fpx_data, scale)
     _check_fp6_format(ebits, mbits)
     torch._check(fpx_data.dim() == 2 and fpx_data.dtype is torch.uint8, lambda: "fpx_data must be a 2d uint8 tensor")
-    N, K = fpx_data.shape[0], fpx_data.shape[1] // 6 * 8
+    N, K = fpx_data.shape[0], fpx_data.shape[1] // (1 + ebits + mbits) * 8
     if scale is not None:
         torch._check(scale.dtype is torch.float16 and scale.numel() == N, lambda: "scale must be float16 of size N")
         scale = scale.contiguous()
@@ -329,12 +329,13 @@ def _fp6_dequantize_cuda(fpx_data, scale, ebits, mbits):
     return out
 
 
-def _fp6_repack_cuda(fpx_data):
+def _fp6_repack_cuda(fpx_data, nbits=6):
     require_cuda(fpx_data)
     torch._check(fpx_data.dim() == 2 and fpx_data.dtype is torch.uint8, lambda: "fpx_data must be a 2d uint8 tensor")
-    N, K = fpx_data.shape[0], fpx_data.shape[1] // 6 * 8
+    torch._check(nbits in (5, 6), lambda: f"TC-FPx codes of {nbits} bits are not supported (5 or 6)")
+    N, K = fpx_data.shape[0], fpx_data.shape[1] // nbits * 8
     native = torch.empty((_fp6_native_numel(N, K),), dtype=torch.int32, device=fpx_data.device)
-    check(lib().ao_amd_fp6_repack(fpx_data.contiguous().data_ptr(), N, K, native.data_ptr(),
+    check(lib().ao_amd_fp6_repack(fpx_data.contiguous().data_ptr(), N, K, nbits, native.data_ptr(),
                                   current_stream(fpx_data.device)))
     return native
 
@@ -373,7 +374,7 @@ def _quant_llm_linear_cuda(EXPONENT, MANTISSA, _in_feats, _weights, _scales, spl
     else:
         if len(_REPACK_CACHE) >= 256:
             _REPACK_CACHE.clear()
-        native = _fp6_repack_cuda(_weights)
+        native = _fp6_repack_cuda(_weights, 1 + EXPONENT + MANTISSA)
         _REPACK_CACHE[key] = (weakref.ref(_weights, lambda _, k=key: _REPACK_CACHE.pop(k, None)),
                               (_weights._version, _weights.data_ptr()), native)
     return _fp6_linear_native_cuda(EXPONENT, MANTISSA, _in_feats, native, _scales)
@@ -505,18 +506,18 @@ def _(EXPONENT, MANTISSA, _in_feats, _weights, _scales, splitK=1):
 
 @torch.library.register_fake("torchao::fp6_quantize_pack")
 def _(w, ebits, mbits):
-    return (w.new_empty((w.shape[0], w.shape[1] // 8 * 6), dtype=torch.uint8),
+    return (w.new_empty((w.shape[0], w.shape[1] // 8 * (1 + ebits + mbits)), dtype=torch.uint8),
             w.new_empty((w.shape[0],), dtype=torch.float16))
 
 
 @torch.library.register_fake("torchao::fp6_dequantize")
 def _(fpx_data, scale, ebits, mbits):
-    return fpx_data.new_empty((fpx_data.shape[0], fpx_data.shape[1] // 6 * 8), dtype=torch.float32)
+    return fpx_data.new_empty((fpx_data.shape[0], fpx_data.shape[1] // (1 + ebits + mbits) * 8), dtype=torch.float32)
 
 
 @torch.library.register_fake("torchao::fp6_repack")
-def _(fpx_data):
-    return fpx_data.new_empty((_fp6_native_numel(fpx_data.shape[0], fpx_data.shape[1] // 6 * 8),), dtype=torch.int32)
+def _(fpx_data, nbits=6):
+    return fpx_data.new_empty((_fp6_native_numel(fpx_data.shape[0], fpx_data.shape[1] // nbits * 8),), dtype=torch.int32)
 
 
 @torch.library.register_fake("torchao::fp6_linear_native")
@@ -545,9 +546,9 @@ def fp6_dequantize(fpx_data: Tensor, scale, ebits: int, mbits: int) -> Tensor:
     return torch.ops.torchao.fp6_dequantize.default(fpx_data, scale, ebits, mbits)
 
 
-def fp6_repack(fpx_data: Tensor) -> Tensor:
+def fp6_repack(fpx_data: Tensor, nbits: int = 6) -> Tensor:
     """TC-FPx bytes -> the kernel's wave64 tile order (int32 words)."""
-    return torch.ops.torchao.fp6_repack.default(fpx_data)
+    return torch.ops.torchao.fp6_repack.default(fpx_data, nbits)
 
 
 def fp6_linear_native(ebits: int, mbits: int, x: Tensor, native: Tensor, scale: Tensor) -> Tensor:

@@ -20,12 +20,14 @@ __all__ = ["to_scaled_tc_fpx", "from_scaled_tc_fpx", "QuantLlmLinearWeight", "qu
 
 
 def _check_fp6(ebits: int, mbits: int):
-    if 1 + ebits + mbits != 6:
-        raise NotImplementedError(f"FP{1 + ebits + mbits} E{ebits}M{mbits}: only 6-bit formats are implemented")
+    # the formats the reference kernel dispatches (torchao/csrc/cuda/fp6_llm/fp6_linear.cu:173-184)
+    if (ebits, mbits) not in ((3, 2), (2, 3), (2, 2), (3, 1)):
+        raise NotImplementedError(f"FP{1 + ebits + mbits} E{ebits}M{mbits} is not supported "
+                                  "(e3m2, e2m3, e2m2 and e3m1 only)")
 
 
 def to_scaled_tc_fpx(tensor: Tensor, ebits: int, mbits: int) -> Tuple[Tensor, Tensor]:
-    """float [N,K] -> (TC-FPx bytes uint8 [N, K*6/8], per-row scale fp16 [N])."""
+    """float [N,K] -> (TC-FPx bytes uint8 [N, K*nbits/8], per-row scale fp16 [N])."""
     _check_fp6(ebits, mbits)
     return ops.fp6_quantize_pack(tensor, ebits, mbits)
 
@@ -60,7 +62,7 @@ class QuantLlmLinearWeight(Tensor):
 
     def native(self) -> Tensor:
         if self._native is None:
-            self._native = ops.fp6_repack(self.fpx_data)
+            self._native = ops.fp6_repack(self.fpx_data, 1 + self.ebits + self.mbits)
         return self._native
 
     def __tensor_flatten__(self):

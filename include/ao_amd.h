@@ -169,28 +169,32 @@ int ao_amd_argmax_bf16(const void* x_bf16, int64_t n, int32_t* out_index, void* 
 /* ---------------------------------------------------------------- FP6-LLM (Quant-LLM FPx, e3m2 / e2m2 ...)
  * Interchange format = the reference's TC-FPx bytes, bit for bit. */
 
-/* replaces to_scaled_tc_fpx, torchao/prototype/quant_llm/quant_llm.py:116-130 for 6-bit formats
- * (ebits + mbits == 5): per-row scale = amax|w| / max_normal (fp32) stored as fp16, codes =
- * _f32_to_fpx_unpacked(w / scale) (torchao/prototype/custom_fp_utils.py:27-140), bytes = _pack_tc_fp6
- * (quant_llm.py:90-106).  w: [N,K] of w_dtype (AO_F32/BF16/F16) contiguous; N % 64 == 0, K % 64 == 0.
- * out_tc: uint8 [N, K*6/8]; out_scale: fp16 [N]. */
+/* replaces to_scaled_tc_fpx, torchao/prototype/quant_llm/quant_llm.py:116-130 for the formats the reference kernel
+ * accepts (torchao/csrc/cuda/fp6_llm/fp6_linear.cu:173-184): e3m2 and e2m3 (6 bits), e2m2 and e3m1 (5 bits).  Per-row
+ * scale = amax|w| / max_normal (fp32) stored as fp16, codes = _f32_to_fpx_unpacked(w / scale)
+ * (torchao/prototype/custom_fp_utils.py:27-140), bytes = _pack_tc_fpx (quant_llm.py:60-86; 6 bits: the 2-bit plane then
+ * the 4-bit plane, = _pack_tc_fp6 :90-106; 5 bits: the 1-bit plane then the 4-bit plane).
+ * w: [N,K] of w_dtype (AO_F32/BF16/F16) contiguous; N % 64 == 0, K % 64 == 0.
+ * out_tc: uint8 [N, K*nbits/8] with nbits = 1 + ebits + mbits; out_scale: fp16 [N]. */
 int ao_amd_fp6_quantize_pack(const void* w, int w_dtype, int64_t N, int64_t K, int ebits, int mbits, void* out_tc,
                              void* out_scale_f16, void* stream);
 
-/* replaces from_scaled_tc_fpx, torchao/prototype/quant_llm/quant_llm.py:203-208 (6-bit formats):
+/* replaces from_scaled_tc_fpx, torchao/prototype/quant_llm/quant_llm.py:203-208 (same four formats):
  * out fp32 [N,K] = fpx_to_f32(unpack(tc)) * float(scale) (scale may be NULL). */
 int ao_amd_fp6_dequantize(const void* tc, const void* scale_f16, int64_t N, int64_t K, int ebits, int mbits,
                           float* out, void* stream);
 
-/* One-time device repack of the TC-FP6 bytes into the kernel's wave64 order (no counterpart in the reference, whose
- * kernel reads the TC bytes directly with 32-lane fragment loads):
+/* One-time device repack of the TC-FPx bytes (nbits = 5 or 6) into the kernel's wave64 order (no counterpart in the
+ * reference, whose kernel reads the TC bytes directly with 32-lane fragment loads).  A 5-bit code is stored as the
+ * 6-bit code of the same value (e2m2 -> e2m3, e3m1 -> e3m2: one more mantissa bit, zero):
  *   native: per 16-row x 128-k tile 1536 bytes = [64 lanes][4 dwords] then [64 lanes][2 dwords]; lane l owns row
  *   16*rb + l%16 and the 32 consecutive k = 128*kb + 32*(l/16) + i, value i at bit 6*i of its 6 dwords; K is padded
  *   with zero codes to a multiple of 128.  ao_amd_fp6_native_bytes gives the buffer size. */
 int ao_amd_fp6_native_bytes(int64_t N, int64_t K, int64_t* bytes);
-int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, void* native, void* stream);
+int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, int nbits, void* native, void* stream);
 
-/* out[M,N] fp16 = x[M,K] fp16 @ W^T with W = fp16(fp6 value * scale), fp32 accumulation.
+/* out[M,N] fp16 = x[M,K] fp16 @ W^T with W = fp16(fpx value * scale), fp32 accumulation; (ebits, mbits) one of
+ * (3,2), (2,3), (2,2), (3,1).
  * replaces torchao::quant_llm_linear, schema torchao/csrc/fp6_llm.cpp:7, CUDA implementation
  * torchao/csrc/cuda/fp6_llm/fp6_linear.cu:139-196.  `weights_native` is the output of ao_amd_fp6_repack. */
 int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,

@@ -67,6 +67,7 @@ class _Sig:
     ao_oracle_pack_tc_fp6 = ([_p, _i64, _i64, _p], _int)
     ao_oracle_unpack_tc_fp6 = ([_p, _i64, _i64, _p], _int)
     ao_oracle_fp6_cuda_read_order = ([_p, _i64, _i64, _p], _int)
+    ao_oracle_fpx_cuda_read_order = ([_p, _i64, _i64, _int, _p], _int)
     ao_oracle_fpx_linear = ([_p, _i64, _i64, _p, _p, _i64, _int, _int, _p], _int)
     ao_oracle_abi_version = ([], _int)
 
@@ -241,6 +242,14 @@ def unpack_tc_fp6(packed, R, C):
     packed = np.ascontiguousarray(packed, np.uint8)
     codes = np.empty((R, C), np.uint8)
     _check(lib().ao_oracle_unpack_tc_fp6(_ptr(packed), R, C, _ptr(codes)), "unpack_tc_fp6")
+    return codes
+
+
+def fpx_cuda_read_order(packed, R, C, nbits):
+    """Codes [R,C] as the reference CUDA kernel reads them out of the TC-FPx bytes (nbits 5 or 6)."""
+    packed = np.ascontiguousarray(packed, np.uint8)
+    codes = np.empty((R, C), np.uint8)
+    _check(lib().ao_oracle_fpx_cuda_read_order(_ptr(packed), R, C, nbits, _ptr(codes)), "fpx_cuda_read_order")
     return codes
 
 

@@ -551,36 +551,44 @@ int ao_oracle_unpack_tc_fp6(const uint8_t* in, int64_t R, int64_t C, uint8_t* co
     return 0;
 }
 
-/* Emulation of how the reference CUDA kernel consumes the TC-FP6 bytes, used as a known-answer
+/* Emulation of how the reference CUDA kernel consumes the TC-FPx bytes, used as a known-answer
  * check of the packer: csrc/cuda/fp6_llm/kernel_matmul.cuh:57-104 (segment bases, tile order),
- * utils_core.cuh:27-35 (lane-strided fragment reads), utils_parallel_dequant.cuh:30-119 (bit
- * extraction into mma.m16n8k16 A fragments).  Reconstructs the 6-bit code of every weight
- * element [R,C] from the packed bytes. R % 256 == 0 (one thread block = 4 warps x 64 rows), C % 64 == 0. */
-int ao_oracle_fp6_cuda_read_order(const uint8_t* packed, int64_t R, int64_t C, uint8_t* codes) {
-    if (R % 64 || C % 64) return -1;
-    const uint32_t* seg2 = (const uint32_t*)packed;                 /* 2-bit plane */
-    const uint32_t* seg4 = (const uint32_t*)(packed + R * C / 4);   /* 4-bit plane */
+ * utils_core.cuh:27-35 (lane-strided fragment reads), utils_parallel_dequant.cuh:30-119 (1 + 2 + 4 bit
+ * extraction into mma.m16n8k16 A fragments).  Reconstructs the nbits-bit code (nbits 5 or 6) of every weight
+ * element [R,C] from the packed bytes: planes in the order 1-bit, 2-bit, 4-bit, those that nbits has.
+ * R % 64 == 0, C % 64 == 0. */
+int ao_oracle_fpx_cuda_read_order(const uint8_t* packed, int64_t R, int64_t C, int nbits, uint8_t* codes) {
+    if (R % 64 || C % 64 || (nbits != 5 && nbits != 6)) return -1;
+    const int use1 = nbits & 1, use2 = nbits & 2;
+    const uint32_t* seg1 = (const uint32_t*)packed;                                    /* 1-bit plane (FP5) */
+    const uint32_t* seg2 = (const uint32_t*)(packed + (use1 ? R * C / 8 : 0));         /* 2-bit plane (FP6) */
+    const uint32_t* seg4 = (const uint32_t*)(packed + (use1 ? R * C / 8 : 0) + (use2 ? R * C / 4 : 0));
     const int64_t KT = C / 64;
     for (int64_t Rb = 0; Rb < R / 64; ++Rb)         /* one warp's 64 rows */
         for (int64_t kb = 0; kb < KT; ++kb) {       /* 64-wide K tile */
-            /* tile base in uint32 words: 64 x 16-byte units for the 2-bit plane, 128 for the 4-bit */
+            /* tile base in uint32 words: 32 / 64 / 128 16-byte units for the 1 / 2 / 4-bit plane */
+            const uint32_t* t1 = seg1 + (Rb * KT + kb) * 32 * 4;
             const uint32_t* t2 = seg2 + (Rb * KT + kb) * 64 * 4;
             const uint32_t* t4 = seg4 + (Rb * KT + kb) * 128 * 4;
             for (int s = 0; s < 4; ++s)             /* 16-column slice */
                 for (int t = 0; t < 32; ++t) {      /* lane */
-                    uint32_t f2[2], f4[4];
-                    for (int i = 0; i < 2; ++i) f2[i] = t2[s * 2 * 32 + i * 32 + t];
+                    uint32_t f1 = 0, f2[2] = {0, 0}, f4[4];
+                    if (use1) f1 = t1[s * 32 + t];
+                    if (use2) for (int i = 0; i < 2; ++i) f2[i] = t2[s * 2 * 32 + i * 32 + t];
                     for (int i = 0; i < 4; ++i) f4[i] = t4[s * 4 * 32 + i * 32 + t];
-                    /* 8 iterations x 4 fp6 -> 16 registers x 2 fp16 = 4 mma tiles x 4 regs */
+                    /* 8 iterations x 4 codes -> 16 registers x 2 fp16 = 4 mma tiles x 4 regs */
                     for (int j = 0; j < 8; ++j) {
-                        uint32_t w2 = f2[j / 4], w4 = f4[j / 2];
-                        uint32_t P = (w2 & 0xC0C0C0C0u) | ((w4 & 0xF0F0F0F0u) >> 2);
-                        f2[j / 4] = w2 << 2;
-                        f4[j / 2] = w4 << 4;
+                        uint32_t P = 0;
+                        if (use1) { P |= (f1 & 0x80808080u) >> (nbits & 0); f1 <<= 1; }
+                        if (use2) { P |= (f2[j / 4] & 0xC0C0C0C0u) >> (nbits & 1); f2[j / 4] <<= 2; }
+                        P |= (f4[j / 2] & 0xF0F0F0F0u) >> (nbits & 3);
+                        f4[j / 2] <<= 4;
                         /* FPx_FP16_Cast_4Way: out1 <- bytes 3,1 ; out2 <- bytes 2,0.  In each
-                         * 32-bit output the high half comes from the higher byte. */
+                         * 32-bit output the high half comes from the higher byte; the code sits in the
+                         * top nbits of its byte. */
+                        const int down = 8 - nbits;
                         uint8_t b3 = (uint8_t)(P >> 24), b2 = (uint8_t)(P >> 16), b1 = (uint8_t)(P >> 8), b0 = (uint8_t)P;
-                        uint8_t c_out1_hi = b3 >> 2, c_out1_lo = b1 >> 2, c_out2_hi = b2 >> 2, c_out2_lo = b0 >> 2;
+                        uint8_t c_out1_hi = b3 >> down, c_out1_lo = b1 >> down, c_out2_hi = b2 >> down, c_out2_lo = b0 >> down;
                         /* register index: iteration j writes regs 2j (out1) and 2j+1 (out2) */
                         int reg1 = 2 * j, reg2 = 2 * j + 1;
                         uint8_t vals[2][2] = {{c_out1_lo, c_out1_hi}, {c_out2_lo, c_out2_hi}};
@@ -600,6 +608,9 @@ int ao_oracle_fp6_cuda_read_order(const uint8_t* packed, int64_t R, int64_t C, u
                 }
         }
     return 0;
+}
+int ao_oracle_fp6_cuda_read_order(const uint8_t* packed, int64_t R, int64_t C, uint8_t* codes) {
+    return ao_oracle_fpx_cuda_read_order(packed, R, C, 6, codes);
 }
 
 /* quant_llm_linear -- csrc/cuda/fp6_llm/fp6_linear.cu:139-196 + utils_parallel_dequant.cuh:47-59:

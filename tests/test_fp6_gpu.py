@@ -102,6 +102,40 @@ def test_e2m3_format(oracle):
     assert rel_l2(y, y_ref) <= 1e-3
 
 
+@pytest.mark.parametrize("fmt", [(2, 2), (3, 1)])
+@pytest.mark.parametrize("shape", [(64, 64), (256, 384), (512, 1024)])
+def test_fp5_formats(oracle, fmt, shape):
+    """e2m2 / e3m1 (torchao/csrc/cuda/fp6_llm/fp6_linear.cu:176-183): quantize + pack bit-exact against the oracle's
+    cast and the generic 1 + 4 bit packer, dequantize exact, linear within the reference test's tolerance
+    (test/test_ops.py:47-62 runs e2m2 alongside e3m2)."""
+    from ao_amd import ops
+    from ao_amd.prototype.quant_llm import QuantLlmLinearWeight
+
+    ebits, mbits = fmt
+    N, K = shape
+    print(f"case fp5 e{ebits}m{mbits} N={N} K={K}", flush=True)
+    dev = _dev()
+    g = torch.Generator().manual_seed(N + K + ebits)
+    w = (torch.randn(N, K, generator=g) * 0.05).half()
+    data, scale = ops.fp6_quantize_pack(w.to(dev), ebits, mbits)
+    codes_ref, scale_ref = oracle.fpx_quantize(bits16(w), oracle.F16, ebits, mbits)
+    assert data.shape == (N, K * 5 // 8)
+    assert np.array_equal(data.cpu().numpy(), oracle.pack_tc_fpx_generic(codes_ref, 5))
+    assert np.array_equal(bits16(scale), scale_ref)
+    dq = ops.fp6_dequantize(data, scale, ebits, mbits).cpu().numpy()
+    assert np.array_equal(dq, oracle.fpx_to_f32(codes_ref, ebits, mbits) * scale_ref.view(np.float16).astype(np.float32)[:, None])
+    for M in (1, 5, 40, 300):
+        x = (torch.rand(M, K, generator=g) + 0.5).half()
+        y = ops.quant_llm_linear(ebits, mbits, x.to(dev), data, scale, 1).float().cpu().numpy()
+        y_ref = oracle.fpx_linear(bits16(x), codes_ref, scale_ref, ebits, mbits).astype(np.float16).astype(np.float32)
+        assert rel_l2(y, y_ref) <= 1e-3, M
+    if N % 256 == 0:
+        qw = QuantLlmLinearWeight.from_float(w.to(dev), ebits, mbits)
+        assert qw.shape == (N, K)
+        y2 = torch.nn.functional.linear(x.to(dev), qw).float().cpu().numpy()
+        assert rel_l2(y2, y_ref) <= 1e-3
+
+
 def test_weight_subclass_and_api(oracle):
     """quantize(model, fp6_llm_weight_only()): shapes the kernel cannot take stay float; forward matches the oracle;
     leading dims and bias work (test/prototype/test_quant_llm.py:68-99)."""

@@ -83,6 +83,56 @@ def test_pack_three_formulations_agree(oracle, shape):
     assert np.array_equal(oracle.fp6_cuda_read_order(a, *shape), codes)
 
 
+def _fpx_value(code, ebits, mbits):
+    """Textbook small float: sign, ebits exponent bits (bias 2^(ebits-1) - 1), mbits mantissa bits, subnormals,
+    no inf / nan."""
+    bias = (1 << (ebits - 1)) - 1
+    s = -1.0 if (code >> (ebits + mbits)) & 1 else 1.0
+    e = (code >> mbits) & ((1 << ebits) - 1)
+    m = code & ((1 << mbits) - 1)
+    frac = m / float(1 << mbits)
+    return s * (2.0 ** (1 - bias) * frac if e == 0 else 2.0 ** (e - bias) * (1 + frac))
+
+
+@pytest.mark.parametrize("fmt", [(2, 2), (3, 1), (2, 3)])
+def test_five_bit_formats_all_codes_and_rounding(oracle, fmt):
+    """e2m2 and e3m1 (the 5-bit formats the reference kernel dispatches, fp6_linear.cu:176-183) and e2m3: every
+    code against the textbook value, every midpoint to the even neighbour, saturation at the largest normal
+    (7.0 for e2m2, 24.0 for e3m1, 7.5 for e2m3)."""
+    ebits, mbits = fmt
+    n = 1 << (ebits + mbits)
+    vals = oracle.fpx_to_f32(np.arange(2 * n, dtype=np.uint8), ebits, mbits)
+    assert np.array_equal(vals, np.array([_fpx_value(c, ebits, mbits) for c in range(2 * n)], np.float32))
+    assert np.array_equal(oracle.f32_to_fpx(vals, ebits, mbits), np.arange(2 * n, dtype=np.uint8))
+    grid = np.array([_fpx_value(c, ebits, mbits) for c in range(n)], np.float64)
+    assert grid[-1] == {(2, 2): 7.0, (3, 1): 24.0, (2, 3): 7.5}[fmt]
+    for c in range(n - 1):
+        mid = np.float32((grid[c] + grid[c + 1]) / 2)
+        even = c if c % 2 == 0 else c + 1
+        assert oracle.f32_to_fpx(np.array([mid], np.float32), ebits, mbits)[0] == even
+        assert oracle.f32_to_fpx(np.array([np.nextafter(mid, np.float32(0), dtype=np.float32)], np.float32), ebits, mbits)[0] == c
+        assert oracle.f32_to_fpx(np.array([np.nextafter(mid, np.float32(100), dtype=np.float32)], np.float32), ebits, mbits)[0] == c + 1
+    assert np.all(oracle.f32_to_fpx(np.array([grid[-1], grid[-1] * 1.2, 1e9, np.inf], np.float32), ebits, mbits) == n - 1)
+    # a 5-bit code and the 6-bit code with one more (zero) mantissa bit are the same number
+    if 1 + ebits + mbits == 5:
+        wide = oracle.fpx_to_f32((np.arange(2 * n, dtype=np.uint8) << 1).astype(np.uint8), ebits, mbits + 1)
+        assert np.array_equal(wide, vals)
+
+
+@pytest.mark.parametrize("shape", [(64, 64), (256, 64), (128, 192)])
+def test_pack_fp5_two_formulations_agree(oracle, shape):
+    """5-bit codes: the generic three-pass packer (1-bit plane, then 4-bit plane) against the order in which the
+    reference CUDA kernel reads those planes back (utils_parallel_dequant.cuh:85-113)."""
+    rng = np.random.default_rng(shape[0] + shape[1])
+    codes = rng.integers(0, 32, shape, dtype=np.uint8)
+    packed = oracle.pack_tc_fpx_generic(codes, 5)
+    assert packed.shape == (shape[0], shape[1] * 5 // 8)
+    assert np.array_equal(oracle.fpx_cuda_read_order(packed, shape[0], shape[1], 5), codes)
+    # the 4-bit plane is the same whatever the high plane is
+    p6 = oracle.pack_tc_fpx_generic(codes, 6).reshape(-1)
+    assert np.array_equal(packed.reshape(-1)[codes.size // 8:], p6[codes.size // 4:])
+
+
 def test_pack_single_element_positions(oracle):
     """One non-zero code at a time: its 2 high bits and 4 low bits land in exactly one byte each, in the
     right plane (first R*C/4 bytes = 2-bit plane)."""
