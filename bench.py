@@ -181,6 +181,22 @@ def cpu_baseline_leg(config, group=64, min_seconds=10.0):
         t_layer += time.perf_counter() - t0
         reps += 1
     per_layer = t_layer / reps
+    # the reference's CPU-runnable case step by step: one bf16 weight [4096, 4096], g = 128, x [1, 4096]
+    w = O.f32_to_bf16_bits((rng.standard_normal((4096, 4096), dtype=np.float32) * 0.02))
+    x = O.f32_to_bf16_bits(rng.standard_normal((1, 4096), dtype=np.float32))
+    c1 = {}
+    t0 = time.perf_counter()
+    codes, scale, zero = O.int4wo_quantize(w, O.BF16, 128, 4096, 4096)
+    c1["choose_qparams+quantize"] = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    O.int4wo_pack(codes, scale, zero, 128)
+    c1["pack"] = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    dq = O.dequantize_affine(codes, O.I32, (1, 128), scale, O.BF16, zero, O.BF16, 0, 15, 1, O.BF16)
+    c1["dequantize"] = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    O.linear(x, O.BF16, dq, O.BF16)
+    c1["linear"] = time.perf_counter() - t0
     head_params = config.vocab_size * dim
     per_token = per_layer * config.n_layer + per_layer * head_params / layer_params
     return {
@@ -191,6 +207,7 @@ def cpu_baseline_leg(config, group=64, min_seconds=10.0):
         "sample": (f"C oracle dequantize_affine+fp32 linear (M=1, g={group}) on one transformer layer's five linears "
                    f"({layer_params / 1e6:.0f}M weights), {reps} repetitions, {per_layer:.2f} s per layer; scaled to "
                    f"{config.n_layer} layers + vocabulary head"),
+        "config0_steps_ms": {k: round(v * 1e3, 1) for k, v in c1.items()},
     }
 
 
