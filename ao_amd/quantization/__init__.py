@@ -1,3 +1,4 @@
+from .GPTQ import Int4WeightOnlyQuantizer, WeightOnlyInt4Linear
 from .quant_api import (
     fp6_llm_weight_only,
     int4_weight_only,
@@ -13,6 +14,7 @@ from .quant_primitives import (
     dequantize_affine,
     quantize_affine,
 )
+from .unified import Quantizer, TwoStepQuantizer
 from .utils import (
     compute_error,
     get_groupwise_affine_qparams,

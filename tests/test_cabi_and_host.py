@@ -185,3 +185,38 @@ def test_llama_model_shapes_on_meta():
     n_lin = sum(p.numel() for name, p in m.named_parameters() if p.dim() == 2 and "tok_embeddings" not in name)
     assert n_lin == 7_504_658_432  # linear weights per decoded token
     assert m.layers[0].attention.wqkv.weight.shape == (6144, 4096)
+
+
+def test_module_swap_host_logic(oracle):
+    """Eligibility rule, module replacement on the meta device and the torch-side interleaving of the reference's
+    [K/g, N, 2] qparams into the kernels' words (checked against the oracle's packer, pads included)."""
+    import numpy as np
+    from ao_amd.quantization.GPTQ import (WeightOnlyInt4Linear, _check_linear_int4_k, interleave_scales_and_zeros,
+                                          replace_linear_int4)
+
+    assert _check_linear_int4_k(4096, 128, 8) and not _check_linear_int4_k(192, 64, 8) and _check_linear_int4_k(192, 64, 2)
+    assert not _check_linear_int4_k(4096 + 64, 128) and _check_linear_int4_k(4096 + 64, 64)
+
+    with torch.device("meta"):
+        m = torch.nn.Sequential(torch.nn.Linear(256, 64, bias=False), torch.nn.ReLU(),
+                                torch.nn.Sequential(torch.nn.Linear(192, 24, bias=False)))
+    replace_linear_int4(m, 64, 8, padding_allowed=False)
+    assert isinstance(m[0], WeightOnlyInt4Linear) and type(m[2][0]) is torch.nn.Linear
+    assert m[0].weight.shape == (4, 2, 64, 4) and m[0].scales_and_zeros.shape == (4, 64, 2)
+    replace_linear_int4(m, 64, 8, padding_allowed=True, skip_layer_func=lambda w: w.shape[0] == 24)
+    assert type(m[2][0]) is torch.nn.Linear
+    replace_linear_int4(m, 64, 8, padding_allowed=True)
+    assert isinstance(m[2][0], WeightOnlyInt4Linear) and m[2][0].in_features == 1024 and m[2][0].origin_in_features == 192
+
+    for (N, K, g) in [(20, 96, 32), (64, 256, 64), (33, 256, 256), (16, 384, 128)]:
+        gen = torch.Generator().manual_seed(N + K)
+        sz = torch.randn(K // g, N, 2, generator=gen).bfloat16()
+        words = interleave_scales_and_zeros(sz, g).numpy().view(np.uint32)
+        Np, Kp = oracle.int4wo_padded_shape(N, K, g)
+        bits = sz.view(torch.int16).numpy().view(np.uint16)
+        spad = np.full((Np, Kp // g), 0x3586, np.uint16)
+        zpad = np.zeros((Np, Kp // g), np.uint16)
+        spad[:N, :K // g] = bits[:, :, 0].T
+        zpad[:N, :K // g] = bits[:, :, 1].T
+        _, q_ref = oracle.int4wo_pack(np.full((Np, Kp), 8, np.int32), spad, zpad, g)
+        assert words.shape == q_ref.shape and np.array_equal(words, q_ref)
