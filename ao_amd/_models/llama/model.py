@@ -226,11 +226,30 @@ class Transformer(nn.Module):
             if not isinstance(lay, Gfx950WaveTiledAQTLayout) or lay.transposed or not w.is_cuda:
                 return False
             groups.add(lay.group_size)
-        return len(groups) == 1 and self.tok_embeddings.weight.dtype is torch.bfloat16
+        return len(groups) == 1 and self.tok_embeddings.weight.dtype is torch.bfloat16 \
+            and self.config.intermediate_size % 16 == 0
+
+    @staticmethod
+    def _gate_up_pair(ff):
+        """w1 and w3 of a feed-forward block as one packed weight with gate and up rows interleaved in eights, built
+        on first use and rebuilt when either weight is replaced.  One launch of twice the row blocks, half the work
+        each, spreads evenly over the CUs where two row-block streams per workgroup do not."""
+        from ... import ops
+
+        g, u = ff.w1.weight.layout_tensor, ff.w3.weight.layout_tensor
+        key = (g.packed_weight.data_ptr(), u.packed_weight.data_ptr(), g.scale_and_zero.data_ptr(),
+               u.scale_and_zero.data_ptr())
+        cached = getattr(ff, "_gate_up_pair_cache", None)
+        if cached is None or cached[0] != key:
+            pair, pair_q = ops.int4wo_interleave_pair(g.packed_weight, g.scale_and_zero, u.packed_weight,
+                                                      u.scale_and_zero, g.N, g.K, g.group_size)
+            cached = (key, pair, pair_q, g.group_size, g.N)
+            ff._gate_up_pair_cache = cached
+        return cached[1:]
 
     def _fused_decode(self, idx: Tensor, input_pos: Tensor) -> Tensor:
         """One token, batch 1: five launches per layer (norm + qkv, attention, wo + residual, norm + gate/up +
-        SwiGLU, down + residual).  Same roundings as the module-by-module path."""
+        SwiGLU over the interleaved pair, down + residual).  Same roundings as the module-by-module path."""
         from ... import ops
 
         cfg = self.config
@@ -251,9 +270,8 @@ class Transformer(nn.Module):
             y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
                                            cfg.n_head, cfg.n_local_heads)
             h = lin(y, att.wo, residual=x)
-            g, u = b.feed_forward.w1.weight.layout_tensor, b.feed_forward.w3.weight.layout_tensor
-            ff = ops.int4wo_rmsnorm_swiglu(h, b.ffn_norm.weight, b.ffn_norm.eps, g.packed_weight, g.scale_and_zero,
-                                           u.packed_weight, u.scale_and_zero, g.group_size, g.N)
+            pair, pair_q, group, n_ff = self._gate_up_pair(b.feed_forward)
+            ff = ops.int4wo_swiglu_interleaved(h, pair, pair_q, group, n_ff, b.ffn_norm.weight, b.ffn_norm.eps)
             x = lin(ff, b.feed_forward.w2, residual=h)
         xn = ops.rmsnorm(x, self.norm.weight, self.norm.eps)
         return lin(xn, self.output).view(1, 1, cfg.vocab_size)

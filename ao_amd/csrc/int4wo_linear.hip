@@ -190,6 +190,8 @@ struct LinearArgs {
     const uint16_t* residual; int64_t ldres;           // [M,N] or null
     void* y; int y_is_f32; int64_t ldy;
     const uint16_t* norm_w; float norm_eps;            // GEMV only: RMSNorm weight [K] applied to x while staging, or null
+    int pair8;                                         // GEMV only: rows 0-7 of every 16-row block are gate rows, rows 8-15
+                                                       // the matching up rows; y[m, 8*rb + r] = silu(gate) * up, N = output rows
 };
 
 __device__ __forceinline__ float silu_bf16(float a) {
@@ -660,7 +662,9 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     }
     __syncthreads();
     if (wave == 0) {
-        const int64_t n = rb * 16 + r;
+        const bool pair8 = !DUAL && a.pair8;
+        const int64_t n = pair8 ? rb * 8 + (r & 7) : rb * 16 + r;
+        const bool writer = n < a.N && !(pair8 && r >= 8);
         float bv = 0.f;
         if (a.bias && n < a.N) bv = bf16_bits_to_f32(a.bias[n]);
 #pragma unroll
@@ -671,9 +675,10 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
                 s += red[0][w][i][lane];
                 if (DUAL) s2 += red[NRED - 1][w][i][lane];
             }
+            if (pair8) s2 = __shfl_xor(s, 8, 64);  // the up row of gate lane r sits in lane r + 8
             const int64_t m = m0 + 4 * qd + i;
-            if (m < a.M && n < a.N) {
-                if (DUAL) {
+            if (m < a.M && writer) {
+                if (DUAL || pair8) {
                     s = hw_rne_bf16(silu_bf16(hw_rne_bf16(s)) * hw_rne_bf16(s2));
                 } else {
                     s += bv;
@@ -902,14 +907,19 @@ static void launch_group(int64_t g, int waves, dim3 grid, size_t smem, hipStream
 static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed, const void* qparams,
                            const void* packed2, const void* qparams2, int64_t N, int64_t g, const void* bias_bf16,
                            const void* residual_bf16, int64_t ldres, void* y, int y_dtype, int64_t ldy, void* stream,
-                           const void* norm_weight_bf16 = nullptr, float norm_eps = 0.f) {
+                           const void* norm_weight_bf16 = nullptr, float norm_eps = 0.f, bool pair8 = false) {
+    // pair8: `packed` / `qparams` hold 2 * N rows (gate and up rows interleaved in eights), the output has N columns
+    const int64_t n_out = N;
+    if (pair8) N *= 2;
     AO_REQUIRE(x_bf16 && packed && qparams && y, "null pointer argument");
     AO_REQUIRE(M >= 0, "negative batch");
     AO_REQUIRE(y_dtype == AO_BF16 || y_dtype == AO_F32, "output dtype must be bf16 or f32, got code %d", y_dtype);
     int64_t Np, Kp;
     if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
-    AO_REQUIRE(ldx >= K && ldy >= N, "row strides (ldx=%lld, ldy=%lld) smaller than the rows (K=%lld, N=%lld)",
-               (long long)ldx, (long long)ldy, (long long)K, (long long)N);
+    AO_REQUIRE(ldx >= K && ldy >= n_out, "row strides (ldx=%lld, ldy=%lld) smaller than the rows (K=%lld, N=%lld)",
+               (long long)ldx, (long long)ldy, (long long)K, (long long)n_out);
+    AO_REQUIRE(!pair8 || n_out % 8 == 0, "interleaved gate/up weights need out_features to be a multiple of 8, got %lld",
+               (long long)n_out);
     AO_REQUIRE(!residual_bf16 || ldres >= N, "residual row stride %lld smaller than N=%lld", (long long)ldres, (long long)N);
     AO_REQUIRE((((uintptr_t)packed) & 15) == 0 && (((uintptr_t)packed2) & 15) == 0, "packed buffer must be 16-byte aligned");
     AO_REQUIRE(Kp / 128 < (1 << 23), "in_features too large: K=%lld", (long long)K);
@@ -928,17 +938,28 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     const bool aligned = (K == Kp) && ((ldx & 7) == 0) && ((((uintptr_t)x_bf16) & 15) == 0);
     const int64_t rows = M < 16 ? M : 16;
     const size_t xbytes = (size_t)rows * (size_t)Kp * 2;
-    // LDS staging only while it leaves room for about 16 waves per CU (160 KB of LDS per CU)
-    int xmode = aligned ? (xbytes <= (size_t)waves * 10 * 1024 ? X_LDS : X_GLOBAL) : X_CHECKED;
+    // the fused RMSNorm and the interleaved gate/up epilogue exist on the LDS-staged path only: use workgroups
+    // large enough for the staged rows to pass the occupancy rule below
+    if (norm_weight_bf16 || pair8)
+        while (waves < 16 && xbytes > (size_t)waves * 10 * 1024 && waves * 2 <= KB) waves *= 2;
+    // LDS staging only while it leaves room for about 16 waves per CU (160 KB of LDS per CU) and, with the kernel's
+    // static arrays (cross-wave reduction: 1 KB per wave and weight, RMSNorm partials), fits one workgroup's limit
+    const size_t static_lds = (size_t)(dual ? 2 : 1) * waves * 1024 + 256;
+    const bool lds_ok = xbytes <= (size_t)waves * 10 * 1024 && xbytes + static_lds <= 160 * 1024;
+    int xmode = aligned ? (lds_ok ? X_LDS : X_GLOBAL) : X_CHECKED;
     LinearArgs a{(const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams,
-                 (const uint4*)packed2, (const uint32_t*)qparams2, N, Kp, (const uint16_t*)bias_bf16,
+                 (const uint4*)packed2, (const uint32_t*)qparams2, n_out, Kp, (const uint16_t*)bias_bf16,
                  (const uint16_t*)residual_bf16, ldres, y, y_dtype == AO_F32, ldy,
-                 (const uint16_t*)norm_weight_bf16, norm_eps};
+                 (const uint16_t*)norm_weight_bf16, norm_eps, pair8 ? 1 : 0};
     hipStream_t st = (hipStream_t)stream;
     // the fused RMSNorm lives in the activation staging of the GEMV kernel only
     AO_REQUIRE(!norm_weight_bf16 || (xmode == X_LDS && M <= 16 && (((uintptr_t)norm_weight_bf16) & 15) == 0),
                "fused rmsnorm needs M <= 16, K a multiple of max(128, group), 16-byte aligned rows and norm weight, and "
                "activations that fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);
+    // so does the interleaved gate/up epilogue
+    AO_REQUIRE(!pair8 || (xmode == X_LDS && M <= 16 && !dual),
+               "interleaved swiglu needs M <= 16, K a multiple of max(128, group), 16-byte aligned rows and activations "
+               "that fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);
     if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16) {
         // 128 x 128 workgroup tiles when they fill a good part of the 256 CUs, else 64 x 64 tiles: four times
         // the workgroups, each dequantizing for 64 activation rows only
@@ -1024,4 +1045,12 @@ extern "C" int ao_amd_int4wo_rmsnorm_swiglu(const void* x_bf16, int64_t M, int64
     AO_REQUIRE(norm_weight_bf16 && packed_up && qparams_up, "null pointer argument");
     return linear_dispatch(x_bf16, M, K, ldx, packed_gate, qparams_gate, packed_up, qparams_up, N, g, nullptr, nullptr, 0,
                            y_bf16, AO_BF16, ldy, stream, norm_weight_bf16, eps);
+}
+
+extern "C" int ao_amd_int4wo_swiglu_interleaved(const void* x_bf16, int64_t M, int64_t K, int64_t ldx,
+                                                const void* norm_weight_bf16, float eps, const void* packed_pair,
+                                                const void* qparams_pair, int64_t N, int64_t g, void* y_bf16, int64_t ldy,
+                                                void* stream) {
+    return linear_dispatch(x_bf16, M, K, ldx, packed_pair, qparams_pair, nullptr, nullptr, N, g, nullptr, nullptr, 0,
+                           y_bf16, AO_BF16, ldy, stream, norm_weight_bf16, eps, true);
 }

@@ -342,6 +342,30 @@ __global__ __launch_bounds__(256) void int4wo_pack_kernel(const int32_t* __restr
     }
 }
 
+// Gate / up interleaving for the fused SwiGLU GEMV: output row block b holds gate rows 8b..8b+7 in lanes r = 0..7 and
+// up rows 8b..8b+7 in lanes r = 8..15.  Every 16-byte lane chunk and every qparam word moves whole, so this is a
+// permutation of the two packed tensors (N a multiple of 16: no padded rows to place).
+__global__ __launch_bounds__(256) void int4wo_interleave_pair_kernel(const uint4* __restrict__ pg, const uint32_t* __restrict__ qg,
+                                                                      const uint4* __restrict__ pu, const uint32_t* __restrict__ qu,
+                                                                      int64_t RBo, int64_t KB, int64_t G, uint4* __restrict__ po,
+                                                                      uint32_t* __restrict__ qo) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < RBo * KB * 64) {
+        const int l = i & 63, r = l & 15, qd = l >> 4;
+        const int64_t kb = (i >> 6) % KB, rbo = (i >> 6) / KB;
+        const int64_t row = rbo * 8 + (r & 7);
+        const uint4* src = r < 8 ? pg : pu;
+        po[i] = src[((row >> 4) * KB + kb) * 64 + qd * 16 + (row & 15)];
+    }
+    if (i < RBo * G * 16) {
+        const int r = i & 15;
+        const int64_t gi = (i >> 4) % G, rbo = (i >> 4) / G;
+        const int64_t row = rbo * 8 + (r & 7);
+        const uint32_t* src = r < 8 ? qg : qu;
+        qo[i] = src[((row >> 4) * G + gi) * 16 + (row & 15)];
+    }
+}
+
 // mode 0: unpack to int32 codes + bf16 scale/zero (logical region); mode 1: dequantize to bf16 [N,K]
 template <int MODE>
 __global__ __launch_bounds__(256) void int4wo_unpack_kernel(const uint32_t* __restrict__ packed,
@@ -387,6 +411,48 @@ __global__ __launch_bounds__(256) void int4wo_unpack_kernel(const uint32_t* __re
                 zero[row * Gl + gi] = (uint16_t)(v >> 16);
             }
         }
+    }
+}
+
+// Dequantize whole tiles: one wave per (16-row block, 128-wide K tile).  Lane (row r, quarter qd) decodes its 32
+// codes, the wave transposes the 4 KB tile through LDS (16-byte chunks XOR-swizzled by the row so that neither the
+// writes nor the reads collide on banks) and every store instruction then writes four full 256-byte row
+// segments.  K must be a multiple of 8 and `out` 16-byte aligned.
+__global__ __launch_bounds__(256) void int4wo_dequantize_tiles_kernel(const uint4* __restrict__ packed,
+                                                                      const uint32_t* __restrict__ qparams, int64_t N,
+                                                                      int64_t K, int64_t RB, int64_t KB, int64_t Gt,
+                                                                      int64_t g, uint16_t* __restrict__ out) {
+    __shared__ uint4 tile_s[4][256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, qd = lane >> 4;
+    const int64_t t = (int64_t)blockIdx.x * 4 + wave;
+    const bool live = t < RB * KB;
+    const int64_t tc = live ? t : 0;
+    const int64_t rb = tc / KB, kb = tc % KB;
+    const uint4 w = packed[tc * 64 + lane];
+    const uint32_t qp = qparams[(rb * Gt + (kb * 128 + qd * 32) / g) * 16 + r];
+    const float s = __uint_as_float(qp << 16), z = __uint_as_float(qp & 0xffff0000u);
+    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+        uint32_t o[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            // dequantize_affine, FLOAT domain (quant_primitives.py:265-274): bf16(bf16((q - 8) * s) + z)
+            const float q0 = (float)(int)((ww[sl] >> (4 * nib_pos(2 * p))) & 15u) - 8.0f;
+            const float q1 = (float)(int)((ww[sl] >> (4 * nib_pos(2 * p + 1))) & 15u) - 8.0f;
+            o[p] = hw_bf16_pack(hw_rne_bf16(q0 * s) + z, hw_rne_bf16(q1 * s) + z);
+        }
+        const int chunk = qd * 4 + sl;
+        tile_s[wave][r * 16 + (chunk ^ r)] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = 4 * j + qd, c = r;  // this lane stores chunk c of tile row `row`
+        const uint4 v = tile_s[wave][row * 16 + (c ^ row)];
+        const int64_t n = rb * 16 + row, k = kb * 128 + c * 8;
+        if (live && n < N && k < K) *reinterpret_cast<uint4*>(out + n * K + k) = v;
     }
 }
 
@@ -522,6 +588,26 @@ extern "C" int ao_amd_int4wo_pack(const int32_t* codes, const void* scale_bf16, 
     return 0;
 }
 
+extern "C" int ao_amd_int4wo_interleave_pair(const void* packed_gate, const void* qparams_gate, const void* packed_up,
+                                             const void* qparams_up, int64_t N, int64_t K, int64_t g, void* packed_pair,
+                                             void* qparams_pair, void* stream) {
+    AO_REQUIRE(packed_gate && qparams_gate && packed_up && qparams_up && packed_pair && qparams_pair, "null pointer argument");
+    int64_t Np, Kp;
+    if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
+    AO_REQUIRE(N % 16 == 0, "gate/up interleaving needs out_features to be a multiple of 16, got %lld", (long long)N);
+    AO_REQUIRE(((((uintptr_t)packed_gate) | ((uintptr_t)packed_up) | ((uintptr_t)packed_pair)) & 15) == 0,
+               "packed buffers must be 16-byte aligned");
+    AO_REQUIRE(packed_pair != packed_gate && packed_pair != packed_up, "the interleaved output cannot alias an input");
+    const int64_t RBo = 2 * N / 16, KB = Kp / 128, G = Kp / g;
+    const int64_t n = RBo * KB * 64;  // >= number of qparam words
+    AO_REQUIRE((n + 255) / 256 <= 0x7fffffff, "weight too large for one launch");
+    hipLaunchKernelGGL(int4wo_interleave_pair_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4*)packed_gate, (const uint32_t*)qparams_gate, (const uint4*)packed_up,
+                       (const uint32_t*)qparams_up, RBo, KB, G, (uint4*)packed_pair, (uint32_t*)qparams_pair);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
 extern "C" int ao_amd_int4wo_unpack(const void* packed, const void* qparams, int64_t N, int64_t K, int64_t g,
                                     int32_t* codes, void* scale_bf16, void* zero_bf16, void* stream) {
     AO_REQUIRE(codes && scale_bf16 && zero_bf16 && packed && qparams, "null pointer argument");
@@ -541,6 +627,15 @@ extern "C" int ao_amd_int4wo_dequantize(const void* packed, const void* qparams,
     AO_REQUIRE(packed && qparams && out_bf16, "null pointer argument");
     int64_t Np, Kp;
     if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
+    if (K % 8 == 0 && (((uintptr_t)out_bf16) & 15) == 0 && (((uintptr_t)packed) & 15) == 0) {
+        const int64_t tiles = (Np / 16) * (Kp / 128);
+        AO_REQUIRE((tiles + 3) / 4 <= 0x7fffffff, "weight too large for one launch");
+        hipLaunchKernelGGL(int4wo_dequantize_tiles_kernel, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0,
+                           (hipStream_t)stream, (const uint4*)packed, (const uint32_t*)qparams, N, K, Np / 16, Kp / 128,
+                           Kp / g, g, (uint16_t*)out_bf16);
+        AO_LAUNCH_CHECK();
+        return 0;
+    }
     const int64_t n = Np * Kp / 8;
     hipLaunchKernelGGL(int4wo_unpack_kernel<1>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                        (const uint32_t*)packed, (const uint32_t*)qparams, N, K, Np, Kp, g, (int32_t*)nullptr,

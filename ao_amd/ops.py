@@ -45,6 +45,8 @@ _LIB.define("int4wo_linear_residual(Tensor x, Tensor packed, Tensor qparams, int
 _LIB.define("int4wo_swiglu(Tensor x, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
 _LIB.define("int4wo_rmsnorm_linear(Tensor x, Tensor norm_weight, float eps, Tensor packed, Tensor qparams, int group_size, int N, Tensor? bias) -> Tensor")
 _LIB.define("int4wo_rmsnorm_swiglu(Tensor x, Tensor norm_weight, float eps, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
+_LIB.define("int4wo_interleave_pair(Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int N, int K, int group_size) -> (Tensor, Tensor)")
+_LIB.define("int4wo_swiglu_interleaved(Tensor x, Tensor? norm_weight, float eps, Tensor packed_pair, Tensor qparams_pair, int group_size, int N) -> Tensor")
 _LIB.define("int8wo_linear(Tensor x, Tensor w_int8, Tensor scale, Tensor? bias, bool fp32_out) -> Tensor")
 _LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
 _LIB.define("argmax_bf16(Tensor x) -> Tensor")
@@ -55,6 +57,20 @@ _LIB.define("fp6_quantize_pack(Tensor w, int ebits, int mbits) -> (Tensor, Tenso
 _LIB.define("fp6_dequantize(Tensor fpx_data, Tensor? scale, int ebits, int mbits) -> Tensor")
 _LIB.define("fp6_repack(Tensor fpx_data, int nbits=6) -> Tensor")
 _LIB.define("fp6_linear_native(int ebits, int mbits, Tensor x, Tensor native, Tensor scale) -> Tensor")
+
+
+# Activation rows from which the int4 linear dequantizes the weight once and calls the library bf16 GEMM.
+# Measured crossovers on MI355X (Llama-3-8B shapes, g = 64): 512 rows for the 14336 x 4096 / 4096 x 14336 weights,
+# 1024 for 4096 x 4096 and for a vocabulary-sized weight, never worth it below about 2048 output features.
+TWO_PASS_MIN_M = 512
+
+
+def int4wo_two_pass(M: int, N: int, K: int) -> bool:
+    if N < 2048:
+        return M >= 8 * TWO_PASS_MIN_M
+    if N > 32768 or N * K < (1 << 25):
+        return M >= 2 * TWO_PASS_MIN_M
+    return M >= TWO_PASS_MIN_M
 
 
 def int4wo_packed_shapes(N: int, K: int, group_size: int):
@@ -144,6 +160,13 @@ def _linear_cuda(x: Tensor, packed: Tensor, qparams: Tensor, group_size: int, N:
     if bias is not None:
         torch._check(bias.dtype is torch.bfloat16 and bias.numel() == N, lambda: "bias must be bfloat16 of size N")
         bias = bias.contiguous()
+    if int4wo_two_pass(M, N, K) and not fp32_out:
+        # Large batches (prefill): dequantize once into a bf16 scratch weight with the HIP kernel, then one plain
+        # bf16 GEMM from the vendor library (hipBLASLt through torch).  A dense library GEMM runs at about twice
+        # the matrix-core utilisation of the fused kernel, whose VALU dequantization is repaid per 128 activation
+        # rows; the extra pass over the weight (N*K*2.5 bytes) costs less than that from about 512 rows on.
+        # This is the reference's own definition of the result: dequantize, then F.linear.
+        return torch.nn.functional.linear(x, _dequantize_cuda(packed, qparams, N, K, group_size), bias)
     y = torch.empty((M, N), dtype=torch.float32 if fp32_out else torch.bfloat16, device=x.device)
     check(lib().ao_amd_int4wo_linear(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, packed.data_ptr(),
                                      qparams.data_ptr(), N, group_size, None if bias is None else bias.data_ptr(),
@@ -246,6 +269,38 @@ def _rmsnorm_swiglu_cuda(x, norm_weight, eps, packed_gate, qparams_gate, packed_
                                              float(eps), packed_gate.data_ptr(), qparams_gate.data_ptr(),
                                              packed_up.data_ptr(), qparams_up.data_ptr(), N, group_size, y.data_ptr(), N,
                                              current_stream(x.device)))
+    return y
+
+
+def _interleave_pair_cuda(packed_gate, qparams_gate, packed_up, qparams_up, N, K, group_size):
+    """Two packed weights of one shape -> the packed weight of 2N rows whose 16-row blocks hold 8 gate rows and the 8
+    up rows of the same outputs (input of `int4wo_swiglu_interleaved`)."""
+    require_cuda(packed_gate, qparams_gate, packed_up, qparams_up)
+    _check_packed(packed_gate, qparams_gate, N, K, group_size)
+    _check_packed(packed_up, qparams_up, N, K, group_size)
+    pshape, qshape = int4wo_packed_shapes(2 * N, K, group_size)
+    packed = torch.empty(pshape, dtype=torch.int32, device=packed_gate.device)
+    qparams = torch.empty(qshape, dtype=torch.int32, device=packed_gate.device)
+    check(lib().ao_amd_int4wo_interleave_pair(packed_gate.data_ptr(), qparams_gate.data_ptr(), packed_up.data_ptr(),
+                                              qparams_up.data_ptr(), N, K, group_size, packed.data_ptr(),
+                                              qparams.data_ptr(), current_stream(packed_gate.device)))
+    return packed, qparams
+
+
+def _swiglu_interleaved_cuda(x, norm_weight, eps, packed_pair, qparams_pair, group_size, N):
+    require_cuda(x, norm_weight, packed_pair, qparams_pair)
+    torch._check(x.dim() == 2 and x.dtype is torch.bfloat16, lambda: "input must be a 2d bfloat16 tensor")
+    if norm_weight is not None:
+        _check_norm(x, norm_weight)
+    M, K = x.shape
+    _check_packed(packed_pair, qparams_pair, 2 * N, K, group_size)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    check(lib().ao_amd_int4wo_swiglu_interleaved(x.data_ptr(), M, K, x.stride(0) if M > 0 else K,
+                                                 None if norm_weight is None else norm_weight.data_ptr(), float(eps),
+                                                 packed_pair.data_ptr(), qparams_pair.data_ptr(), N, group_size,
+                                                 y.data_ptr(), N, current_stream(x.device)))
     return y
 
 
@@ -389,6 +444,8 @@ _LIB.impl("int4wo_linear_residual", _linear_residual_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu", _swiglu_cuda, "CUDA")
 _LIB.impl("int4wo_rmsnorm_linear", _rmsnorm_linear_cuda, "CUDA")
 _LIB.impl("int4wo_rmsnorm_swiglu", _rmsnorm_swiglu_cuda, "CUDA")
+_LIB.impl("int4wo_interleave_pair", _interleave_pair_cuda, "CUDA")
+_LIB.impl("int4wo_swiglu_interleaved", _swiglu_interleaved_cuda, "CUDA")
 _LIB.impl("int8wo_linear", _int8wo_linear_cuda, "CUDA")
 _LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
 _LIB.impl("llama_decode_attention", _decode_attention_cuda, "CUDA")
@@ -407,7 +464,8 @@ def _no_cpu(name):
 
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
-              "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int8wo_linear", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
+              "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int4wo_interleave_pair",
+              "int4wo_swiglu_interleaved", "int8wo_linear", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
               "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
@@ -465,6 +523,17 @@ def _(x, norm_weight, eps, packed, qparams, group_size, N, bias):
 
 @torch.library.register_fake("torchao::int4wo_rmsnorm_swiglu")
 def _(x, norm_weight, eps, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
+    return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::int4wo_interleave_pair")
+def _(packed_gate, qparams_gate, packed_up, qparams_up, N, K, group_size):
+    pshape, qshape = int4wo_packed_shapes(2 * N, K, group_size)
+    return packed_gate.new_empty(pshape), qparams_gate.new_empty(qshape)
+
+
+@torch.library.register_fake("torchao::int4wo_swiglu_interleaved")
+def _(x, norm_weight, eps, packed_pair, qparams_pair, group_size, N):
     return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
 
 
@@ -575,6 +644,19 @@ def int4wo_rmsnorm_swiglu(x, norm_weight, eps: float, packed_gate, qparams_gate,
     """swiglu(rmsnorm(x, norm_weight, eps)) in one launch, for M <= 16 rows (decode)."""
     return torch.ops.torchao.int4wo_rmsnorm_swiglu.default(x, norm_weight, eps, packed_gate, qparams_gate, packed_up,
                                                            qparams_up, group_size, N)
+
+
+def int4wo_interleave_pair(packed_gate, qparams_gate, packed_up, qparams_up, N: int, K: int, group_size: int):
+    """Gate and up weights [N,K] (packed) -> one packed weight of 2N rows, 8 gate rows then the 8 matching up rows
+    in every 16-row block."""
+    return torch.ops.torchao.int4wo_interleave_pair.default(packed_gate, qparams_gate, packed_up, qparams_up, N, K,
+                                                            group_size)
+
+
+def int4wo_swiglu_interleaved(x, packed_pair, qparams_pair, group_size, N, norm_weight=None, eps: float = 0.0):
+    """silu(x' W_gate^T) * (x' W_up^T) from the interleaved pair, x' = x or rmsnorm(x, norm_weight, eps); M <= 16 rows."""
+    return torch.ops.torchao.int4wo_swiglu_interleaved.default(x, norm_weight, eps, packed_pair, qparams_pair,
+                                                               group_size, N)
 
 
 def int8wo_linear(x: Tensor, w_int8: Tensor, scale: Tensor, bias=None, fp32_out: bool = False) -> Tensor:

@@ -8,7 +8,7 @@ A step is one decoded token (one pass of every quantized linear over one activat
 region is K replays of the HIP graph of the decode step with all weights resident in HBM, bracketed by
 torch.cuda.synchronize().  One JSON line is printed with:
   value        tokens/s
-  roofline     the int4wo GEMV kernel over the 161 linear launches of one token: algorithmic bytes
+  roofline     the int4wo GEMV kernel over the 129 linear launches of one decoded token: algorithmic bytes
                (N*K*(1/2 + 4/g) + 2*M*K + 2*M*N per launch) / kernel time, kernel time taken from HIP events
                that carry each kernel's own begin / end timestamps
   cpu_baseline the C oracle (dequantize_affine + fp32 linear, 1 thread) timed on one transformer layer's
@@ -67,50 +67,70 @@ class KernelTimer:
             self.hip.hipEventDestroy(b)
 
 
-def quantized_linears(model):
-    """(name, AffineQuantizedTensor) of every int4 linear in execution order of one forward pass."""
-    from ao_amd.dtypes import AffineQuantizedTensor
-
-    out = []
-    for layer_idx, layer in enumerate(model.layers):
-        for name, lin in (("wqkv", layer.attention.wqkv), ("wo", layer.attention.wo), ("w1", layer.feed_forward.w1),
-                          ("w3", layer.feed_forward.w3), ("w2", layer.feed_forward.w2)):
-            out.append((f"layers.{layer_idx}.{name}", lin.weight))
-    out.append(("output", model.output.weight))
-    assert all(isinstance(w, AffineQuantizedTensor) for _, w in out)
-    return out
-
-
 def roofline_leg(model, passes=3):
-    """Time the GEMV kernel alone over the linear launches of one token (M=1), `passes` times."""
+    """Time the GEMV kernel alone over the linear launches of one decoded token (M=1), `passes` times: per layer
+    norm + wqkv, wo + residual, norm + gate/up SwiGLU over the interleaved pair, w2 + residual, then the head:
+    the same entry points, weights and order as the decode step, 4 * n_layer + 1 launches."""
     import torch
 
     from ao_amd import _lib
 
     L = _lib.lib()
-    lins = quantized_linears(model)
     dev = torch.device("cuda:0")
-    timer = KernelTimer(len(lins))
     st = torch.cuda.current_stream().cuda_stream
-    xs = {}
-    total_bytes = 0.0
-    for _, w in lins:
-        lay = w.layout_tensor
-        if lay.K not in xs:
-            xs[lay.K] = torch.randn(1, lay.K, device=dev).bfloat16()
-        total_bytes += int4wo_bytes(lay.N, lay.K, lay.group_size)
-    ys = {n: torch.empty(1, n, dtype=torch.bfloat16, device=dev) for n in {w.layout_tensor.N for _, w in lins}}
+    cfg = model.config
+    x = torch.randn(1, cfg.dim, device=dev).bfloat16()
+    xf = torch.randn(1, cfg.intermediate_size, device=dev).bfloat16()
+    res = torch.randn(1, cfg.dim, device=dev).bfloat16()
+    launches = []  # (callable, algorithmic bytes)
+
+    def add(fn, nbytes):
+        launches.append((fn, nbytes))
+
+    def plain(lay, xin, residual=None, norm=None):
+        y = torch.empty(1, lay.N, dtype=torch.bfloat16, device=dev)
+        common = (lay.packed_weight.data_ptr(), lay.scale_and_zero.data_ptr(), lay.N, lay.group_size, None)
+        if norm is not None:
+            return lambda: L.ao_amd_int4wo_rmsnorm_linear(xin.data_ptr(), 1, lay.K, lay.K, norm.weight.data_ptr(),
+                                                          float(norm.eps), *common, y.data_ptr(), _lib.BF16, lay.N, st), y
+        if residual is not None:
+            return lambda: L.ao_amd_int4wo_linear_residual(xin.data_ptr(), 1, lay.K, lay.K, *common, residual.data_ptr(),
+                                                           lay.N, y.data_ptr(), lay.N, st), y
+        return lambda: L.ao_amd_int4wo_linear(xin.data_ptr(), 1, lay.K, lay.K, *common, y.data_ptr(), _lib.BF16,
+                                              lay.N, st), y
+
+    keep = []
+    for b in model.layers:
+        lay = b.attention.wqkv.weight.layout_tensor
+        fn, y = plain(lay, x, norm=b.attention_norm)
+        add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(y)
+        lay = b.attention.wo.weight.layout_tensor
+        fn, y = plain(lay, x, residual=res)
+        add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(y)
+        pair, pair_q, group, n_ff = model._gate_up_pair(b.feed_forward)
+        yff = torch.empty(1, n_ff, dtype=torch.bfloat16, device=dev)
+        norm = b.ffn_norm
+        add(lambda pair=pair, pair_q=pair_q, group=group, n_ff=n_ff, norm=norm, yff=yff:
+            L.ao_amd_int4wo_swiglu_interleaved(x.data_ptr(), 1, cfg.dim, cfg.dim, norm.weight.data_ptr(), float(norm.eps),
+                                               pair.data_ptr(), pair_q.data_ptr(), n_ff, group, yff.data_ptr(), n_ff, st),
+            int4wo_bytes(2 * n_ff, cfg.dim, group) - 2 * n_ff)
+        keep.append(yff)
+        lay = b.feed_forward.w2.weight.layout_tensor
+        fn, y = plain(lay, xf, residual=res)
+        add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(y)
+    lay = model.output.weight.layout_tensor
+    fn, y = plain(lay, x)
+    add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(y)
+
+    timer = KernelTimer(len(launches))
+    total_bytes = sum(nb for _, nb in launches)
     best = None
     for _ in range(passes):
-        for i, (_, w) in enumerate(lins):
-            lay = w.layout_tensor
-            x = xs[lay.K]
+        for i, (fn, _) in enumerate(launches):
             L.ao_amd_profile_next_linear(timer.pairs[i][0], timer.pairs[i][1])
-            _lib.check(L.ao_amd_int4wo_linear(x.data_ptr(), 1, lay.K, lay.K, lay.packed_weight.data_ptr(),
-                                              lay.scale_and_zero.data_ptr(), lay.N, lay.group_size, None,
-                                              ys[lay.N].data_ptr(), _lib.BF16, lay.N, st))
+            _lib.check(fn())
         torch.cuda.synchronize()
-        durs = [timer.elapsed_us(i) for i in range(len(lins))]
+        durs = [timer.elapsed_us(i) for i in range(len(launches))]
         if best is None or sum(durs) < sum(best):
             best = durs
     timer.close()
@@ -123,9 +143,12 @@ def roofline_leg(model, passes=3):
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "launches": len(lins),
-        "bytes_per_launch": round(total_bytes / len(lins)),
-        "avg_launch_us": round(total_us / len(lins), 3),
+        "launches": len(launches),
+        "bytes_per_launch": round(total_bytes / len(launches)),
+        "avg_launch_us": round(total_us / len(launches), 3),
+        "us_by_linear": {k: round(sum(best[i] for i in range(j, len(launches) - 1, 4)) / len(model.layers), 2)
+                         for j, k in enumerate(("norm_wqkv", "wo_residual", "norm_w1w3_swiglu", "w2_residual"))}
+        | {"output": round(best[-1], 2)},
         "traffic": _traffic_from_profile(),
     }
 
@@ -217,14 +240,24 @@ SWEEP_ROTATE_BYTES = 640 << 20  # the sweeps rotate over weight copies totalling
 LLAMA3_8B_SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)]  # (N, K)
 
 
-def _time_linear(L, launch, iters):
-    """Median of the kernel's own duration (us) over `iters` armed launches; launch(i) is given the iteration
-    number so that it can rotate over copies of the weight (each launch then reads HBM, not the last-level cache)."""
+def _time_linear(L, launch, iters, armed=True):
+    """Median of the kernel's own duration (us) over `iters` launches; launch(i) is given the iteration number so
+    that it can rotate over copies of the weight (each launch then reads HBM, not the last-level cache).  Linear
+    kernels are timed by events armed on the launch itself; entry points without that hook (`armed=False`) by
+    stream events recorded around the launch."""
     import torch
 
-    timer = KernelTimer(iters)
     for i in range(3):
         launch(i)
+    if not armed:
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        for i in range(iters):
+            evs[i][0].record()
+            launch(i + 3)
+            evs[i][1].record()
+        torch.cuda.synchronize()
+        return sorted(a.elapsed_time(b) * 1e3 for a, b in evs)[iters // 2]
+    timer = KernelTimer(iters)
     for i in range(iters):
         L.ao_amd_profile_next_linear(timer.pairs[i][0], timer.pairs[i][1])
         launch(i + 3)
@@ -268,6 +301,36 @@ def sweep(kind, iters=15):
             print(json.dumps({"kernel": "int4wo_linear", "N": N, "K": K, "M": M, "group": g, "us": round(us, 2),
                               "GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
                               "TFLOPs": round(tfs, 2), "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
+            if kind == "gemm":
+                from ao_amd import ops
+
+                if ops.int4wo_two_pass(M, N, K):
+                    # what torch.ops.torchao.int4wo_linear runs at this size: the dequantize kernel into a bf16
+                    # scratch weight, then the library bf16 GEMM; timed with stream events around the op
+                    shp_p, shp_q = ops.int4wo_packed_shapes(N, K, g)
+                    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+                    for i in range(iters + 3):
+                        pi, qi = packed[i % copies].view(shp_p), qp[i % copies].view(shp_q)
+                        if i >= 3:
+                            evs[i - 3][0].record()
+                        ops.int4wo_linear(x, pi, qi, g, N)
+                        if i >= 3:
+                            evs[i - 3][1].record()
+                    torch.cuda.synchronize()
+                    us2 = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)[iters // 2]
+                    tfs2 = 2.0 * M * N * K / us2 / 1e6
+                    print(json.dumps({"kernel": "int4wo_linear op: int4wo_dequantize + library bf16 GEMM", "N": N, "K": K,
+                                      "M": M, "group": g, "us": round(us2, 2), "TFLOPs": round(tfs2, 2),
+                                      "mfma_frac": round(tfs2 / MFMA_PEAK_TFLOPS, 4)}), flush=True)
+                if M == 2048 or (M == 512 and N * 2048 >= 1 << 28):
+                    wd = torch.empty(N, K, dtype=torch.bfloat16, device=dev)
+                    usd = _time_linear(L, lambda i: _lib.check(L.ao_amd_int4wo_dequantize(
+                        packed[i % copies].data_ptr(), qp[i % copies].data_ptr(), N, K, g, wd.data_ptr(), st)), iters,
+                        armed=False)
+                    gbd = (N * K * (0.5 + 4.0 / g) + 2.0 * N * K) / usd / 1e3
+                    print(json.dumps({"kernel": "int4wo_dequantize", "N": N, "K": K, "group": g, "us": round(usd, 2),
+                                      "GBs": round(gbd, 1), "hbm_frac": round(gbd / HBM_PEAK_GBS, 4)}), flush=True)
+                    del wd
             del w, packed, qp, x, y
     elif kind == "fp6":
         for N, K in [(4096, 4096), (14336, 4096), (4096, 14336)]:

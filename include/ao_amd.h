@@ -135,6 +135,20 @@ int ao_amd_int4wo_rmsnorm_swiglu(const void* x_bf16, int64_t M, int64_t K, int64
                                  float eps, const void* packed_gate, const void* qparams_gate, const void* packed_up,
                                  const void* qparams_up, int64_t N, int64_t g, void* y_bf16, int64_t ldy, void* stream);
 
+/* SwiGLU over ONE interleaved weight: `ao_amd_int4wo_interleave_pair` permutes two packed weights of the same shape
+ * (N a multiple of 16) into a packed weight of 2N rows whose 16-row blocks hold 8 gate rows followed by the 8 up rows of
+ * the same outputs (buffers sized by ao_amd_int4wo_packed_shape(2N, K, g)); `ao_amd_int4wo_swiglu_interleaved` computes
+ * y[M,N] = bf16( silu(bf16(x' Wg^T)) * bf16(x' Wu^T) ) from it, x' = x or, with `norm_weight_bf16` non-null, the RMSNorm
+ * of x as in ao_amd_int4wo_rmsnorm_swiglu.  Same arithmetic and roundings as ao_amd_int4wo_swiglu (FeedForward.forward,
+ * torchao/_models/llama/model.py:209-214); the point of the layout is the launch shape: 2N/16 workgroups of half the
+ * work each (7 per CU instead of 3.5 for Llama-3-8B's 14336 x 4096 pair on 256 CUs).  Decode shapes only, as above. */
+int ao_amd_int4wo_interleave_pair(const void* packed_gate, const void* qparams_gate, const void* packed_up,
+                                  const void* qparams_up, int64_t N, int64_t K, int64_t g, void* packed_pair,
+                                  void* qparams_pair, void* stream);
+int ao_amd_int4wo_swiglu_interleaved(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* norm_weight_bf16,
+                                     float eps, const void* packed_pair, const void* qparams_pair, int64_t N, int64_t g,
+                                     void* y_bf16, int64_t ldy, void* stream);
+
 /* ---------------------------------------------------------------- int8 weight-only linear
  * y[M,N] = bf16( bf16(x[M,K] @ bf16(w)^T) * scale[N] ) (+ bias, rounded to bf16 again): the per-channel int8
  * weight-only branch of _quantized_linear_op, torchao/dtypes/affine_quantized_tensor.py:641-665

@@ -116,6 +116,91 @@ def test_rmsnorm_swiglu_fused(M):
     assert np.count_nonzero(out != ref) <= 0.05 * out.size
 
 
+@pytest.mark.parametrize("N,K,g", [(512, 1024, 64), (48, 256, 32), (1024, 4096, 128), (32, 512, 256)])
+def test_interleave_pair_is_the_row_permutation(N, K, g):
+    """Unpacking the interleaved weight gives, in every 16-row block, 8 gate rows then the 8 up rows of the same
+    outputs: codes, scales and zeros bit for bit."""
+    from ao_amd import ops
+
+    dev = _dev()
+    wg = make_weight(N, K, seed=71 + N).to(dev)
+    wu = make_weight(N, K, seed=72 + N).to(dev)
+    pg, qg = ops.int4wo_quantize_pack(wg, g)
+    pu, qu = ops.int4wo_quantize_pack(wu, g)
+    pp, qq = ops.int4wo_interleave_pair(pg, qg, pu, qu, N, K, g)
+    got = [t.cpu() for t in ops.int4wo_unpack(pp, qq, 2 * N, K, g)]
+    gate = [t.cpu() for t in ops.int4wo_unpack(pg, qg, N, K, g)]
+    up = [t.cpu() for t in ops.int4wo_unpack(pu, qu, N, K, g)]
+    for t, a, b in zip(got, gate, up):
+        expect = torch.stack([a.reshape(N // 8, 8, -1), b.reshape(N // 8, 8, -1)], dim=1).reshape(2 * N, -1)
+        assert torch.equal(t.view(torch.int16) if t.dtype is torch.bfloat16 else t,
+                           expect.view(torch.int16) if expect.dtype is torch.bfloat16 else expect)
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("N,K,g", [(1024, 4096, 64), (48, 256, 32), (14336, 4096, 64)])
+def test_swiglu_interleaved_matches_two_weight_kernel(M, N, K, g):
+    """Same products, same roundings as the two-weight SwiGLU kernel; the K tiles may be split over a different
+    number of waves, which reorders the fp32 sums (1e-3 relative L2, nearly all elements identical).  With the
+    RMSNorm fused as well."""
+    from ao_amd import ops
+
+    print(f"case swiglu interleaved M={M} N={N} K={K} g={g}", flush=True)
+    dev = _dev()
+    wg = make_weight(N, K, seed=81).to(dev)
+    wu = make_weight(N, K, seed=82).to(dev)
+    x = (make_act(M, K, seed=83) * 0.5).to(dev)
+    nw = (1 + 0.1 * torch.randn(K, generator=torch.Generator().manual_seed(84))).bfloat16().to(dev)
+    pg, qg = ops.int4wo_quantize_pack(wg, g)
+    pu, qu = ops.int4wo_quantize_pack(wu, g)
+    pp, qq = ops.int4wo_interleave_pair(pg, qg, pu, qu, N, K, g)
+    ref = ops.int4wo_swiglu(x, pg, qg, pu, qu, g, N).float().cpu().numpy()
+    out = ops.int4wo_swiglu_interleaved(x, pp, qq, g, N).float().cpu().numpy()
+    assert rel_l2(out, ref) <= 1e-3
+    assert np.count_nonzero(out != ref) <= 0.02 * out.size
+    # norm fused into the staging against the two-launch chain (statistics summed in another order: an ulp of the
+    # normalised activation on rare elements)
+    ref_n = ops.int4wo_swiglu(ops.rmsnorm(x, nw, 1e-5), pg, qg, pu, qu, g, N).float().cpu().numpy()
+    out_n = ops.int4wo_swiglu_interleaved(x, pp, qq, g, N, nw, 1e-5).float().cpu().numpy()
+    assert rel_l2(out_n, ref_n) <= 1e-3
+    assert np.count_nonzero(out_n != ref_n) <= 0.05 * out_n.size
+
+
+def test_two_weight_swiglu_at_16_rows_of_4096():
+    """16 activation rows of 4096 fill 128 KB of LDS; with two weights the cross-wave reduction arrays no longer fit
+    beside them, so the launch must take the path that reads activations from global memory (and the fused-norm
+    variant, which only exists on the LDS path, must say so)."""
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K, g, M = 256, 4096, 64, 16
+    pg, qg = ops.int4wo_quantize_pack(make_weight(N, K, seed=95).to(dev), g)
+    pu, qu = ops.int4wo_quantize_pack(make_weight(N, K, seed=96).to(dev), g)
+    x = (make_act(M, K, seed=97) * 0.5).to(dev)
+    a = ops.int4wo_linear(x, pg, qg, g, N, None, False)
+    b = ops.int4wo_linear(x, pu, qu, g, N, None, False)
+    expect = (torch.nn.functional.silu(a) * b).float().cpu().numpy()
+    y = ops.int4wo_swiglu(x, pg, qg, pu, qu, g, N).float().cpu().numpy()
+    assert rel_l2(y, expect) <= 1e-3
+    nw = torch.ones(K, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="fused rmsnorm"):
+        ops.int4wo_rmsnorm_swiglu(x, nw, 1e-5, pg, qg, pu, qu, g, N)
+
+
+def test_swiglu_interleaved_rejects_what_it_cannot_take():
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K, g = 64, 512, 64
+    pg, qg = ops.int4wo_quantize_pack(make_weight(N, K, seed=91).to(dev), g)
+    pp, qq = ops.int4wo_interleave_pair(pg, qg, pg, qg, N, K, g)
+    with pytest.raises(RuntimeError, match="interleaved swiglu"):
+        ops.int4wo_swiglu_interleaved(make_act(17, K, seed=92).to(dev), pp, qq, g, N)
+    p24, q24 = ops.int4wo_quantize_pack(make_weight(24, K, seed=93).to(dev), g)
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        ops.int4wo_interleave_pair(p24, q24, p24, q24, 24, K, g)
+
+
 def test_rmsnorm_linear_rejects_prefill_shapes():
     from ao_amd import ops
 

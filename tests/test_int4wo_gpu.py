@@ -219,6 +219,48 @@ def test_linear_gemm_path(cabi, oracle, case, g):
     assert rel_l2(y16.float().cpu().numpy(), y_ref16) <= REL_L2_TOL
 
 
+@pytest.mark.parametrize("case", [(272, 1024, 512, 64, True), (1040, 2048, 700, 128, False), (48, 192, 600, 32, True)])
+def test_linear_op_prefill_two_pass(oracle, case, monkeypatch):
+    """From 512 activation rows on (large weights) the op dequantizes the weight once (tiled HIP kernel, bit-exact
+    against the oracle's dequantize_affine) and calls the library bf16 GEMM: same tolerance against the oracle as
+    the fused kernel, and close to the fused kernel's own result."""
+    from ao_amd import ops
+
+    N, K, M, g, with_bias = case
+    print(f"case two-pass N={N} K={K} M={M} g={g}", flush=True)
+    dev = _dev()
+    w = make_weight(N, K, seed=88 + N + g)
+    x = make_act(M, K, seed=M + K + 2)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(3)) * 0.1).bfloat16() if with_bias else None
+    bias_d = None if bias is None else bias.to(dev)
+    packed, qp = ops.int4wo_quantize_pack(w.to(dev), g)
+    dq = ops.int4wo_dequantize(packed, qp, N, K, g)
+    Np, Kp = oracle.int4wo_padded_shape(N, K, g)
+    codes, scale, zero = oracle.int4wo_quantize(bits16(w), oracle.BF16, g, Np, Kp)
+    dq_ref = oracle.dequantize_affine(codes, oracle.I32, (1, g), scale, oracle.BF16, zero, oracle.BF16, 0, 15, 1, oracle.BF16)
+    assert np.array_equal(bits16(dq), dq_ref[:N, :K])
+    monkeypatch.setattr(ops, "TWO_PASS_MIN_M", 1)  # these small weights would otherwise stay on the fused kernel
+    assert ops.int4wo_two_pass(M, N, K)
+    y = ops.int4wo_linear(x.to(dev), packed, qp, g, N, bias_d)
+    monkeypatch.setattr(ops, "TWO_PASS_MIN_M", 1 << 30)
+    assert not ops.int4wo_two_pass(M, N, K)
+    y_fused = ops.int4wo_linear(x.to(dev), packed, qp, g, N, bias_d)
+    assert y.dtype is torch.bfloat16 and y.shape == (M, N)
+    _, y_ref = _oracle_linear(oracle, w, x, g, bias)
+    y_ref16 = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(y_ref))
+    assert rel_l2(y.float().cpu().numpy(), y_ref16) <= REL_L2_TOL
+    assert rel_l2(y.float().cpu().numpy(), y_fused.float().cpu().numpy()) <= REL_L2_TOL
+
+
+def test_two_pass_rule():
+    from ao_amd import ops
+
+    assert ops.int4wo_two_pass(512, 14336, 4096) and ops.int4wo_two_pass(512, 4096, 14336)
+    assert not ops.int4wo_two_pass(512, 4096, 4096) and ops.int4wo_two_pass(1024, 4096, 4096)
+    assert not ops.int4wo_two_pass(512, 128256, 4096) and ops.int4wo_two_pass(1024, 128256, 4096)
+    assert not ops.int4wo_two_pass(2048, 1024, 4096) and not ops.int4wo_two_pass(511, 14336, 4096)
+
+
 def test_linear_rejects_bad_arguments(cabi):
     dev = _dev()
     x = torch.zeros(1, 128, dtype=torch.bfloat16, device=dev)
