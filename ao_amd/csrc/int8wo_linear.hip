@@ -118,6 +118,26 @@ __global__ __launch_bounds__(WAVES * 64) void int8wo_linear_kernel(const Int8Arg
     }
 }
 
+// int8 [N,K] (row stride ldw) -> bf16 [N,K]: the `w_int8.to(x.dtype)` of the reference's formula as its own pass, for
+// batches large enough that a plain bf16 GEMM on the converted weight beats re-streaming the int8 weight per 16 rows.
+// 16 codes in, 32 bytes out per thread; every int8 value is exact in bf16.
+__global__ __launch_bounds__(256) void int8_to_bf16_kernel(const int8_t* __restrict__ w, int64_t N, int64_t K, int64_t ldw,
+                                                           uint16_t* __restrict__ out) {
+    const int64_t per_row = K / 16;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N * per_row) return;
+    const int64_t n = i / per_row, c = i % per_row;
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(w + n * ldw + c * 16);
+    uint32_t o[8];
+    int8x4_to_bf16(v.x, o[0], o[1]);
+    int8x4_to_bf16(v.y, o[2], o[3]);
+    int8x4_to_bf16(v.z, o[4], o[5]);
+    int8x4_to_bf16(v.w, o[6], o[7]);
+    u32x4_t* dst = reinterpret_cast<u32x4_t*>(out + n * K + c * 16);
+    dst[0] = u32x4_t{o[0], o[1], o[2], o[3]};
+    dst[1] = u32x4_t{o[4], o[5], o[6], o[7]};
+}
+
 template <int WAVES>
 static void launch_int8(dim3 grid, hipStream_t st, const Int8Args& a) {
     hipEvent_t ev0 = g_prof_start, ev1 = g_prof_stop;  // optional per-kernel timing, see common.h
@@ -156,6 +176,20 @@ extern "C" int ao_amd_int8wo_linear(const void* x_bf16, int64_t M, int64_t K, in
         case 8: launch_int8<8>(grid, st, a); break;
         default: launch_int8<16>(grid, st, a); break;
     }
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_int8_to_bf16(const void* w_int8, int64_t N, int64_t K, int64_t ldw, void* out_bf16, void* stream) {
+    AO_REQUIRE(w_int8 && out_bf16, "null pointer argument");
+    AO_REQUIRE(N > 0 && K > 0 && K % 16 == 0, "int8 -> bf16 conversion needs K to be a positive multiple of 16, got N=%lld K=%lld",
+               (long long)N, (long long)K);
+    AO_REQUIRE(ldw >= K && (ldw & 15) == 0 && (((uintptr_t)w_int8) & 15) == 0 && (((uintptr_t)out_bf16) & 15) == 0,
+               "rows must be 16-byte aligned (ldw=%lld)", (long long)ldw);
+    const int64_t n = N * (K / 16);
+    AO_REQUIRE((n + 255) / 256 <= 0x7fffffff, "weight too large for one launch");
+    hipLaunchKernelGGL(int8_to_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const int8_t*)w_int8, N, K, ldw, (uint16_t*)out_bf16);
     AO_LAUNCH_CHECK();
     return 0;
 }

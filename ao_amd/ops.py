@@ -65,6 +65,9 @@ _LIB.define("fp6_linear_native(int ebits, int mbits, Tensor x, Tensor native, Te
 TWO_PASS_MIN_M = 512
 
 
+INT8_TWO_PASS_MIN_M = 128
+
+
 def int4wo_two_pass(M: int, N: int, K: int) -> bool:
     if N < 2048:
         return M >= 8 * TWO_PASS_MIN_M
@@ -224,6 +227,14 @@ def _int8wo_linear_cuda(x, w_int8, scale, bias, fp32_out):
     if bias is not None:
         torch._check(bias.dtype is torch.bfloat16 and bias.numel() == N, lambda: "bias must be bfloat16 of size N")
         bias = bias.contiguous()
+    if M >= INT8_TWO_PASS_MIN_M and not fp32_out and K % 16 == 0:
+        # prefill-sized batch: bf16 copy of the codes (HIP kernel), library bf16 GEMM, scale, bias: the reference's
+        # `torch.mm(x, w_int8.t().to(x.dtype)) * scale` (+ bias) op by op.  The streaming kernel below re-reads the
+        # weight for every 16 activation rows and falls behind from about 128 rows on.
+        wb = torch.empty((N, K), dtype=torch.bfloat16, device=x.device)
+        check(lib().ao_amd_int8_to_bf16(w_int8.data_ptr(), N, K, w_int8.stride(0), wb.data_ptr(), current_stream(x.device)))
+        y = torch.nn.functional.linear(x, wb) * scale
+        return y if bias is None else y + bias
     y = torch.empty((M, N), dtype=torch.float32 if fp32_out else torch.bfloat16, device=x.device)
     check(lib().ao_amd_int8wo_linear(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, w_int8.data_ptr(),
                                      w_int8.stride(0), scale.data_ptr(), N, None if bias is None else bias.data_ptr(),

@@ -161,6 +161,10 @@ int ao_amd_int8wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, 
                          const void* scale_bf16, int64_t N, const void* bias_bf16, void* y, int y_dtype, int64_t ldy,
                          void* stream);
 
+/* bf16 copy of the int8 codes (`w_int8.to(x.dtype)` of the same formula) for prefill-sized batches: the caller then
+ * runs a plain bf16 GEMM on it and multiplies by the scale.  K a multiple of 16, 16-byte aligned rows. */
+int ao_amd_int8_to_bf16(const void* w_int8, int64_t N, int64_t K, int64_t ldw, void* out_bf16, void* stream);
+
 /* ---------------------------------------------------------------- Llama decode harness kernels (bf16)
  * out[rows,dim] = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * weight ): RMSNorm.forward,
  * torchao/_models/llama/model.py:232-244. */
