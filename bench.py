@@ -342,7 +342,7 @@ def sweep(kind, iters=15):
             _lib.check(L.ao_amd_fp6_native_bytes(N, K, ctypes.byref(nbytes)))
             copies = max(2, -(-SWEEP_ROTATE_BYTES // nbytes.value))
             native = torch.empty(copies, nbytes.value, dtype=torch.uint8, device=dev)
-            _lib.check(L.ao_amd_fp6_repack(tc.data_ptr(), N, K, native.data_ptr(), st))
+            _lib.check(L.ao_amd_fp6_repack(tc.data_ptr(), N, K, 6, native.data_ptr(), st))
             native[1:] = native[0]
             for M in (1, 16, 128, 512):
                 x = torch.randn(M, K, device=dev, generator=gen).half()
