@@ -247,27 +247,27 @@ def _time_linear(L, launch, iters, armed=True):
     stream events recorded around the launch."""
     import torch
 
-    for i in range(3):
+    for i in range(10):
         launch(i)
     if not armed:
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
         for i in range(iters):
             evs[i][0].record()
-            launch(i + 3)
+            launch(i + 10)
             evs[i][1].record()
         torch.cuda.synchronize()
         return sorted(a.elapsed_time(b) * 1e3 for a, b in evs)[iters // 2]
     timer = KernelTimer(iters)
     for i in range(iters):
         L.ao_amd_profile_next_linear(timer.pairs[i][0], timer.pairs[i][1])
-        launch(i + 3)
+        launch(i + 10)
     torch.cuda.synchronize()
     durs = sorted(timer.elapsed_us(i) for i in range(iters))
     timer.close()
     return durs[len(durs) // 2]
 
 
-def sweep(kind, iters=15):
+def sweep(kind, iters=100):
     """Per-kernel lines for the shapes of the other benchmark configurations: int4 GEMV (M in 1, 4; g in 64, 128),
     int4 GEMM (M in 16 .. 2048, g=64), the FP6 e3m2 linear (M in 1, 16, 128, 512) and the int8 weight-only linear
     (M in 1, 4, 16); one JSON line per case."""
@@ -298,9 +298,16 @@ def sweep(kind, iters=15):
                 y.data_ptr(), _lib.BF16, N, st)), iters)
             gbs = int4wo_bytes(N, K, g, M) / us / 1e3
             tfs = 2.0 * M * N * K / us / 1e6
-            print(json.dumps({"kernel": "int4wo_linear", "N": N, "K": K, "M": M, "group": g, "us": round(us, 2),
-                              "GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
-                              "TFLOPs": round(tfs, 2), "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
+            line = {"kernel": "int4wo_linear", "N": N, "K": K, "M": M, "group": g, "us": round(us, 2),
+                    "GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+                    "TFLOPs": round(tfs, 2), "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}
+            if kind == "gemv":
+                # for information: the same launch on one copy of the weight (served from the 256 MB last-level
+                # cache when it fits); every other figure is the cold one above
+                line["us_warm"] = round(_time_linear(L, lambda i: _lib.check(L.ao_amd_int4wo_linear(
+                    x.data_ptr(), M, K, K, packed[0].data_ptr(), qp[0].data_ptr(), N, g, None, y.data_ptr(), _lib.BF16,
+                    N, st)), iters), 2)
+            print(json.dumps(line), flush=True)
             if kind == "gemm":
                 from ao_amd import ops
 
@@ -309,13 +316,13 @@ def sweep(kind, iters=15):
                     # scratch weight, then the library bf16 GEMM; timed with stream events around the op
                     shp_p, shp_q = ops.int4wo_packed_shapes(N, K, g)
                     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
-                    for i in range(iters + 3):
+                    for i in range(iters + 10):
                         pi, qi = packed[i % copies].view(shp_p), qp[i % copies].view(shp_q)
-                        if i >= 3:
-                            evs[i - 3][0].record()
+                        if i >= 10:
+                            evs[i - 10][0].record()
                         ops.int4wo_linear(x, pi, qi, g, N)
-                        if i >= 3:
-                            evs[i - 3][1].record()
+                        if i >= 10:
+                            evs[i - 10][1].record()
                     torch.cuda.synchronize()
                     us2 = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)[iters // 2]
                     tfs2 = 2.0 * M * N * K / us2 / 1e6
