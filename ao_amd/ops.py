@@ -11,7 +11,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from ._lib import BF16, DTYPE_CODE, F32, check, current_stream, lib, require_cuda
+from ._lib import BF16, DTYPE_CODE, F16, F32, check, current_stream, lib, require_cuda
 
 __all__ = [
     "quant_llm_linear",
@@ -48,6 +48,7 @@ _LIB.define("int4wo_rmsnorm_swiglu(Tensor x, Tensor norm_weight, float eps, Tens
 _LIB.define("int4wo_interleave_pair(Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int N, int K, int group_size) -> (Tensor, Tensor)")
 _LIB.define("int4wo_swiglu_interleaved(Tensor x, Tensor? norm_weight, float eps, Tensor packed_pair, Tensor qparams_pair, int group_size, int N) -> Tensor")
 _LIB.define("int8wo_linear(Tensor x, Tensor w_int8, Tensor scale, Tensor? bias, bool fp32_out) -> Tensor")
+_LIB.define("hqq_dequantize(Tensor packed_2xint4, Tensor scales, Tensor zeros, int group_size) -> Tensor")
 _LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
 _LIB.define("argmax_bf16(Tensor x) -> Tensor")
 _LIB.define("llama_decode_attention(Tensor qkv, Tensor freqs_cis, Tensor input_pos, Tensor(a!) k_cache, Tensor(b!) v_cache, int n_head, int n_kv) -> Tensor")
@@ -315,6 +316,26 @@ def _swiglu_interleaved_cuda(x, norm_weight, eps, packed_pair, qparams_pair, gro
     return y
 
 
+def _hqq_dequantize_cuda(packed_2xint4, scales, zeros, group_size):
+    """uint8 / int8 [K/2, N] two-per-byte codes + scales / zeros [K/group, N] (fp16 or bf16) -> [K, N] in that dtype."""
+    require_cuda(packed_2xint4, scales, zeros)
+    torch._check(packed_2xint4.dim() == 2 and packed_2xint4.dtype in (torch.uint8, torch.int8),
+                 lambda: "b must be a 2d int8 or uint8 tensor")
+    torch._check(scales.dtype in (torch.float16, torch.bfloat16) and zeros.dtype is scales.dtype,
+                 lambda: f"scales and zeros must both be float16 or bfloat16, got {scales.dtype} and {zeros.dtype}")
+    K2, N = packed_2xint4.shape
+    K = 2 * K2
+    torch._check(scales.dim() == 2 and scales.shape == zeros.shape and scales.shape == (K // group_size, N),
+                 lambda: f"scales / zeros must have shape ({K // group_size}, {N}), got {tuple(scales.shape)} and {tuple(zeros.shape)}")
+    packed_2xint4, scales, zeros = packed_2xint4.contiguous(), scales.contiguous(), zeros.contiguous()
+    out = torch.empty((K, N), dtype=scales.dtype, device=scales.device)
+    check(lib().ao_amd_hqq_dequantize(packed_2xint4.data_ptr(), int(packed_2xint4.dtype is torch.int8), K, N,
+                                      scales.data_ptr(), zeros.data_ptr(), group_size,
+                                      BF16 if scales.dtype is torch.bfloat16 else F16, out.data_ptr(),
+                                      current_stream(scales.device)))
+    return out
+
+
 def _rmsnorm_cuda(x, weight, eps):
     require_cuda(x, weight)
     torch._check(x.dtype is torch.bfloat16 and weight.dtype is torch.bfloat16, lambda: "rmsnorm needs bfloat16 tensors")
@@ -458,6 +479,7 @@ _LIB.impl("int4wo_rmsnorm_swiglu", _rmsnorm_swiglu_cuda, "CUDA")
 _LIB.impl("int4wo_interleave_pair", _interleave_pair_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu_interleaved", _swiglu_interleaved_cuda, "CUDA")
 _LIB.impl("int8wo_linear", _int8wo_linear_cuda, "CUDA")
+_LIB.impl("hqq_dequantize", _hqq_dequantize_cuda, "CUDA")
 _LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
 _LIB.impl("llama_decode_attention", _decode_attention_cuda, "CUDA")
 _LIB.impl("argmax_bf16", _argmax_bf16_cuda, "CUDA")
@@ -476,7 +498,7 @@ def _no_cpu(name):
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
               "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int4wo_interleave_pair",
-              "int4wo_swiglu_interleaved", "int8wo_linear", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
+              "int4wo_swiglu_interleaved", "int8wo_linear", "hqq_dequantize", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
               "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
@@ -556,6 +578,11 @@ def _(x, w_int8, scale, bias, fp32_out):
 @torch.library.register_fake("torchao::argmax_bf16")
 def _(x):
     return x.new_empty((1,), dtype=torch.int32)
+
+
+@torch.library.register_fake("torchao::hqq_dequantize")
+def _(packed_2xint4, scales, zeros, group_size):
+    return scales.new_empty((2 * packed_2xint4.shape[0], packed_2xint4.shape[1]))
 
 
 @torch.library.register_fake("torchao::rmsnorm")
@@ -673,6 +700,11 @@ def int4wo_swiglu_interleaved(x, packed_pair, qparams_pair, group_size, N, norm_
 def int8wo_linear(x: Tensor, w_int8: Tensor, scale: Tensor, bias=None, fp32_out: bool = False) -> Tensor:
     """bf16(bf16(x @ w_int8^T) * scale) (+ bias): x bf16 [M,K], w_int8 int8 [N,K] (plain layout), scale bf16 [N]."""
     return torch.ops.torchao.int8wo_linear.default(x, w_int8, scale, bias, fp32_out)
+
+
+def hqq_dequantize(packed_2xint4: Tensor, scales: Tensor, zeros: Tensor, group_size: int) -> Tensor:
+    """HQQ two-per-byte codes [K/2, N] -> (q - zero) * scale as a [K, N] matrix in the dtype of the scales."""
+    return torch.ops.torchao.hqq_dequantize.default(packed_2xint4, scales, zeros, group_size)
 
 
 def rmsnorm(x, weight, eps: float):

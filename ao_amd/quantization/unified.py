@@ -1,24 +1,23 @@
-"""Quantizer base classes (reference torchao/quantization/unified.py:15-37)."""
-from abc import ABC, abstractmethod
-from typing import Any
+"""The two quantizer interfaces of the module-swap flows (reference torchao/quantization/unified.py:15-37)."""
+import abc
 
 import torch
 
 
-class Quantizer(ABC):
-    """One-step flow: `quantize(model)` returns the quantized model."""
+class Quantizer(abc.ABC):
+    """One call: `quantize(model, ...)` returns the quantized model."""
 
-    @abstractmethod
-    def quantize(self, model: torch.nn.Module, *args: Any, **kwargs: Any) -> torch.nn.Module:
-        pass
+    @abc.abstractmethod
+    def quantize(self, model: torch.nn.Module, *args, **kwargs) -> torch.nn.Module:
+        ...
 
 
 class TwoStepQuantizer:
-    """Flow with a calibration or training phase between `prepare` and `convert`."""
+    """`prepare(model)` inserts what calibration or training needs, `convert(model)` produces the quantized model."""
 
-    @abstractmethod
-    def prepare(self, model: torch.nn.Module, *args: Any, **kwargs: Any) -> torch.nn.Module:
-        pass
+    @abc.abstractmethod
+    def prepare(self, model: torch.nn.Module, *args, **kwargs) -> torch.nn.Module:
+        ...
 
-    def convert(self, model: torch.nn.Module, *args: Any, **kwargs: Any) -> torch.nn.Module:
-        pass
+    def convert(self, model: torch.nn.Module, *args, **kwargs) -> torch.nn.Module:
+        ...

@@ -149,6 +149,17 @@ int ao_amd_int4wo_swiglu_interleaved(const void* x_bf16, int64_t M, int64_t K, i
                                      float eps, const void* packed_pair, const void* qparams_pair, int64_t N, int64_t g,
                                      void* y_bf16, int64_t ldy, void* stream);
 
+/* ---------------------------------------------------------------- HQQ-format int4 weight (prototype/hqq mixed matmul)
+ * W[k][n] = (q[k][n] - zeros[k/group][n]) * scales[k/group][n], each op rounded to `dtype` (AO_BF16 or AO_F16), from
+ * `packed_2xint4` uint8/int8 [K/2, N] whose byte (k2, n) holds q[2*k2][n] in the low and q[2*k2+1][n] in the high nibble
+ * (pack_2xint4, torchao/prototype/hqq/mixed_mm.py:13-35; unsigned nibbles, or sign-extended ones when `is_signed`).
+ * This is the dequantization inside the reference's Triton kernel (torchao/prototype/hqq/kernels.py:318-358) as a pass
+ * of its own: `out` is the [K, N] matrix in `dtype`; the caller multiplies x[M,K] @ out for the forward product and
+ * x[M,N] @ out^T for the transposed one (triton_mixed_mm(..., transposed=True), mixed_mm.py:38-62) with a library GEMM.
+ * N a multiple of 16, group_size even and dividing K, 16-byte aligned buffers. */
+int ao_amd_hqq_dequantize(const void* packed_2xint4, int is_signed, int64_t K, int64_t N, const void* scales,
+                          const void* zeros, int64_t group_size, int dtype, void* out, void* stream);
+
 /* ---------------------------------------------------------------- int8 weight-only linear
  * y[M,N] = bf16( bf16(x[M,K] @ bf16(w)^T) * scale[N] ) (+ bias, rounded to bf16 again): the per-channel int8
  * weight-only branch of _quantized_linear_op, torchao/dtypes/affine_quantized_tensor.py:641-665

@@ -69,6 +69,7 @@ class _Sig:
     ao_oracle_fp6_cuda_read_order = ([_p, _i64, _i64, _p], _int)
     ao_oracle_fpx_cuda_read_order = ([_p, _i64, _i64, _int, _p], _int)
     ao_oracle_fpx_linear = ([_p, _i64, _i64, _p, _p, _i64, _int, _int, _p], _int)
+    ao_oracle_hqq_dequantize = ([_p, _int, _i64, _i64, _p, _p, _i64, _int, _p], _int)
     ao_oracle_abi_version = ([], _int)
 
 
@@ -269,6 +270,18 @@ def fpx_linear(x_f16_bits, codes, scale_f16_bits, ebits, mbits):
     _check(lib().ao_oracle_fpx_linear(_ptr(x), M, K, _ptr(codes), _ptr(_c(scale_f16_bits, F16)), N, ebits, mbits,
                                       _ptr(y)), "fpx_linear")
     return y
+
+
+def hqq_dequantize(packed, scales_bits, zeros_bits, group, dtype):
+    """pack_2xint4 bytes [K/2, N] (uint8: unsigned nibbles, int8: sign-extended) + scales / zeros [K/group, N] bit
+    patterns -> [K, N] bit patterns of (q - zero) * scale computed op by op in `dtype` (BF16 or F16)."""
+    is_signed = int(packed.dtype == np.int8)
+    pk = np.ascontiguousarray(packed).view(np.uint8)
+    K2, N = pk.shape
+    out = np.empty((2 * K2, N), np.uint16)
+    _check(lib().ao_oracle_hqq_dequantize(_ptr(pk), is_signed, 2 * K2, N, _ptr(_c(scales_bits, dtype)),
+                                          _ptr(_c(zeros_bits, dtype)), group, dtype, _ptr(out)), "hqq_dequantize")
+    return out
 
 
 # numpy restatement of the generic three-pass packer _pack_tc_fpx (quant_llm.py:15-86): a second,

@@ -640,4 +640,37 @@ int ao_oracle_fpx_linear(const uint16_t* x_f16, int64_t M, int64_t K, const uint
     return 0;
 }
 
+/* HQQ-format mixed matmul weight (torchao/prototype/hqq): byte (k2, n) of `packed` [K/2, N] holds W_q[n][2*k2] in its low
+ * nibble and W_q[n][2*k2+1] in its high nibble (pack_2xint4, mixed_mm.py:13-35); the kernel unpacks with
+ * (qb << 4) >> 4 and qb >> 4 in the storage dtype (kernels.py:324-326: logical shifts for uint8, sign-extending for int8)
+ * and dequantizes op by op in the activation dtype: w = (q - zero) * scale (kernels.py:358), scales / zeros [K/group, N].
+ * Output: [K, N] bit patterns of `dtype`.  Both intermediate results are exact in fp32 (small integer minus a 16-bit
+ * float; product of two 16-bit floats), so rounding each to `dtype` is the op-by-op result. */
+int ao_oracle_hqq_dequantize(const uint8_t* packed, int is_signed, int64_t K, int64_t N, const uint16_t* scales,
+                             const uint16_t* zeros, int64_t group, int dtype, uint16_t* out) {
+    if (dtype != AO_BF16 && dtype != AO_F16) return 1;
+    if (K % 2 || group <= 0 || K % group || group % 2) return 2;
+    for (int64_t k2 = 0; k2 < K / 2; ++k2)
+        for (int64_t n = 0; n < N; ++n) {
+            const uint8_t b = packed[k2 * N + n];
+            int q[2];
+            if (is_signed) {
+                q[0] = ((int8_t)(uint8_t)(b << 4)) >> 4;
+                q[1] = ((int8_t)b) >> 4;
+            } else {
+                q[0] = b & 15;
+                q[1] = b >> 4;
+            }
+            const int64_t g = (2 * k2) / group;
+            const float sc = dtype == AO_BF16 ? bf16_to_f32(scales[g * N + n]) : f16_to_f32(scales[g * N + n]);
+            const float zp = dtype == AO_BF16 ? bf16_to_f32(zeros[g * N + n]) : f16_to_f32(zeros[g * N + n]);
+            for (int h = 0; h < 2; ++h) {
+                const float d = rd(dtype, (float)q[h] - zp);
+                const float w = d * sc;
+                out[(2 * k2 + h) * N + n] = dtype == AO_BF16 ? f32_to_bf16(w) : f32_to_f16(w);
+            }
+        }
+    return 0;
+}
+
 int ao_oracle_abi_version(void) { return 1; }

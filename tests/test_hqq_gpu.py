@@ -1,0 +1,142 @@
+"""GPU tests of the HQQ prototype path: the dequantize kernel bit-exact against the oracle, the mixed matmul (forward and
+transposed) at the reference test's shapes against `x @ W_dq` / `x @ W_dq.T` (test/hqq/test_triton_mm.py:18-29, 118-139),
+and the HQQ -> int4 weight-only converter module."""
+import numpy as np
+import pytest
+import torch
+
+from _util import bits16, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    assert torch.cuda.is_available()
+    return torch.device("cuda:0")
+
+
+def _hqq_like(N, K, g, dtype, seed, signed=False):
+    """Codes, scales and zeros shaped as HQQ leaves them with axis = 1 grouping of an [N, K] weight: W_q [N, K],
+    scale / zero [N, K/g] (meta tensors reshaped as in the reference test)."""
+    gen = torch.Generator().manual_seed(seed)
+    lo, hi = (-8, 8) if signed else (0, 16)
+    W_q = torch.randint(lo, hi, (N, K), generator=gen).to(torch.int8 if signed else torch.uint8)
+    scale = (torch.rand(N, K // g, generator=gen) * 0.02 + 1e-3).to(dtype)
+    zero = (torch.rand(N, K // g, generator=gen) * 6 + (-3 if signed else 5)).to(dtype)
+    return W_q, scale, zero
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(128, 128, 64), (48, 256, 32), (4096, 4096, 128)])
+def test_dequantize_bit_exact(oracle, shape, dtype, signed):
+    from ao_amd import ops
+    from ao_amd.prototype.hqq import pack_2xint4
+
+    N, K, g = shape
+    print(f"case hqq dequantize N={N} K={K} g={g} {dtype} signed={signed}", flush=True)
+    dev = _dev()
+    W_q, scale, zero = _hqq_like(N, K, g, dtype, seed=N + g, signed=signed)
+    packed = pack_2xint4(W_q.T.contiguous())
+    w = ops.hqq_dequantize(packed.to(dev), scale.T.contiguous().to(dev), zero.T.contiguous().to(dev), g)
+    assert w.shape == (K, N) and w.dtype is dtype
+    ref = oracle.hqq_dequantize(packed.numpy(), bits16(scale.T.contiguous()), bits16(zero.T.contiguous()), g,
+                                oracle.BF16 if dtype is torch.bfloat16 else oracle.F16)
+    assert np.array_equal(bits16(w), ref)
+
+
+@pytest.mark.parametrize("transposed", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("group_size", [64, 128])
+@pytest.mark.parametrize("shape", [(16, 128, 128), (16, 4096, 4096), (300, 512, 1024)])
+def test_mixed_mm(oracle, shape, group_size, dtype, transposed):
+    """Arguments passed as the reference test passes them: packed W_q.T, scales.T and zeros.T as (non-contiguous)
+    transposed views of the [N, K/g] parameters."""
+    from ao_amd.prototype.hqq import pack_2xint4, triton_mixed_mm
+
+    M, N, K = shape
+    print(f"case mixed_mm M={M} N={N} K={K} g={group_size} {dtype} transposed={transposed}", flush=True)
+    dev = _dev()
+    W_q, scale, zero = _hqq_like(N, K, group_size, dtype, seed=M + N + group_size)
+    W_q, scale, zero = W_q.to(dev), scale.to(dev), zero.to(dev)
+    # HQQ's dequantize: ((W_q - zero) * scale) on the grouped view, in the compute dtype
+    W_dq = ((W_q.to(dtype).reshape(-1, group_size) - zero.reshape(-1, 1)) * scale.reshape(-1, 1)).reshape(N, K)
+    packed_w = pack_2xint4(W_q.T)
+    gen = torch.Generator(device=dev).manual_seed(7)
+    if transposed:
+        x = torch.randn(M, N, dtype=dtype, device=dev, generator=gen)
+        expect = x @ W_dq
+    else:
+        x = torch.randn(M, K, dtype=dtype, device=dev, generator=gen)
+        expect = x @ W_dq.T
+    out = triton_mixed_mm(x, packed_w, scale.T, zero.T, transposed=transposed, group_size=group_size,
+                          fp8_fast_accum=False, kernel_type="compute_bound")
+    assert out.shape == expect.shape and out.dtype is dtype
+    # The reference test asks for atol = rtol = 1e-3 between its kernel and torch's matmul.  Two GEMMs that sum in a
+    # different order may round an element to neighbouring values of the output dtype, and one bf16 step is 2^-7
+    # relative, so the bound here is one step of the dtype (plus the reference's atol), on few elements.
+    step = 2.0 ** -7 if dtype is torch.bfloat16 else 2.0 ** -10
+    assert torch.allclose(expect, out, atol=1e-3, rtol=step)
+    assert (expect != out).float().mean().item() <= 0.05
+    # and against fp32 accumulation on the CPU for the small cases
+    if N * K <= 512 * 1024:
+        ref = (x.double().cpu() @ (W_dq.double().cpu() if transposed else W_dq.double().cpu().T)).numpy()
+        assert rel_l2(out.float().cpu().numpy(), ref) <= 4e-3  # one rounding of the result to bf16 / fp16
+
+
+def test_mixed_mm_argument_checks():
+    from ao_amd.prototype.hqq import mixed_mm, pack_2xint4
+
+    dev = _dev()
+    W_q, scale, zero = _hqq_like(64, 128, 64, torch.float16, seed=1)
+    b = pack_2xint4(W_q.T.contiguous()).to(dev)
+    s, z = scale.T.contiguous().to(dev), zero.T.contiguous().to(dev)
+    x = torch.randn(4, 128, dtype=torch.float16, device=dev)
+    with pytest.raises(AssertionError, match="incompatible dimensions"):
+        mixed_mm(x[:, :64], b, s, z, 64)
+    with pytest.raises(AssertionError, match="transpose requires"):
+        mixed_mm(x, b, s, z, 64, transposed=True)
+    with pytest.raises(AssertionError):
+        mixed_mm(x.bfloat16(), b, s, z, 64)
+    with pytest.raises(AssertionError, match="int8 or uint8"):
+        mixed_mm(x, b.to(torch.int32), s, z, 64)
+
+
+@pytest.mark.parametrize("g", [64, 128])
+def test_converter_module_runs_hqq_weights_on_the_int4_kernels(oracle, g):
+    from ao_amd import ops
+    from ao_amd.prototype.hqq import HQQLinearTorchWeightOnlyInt4
+
+    dev = _dev()
+    N, K = 256, 1024
+    W_q, scale, zero = _hqq_like(N, K, g, torch.bfloat16, seed=3 + g)
+    meta = {"scale": scale.reshape(-1, 1).to(dev), "zero": zero.reshape(-1, 1).to(dev), "shape": (N, K),
+            "packing": None, "nbits": 4, "group_size": g, "axis": 1}
+    cfg = {"weight_quant_params": {"nbits": 4, "group_size": g, "axis": 1}}
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(1)) * 0.1).bfloat16().to(dev)
+    mod = HQQLinearTorchWeightOnlyInt4(None, cfg, initialize=False).initialize_with_hqq_quants(
+        W_q.reshape(-1, g).to(dev).float(), meta, bias=bias)
+    assert mod.ready and mod.in_features == K and mod.out_features == N and not mod.padding
+    assert mod.scales_and_zeros.shape == (K // g, N, 2) and mod.scales_and_zeros.dtype is torch.bfloat16
+    codes, s, z_aff = ops.int4wo_unpack(mod.weight_int4pack, mod._qparams, N, K, g)
+    assert torch.equal(codes.cpu(), W_q.to(torch.int32))           # the conversion keeps the codes
+    assert torch.equal(s.cpu(), scale)                              # and the scales
+    assert torch.equal(mod.scales_and_zeros[:, :, 0].t().cpu(), scale)
+    assert torch.equal(mod.scales_and_zeros[:, :, 1].t().cpu(), z_aff.cpu())
+    # forward = linear over the affine reconstruction (the int4 kernels' own oracle) ...
+    x = torch.randn(2, 5, K, generator=torch.Generator().manual_seed(2)).bfloat16()
+    y = mod(x.to(dev))
+    assert y.shape == (2, 5, N) and y.dtype is torch.bfloat16
+    dq = oracle.dequantize_affine(codes.cpu().numpy(), oracle.I32, (1, g), bits16(s), oracle.BF16, bits16(z_aff),
+                                  oracle.BF16, 0, 15, 1, oracle.BF16)
+    assert np.array_equal(bits16(mod.dequantize()), dq)
+    y_ref = oracle.linear(bits16(x.reshape(-1, K)), oracle.BF16, dq, oracle.BF16)
+    y_ref = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(y_ref)) + bias.float().cpu().numpy()
+    assert rel_l2(y.float().cpu().numpy().reshape(-1, N), y_ref) <= 4e-3
+    # ... which is HQQ's own reconstruction up to the bf16 rounding of the converted zero point
+    hqq_w = ((W_q.double().reshape(-1, g) - zero.double().reshape(-1, 1)) * scale.double().reshape(-1, 1)).reshape(N, K)
+    y_hqq = x.double().reshape(-1, K) @ hqq_w.T + bias.double().cpu()
+    assert rel_l2(y.float().cpu().numpy().reshape(-1, N), y_hqq.numpy()) <= 2e-2
+
+    with pytest.raises(ImportError, match="hqq"):
+        HQQLinearTorchWeightOnlyInt4(torch.nn.Linear(K, N, bias=False), cfg, initialize=True)
