@@ -960,7 +960,12 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     AO_REQUIRE(!pair8 || (xmode == X_LDS && M <= 16 && !dual),
                "interleaved swiglu needs M <= 16, K a multiple of max(128, group), 16-byte aligned rows and activations "
                "that fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);
-    if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16) {
+    // Between 17 and 64 rows a small weight gives the GEMM too few tiles to occupy the chip (64 x 64 tiles over
+    // N = 4096: 64 workgroups on 256 CUs, each walking all of K); the streaming kernel over chunks of 16 rows
+    // keeps every CU busy there and re-reads the weight from the last-level cache.
+    const int64_t gemm_small_wgs = ((RB + 3) / 4) * ((M + 63) / 64);
+    const bool gemm_starved = (M <= 32 && gemm_small_wgs < 128) || (M <= 64 && gemm_small_wgs <= 64);
+    if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16 && !gemm_starved) {
         // 128 x 128 workgroup tiles when they fill a good part of the 256 CUs, else 64 x 64 tiles: four times
         // the workgroups, each dequantizing for 64 activation rows only
         const bool big = ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
