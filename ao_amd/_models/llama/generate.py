@@ -12,7 +12,7 @@ from typing import Optional
 
 import torch
 
-from ...quantization import int4_weight_only, quantize
+from ...quantization import int4_weight_only, int8_weight_only, quantize
 from ...utils import get_model_size_in_bytes
 from .model import Transformer, prepare_inputs_for_model
 
@@ -157,7 +157,8 @@ def random_init_(model: torch.nn.Module, std: float = 0.02, seed: int = 1234) ->
 
 
 def build_random_model(name: str, device, quantization: Optional[str] = None, seed: int = 1234) -> Transformer:
-    """Random-init bf16 model on `device`, optionally quantized ("int4wo-<group>")."""
+    """Random-init bf16 model on `device`, optionally quantized ("int4wo-<group>" or "int8wo", the names of the
+    reference's generate.py:199-215)."""
     prev = torch.get_default_dtype()
     torch.set_default_dtype(torch.bfloat16)
     try:
@@ -167,7 +168,9 @@ def build_random_model(name: str, device, quantization: Optional[str] = None, se
         torch.set_default_dtype(prev)
     random_init_(model, seed=seed)
     model.eval()
-    if quantization:
+    if quantization == "int8wo":
+        quantize(model, int8_weight_only())
+    elif quantization:
         assert quantization.startswith("int4wo-"), f"unsupported quantization {quantization}"
         group = int(quantization.split("-")[-1])
         assert group in (32, 64, 128, 256), f"int4wo groupsize needs to be one of [32,64,128,256] but got {group}"

@@ -207,27 +207,42 @@ class Transformer(nn.Module):
                                               dtype, device)
         self.causal_mask = torch.tril(torch.ones(max_seq_length, max_seq_length, dtype=torch.bool, device=device))
 
-    def fused_decode_ready(self) -> bool:
-        """True when a batch-1 single-token step can run on the fused HIP path: every linear is an int4
-        weight in the gfx950 layout with one group size, bf16 everywhere, head_dim 128, caches set up."""
-        from ...dtypes.affine_quantized_tensor import AffineQuantizedTensor, Gfx950WaveTiledAQTLayout
+    def _decode_linears(self):
+        return [self.output] + [m for b in self.layers for m in (b.attention.wqkv, b.attention.wo, b.feed_forward.w1,
+                                                                 b.feed_forward.w3, b.feed_forward.w2)]
+
+    def fused_decode_kind(self) -> Optional[str]:
+        """"int4" / "int8" when a batch-1 single-token step can run on the HIP decode path, else None.  int4: every
+        linear an int4 weight in the gfx950 layout with one group size; int8: every linear a per-channel int8
+        weight in the plain layout with in_features a multiple of 128; in both cases bf16 everywhere, head_dim 128,
+        caches set up for batch 1."""
+        from ...dtypes.affine_quantized_tensor import AffineQuantizedTensor, Gfx950WaveTiledAQTLayout, PlainAQTLayout
 
         if self.freqs_cis is None or self.max_batch_size != 1 or self.config.head_dim != 128 \
-                or self.max_seq_length > 8192:
-            return False
-        lins = [self.output] + [m for b in self.layers for m in (b.attention.wqkv, b.attention.wo, b.feed_forward.w1,
-                                                                  b.feed_forward.w3, b.feed_forward.w2)]
-        groups = set()
-        for lin in lins:
+                or self.max_seq_length > 8192 or self.tok_embeddings.weight.dtype is not torch.bfloat16:
+            return None
+        kinds, groups = set(), set()
+        for lin in self._decode_linears():
             w = lin.weight
-            if lin.bias is not None or not isinstance(w, AffineQuantizedTensor) or w.dtype is not torch.bfloat16:
-                return False
+            if lin.bias is not None or not isinstance(w, AffineQuantizedTensor) or w.dtype is not torch.bfloat16 \
+                    or not w.is_cuda:
+                return None
             lay = w.layout_tensor
-            if not isinstance(lay, Gfx950WaveTiledAQTLayout) or lay.transposed or not w.is_cuda:
-                return False
-            groups.add(lay.group_size)
-        return len(groups) == 1 and self.tok_embeddings.weight.dtype is torch.bfloat16 \
-            and self.config.intermediate_size % 16 == 0
+            if isinstance(lay, Gfx950WaveTiledAQTLayout) and not lay.transposed:
+                kinds.add("int4")
+                groups.add(lay.group_size)
+            elif isinstance(lay, PlainAQTLayout) and lay.int_data.dtype is torch.int8 and lay.int_data.dim() == 2 \
+                    and lay.int_data.is_contiguous() and lay.int_data.shape[1] % 128 == 0 \
+                    and lay.scale.numel() == lay.int_data.shape[0] and lay.scale.dtype is torch.bfloat16:
+                kinds.add("int8")
+            else:
+                return None
+        if kinds == {"int4"} and len(groups) == 1 and self.config.intermediate_size % 16 == 0:
+            return "int4"
+        return "int8" if kinds == {"int8"} else None
+
+    def fused_decode_ready(self) -> bool:
+        return self.fused_decode_kind() is not None
 
     @staticmethod
     def _gate_up_pair(ff):
@@ -276,11 +291,37 @@ class Transformer(nn.Module):
         xn = ops.rmsnorm(x, self.norm.weight, self.norm.eps)
         return lin(xn, self.output).view(1, 1, cfg.vocab_size)
 
+    def _fused_decode_int8(self, idx: Tensor, input_pos: Tensor) -> Tensor:
+        """The same step over int8 weight-only linears: the streaming int8 kernel per linear, the RMSNorm and decode
+        attention kernels, and the module's own elementwise ops (residual add, SiLU * up) in between."""
+        from ... import ops
+
+        cfg = self.config
+
+        def lin(x, layer):
+            lay = layer.weight.layout_tensor
+            return ops.int8wo_linear(x, lay.int_data, lay.scale.reshape(-1))
+
+        x = self.tok_embeddings(idx).view(1, cfg.dim)
+        pos = input_pos.to(torch.int32) if input_pos.dtype is not torch.int32 else input_pos
+        for b in self.layers:
+            att, ffn = b.attention, b.feed_forward
+            qkv = lin(ops.rmsnorm(x, b.attention_norm.weight, b.attention_norm.eps), att.wqkv)
+            y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
+                                           cfg.n_head, cfg.n_local_heads)
+            h = x + lin(y, att.wo)
+            hn = ops.rmsnorm(h, b.ffn_norm.weight, b.ffn_norm.eps)
+            x = h + lin(F.silu(lin(hn, ffn.w1)) * lin(hn, ffn.w3), ffn.w2)
+        return lin(ops.rmsnorm(x, self.norm.weight, self.norm.eps), self.output).view(1, 1, cfg.vocab_size)
+
     def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None) -> Tensor:
         assert self.freqs_cis is not None, "Caches must be initialized first"
-        if self.use_fused_decode and idx.numel() == 1 and input_pos is not None and input_pos.numel() == 1 \
-                and self.fused_decode_ready():
-            return self._fused_decode(idx, input_pos)
+        if self.use_fused_decode and idx.numel() == 1 and input_pos is not None and input_pos.numel() == 1:
+            kind = self.fused_decode_kind()
+            if kind == "int4":
+                return self._fused_decode(idx, input_pos)
+            if kind == "int8":
+                return self._fused_decode_int8(idx, input_pos)
         mask = self.causal_mask[None, None, input_pos]
         freqs_cis = self.freqs_cis[input_pos]
         x = self.tok_embeddings(idx)

@@ -396,6 +396,9 @@ def main():
     ap.add_argument("--roofline-only", action="store_true",
                     help="build the model, run one pass of the roofline leg and a copy kernel of known size, no decode "
                          "loop: the command to put under rocprofv3 --pmc")
+    ap.add_argument("--quantization", default=None,
+                    help="int4wo-<group> (default: int4wo-<--group>, the headline configuration) or int8wo: the decode "
+                         "loop of the reference's other weight-only configuration, reported without the int4 roofline leg")
     ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6", "int8"), default=None,
                     help="instead of the decode benchmark, print one line per kernel case of the named sweep")
     args = ap.parse_args()
@@ -418,7 +421,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    quant = f"int4wo-{args.group}"
+    quant = args.quantization or f"int4wo-{args.group}"
+    if not quant.startswith("int4wo-"):
+        args.no_roofline = args.no_cpu_baseline = True  # both legs describe the int4 kernels
     model = build_random_model(args.model, device, quant)
     cfg = model.config
     model_size = get_model_size_in_bytes(model, ignore_embeddings=True)
@@ -448,7 +453,8 @@ def main():
 
     tok_s = args.steps / elapsed
     line = {
-        "metric": "tok/s Llama-3-8B-arch int4wo-64 bs=1; int4 GEMV HBM GB/s vs peak",
+        "metric": ("tok/s Llama-3-8B-arch int4wo-64 bs=1; int4 GEMV HBM GB/s vs peak" if quant.startswith("int4wo-")
+                   else f"tok/s Llama-3-8B-arch {quant} bs=1"),
         "value": round(tok_s, 2),
         "unit": "tokens/s",
         "n_gpus": 1,

@@ -292,3 +292,27 @@ def test_fused_decode_step_matches_module_path():
     a = generate(model, prompt, 10, use_graph=True, greedy=True)
     b = generate(model, prompt, 10, use_graph=False, greedy=True)
     assert torch.equal(a, b)
+
+
+def test_fused_decode_step_int8_weight_only():
+    """The same comparison for an int8 weight-only model: streaming int8 kernel + RMSNorm / attention kernels
+    against the module-by-module forward; then graph replay against the eager loop."""
+    from ao_amd._models.llama.generate import build_random_model, generate
+
+    dev = _dev()
+    model = build_random_model("tiny128", dev, "int8wo")
+    prompt = torch.randint(0, model.config.vocab_size, (12,), device=dev, dtype=torch.int)
+    with torch.no_grad():
+        model.setup_caches(1, 64)
+        assert model.fused_decode_kind() == "int8"
+        model(prompt.view(1, -1), torch.arange(12, device=dev))
+        tok = torch.tensor([[7]], device=dev, dtype=torch.int)
+        p = torch.tensor([12], device=dev, dtype=torch.int)
+        model.use_fused_decode = False
+        ref = model(tok, p).float()
+        model.use_fused_decode = True
+        out = model(tok, p).float()
+    assert rel_l2(out.cpu().numpy(), ref.cpu().numpy()) <= 3e-2
+    a = generate(model, prompt, 10, use_graph=True, greedy=True)
+    b = generate(model, prompt, 10, use_graph=False, greedy=True)
+    assert torch.equal(a, b)
