@@ -161,13 +161,15 @@ def test_linear_one_hot_is_exact_dequant(cabi, oracle, g):
     w = make_weight(N, K, seed=99 + g)
     packed, qparams, _, _ = _quantize_pack(cabi, w.to(_dev()), g)
     ks = [0, 1, 7, 8, 31, 32, 33, 63, 64, 127, 128, 255, 256, 300, 510, 511, 200, 77]
+    ks += [(37 * i + 5) % K for i in range(70 - len(ks))]
     x = torch.zeros(len(ks), K, dtype=torch.bfloat16)
     for m, k in enumerate(ks):
         x[m, k] = 1.0
     dq, _ = _oracle_linear(oracle, w, x, g)
     dqf = oracle.bf16_bits_to_f32(dq)
-    # 18 rows run on the tiled kernel (M > 16), 16 and 1 on the decode kernel: each has its own dequantization code
-    for rows in (len(ks), 16, 1):
+    # 70 rows run on the tiled GEMM kernel, 18 on the streaming kernel in two chunks, 16 and 1 on the decode kernel:
+    # each has its own dequantization code
+    for rows in (len(ks), 18, 16, 1):
         y = _linear(cabi, x[:rows].contiguous().to(_dev()), packed, qparams, N, g, fp32=True).cpu().numpy()
         for m, k in enumerate(ks[:rows]):
             assert np.array_equal(y[m], dqf[:, k]), (rows, m, k)
