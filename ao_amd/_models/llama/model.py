@@ -245,6 +245,14 @@ class Transformer(nn.Module):
         return self.fused_decode_kind() is not None
 
     @staticmethod
+    def qkv_ksplit(n_rows: int, n_cu: int = 256) -> int:
+        """2 when the fused qkv weight's 16-row blocks would leave half of the CUs with one workgroup more than the
+        others (Llama-3-8B: 384 blocks on 256 CUs), else 1."""
+        blocks = (n_rows + 15) // 16
+        frac = (blocks % n_cu) / n_cu
+        return 2 if blocks < 4 * n_cu and 0.25 <= frac <= 0.75 else 1
+
+    @staticmethod
     def _gate_up_pair(ff):
         """w1 and w3 of a feed-forward block as one packed weight with gate and up rows interleaved in eights, built
         on first use and rebuilt when either weight is replaced.  One launch of twice the row blocks, half the work
@@ -280,8 +288,13 @@ class Transformer(nn.Module):
         for b in self.layers:
             att = b.attention
             qw = att.wqkv.weight.layout_tensor
-            qkv = ops.int4wo_rmsnorm_linear(x, b.attention_norm.weight, b.attention_norm.eps, qw.packed_weight,
-                                            qw.scale_and_zero, qw.group_size, qw.N)
+            if self.qkv_ksplit(qw.N) > 1:
+                # fp32 partial rows over two halves of K; the attention kernel adds and rounds them
+                qkv = ops.int4wo_linear_partials(x, qw.packed_weight, qw.scale_and_zero, qw.group_size, qw.N,
+                                                 self.qkv_ksplit(qw.N), b.attention_norm.weight, b.attention_norm.eps)
+            else:
+                qkv = ops.int4wo_rmsnorm_linear(x, b.attention_norm.weight, b.attention_norm.eps, qw.packed_weight,
+                                                qw.scale_and_zero, qw.group_size, qw.N)
             y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
                                            cfg.n_head, cfg.n_local_heads)
             h = lin(y, att.wo, residual=x)

@@ -190,6 +190,8 @@ struct LinearArgs {
     const uint16_t* residual; int64_t ldres;           // [M,N] or null
     void* y; int y_is_f32; int64_t ldy;
     const uint16_t* norm_w; float norm_eps;            // GEMV only: RMSNorm weight [K] applied to x while staging, or null
+    int ksplit;                                        // GEMV only: blockIdx.z takes the z-th of `ksplit` contiguous runs of K tiles and
+                                                       // stores its fp32 partial sums at y + z * M * ldy (the consumer adds them)
     int pair8;                                         // GEMV only: rows 0-7 of every 16-row block are gate rows, rows 8-15
                                                        // the matching up rows; y[m, 8*rb + r] = silu(gate) * up, N = output rows
 };
@@ -541,8 +543,13 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
         buf[j].q = 0;
         buf[j].q2 = 0;
     }
-    // tiles of this wave: kb = wave + i*WAVES, i = 0..nt-1; tile i lives in buf[i % D]
-    const int nt = wave < KB ? (KB - wave + WAVES - 1) / WAVES : 0;
+    // K tiles of this workgroup: all of them, or the blockIdx.z-th run when K is split across workgroups;
+    // tiles of this wave: kb = kb0 + i*WAVES, i = 0..nt-1; tile i lives in buf[i % D]
+    const int kbs = (KB + a.ksplit - 1) / a.ksplit;
+    const int kbeg = (int)blockIdx.z * kbs;
+    const int kcnt = KB - kbeg < kbs ? (KB - kbeg > 0 ? KB - kbeg : 0) : kbs;
+    const int kb0 = kbeg + wave;
+    const int nt = wave < kcnt ? (kcnt - wave + WAVES - 1) / WAVES : 0;
 
     // ---- activations -> LDS.  Decode shape (one row that fits two 16-byte chunks per thread): the row is
     // requested BEFORE the weight prefetch, so it does not queue behind megabytes of weight traffic, and is
@@ -566,7 +573,7 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     // always D-1 tiles' worth of weight loads (a wave with fewer tiles requests its last one again), so that the
     // count below is a constant; later waits only ever wait for more than they need because of it
 #pragma unroll
-    for (int j = 0; j < D - 1; ++j) load_tile(buf[j], wave + (j < nt ? j : (nt > 0 ? nt - 1 : 0)) * WAVES);
+    for (int j = 0; j < D - 1; ++j) load_tile(buf[j], (nt > 0 ? kb0 : 0) + (j < nt ? j : (nt > 0 ? nt - 1 : 0)) * WAVES);
     asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(xv0), "+v"(xv1), "+v"(nv0), "+v"(nv1) : [n] "n"((D - 1) * LPT) : "memory");
     {
         __shared__ float norm_part[WAVES];
@@ -647,9 +654,9 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
             const int i = i0 + j;
             if (i < nt) {
                 const int nxt = i + (D - 1);
-                if (nxt < nt) load_tile(buf[(j + D - 1) % D], wave + nxt * WAVES);
+                if (nxt < nt) load_tile(buf[(j + D - 1) % D], kb0 + nxt * WAVES);
                 wait_tiles<LPT>(younger(i, D - 1));
-                compute_tile(buf[j], wave + i * WAVES, buf[(j + 1) % D], i + 1 < nt, younger(i + 1, D - 2));
+                compute_tile(buf[j], kb0 + i * WAVES, buf[(j + 1) % D], i + 1 < nt, younger(i + 1, D - 2));
             }
         }
     }
@@ -684,7 +691,7 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
                     s += bv;
                     if (a.residual) s = hw_rne_bf16(s) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
                 }
-                if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = s;
+                if (a.y_is_f32) ((float*)a.y)[((int64_t)blockIdx.z * a.M + m) * a.ldy + n] = s;
                 else ((uint16_t*)a.y)[m * a.ldy + n] = hw_bf16_bits(s);
             }
         }
@@ -907,7 +914,8 @@ static void launch_group(int64_t g, int waves, dim3 grid, size_t smem, hipStream
 static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed, const void* qparams,
                            const void* packed2, const void* qparams2, int64_t N, int64_t g, const void* bias_bf16,
                            const void* residual_bf16, int64_t ldres, void* y, int y_dtype, int64_t ldy, void* stream,
-                           const void* norm_weight_bf16 = nullptr, float norm_eps = 0.f, bool pair8 = false) {
+                           const void* norm_weight_bf16 = nullptr, float norm_eps = 0.f, bool pair8 = false,
+                           int ksplit = 1) {
     // pair8: `packed` / `qparams` hold 2 * N rows (gate and up rows interleaved in eights), the output has N columns
     const int64_t n_out = N;
     if (pair8) N *= 2;
@@ -928,10 +936,13 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     AO_REQUIRE(!dual || qparams2, "null pointer argument");
     const int64_t mchunks = (M + 15) / 16;
     AO_REQUIRE(mchunks <= 65535, "batch too large for one launch: M=%lld", (long long)M);
-    const int64_t KB = Kp / 128, RB = Np / 16;
+    const int64_t KB_all = Kp / 128, RB = Np / 16;
+    AO_REQUIRE(ksplit >= 1 && ksplit <= 8 && ksplit <= KB_all, "K split %d out of range for %lld K tiles", ksplit,
+               (long long)KB_all);
+    const int64_t KB = (KB_all + ksplit - 1) / ksplit;  // K tiles per workgroup: what the wave count is sized for
     // about 16 waves per CU over 256 CUs, each with as many K tiles as the shape allows
     int waves = 1;
-    while (waves < 16 && RB * mchunks * waves * 2 <= 4096 + RB * mchunks && waves * 2 <= KB) waves *= 2;
+    while (waves < 16 && RB * ksplit * mchunks * waves * 2 <= 4096 + RB * ksplit * mchunks && waves * 2 <= KB) waves *= 2;
     // a single activation row is staged fastest when the workgroup's threads cover it with two 16-byte chunks each
     if (M == 1)
         while (waves < 16 && (int64_t)waves * 128 < Kp / 8 && waves * 2 <= KB) waves *= 2;
@@ -950,7 +961,7 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     LinearArgs a{(const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams,
                  (const uint4*)packed2, (const uint32_t*)qparams2, n_out, Kp, (const uint16_t*)bias_bf16,
                  (const uint16_t*)residual_bf16, ldres, y, y_dtype == AO_F32, ldy,
-                 (const uint16_t*)norm_weight_bf16, norm_eps, pair8 ? 1 : 0};
+                 (const uint16_t*)norm_weight_bf16, norm_eps, ksplit, pair8 ? 1 : 0};
     hipStream_t st = (hipStream_t)stream;
     // the fused RMSNorm lives in the activation staging of the GEMV kernel only
     AO_REQUIRE(!norm_weight_bf16 || (xmode == X_LDS && M <= 16 && (((uintptr_t)norm_weight_bf16) & 15) == 0),
@@ -965,6 +976,9 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // keeps every CU busy there and re-reads the weight from the last-level cache.
     const int64_t gemm_small_wgs = ((RB + 3) / 4) * ((M + 63) / 64);
     const bool gemm_starved = (M <= 32 && gemm_small_wgs < 128) || (M <= 64 && gemm_small_wgs <= 64);
+    AO_REQUIRE(ksplit == 1 || (xmode == X_LDS && M <= 16 && !dual && !pair8 && !bias_bf16 && !residual_bf16 && y_dtype == AO_F32),
+               "partial sums over a split K need M <= 16, fp32 output, no bias / residual epilogue and activations that "
+               "fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);
     if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16 && !gemm_starved) {
         // 128 x 128 workgroup tiles when they fill a good part of the 256 CUs, else 64 x 64 tiles: four times
         // the workgroups, each dequantizing for 64 activation rows only
@@ -985,7 +999,7 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
         AO_LAUNCH_CHECK();
         return 0;
     }
-    dim3 grid((unsigned)RB, (unsigned)mchunks);
+    dim3 grid((unsigned)RB, (unsigned)mchunks, (unsigned)ksplit);
     const size_t smem = xmode == X_LDS ? xbytes : 0;
     if (dual) {
         if (xmode == X_LDS) launch_gemv<true>(g, waves, grid, smem, st, a);
@@ -1058,4 +1072,12 @@ extern "C" int ao_amd_int4wo_swiglu_interleaved(const void* x_bf16, int64_t M, i
                                                 void* stream) {
     return linear_dispatch(x_bf16, M, K, ldx, packed_pair, qparams_pair, nullptr, nullptr, N, g, nullptr, nullptr, 0,
                            y_bf16, AO_BF16, ldy, stream, norm_weight_bf16, eps, true);
+}
+
+extern "C" int ao_amd_int4wo_linear_partials(const void* x_bf16, int64_t M, int64_t K, int64_t ldx,
+                                             const void* norm_weight_bf16, float eps, const void* packed,
+                                             const void* qparams, int64_t N, int64_t g, int ksplit, void* y_f32_parts,
+                                             int64_t ldy, void* stream) {
+    return linear_dispatch(x_bf16, M, K, ldx, packed, qparams, nullptr, nullptr, N, g, nullptr, nullptr, 0, y_f32_parts,
+                           AO_F32, ldy, stream, norm_weight_bf16, eps, false, ksplit);
 }

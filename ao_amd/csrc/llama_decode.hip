@@ -106,6 +106,7 @@ constexpr int ATT_U = 8;                 // passes per chunk
 constexpr int ATT_CHUNK = 64 * ATT_U;    // positions per chunk
 
 __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uint16_t* __restrict__ qkv,
+                                                                        const float* __restrict__ qkv_parts, int nparts,
                                                                         const uint16_t* __restrict__ freqs,
                                                                         const int32_t* __restrict__ pos_ptr,
                                                                         uint16_t* __restrict__ k_cache,
@@ -128,9 +129,16 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     const int pos = pos_ptr[0];
     const int T = pos + 1;
 
-    const uint16_t* qp = qkv + (int64_t)h * HD;
-    const uint16_t* kp = qkv + (int64_t)(n_head + hk) * HD;
-    const uint16_t* vp = qkv + (int64_t)(n_head + n_kv + hk) * HD;
+    // element i of the fused qkv row: a bf16 value, or the bf16 rounding of the sum of `nparts` fp32 partial rows
+    // (a linear whose K range was split across workgroups leaves the last add to its consumer)
+    const int64_t qkv_len = (int64_t)(n_head + 2 * n_kv) * HD;
+    auto qkv_at = [&](int64_t i) -> uint16_t {
+        if (nparts == 0) return qkv[i];
+        float t = qkv_parts[i];
+        for (int p = 1; p < nparts; ++p) t += qkv_parts[p * qkv_len + i];
+        return f32_to_bf16_bits(t);
+    };
+    const int64_t qp = (int64_t)h * HD, kp = (int64_t)(n_head + hk) * HD, vp = (int64_t)(n_head + n_kv + hk) * HD;
     uint16_t* kc = k_cache + (int64_t)hk * S * HD;
     uint16_t* vc = v_cache + (int64_t)hk * S * HD;
 
@@ -151,8 +159,8 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     // rotary embedding on pairs (2i, 2i+1), fp32 math, result rounded to bf16 like the module does
     if (tid < 128) {
         const int which = tid >> 6, i = tid & 63;   // 0: q, 1: k
-        const uint16_t* src = which ? kp : qp;
-        const float x0 = bf16_bits_to_f32(src[2 * i]), x1 = bf16_bits_to_f32(src[2 * i + 1]);
+        const int64_t src = which ? kp : qp;
+        const float x0 = bf16_bits_to_f32(qkv_at(src + 2 * i)), x1 = bf16_bits_to_f32(qkv_at(src + 2 * i + 1));
         const float c = bf16_bits_to_f32(freqs[((int64_t)pos * 64 + i) * 2]);
         const float sn = bf16_bits_to_f32(freqs[((int64_t)pos * 64 + i) * 2 + 1]);
         const float o0 = rne_bf16(x0 * c - x1 * sn), o1 = rne_bf16(x1 * c + x0 * sn);
@@ -165,7 +173,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
         }
     } else if (tid < 256) {
         const int i = tid - 128;
-        const uint16_t v = vp[i];
+        const uint16_t v = qkv_at(vp + i);
         vnew_s[i] = bf16_bits_to_f32(v);
         if ((h % rep) == 0) vc[(int64_t)pos * HD + i] = v;
     }
@@ -390,8 +398,24 @@ extern "C" int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* f
     AO_REQUIRE(max_seq > 0 && max_seq <= 8192, "max_seq=%lld outside (0, 8192]", (long long)max_seq);
     const size_t smem = (size_t)(3 * 128 + 32 + 16 * 128 + max_seq + 8) * sizeof(float);
     hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head), dim3(ATT_THREADS), smem, (hipStream_t)stream,
-                       (const uint16_t*)qkv_bf16, (const uint16_t*)freqs_cis_bf16, pos_dev, (uint16_t*)k_cache,
-                       (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16);
+                       (const uint16_t*)qkv_bf16, (const float*)nullptr, 0, (const uint16_t*)freqs_cis_bf16, pos_dev,
+                       (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_llama_decode_attention_parts(const void* qkv_f32_parts, int nparts, const void* freqs_cis_bf16,
+                                                   const int32_t* pos_dev, void* k_cache, void* v_cache, int n_head,
+                                                   int n_kv, int head_dim, int64_t max_seq, void* out_bf16, void* stream) {
+    AO_REQUIRE(qkv_f32_parts && freqs_cis_bf16 && pos_dev && k_cache && v_cache && out_bf16, "null pointer argument");
+    AO_REQUIRE(nparts >= 1 && nparts <= 8, "number of partial rows %d outside [1, 8]", nparts);
+    AO_REQUIRE(head_dim == 128, "decode attention kernel is built for head_dim 128, got %d", head_dim);
+    AO_REQUIRE(n_kv > 0 && n_head % n_kv == 0, "n_head=%d must be a multiple of n_kv=%d", n_head, n_kv);
+    AO_REQUIRE(max_seq > 0 && max_seq <= 8192, "max_seq=%lld outside (0, 8192]", (long long)max_seq);
+    const size_t smem = (size_t)(3 * 128 + 32 + 16 * 128 + max_seq + 8) * sizeof(float);
+    hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head), dim3(ATT_THREADS), smem, (hipStream_t)stream,
+                       (const uint16_t*)nullptr, (const float*)qkv_f32_parts, nparts, (const uint16_t*)freqs_cis_bf16,
+                       pos_dev, (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16);
     AO_LAUNCH_CHECK();
     return 0;
 }

@@ -45,6 +45,7 @@ _LIB.define("int4wo_linear_residual(Tensor x, Tensor packed, Tensor qparams, int
 _LIB.define("int4wo_swiglu(Tensor x, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
 _LIB.define("int4wo_rmsnorm_linear(Tensor x, Tensor norm_weight, float eps, Tensor packed, Tensor qparams, int group_size, int N, Tensor? bias) -> Tensor")
 _LIB.define("int4wo_rmsnorm_swiglu(Tensor x, Tensor norm_weight, float eps, Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int group_size, int N) -> Tensor")
+_LIB.define("int4wo_linear_partials(Tensor x, Tensor? norm_weight, float eps, Tensor packed, Tensor qparams, int group_size, int N, int ksplit) -> Tensor")
 _LIB.define("int4wo_interleave_pair(Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int N, int K, int group_size) -> (Tensor, Tensor)")
 _LIB.define("int4wo_swiglu_interleaved(Tensor x, Tensor? norm_weight, float eps, Tensor packed_pair, Tensor qparams_pair, int group_size, int N) -> Tensor")
 _LIB.define("int8wo_linear(Tensor x, Tensor w_int8, Tensor scale, Tensor? bias, bool fp32_out) -> Tensor")
@@ -284,6 +285,24 @@ def _rmsnorm_swiglu_cuda(x, norm_weight, eps, packed_gate, qparams_gate, packed_
     return y
 
 
+def _linear_partials_cuda(x, norm_weight, eps, packed, qparams, group_size, N, ksplit):
+    """fp32 [ksplit, M, N]: partial sums of (rmsnorm(x) or x) @ W^T over `ksplit` runs of K; decode shapes only."""
+    require_cuda(x, norm_weight, packed, qparams)
+    torch._check(x.dim() == 2 and x.dtype is torch.bfloat16, lambda: "input must be a 2d bfloat16 tensor")
+    if norm_weight is not None:
+        _check_norm(x, norm_weight)
+    M, K = x.shape
+    _check_packed(packed, qparams, N, K, group_size)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    y = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
+    check(lib().ao_amd_int4wo_linear_partials(x.data_ptr(), M, K, x.stride(0) if M > 0 else K,
+                                              None if norm_weight is None else norm_weight.data_ptr(), float(eps),
+                                              packed.data_ptr(), qparams.data_ptr(), N, group_size, ksplit, y.data_ptr(), N,
+                                              current_stream(x.device)))
+    return y
+
+
 def _interleave_pair_cuda(packed_gate, qparams_gate, packed_up, qparams_up, N, K, group_size):
     """Two packed weights of one shape -> the packed weight of 2N rows whose 16-row blocks hold 8 gate rows and the 8
     up rows of the same outputs (input of `int4wo_swiglu_interleaved`)."""
@@ -359,17 +378,28 @@ def _argmax_bf16_cuda(x):
 
 def _decode_attention_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv):
     require_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache)
-    torch._check(qkv.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16 and v_cache.dtype is torch.bfloat16
-                 and freqs_cis.dtype is torch.bfloat16, lambda: "decode attention needs bfloat16 tensors")
+    torch._check(qkv.dtype in (torch.bfloat16, torch.float32) and k_cache.dtype is torch.bfloat16
+                 and v_cache.dtype is torch.bfloat16 and freqs_cis.dtype is torch.bfloat16,
+                 lambda: "decode attention needs bfloat16 tensors (or fp32 partial rows for qkv)")
     torch._check(input_pos.dtype is torch.int32 and input_pos.numel() == 1, lambda: "input_pos must be one int32")
     torch._check(k_cache.dim() == 4 and k_cache.shape[0] == 1 and k_cache.shape[1] == n_kv and k_cache.is_contiguous()
                  and v_cache.shape == k_cache.shape and v_cache.is_contiguous(),
                  lambda: "caches must be contiguous [1, n_kv, max_seq, head_dim]")
     head_dim, max_seq = k_cache.shape[3], k_cache.shape[2]
-    torch._check(qkv.numel() == (n_head + 2 * n_kv) * head_dim and qkv.is_contiguous(),
-                 lambda: "qkv must be the contiguous fused projection of one token")
+    row = (n_head + 2 * n_kv) * head_dim
     torch._check(freqs_cis.is_contiguous() and freqs_cis.shape[-2:] == (head_dim // 2, 2), lambda: "bad freqs_cis shape")
     out = torch.empty((1, n_head * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    if qkv.dtype is torch.float32:
+        # fp32 partial rows of a linear whose K range was split (int4wo_linear_partials): added and rounded in the kernel
+        nparts = qkv.numel() // row
+        torch._check(qkv.is_contiguous() and qkv.numel() == nparts * row and 1 <= nparts <= 8,
+                     lambda: "fp32 qkv must be [parts, 1, (n_head + 2 n_kv) * head_dim] contiguous, 1..8 parts")
+        check(lib().ao_amd_llama_decode_attention_parts(qkv.data_ptr(), nparts, freqs_cis.data_ptr(), input_pos.data_ptr(),
+                                                        k_cache.data_ptr(), v_cache.data_ptr(), n_head, n_kv, head_dim,
+                                                        max_seq, out.data_ptr(), current_stream(qkv.device)))
+        return out
+    torch._check(qkv.numel() == row and qkv.is_contiguous(),
+                 lambda: "qkv must be the contiguous fused projection of one token")
     check(lib().ao_amd_llama_decode_attention(qkv.data_ptr(), freqs_cis.data_ptr(), input_pos.data_ptr(),
                                               k_cache.data_ptr(), v_cache.data_ptr(), n_head, n_kv, head_dim, max_seq,
                                               out.data_ptr(), current_stream(qkv.device)))
@@ -476,6 +506,7 @@ _LIB.impl("int4wo_linear_residual", _linear_residual_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu", _swiglu_cuda, "CUDA")
 _LIB.impl("int4wo_rmsnorm_linear", _rmsnorm_linear_cuda, "CUDA")
 _LIB.impl("int4wo_rmsnorm_swiglu", _rmsnorm_swiglu_cuda, "CUDA")
+_LIB.impl("int4wo_linear_partials", _linear_partials_cuda, "CUDA")
 _LIB.impl("int4wo_interleave_pair", _interleave_pair_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu_interleaved", _swiglu_interleaved_cuda, "CUDA")
 _LIB.impl("int8wo_linear", _int8wo_linear_cuda, "CUDA")
@@ -497,7 +528,7 @@ def _no_cpu(name):
 
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
-              "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int4wo_interleave_pair",
+              "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int4wo_linear_partials", "int4wo_interleave_pair",
               "int4wo_swiglu_interleaved", "int8wo_linear", "hqq_dequantize", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
               "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
@@ -557,6 +588,11 @@ def _(x, norm_weight, eps, packed, qparams, group_size, N, bias):
 @torch.library.register_fake("torchao::int4wo_rmsnorm_swiglu")
 def _(x, norm_weight, eps, packed_gate, qparams_gate, packed_up, qparams_up, group_size, N):
     return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::int4wo_linear_partials")
+def _(x, norm_weight, eps, packed, qparams, group_size, N, ksplit):
+    return x.new_empty((ksplit, x.shape[0], N), dtype=torch.float32)
 
 
 @torch.library.register_fake("torchao::int4wo_interleave_pair")
@@ -682,6 +718,12 @@ def int4wo_rmsnorm_swiglu(x, norm_weight, eps: float, packed_gate, qparams_gate,
     """swiglu(rmsnorm(x, norm_weight, eps)) in one launch, for M <= 16 rows (decode)."""
     return torch.ops.torchao.int4wo_rmsnorm_swiglu.default(x, norm_weight, eps, packed_gate, qparams_gate, packed_up,
                                                            qparams_up, group_size, N)
+
+
+def int4wo_linear_partials(x, packed, qparams, group_size, N, ksplit: int, norm_weight=None, eps: float = 0.0):
+    """fp32 [ksplit, M, N] partial sums of x' @ W^T over `ksplit` runs of K (x' = x or rmsnorm(x)); the consumer adds
+    them (llama_decode_attention does when given fp32 rows).  M <= 16."""
+    return torch.ops.torchao.int4wo_linear_partials.default(x, norm_weight, eps, packed, qparams, group_size, N, ksplit)
 
 
 def int4wo_interleave_pair(packed_gate, qparams_gate, packed_up, qparams_up, N: int, K: int, group_size: int):

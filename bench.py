@@ -102,8 +102,17 @@ def roofline_leg(model, passes=3):
     keep = []
     for b in model.layers:
         lay = b.attention.wqkv.weight.layout_tensor
-        fn, y = plain(lay, x, norm=b.attention_norm)
-        add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(y)
+        ks = model.qkv_ksplit(lay.N)
+        if ks > 1:  # as the decode step launches it: fp32 partial rows over `ks` runs of K
+            yp = torch.empty(ks, 1, lay.N, dtype=torch.float32, device=dev)
+            norm = b.attention_norm
+            fn = (lambda lay=lay, norm=norm, yp=yp, ks=ks: L.ao_amd_int4wo_linear_partials(
+                x.data_ptr(), 1, lay.K, lay.K, norm.weight.data_ptr(), float(norm.eps), lay.packed_weight.data_ptr(),
+                lay.scale_and_zero.data_ptr(), lay.N, lay.group_size, ks, yp.data_ptr(), lay.N, st))
+            add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(yp)
+        else:
+            fn, y = plain(lay, x, norm=b.attention_norm)
+            add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(y)
         lay = b.attention.wo.weight.layout_tensor
         fn, y = plain(lay, x, residual=res)
         add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(y)

@@ -135,6 +135,16 @@ int ao_amd_int4wo_rmsnorm_swiglu(const void* x_bf16, int64_t M, int64_t K, int64
                                  float eps, const void* packed_gate, const void* qparams_gate, const void* packed_up,
                                  const void* qparams_up, int64_t N, int64_t g, void* y_bf16, int64_t ldy, void* stream);
 
+/* Linear with the K range split over `ksplit` (1..8) groups of workgroups, for weights whose row-block count does not fill
+ * the CUs evenly (Llama-3-8B wqkv: 384 row blocks on 256 CUs): y_f32_parts[z][M][ldy] = sum over the z-th run of K tiles
+ * of x' W^T in fp32, x' = x or its RMSNorm as in ao_amd_int4wo_rmsnorm_linear.  The consumer adds the parts and rounds
+ * (ao_amd_llama_decode_attention_parts); no cross-workgroup reduction, no scratch memory.  Decode shapes only (M <= 16).
+ * Same product as ao_amd_int4wo_linear (`aten::_weight_int4pack_mm`, affine_quantized_tensor.py:600-640), summed in
+ * another order. */
+int ao_amd_int4wo_linear_partials(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* norm_weight_bf16,
+                                  float eps, const void* packed, const void* qparams, int64_t N, int64_t g, int ksplit,
+                                  void* y_f32_parts, int64_t ldy, void* stream);
+
 /* SwiGLU over ONE interleaved weight: `ao_amd_int4wo_interleave_pair` permutes two packed weights of the same shape
  * (N a multiple of 16) into a packed weight of 2N rows whose 16-row blocks hold 8 gate rows followed by the 8 up rows of
  * the same outputs (buffers sized by ao_amd_int4wo_packed_shape(2N, K, g)); `ao_amd_int4wo_swiglu_interleaved` computes
@@ -189,6 +199,12 @@ int ao_amd_rmsnorm_bf16(const void* x, const void* weight, int64_t rows, int64_t
 int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* freqs_cis_bf16, const int32_t* pos_dev,
                                   void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim, int64_t max_seq,
                                   void* out_bf16, void* stream);
+
+/* The same step reading the fused qkv row as `nparts` fp32 partial rows [nparts][(n_head + 2 n_kv) * head_dim] that it adds
+ * and rounds to bf16 itself: the output of ao_amd_int4wo_linear_partials, which splits K across workgroups. */
+int ao_amd_llama_decode_attention_parts(const void* qkv_f32_parts, int nparts, const void* freqs_cis_bf16,
+                                        const int32_t* pos_dev, void* k_cache, void* v_cache, int n_head, int n_kv,
+                                        int head_dim, int64_t max_seq, void* out_bf16, void* stream);
 
 /* out_index[0] = index of the largest of n bf16 values (lowest index among equals; NaN counts as largest): the greedy
  * branch of `sample` in the decode harness, torch.argmax over the last position's logits

@@ -316,3 +316,52 @@ def test_fused_decode_step_int8_weight_only():
     a = generate(model, prompt, 10, use_graph=True, greedy=True)
     b = generate(model, prompt, 10, use_graph=False, greedy=True)
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("ksplit", [1, 2, 3])
+@pytest.mark.parametrize("M,N,K,g", [(1, 6144, 4096, 64), (1, 512, 1024, 128), (5, 256, 2048, 32)])
+def test_linear_partials_sum_to_the_linear(M, N, K, g, ksplit):
+    """K split over workgroups: the fp32 partial rows add up to the unsplit fp32 result (another summation order:
+    1e-5 relative), with and without the fused RMSNorm; an uneven split (3 over 8 or 32 tiles) included."""
+    from ao_amd import ops
+
+    dev = _dev()
+    w = make_weight(N, K, seed=101).to(dev)
+    x = (make_act(M, K, seed=102) * 2).to(dev)
+    nw = (1 + 0.1 * torch.randn(K, generator=torch.Generator().manual_seed(103))).bfloat16().to(dev)
+    packed, qp = ops.int4wo_quantize_pack(w, g)
+    parts = ops.int4wo_linear_partials(x, packed, qp, g, N, ksplit)
+    assert parts.shape == (ksplit, M, N) and parts.dtype is torch.float32
+    full = ops.int4wo_linear(x, packed, qp, g, N, None, True)
+    assert rel_l2(parts.sum(0).cpu().numpy(), full.cpu().numpy()) <= 1e-5
+    parts_n = ops.int4wo_linear_partials(x, packed, qp, g, N, ksplit, nw, 1e-5)
+    full_n = ops.int4wo_linear(ops.rmsnorm(x, nw, 1e-5), packed, qp, g, N, None, True)
+    assert rel_l2(parts_n.sum(0).cpu().numpy(), full_n.cpu().numpy()) <= 1e-3
+
+
+def test_decode_attention_from_partial_rows():
+    """fp32 partial qkv rows are added and rounded to bf16 inside the attention kernel: same result as handing it the
+    rounded sum."""
+    from ao_amd import ops
+
+    dev = _dev()
+    n_head, n_kv, hd, S = 8, 2, 128, 64
+    gen = torch.Generator().manual_seed(5)
+    parts = torch.randn(2, 1, (n_head + 2 * n_kv) * hd, generator=gen).to(dev)
+    qkv = parts.sum(0).bfloat16()
+    freqs = torch.randn(S, hd // 2, 2, generator=gen).bfloat16().to(dev)
+    pos = torch.tensor([9], dtype=torch.int32, device=dev)
+    caches = [torch.randn(1, n_kv, S, hd, generator=gen).bfloat16().to(dev) for _ in range(2)]
+    k1, v1 = caches[0].clone(), caches[1].clone()
+    k2, v2 = caches[0].clone(), caches[1].clone()
+    a = ops.llama_decode_attention(qkv, freqs, pos, k1, v1, n_head, n_kv)
+    b = ops.llama_decode_attention(parts, freqs, pos, k2, v2, n_head, n_kv)
+    assert torch.equal(a, b) and torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
+def test_qkv_split_rule():
+    from ao_amd._models.llama.model import Transformer
+
+    assert Transformer.qkv_ksplit(6144) == 2       # Llama-3-8B: 384 row blocks on 256 CUs
+    assert Transformer.qkv_ksplit(4096) == 1 and Transformer.qkv_ksplit(12288) == 1 and Transformer.qkv_ksplit(512) == 1
+    assert Transformer.qkv_ksplit(2048) == 2       # half of the CUs idle otherwise
