@@ -260,8 +260,8 @@ class Transformer(nn.Module):
         from ... import ops
 
         g, u = ff.w1.weight.layout_tensor, ff.w3.weight.layout_tensor
-        key = (g.packed_weight.data_ptr(), u.packed_weight.data_ptr(), g.scale_and_zero.data_ptr(),
-               u.scale_and_zero.data_ptr())
+        srcs = (g.packed_weight, u.packed_weight, g.scale_and_zero, u.scale_and_zero)
+        key = tuple((t.data_ptr(), t._version) for t in srcs)
         cached = getattr(ff, "_gate_up_pair_cache", None)
         if cached is None or cached[0] != key:
             pair, pair_q = ops.int4wo_interleave_pair(g.packed_weight, g.scale_and_zero, u.packed_weight,
