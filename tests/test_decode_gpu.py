@@ -365,3 +365,49 @@ def test_qkv_split_rule():
     assert Transformer.qkv_ksplit(6144) == 2       # Llama-3-8B: 384 row blocks on 256 CUs
     assert Transformer.qkv_ksplit(4096) == 1 and Transformer.qkv_ksplit(12288) == 1 and Transformer.qkv_ksplit(512) == 1
     assert Transformer.qkv_ksplit(2048) == 2       # half of the CUs idle otherwise
+
+
+@pytest.mark.parametrize("g", [32, 64, 128, 256])
+@pytest.mark.parametrize("N,K", [(8192, 512), (8192 + 16, 1024), (28672, 4096), (16384 + 48, 256)])
+def test_single_row_over_many_row_blocks(N, K, g):
+    """Large row counts (two and more row blocks per CU, ragged last block) at M = 1 against the same product at
+    M = 2, whose second row takes another staging path and wave count: 1e-5 relative in fp32; bf16 outputs with bias
+    and residual identical but for rare boundary roundings."""
+    from ao_amd import ops
+
+    if K % max(128, g):
+        pytest.skip("K must be a multiple of max(128, group)")
+    print(f"case many row blocks N={N} K={K} g={g}", flush=True)
+    dev = _dev()
+    w = make_weight(N, K, seed=111 + g).to(dev)
+    x = make_act(2, K, seed=112).to(dev)
+    x[1] = x[0]
+    packed, qp = ops.int4wo_quantize_pack(w, g)
+    y1 = ops.int4wo_linear(x[:1], packed, qp, g, N, None, True)
+    y2 = ops.int4wo_linear(x, packed, qp, g, N, None, True)
+    assert rel_l2(y1.cpu().numpy(), y2[:1].cpu().numpy()) <= 1e-5
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(113)) * 0.1).bfloat16().to(dev)
+    res = make_act(2, N, seed=114).to(dev)
+    res[1] = res[0]
+    z1 = ops.int4wo_linear_residual(x[:1], packed, qp, g, N, res[:1], bias).float().cpu().numpy()
+    z2 = ops.int4wo_linear_residual(x, packed, qp, g, N, res, bias)[:1].float().cpu().numpy()
+    assert rel_l2(z1, z2) <= 1e-3 and np.count_nonzero(z1 != z2) <= 0.01 * z1.size
+
+
+def test_single_row_many_row_blocks_one_hot_is_exact(oracle):
+    """One-hot activation over a weight with many row blocks: every output is a single dequantized weight, bit for
+    bit the oracle's dequantize_affine."""
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K, g = 8192 + 32, 512, 64
+    w = make_weight(N, K, seed=121)
+    packed, qp = ops.int4wo_quantize_pack(w.to(dev), g)
+    codes, scale, zero = oracle.int4wo_quantize(bits16(w), oracle.BF16, g, N, K)
+    dq = oracle.bf16_bits_to_f32(oracle.dequantize_affine(codes, oracle.I32, (1, g), scale, oracle.BF16, zero,
+                                                          oracle.BF16, 0, 15, 1, oracle.BF16))
+    for k in (0, 33, 127, 128, 300, 511):
+        x = torch.zeros(1, K, dtype=torch.bfloat16)
+        x[0, k] = 1.0
+        y = ops.int4wo_linear(x.to(dev), packed, qp, g, N, None, True).cpu().numpy()
+        assert np.array_equal(y[0], dq[:, k]), k
