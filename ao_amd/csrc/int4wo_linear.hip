@@ -475,8 +475,14 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     const uint32_t qoff = (uint32_t)(r + (G < 128 ? (qd * 32 / G) * 16 : 0)) * 4;
     auto tile_group_bytes = [&](int kb) -> int { return (G <= 128 ? kb * (128 / G) : kb / (G / 128)) * 64; };
 
+    // MFMA row r multiplies activation row m0 + r: lanes of live rows read their 64 bytes of the staged row per tile,
+    // lanes of rows past M read the same 64 zero bytes each time (no branch or exec masking in the tile loop)
+    __shared__ __align__(16) uint4 zero_s[4];
+    if (threadIdx.x < 4) zero_s[threadIdx.x] = make_uint4(0, 0, 0, 0);
     const bool xact = (m0 + r) < a.M;
-    const uint16_t* xs_lane = xs + (int64_t)r * a.Kp + qd * 32;
+    const char* xs_lane = xact ? reinterpret_cast<const char*>(xs + (int64_t)r * a.Kp + qd * 32)
+                               : reinterpret_cast<const char*>(zero_s);
+    const int xs_step = xact ? 256 : 0;  // bytes per K tile
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     f32x4_t acc2 = {0.f, 0.f, 0.f, 0.f};
 
@@ -490,8 +496,6 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     };
 
     uint4 xl[4];
-#pragma unroll
-    for (int sl = 0; sl < 4; ++sl) xl[sl] = make_uint4(0, 0, 0, 0);  // rows >= M stay zero
     constexpr int LPT = DUAL ? 4 : 2;  // loads per tile
     u32x4_t tcur = {0, 0, 0, 0};  // stage-1 result of the dword that enters stage 2 next
     GroupRegs gnext;              // group constants of the tile whose dword 0 is in tcur
@@ -499,8 +503,8 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     gnext.zz = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     auto compute_tile = [&](const GemvTile& b, int kb, const GemvTile& nb, bool has_next, int younger_of_next) {
-        if (xact) {
-            const uint4* xv = reinterpret_cast<const uint4*>(xs_lane + kb * 128);
+        {
+            const uint4* xv = reinterpret_cast<const uint4*>(xs_lane + kb * xs_step);
 #pragma unroll
             for (int sl = 0; sl < 4; ++sl) xl[sl] = xv[sl];
         }
@@ -648,7 +652,18 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
         gnext = make_group_asm(buf[0].q);
         tcur = first_half(buf[0].w.x, gnext.g, magic);
     }
-    for (int i0 = 0; i0 < nt; i0 += D) {
+    int i0 = 0;
+    // steady state: every tile of the group has a tile D-1 ahead to request, so the waits are compile-time counts
+    // and nothing in the group is conditional
+    for (; i0 + 2 * D - 1 <= nt; i0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            load_tile(buf[(j + D - 1) % D], kb0 + (i0 + j + D - 1) * WAVES);
+            wait_tiles<LPT>(D - 1);
+            compute_tile(buf[j], kb0 + (i0 + j) * WAVES, buf[(j + 1) % D], true, D - 2);
+        }
+    }
+    for (; i0 < nt; i0 += D) {
 #pragma unroll
         for (int j = 0; j < D; ++j) {
             const int i = i0 + j;
