@@ -301,8 +301,10 @@ class Transformer(nn.Module):
             pair, pair_q, group, n_ff = self._gate_up_pair(b.feed_forward)
             ff = ops.int4wo_swiglu_interleaved(h, pair, pair_q, group, n_ff, b.ffn_norm.weight, b.ffn_norm.eps)
             x = lin(ff, b.feed_forward.w2, residual=h)
-        xn = ops.rmsnorm(x, self.norm.weight, self.norm.eps)
-        return lin(xn, self.output).view(1, 1, cfg.vocab_size)
+        ow = self.output.weight.layout_tensor
+        logits = ops.int4wo_rmsnorm_linear(x, self.norm.weight, self.norm.eps, ow.packed_weight, ow.scale_and_zero,
+                                           ow.group_size, ow.N)
+        return logits.view(1, 1, cfg.vocab_size)
 
     def _fused_decode_int8(self, idx: Tensor, input_pos: Tensor) -> Tensor:
         """The same step over int8 weight-only linears: the streaming int8 kernel per linear, the RMSNorm and decode

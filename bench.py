@@ -69,7 +69,7 @@ class KernelTimer:
 
 def roofline_leg(model, passes=3):
     """Time the GEMV kernel alone over the linear launches of one decoded token (M=1), `passes` times: per layer
-    norm + wqkv, wo + residual, norm + gate/up SwiGLU over the interleaved pair, w2 + residual, then the head:
+    norm + wqkv, wo + residual, norm + gate/up SwiGLU over the interleaved pair, w2 + residual, then norm + head:
     the same entry points, weights and order as the decode step, 4 * n_layer + 1 launches."""
     import torch
 
@@ -128,7 +128,7 @@ def roofline_leg(model, passes=3):
         fn, y = plain(lay, xf, residual=res)
         add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(y)
     lay = model.output.weight.layout_tensor
-    fn, y = plain(lay, x)
+    fn, y = plain(lay, x, norm=model.norm)
     add(fn, int4wo_bytes(lay.N, lay.K, lay.group_size)); keep.append(y)
 
     timer = KernelTimer(len(launches))
