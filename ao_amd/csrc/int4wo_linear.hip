@@ -997,12 +997,15 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16 && !gemm_starved) {
         // 128 x 128 workgroup tiles when they fill a good part of the 256 CUs, else 64 x 64 tiles: four times
         // the workgroups, each dequantizing for 64 activation rows only
+        // ... and 32 x 64 tiles when even those leave CUs idle
         const bool big = ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
+        const bool tiny = !big && gemm_small_wgs < 192;
         dim3 ggrid(big ? (unsigned)((RB + 7) / 8) : (unsigned)((RB + 3) / 4),
-                   big ? (unsigned)((M + 127) / 128) : (unsigned)((M + 63) / 64));
+                   big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64));
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
 #define AO_GEMM_LAUNCH(GG)                                                                        \
     if (big) launch_timed(int4wo_gemm_kernel<GG, 2, 8>, ggrid, dim3(256), 0, st, a);              \
+    else if (tiny) launch_timed(int4wo_gemm_kernel<GG, 1, 2>, ggrid, dim3(256), 0, st, a);        \
     else launch_timed(int4wo_gemm_kernel<GG, 1, 4>, ggrid, dim3(256), 0, st, a)
         switch (g) {
             case 32: AO_GEMM_LAUNCH(32); break;
