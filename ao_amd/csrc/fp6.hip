@@ -548,15 +548,19 @@ extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const 
     g_prof_start = g_prof_stop = nullptr;
     // tiled kernel: 128 x 128 workgroup tiles when they give at least one workgroup per CU, else 64 x 64
     if (M > 16 && K % 128 == 0) {
+        // ... and 32 x 64 tiles when even those leave CUs idle
         const bool big = ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
+        const bool tiny = !big && ((RB + 3) / 4) * ((M + 63) / 64) < 192;
         dim3 ggrid(big ? (unsigned)((RB + 7) / 8) : (unsigned)((RB + 3) / 4),
-                   big ? (unsigned)((M + 127) / 128) : (unsigned)((M + 63) / 64));
+                   big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64));
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
         if (ebits == 3) {
             if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 2, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 2>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
             else hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
         } else {
             if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 2, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 2>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
             else hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
         }
         AO_LAUNCH_CHECK();
