@@ -308,13 +308,17 @@ class Transformer(nn.Module):
 
     def _fused_decode_int8(self, idx: Tensor, input_pos: Tensor) -> Tensor:
         """The same step over int8 weight-only linears: the streaming int8 kernel per linear, the RMSNorm and decode
-        attention kernels, and the module's own elementwise ops (residual add, SiLU * up) in between."""
+        attention kernels, with the residual add and the SiLU(gate) * up product fused into the linear that precedes them."""
         from ... import ops
 
         cfg = self.config
 
-        def lin(x, layer):
+        def lin(x, layer, residual=None, gate=None):
             lay = layer.weight.layout_tensor
+            if residual is not None:
+                return ops.int8wo_linear_residual(x, lay.int_data, lay.scale.reshape(-1), residual)
+            if gate is not None:
+                return ops.int8wo_linear_gated(x, lay.int_data, lay.scale.reshape(-1), gate)
             return ops.int8wo_linear(x, lay.int_data, lay.scale.reshape(-1))
 
         x = self.tok_embeddings(idx).view(1, cfg.dim)
@@ -324,9 +328,9 @@ class Transformer(nn.Module):
             qkv = lin(ops.rmsnorm(x, b.attention_norm.weight, b.attention_norm.eps), att.wqkv)
             y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
                                            cfg.n_head, cfg.n_local_heads)
-            h = x + lin(y, att.wo)
+            h = lin(y, att.wo, residual=x)
             hn = ops.rmsnorm(h, b.ffn_norm.weight, b.ffn_norm.eps)
-            x = h + lin(F.silu(lin(hn, ffn.w1)) * lin(hn, ffn.w3), ffn.w2)
+            x = lin(lin(hn, ffn.w3, gate=lin(hn, ffn.w1)), ffn.w2, residual=h)
         return lin(ops.rmsnorm(x, self.norm.weight, self.norm.eps), self.output).view(1, 1, cfg.vocab_size)
 
     def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None) -> Tensor:

@@ -37,6 +37,8 @@ struct Int8Args {
     const uint16_t* bias;
     int64_t N;
     void* y; int y_is_f32; int64_t ldy;
+    const uint16_t* residual; int64_t ldres;  // y = bf16(result) + residual, or null
+    const uint16_t* gate; int64_t ldgate;     // y = silu(gate) * bf16(result) (SwiGLU with the gate already computed), or null
 };
 
 // One workgroup = one 16-row block of W and one chunk of 16 activation rows; its WAVES waves take the 128-wide
@@ -110,6 +112,12 @@ __global__ __launch_bounds__(WAVES * 64) void int8wo_linear_kernel(const Int8Arg
                     // mm result rounded to bf16, times scale rounded to bf16, plus bias rounded to bf16
                     float v = hw_rne_bf16(s) * sc;
                     if (a.bias) v = hw_rne_bf16(v) + bv;
+                    // the module's next elementwise op on the bf16 result, fused: h + linear(...) or silu(w1 x) * linear(...)
+                    if (a.residual) v = hw_rne_bf16(v) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
+                    if (a.gate) {
+                        const float gt = bf16_bits_to_f32(a.gate[m * a.ldgate + n]);
+                        v = hw_rne_bf16(gt / (1.0f + expf(-gt))) * hw_rne_bf16(v);
+                    }
                     if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = v;
                     else ((uint16_t*)a.y)[m * a.ldy + n] = hw_bf16_bits(v);
                 }
@@ -149,10 +157,14 @@ static void launch_int8(dim3 grid, hipStream_t st, const Int8Args& a) {
 
 using namespace ao;
 
-extern "C" int ao_amd_int8wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* w_int8, int64_t ldw,
-                                    const void* scale_bf16, int64_t N, const void* bias_bf16, void* y, int y_dtype,
-                                    int64_t ldy, void* stream) {
+static int int8wo_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* w_int8, int64_t ldw,
+                           const void* scale_bf16, int64_t N, const void* bias_bf16, void* y, int y_dtype, int64_t ldy,
+                           const void* residual_bf16, int64_t ldres, const void* gate_bf16, int64_t ldgate, void* stream) {
     AO_REQUIRE(x_bf16 && w_int8 && scale_bf16 && y, "null pointer argument");
+    AO_REQUIRE(!(residual_bf16 && gate_bf16), "residual and gate epilogues are exclusive");
+    AO_REQUIRE((!residual_bf16 || ldres >= N) && (!gate_bf16 || ldgate >= N), "epilogue operand rows shorter than N=%lld",
+               (long long)N);
+    AO_REQUIRE(!(residual_bf16 || gate_bf16) || y_dtype == AO_BF16, "fused epilogues produce bf16");
     AO_REQUIRE(M >= 0 && N > 0 && K > 0, "bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
     AO_REQUIRE(y_dtype == AO_BF16 || y_dtype == AO_F32, "output dtype must be bf16 or f32, got code %d", y_dtype);
     AO_REQUIRE(K % 128 == 0, "int8 weight-only linear needs in_features to be a multiple of 128, got %lld", (long long)K);
@@ -166,7 +178,8 @@ extern "C" int ao_amd_int8wo_linear(const void* x_bf16, int64_t M, int64_t K, in
     int waves = 1;
     while (waves < 16 && RB * mchunks * waves * 2 <= 4096 + RB * mchunks && waves * 2 <= KB) waves *= 2;
     Int8Args a{(const uint16_t*)x_bf16, M, K, ldx, (const int8_t*)w_int8, ldw, (const uint16_t*)scale_bf16,
-               (const uint16_t*)bias_bf16, N, y, y_dtype == AO_F32, ldy};
+               (const uint16_t*)bias_bf16, N, y, y_dtype == AO_F32, ldy, (const uint16_t*)residual_bf16, ldres,
+               (const uint16_t*)gate_bf16, ldgate};
     dim3 grid((unsigned)RB, (unsigned)mchunks);
     hipStream_t st = (hipStream_t)stream;
     switch (waves) {
@@ -178,6 +191,29 @@ extern "C" int ao_amd_int8wo_linear(const void* x_bf16, int64_t M, int64_t K, in
     }
     AO_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" int ao_amd_int8wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* w_int8, int64_t ldw,
+                                    const void* scale_bf16, int64_t N, const void* bias_bf16, void* y, int y_dtype,
+                                    int64_t ldy, void* stream) {
+    return int8wo_dispatch(x_bf16, M, K, ldx, w_int8, ldw, scale_bf16, N, bias_bf16, y, y_dtype, ldy, nullptr, 0, nullptr, 0,
+                           stream);
+}
+
+extern "C" int ao_amd_int8wo_linear_residual(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* w_int8,
+                                             int64_t ldw, const void* scale_bf16, int64_t N, const void* residual_bf16,
+                                             int64_t ldres, void* y_bf16, int64_t ldy, void* stream) {
+    AO_REQUIRE(residual_bf16, "null pointer argument");
+    return int8wo_dispatch(x_bf16, M, K, ldx, w_int8, ldw, scale_bf16, N, nullptr, y_bf16, AO_BF16, ldy, residual_bf16, ldres,
+                           nullptr, 0, stream);
+}
+
+extern "C" int ao_amd_int8wo_linear_gated(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* w_int8,
+                                          int64_t ldw, const void* scale_bf16, int64_t N, const void* gate_bf16,
+                                          int64_t ldgate, void* y_bf16, int64_t ldy, void* stream) {
+    AO_REQUIRE(gate_bf16, "null pointer argument");
+    return int8wo_dispatch(x_bf16, M, K, ldx, w_int8, ldw, scale_bf16, N, nullptr, y_bf16, AO_BF16, ldy, nullptr, 0, gate_bf16,
+                           ldgate, stream);
 }
 
 extern "C" int ao_amd_int8_to_bf16(const void* w_int8, int64_t N, int64_t K, int64_t ldw, void* out_bf16, void* stream) {

@@ -49,6 +49,7 @@ _LIB.define("int4wo_linear_partials(Tensor x, Tensor? norm_weight, float eps, Te
 _LIB.define("int4wo_interleave_pair(Tensor packed_gate, Tensor qparams_gate, Tensor packed_up, Tensor qparams_up, int N, int K, int group_size) -> (Tensor, Tensor)")
 _LIB.define("int4wo_swiglu_interleaved(Tensor x, Tensor? norm_weight, float eps, Tensor packed_pair, Tensor qparams_pair, int group_size, int N) -> Tensor")
 _LIB.define("int8wo_linear(Tensor x, Tensor w_int8, Tensor scale, Tensor? bias, bool fp32_out) -> Tensor")
+_LIB.define("int8wo_linear_fused(Tensor x, Tensor w_int8, Tensor scale, Tensor other, bool gated) -> Tensor")
 _LIB.define("hqq_dequantize(Tensor packed_2xint4, Tensor scales, Tensor zeros, int group_size) -> Tensor")
 _LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
 _LIB.define("argmax_bf16(Tensor x) -> Tensor")
@@ -241,6 +242,28 @@ def _int8wo_linear_cuda(x, w_int8, scale, bias, fp32_out):
     check(lib().ao_amd_int8wo_linear(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, w_int8.data_ptr(),
                                      w_int8.stride(0), scale.data_ptr(), N, None if bias is None else bias.data_ptr(),
                                      y.data_ptr(), F32 if fp32_out else BF16, N, current_stream(x.device)))
+    return y
+
+
+def _int8wo_linear_fused_cuda(x, w_int8, scale, other, gated):
+    """bf16(linear) + other (gated = False) or silu(other) * bf16(linear) (gated = True) in one launch."""
+    require_cuda(x, w_int8, scale, other)
+    torch._check(x.dim() == 2 and x.dtype is torch.bfloat16, lambda: "input must be a 2d bfloat16 tensor")
+    torch._check(w_int8.dim() == 2 and w_int8.dtype is torch.int8 and w_int8.stride(1) == 1,
+                 lambda: "weight must be a 2d int8 tensor with unit inner stride")
+    M, K = x.shape
+    N = w_int8.shape[0]
+    torch._check(w_int8.shape[1] == K, lambda: f"weight in_features {w_int8.shape[1]} != input features {K}")
+    torch._check(scale.dtype is torch.bfloat16 and scale.numel() == N, lambda: "scale must be bfloat16 of size N")
+    torch._check(other.dtype is torch.bfloat16 and tuple(other.shape) == (M, N) and other.stride(1) == 1,
+                 lambda: "the fused operand must be a bfloat16 [M, N] tensor with unit inner stride")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    scale = scale.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    fn = lib().ao_amd_int8wo_linear_gated if gated else lib().ao_amd_int8wo_linear_residual
+    check(fn(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, w_int8.data_ptr(), w_int8.stride(0), scale.data_ptr(), N,
+             other.data_ptr(), other.stride(0) if M > 0 else N, y.data_ptr(), N, current_stream(x.device)))
     return y
 
 
@@ -510,6 +533,7 @@ _LIB.impl("int4wo_linear_partials", _linear_partials_cuda, "CUDA")
 _LIB.impl("int4wo_interleave_pair", _interleave_pair_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu_interleaved", _swiglu_interleaved_cuda, "CUDA")
 _LIB.impl("int8wo_linear", _int8wo_linear_cuda, "CUDA")
+_LIB.impl("int8wo_linear_fused", _int8wo_linear_fused_cuda, "CUDA")
 _LIB.impl("hqq_dequantize", _hqq_dequantize_cuda, "CUDA")
 _LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
 _LIB.impl("llama_decode_attention", _decode_attention_cuda, "CUDA")
@@ -529,7 +553,7 @@ def _no_cpu(name):
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
               "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int4wo_linear_partials", "int4wo_interleave_pair",
-              "int4wo_swiglu_interleaved", "int8wo_linear", "hqq_dequantize", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
+              "int4wo_swiglu_interleaved", "int8wo_linear", "int8wo_linear_fused", "hqq_dequantize", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
               "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
@@ -604,6 +628,11 @@ def _(packed_gate, qparams_gate, packed_up, qparams_up, N, K, group_size):
 @torch.library.register_fake("torchao::int4wo_swiglu_interleaved")
 def _(x, norm_weight, eps, packed_pair, qparams_pair, group_size, N):
     return x.new_empty((x.shape[0], N), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::int8wo_linear_fused")
+def _(x, w_int8, scale, other, gated):
+    return x.new_empty((x.shape[0], w_int8.shape[0]), dtype=torch.bfloat16)
 
 
 @torch.library.register_fake("torchao::int8wo_linear")
@@ -747,6 +776,16 @@ def int8wo_linear(x: Tensor, w_int8: Tensor, scale: Tensor, bias=None, fp32_out:
 def hqq_dequantize(packed_2xint4: Tensor, scales: Tensor, zeros: Tensor, group_size: int) -> Tensor:
     """HQQ two-per-byte codes [K/2, N] -> (q - zero) * scale as a [K, N] matrix in the dtype of the scales."""
     return torch.ops.torchao.hqq_dequantize.default(packed_2xint4, scales, zeros, group_size)
+
+
+def int8wo_linear_residual(x: Tensor, w_int8: Tensor, scale: Tensor, residual: Tensor) -> Tensor:
+    """bf16(int8wo_linear(x)) + residual in one launch."""
+    return torch.ops.torchao.int8wo_linear_fused.default(x, w_int8, scale, residual, False)
+
+
+def int8wo_linear_gated(x: Tensor, w_int8: Tensor, scale: Tensor, gate: Tensor) -> Tensor:
+    """silu(gate) * bf16(int8wo_linear(x)) in one launch (SwiGLU with the gate projection already computed)."""
+    return torch.ops.torchao.int8wo_linear_fused.default(x, w_int8, scale, gate, True)
 
 
 def rmsnorm(x, weight, eps: float):

@@ -182,6 +182,17 @@ int ao_amd_int8wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, 
                          const void* scale_bf16, int64_t N, const void* bias_bf16, void* y, int y_dtype, int64_t ldy,
                          void* stream);
 
+/* The same linear with the module's next elementwise op on its bf16 result fused into the epilogue, for the decode step:
+ * `_residual`: y = bf16(linear) + residual (h + attention(...) and h + feed_forward(...), TransformerBlock.forward,
+ * torchao/_models/llama/model.py:160-163); `_gated`: y = bf16(silu(gate)) * bf16(linear) with the gate projection already
+ * computed (F.silu(self.w1(x)) * self.w3(x), FeedForward.forward, model.py:209-214).  bf16 output, no bias. */
+int ao_amd_int8wo_linear_residual(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* w_int8, int64_t ldw,
+                                  const void* scale_bf16, int64_t N, const void* residual_bf16, int64_t ldres,
+                                  void* y_bf16, int64_t ldy, void* stream);
+int ao_amd_int8wo_linear_gated(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* w_int8, int64_t ldw,
+                               const void* scale_bf16, int64_t N, const void* gate_bf16, int64_t ldgate, void* y_bf16,
+                               int64_t ldy, void* stream);
+
 /* bf16 copy of the int8 codes (`w_int8.to(x.dtype)` of the same formula) for prefill-sized batches: the caller then
  * runs a plain bf16 GEMM on it and multiplies by the scale.  K a multiple of 16, 16-byte aligned rows. */
 int ao_amd_int8_to_bf16(const void* w_int8, int64_t N, int64_t K, int64_t ldw, void* out_bf16, void* stream);

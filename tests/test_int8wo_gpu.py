@@ -128,3 +128,23 @@ def test_rejects_bad_arguments(cabi):
     rc = cabi.lib().ao_amd_int8wo_linear(x.data_ptr(), 1, 192, 192, w.data_ptr(), 192, s.data_ptr(), 16, None, y.data_ptr(),
                                          cabi.BF16, 16, None)
     assert rc != 0 and b"multiple of 128" in cabi.lib().ao_amd_last_error()
+
+
+@pytest.mark.parametrize("M", [1, 3, 16])
+def test_fused_epilogues_match_the_module_chain(M):
+    """residual add and SiLU(gate) * up fused into the linear: identical to the separate bf16 ops but for rare
+    elements where the device's expf differs from torch's by an ulp."""
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K = 512, 1024
+    gen = torch.Generator().manual_seed(77)
+    q = torch.randint(-127, 128, (N, K), generator=gen, dtype=torch.int8).to(dev)
+    s = (torch.rand(N, generator=gen) * 1e-3 + 1e-4).bfloat16().to(dev)
+    x = make_act(M, K, seed=78).to(dev)
+    other = make_act(M, N, seed=79).to(dev)
+    y = ops.int8wo_linear(x, q, s)
+    assert torch.equal(ops.int8wo_linear_residual(x, q, s, other), other + y)
+    got = ops.int8wo_linear_gated(x, q, s, other).float().cpu().numpy()
+    want = (torch.nn.functional.silu(other) * y).float().cpu().numpy()
+    assert np.count_nonzero(got != want) <= 0.002 * got.size + 1 and rel_l2(got, want) <= 1e-3
