@@ -280,15 +280,30 @@ __global__ __launch_bounds__(256) void int4wo_quantize_pack_kernel(const uint16_
         const float s = (!(s0 >= epsv) && s0 == s0) ? epsv : s0;
         // quantize_affine, FLOAT domain (quant_primitives.py:195-203)
         const float mv = rne_bf16(zp - rne_bf16(s * 8.0f));
+        // bf16((w - mv) / s): the quotient is only needed to bf16 precision, so it is first formed as (w - mv) * rcp(s)
+        // (within 3 fp32 ulp of the correctly rounded fp32 quotient) and rounded to bf16; that is the reference's
+        // result unless the approximate quotient lies within 4 fp32 ulp of a bf16 rounding boundary (low 16 bits near
+        // 0x8000), in which case the dword is redone with the IEEE division.  About 1 % of the dwords take that path.
+        const float rs = __builtin_amdgcn_rcpf(s);
         uint32_t words[4];
 #pragma unroll
         for (int sl = 0; sl < 4; ++sl) {
+            float tq[8];
+            bool risky = false;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float t = hw_rne_bf16(v[ss][sl][e] - mv);
+                tq[e] = t * rs;
+                risky |= ((__float_as_uint(tq[e]) & 0xffffu) - 0x7ffcu) <= 8u;
+            }
+            if (__any(risky)) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) tq[e] = __fdiv_rn(hw_rne_bf16(v[ss][sl][e] - mv), s);
+            }
             uint32_t word = 0;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                float t = rne_bf16(v[ss][sl][e] - mv);
-                t = rne_bf16(__fdiv_rn(t, s));
-                float q = __builtin_rintf(t);
+                float q = __builtin_rintf(hw_rne_bf16(tq[e]));
                 q = q < 0.f ? 0.f : (q > 15.f ? 15.f : q);
                 if (q != q) q = 0.f;
                 word |= (uint32_t)(int)q << (4 * nib_pos(e));
