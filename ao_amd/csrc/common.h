@@ -96,6 +96,40 @@ __device__ __forceinline__ uint32_t hw_bf16_pack(float lo, float hi) {
     return u;
 }
 
+// Cross-lane reductions on the VALU's data-parallel-primitive path instead of ds_bpermute (an LDS round trip per
+// step): DPP control words for gfx9: quad_perm [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E, row_half_mirror = 0x141 (lane i <-> 7-i
+// of each 8), row_mirror = 0x140 (lane i <-> 15-i of each 16).  After the four steps every lane of a 16-lane row holds
+// the row's total; the four rows of a wave are then combined through v_readlane.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    v += dpp_move<0x140>(v);
+    return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_move<0xB1>(v));
+    v = fmaxf(v, dpp_move<0x4E>(v));
+    v = fmaxf(v, dpp_move<0x141>(v));
+    v = fmaxf(v, dpp_move<0x140>(v));
+    return v;
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = row16_max(v);
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
+}
+
 __device__ __forceinline__ bool is_float_dt(int d) { return d == AO_F32 || d == AO_BF16 || d == AO_F16; }
 __device__ __forceinline__ int promote(int a, int b) {
     if (!is_float_dt(a)) return b;

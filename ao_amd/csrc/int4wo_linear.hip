@@ -605,8 +605,7 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
             return make_uint4(o[0], o[1], o[2], o[3]);
         };
         auto block_sum = [&](float ss) {  // the same total in every thread; one barrier
-#pragma unroll
-            for (int o = 32; o >= 1; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            ss = wave_sum(ss);
             if (lane == 0) norm_part[wave] = ss;
             __syncthreads();
             float tot = 0.f;

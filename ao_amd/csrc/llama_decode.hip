@@ -9,17 +9,6 @@
 
 namespace ao {
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
-}
-
 // out = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * w ), statistics in fp32.  One workgroup per row.
 // VEC: dim is a multiple of 8 and the rows are 16-byte aligned; every thread then issues all of its
 // 16-byte loads (up to 4 chunks, dim <= 8192) before the first use so the row is read in one round trip.
@@ -118,8 +107,8 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     float* knew_s = smem + HD;     // [128] rotated new k
     float* vnew_s = smem + 2 * HD; // [128] new v
     float* red = smem + 3 * HD;    // [32] reductions
-    float* po = red + 32;          // [16][128] per-wave partial outputs
-    float* sc = po + 16 * HD;      // [pos + 1] scores, then probabilities
+    float* po = red + 32;          // [64][128] partial outputs of the 64 position slots
+    float* sc = po + 64 * HD;      // [pos + 1] scores, then probabilities
     const int h = blockIdx.x;
     const int rep = n_head / n_kv;
     const int hk = h / rep;
@@ -211,8 +200,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
                     d += qreg[2 * j + 1] * __uint_as_float(w4[j] & 0xffff0000u);
                 }
             }
-#pragma unroll
-            for (int o = 8; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);
+            d = row16_sum(d);
             d *= scale;
             if (t < T) {
                 if (l16 == 0) sc[t] = d;
@@ -272,21 +260,17 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
             }
         }
     }
-    // fold the 4 position slots of a wave, then the 16 waves
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        oacc[e] += __shfl_xor(oacc[e], 16, 64);
-        oacc[e] += __shfl_xor(oacc[e], 32, 64);
-    }
-    if (sub == 0) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) po[wave * HD + l16 * 8 + e] = oacc[e];
+    // every 16-lane position slot parks its partial output row; 128 threads then add the 64 rows in a fixed order
+    {
+        float4* dst = reinterpret_cast<float4*>(po + rg * HD + l16 * 8);
+        dst[0] = make_float4(oacc[0], oacc[1], oacc[2], oacc[3]);
+        dst[1] = make_float4(oacc[4], oacc[5], oacc[6], oacc[7]);
     }
     __syncthreads();
     if (tid < HD) {
         float o = 0.f;
-#pragma unroll
-        for (int w = 0; w < 16; ++w) o += po[w * HD + tid];
+#pragma unroll 16
+        for (int w = 0; w < 64; ++w) o += po[w * HD + tid];
         out[(int64_t)h * HD + tid] = f32_to_bf16_bits(o * inv);
     }
 }
@@ -396,7 +380,7 @@ extern "C" int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* f
     AO_REQUIRE(head_dim == 128, "decode attention kernel is built for head_dim 128, got %d", head_dim);
     AO_REQUIRE(n_kv > 0 && n_head % n_kv == 0, "n_head=%d must be a multiple of n_kv=%d", n_head, n_kv);
     AO_REQUIRE(max_seq > 0 && max_seq <= 8192, "max_seq=%lld outside (0, 8192]", (long long)max_seq);
-    const size_t smem = (size_t)(3 * 128 + 32 + 16 * 128 + max_seq + 8) * sizeof(float);
+    const size_t smem = (size_t)(3 * 128 + 32 + 64 * 128 + max_seq + 8) * sizeof(float);
     hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head), dim3(ATT_THREADS), smem, (hipStream_t)stream,
                        (const uint16_t*)qkv_bf16, (const float*)nullptr, 0, (const uint16_t*)freqs_cis_bf16, pos_dev,
                        (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16);
@@ -412,7 +396,7 @@ extern "C" int ao_amd_llama_decode_attention_parts(const void* qkv_f32_parts, in
     AO_REQUIRE(head_dim == 128, "decode attention kernel is built for head_dim 128, got %d", head_dim);
     AO_REQUIRE(n_kv > 0 && n_head % n_kv == 0, "n_head=%d must be a multiple of n_kv=%d", n_head, n_kv);
     AO_REQUIRE(max_seq > 0 && max_seq <= 8192, "max_seq=%lld outside (0, 8192]", (long long)max_seq);
-    const size_t smem = (size_t)(3 * 128 + 32 + 16 * 128 + max_seq + 8) * sizeof(float);
+    const size_t smem = (size_t)(3 * 128 + 32 + 64 * 128 + max_seq + 8) * sizeof(float);
     hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head), dim3(ATT_THREADS), smem, (hipStream_t)stream,
                        (const uint16_t*)nullptr, (const float*)qkv_f32_parts, nparts, (const uint16_t*)freqs_cis_bf16,
                        pos_dev, (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16);
