@@ -219,7 +219,7 @@ class Transformer(nn.Module):
         from ...dtypes.affine_quantized_tensor import AffineQuantizedTensor, Gfx950WaveTiledAQTLayout, PlainAQTLayout
 
         if self.freqs_cis is None or self.max_batch_size != 1 or self.config.head_dim != 128 \
-                or self.max_seq_length > 8192 or self.tok_embeddings.weight.dtype is not torch.bfloat16:
+                or self.max_seq_length > 16384 or self.tok_embeddings.weight.dtype is not torch.bfloat16:
             return None
         kinds, groups = set(), set()
         for lin in self._decode_linears():

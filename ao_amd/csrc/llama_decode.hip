@@ -100,7 +100,8 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
                                                                         const int32_t* __restrict__ pos_ptr,
                                                                         uint16_t* __restrict__ k_cache,
                                                                         uint16_t* __restrict__ v_cache, int n_head,
-                                                                        int n_kv, int64_t S, uint16_t* __restrict__ out) {
+                                                                        int n_kv, int64_t S, uint16_t* __restrict__ out,
+                                                                        int nsplit, float* __restrict__ part) {
     constexpr int HD = 128, U = ATT_U;
     extern __shared__ float smem[];
     float* q_s = smem;             // [128] rotated q (bf16-rounded values)
@@ -117,6 +118,13 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     const int rg = wave * 4 + sub;  // row group 0..63
     const int pos = pos_ptr[0];
     const int T = pos + 1;
+    // Long contexts: `nsplit` workgroups per head (blockIdx.y = z) take the 64-position rows z, z + nsplit, ... of
+    // the context, so that any context length spreads evenly over them; each leaves (max, sum, unnormalised output) in
+    // `part` and attention_merge_kernel combines them.  Row `ridx` of this workgroup covers positions
+    // (ridx * nsplit + z) * 64 .. + 63; with nsplit = 1 that is the plain order.
+    const int z = blockIdx.y;
+    auto tpos = [&](int ridx) { return (ridx * nsplit + z) * 64 + rg; };
+    const int nchunk = (T + ATT_CHUNK * nsplit - 1) / (ATT_CHUNK * nsplit);  // chunk iterations of this workgroup
 
     // element i of the fused qkv row: a bf16 value, or the bf16 rounding of the sum of `nparts` fp32 partial rows
     // (a linear whose K range was split across workgroups leaves the last add to its consumer)
@@ -136,7 +144,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     uint4 rawk[U], rawv[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        const int t = u * 64 + rg;
+        const int t = tpos(u);
         rawk[u] = make_uint4(0, 0, 0, 0);
         rawv[u] = make_uint4(0, 0, 0, 0);
         if (t < pos) {
@@ -156,7 +164,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
         float* dst = which ? knew_s : q_s;
         dst[2 * i] = o0;
         dst[2 * i + 1] = o1;
-        if (which && (h % rep) == 0) {
+        if (which && (h % rep) == 0 && z == 0) {
             kc[(int64_t)pos * HD + 2 * i] = f32_to_bf16_bits(o0);
             kc[(int64_t)pos * HD + 2 * i + 1] = f32_to_bf16_bits(o1);
         }
@@ -164,7 +172,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
         const int i = tid - 128;
         const uint16_t v = qkv_at(vp + i);
         vnew_s[i] = bf16_bits_to_f32(v);
-        if ((h % rep) == 0) vc[(int64_t)pos * HD + i] = v;
+        if ((h % rep) == 0 && z == 0) vc[(int64_t)pos * HD + i] = v;
     }
     __syncthreads();
 
@@ -176,18 +184,18 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     }
     const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
     float lmax = -INFINITY;
-    for (int t0 = 0; t0 < T; t0 += ATT_CHUNK) {
-        if (t0 > 0) {
+    for (int c = 0; c < nchunk; ++c) {
+        if (c > 0) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int t = t0 + u * 64 + rg;
+                const int t = tpos(c * U + u);
                 rawk[u] = make_uint4(0, 0, 0, 0);
                 if (t < pos) rawk[u] = *reinterpret_cast<const uint4*>(kc + (int64_t)t * HD + l16 * 8);
             }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int t = t0 + u * 64 + rg;
+            const int t = tpos(c * U + u);
             const uint32_t w4[4] = {rawk[u].x, rawk[u].y, rawk[u].z, rawk[u].w};
             float d = 0.f;
             if (t == pos) {
@@ -202,10 +210,8 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
             }
             d = row16_sum(d);
             d *= scale;
-            if (t < T) {
-                if (l16 == 0) sc[t] = d;
-                lmax = fmaxf(lmax, d);
-            }
+            if (l16 == 0) sc[(c * U + u) * 64 + rg] = t < T ? d : -INFINITY;  // local slot; -inf -> probability 0
+            if (t < T) lmax = fmaxf(lmax, d);
         }
     }
     lmax = wave_max(lmax);
@@ -214,10 +220,11 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     float gmax = red[0];
 #pragma unroll
     for (int w = 1; w < 16; ++w) gmax = fmaxf(gmax, red[w]);
+    const float gsub = gmax == -INFINITY ? 0.f : gmax;  // a workgroup without positions (split mode, short context)
     float lsum = 0.f;
-    for (int t = tid; t < T; t += ATT_THREADS) {
-        const float p = expf(sc[t] - gmax);
-        sc[t] = p;
+    for (int li = tid; li < nchunk * ATT_CHUNK; li += ATT_THREADS) {
+        const float p = expf(sc[li] - gsub);
+        sc[li] = p;
         lsum += p;
     }
     lsum = wave_sum(lsum);
@@ -232,20 +239,20 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     float oacc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) oacc[e] = 0.f;
-    for (int t0 = 0; t0 < T; t0 += ATT_CHUNK) {
-        if (t0 > 0) {
+    for (int c = 0; c < nchunk; ++c) {
+        if (c > 0) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int t = t0 + u * 64 + rg;
+                const int t = tpos(c * U + u);
                 rawv[u] = make_uint4(0, 0, 0, 0);
                 if (t < pos) rawv[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)t * HD + l16 * 8);
             }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int t = t0 + u * 64 + rg;
+            const int t = tpos(c * U + u);
             if (t < T) {
-                const float p = sc[t];
+                const float p = sc[(c * U + u) * 64 + rg];
                 if (t == pos) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) oacc[e] += p * vnew_s[l16 * 8 + e];
@@ -271,8 +278,32 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
         float o = 0.f;
 #pragma unroll 16
         for (int w = 0; w < 64; ++w) o += po[w * HD + tid];
-        out[(int64_t)h * HD + tid] = f32_to_bf16_bits(o * inv);
+        if (nsplit == 1) {
+            out[(int64_t)h * HD + tid] = f32_to_bf16_bits(o * inv);
+        } else {
+            float* dst = part + ((int64_t)h * nsplit + z) * (HD + 2);
+            dst[2 + tid] = o;
+            if (tid == 0) { dst[0] = gmax; dst[1] = tot; }
+        }
     }
+}
+
+// Combines the `nsplit` partial results of one head: out = sum_z e^(m_z - M) o_z / sum_z e^(m_z - M) l_z, M = max_z m_z.
+__global__ __launch_bounds__(128) void attention_merge_kernel(const float* __restrict__ part, int nsplit,
+                                                              uint16_t* __restrict__ out) {
+    constexpr int HD = 128;
+    const int h = blockIdx.x, d = threadIdx.x;
+    const float* p = part + (int64_t)h * nsplit * (HD + 2);
+    float M = -INFINITY;
+    for (int z = 0; z < nsplit; ++z) M = fmaxf(M, p[z * (HD + 2)]);
+    float L = 0.f, o = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+        const float m = p[z * (HD + 2)];
+        const float w = m == -INFINITY ? 0.f : expf(m - M);
+        L += w * p[z * (HD + 2) + 1];
+        o += w * p[z * (HD + 2) + 2 + d];
+    }
+    out[(int64_t)h * HD + d] = f32_to_bf16_bits(o / L);
 }
 
 // Index of the largest of n bf16 values (the lowest such index; a NaN counts as larger than any number), for
@@ -373,35 +404,60 @@ extern "C" int ao_amd_rmsnorm_bf16(const void* x, const void* weight, int64_t ro
     return 0;
 }
 
+static int attention_dispatch(const void* qkv_bf16, const void* qkv_f32_parts, int nparts, const void* freqs_cis_bf16,
+                              const int32_t* pos_dev, void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim,
+                              int64_t max_seq, int nsplit, void* workspace_f32, void* out_bf16, void* stream) {
+    AO_REQUIRE((qkv_bf16 || qkv_f32_parts) && freqs_cis_bf16 && pos_dev && k_cache && v_cache && out_bf16,
+               "null pointer argument");
+    AO_REQUIRE(head_dim == 128, "decode attention kernel is built for head_dim 128, got %d", head_dim);
+    AO_REQUIRE(n_kv > 0 && n_head > 0 && n_head % n_kv == 0, "n_head=%d must be a multiple of n_kv=%d", n_head, n_kv);
+    AO_REQUIRE(max_seq > 0 && max_seq <= 32768, "max_seq=%lld outside (0, 32768]", (long long)max_seq);
+    AO_REQUIRE(nsplit >= 1 && nsplit <= 16, "context split %d outside [1, 16]", nsplit);
+    AO_REQUIRE(nsplit == 1 || workspace_f32, "a split context needs a workspace of n_head * nsplit * 130 floats");
+    // one workgroup keeps the scores of its share of the context in LDS
+    const int64_t local = (max_seq + nsplit - 1) / nsplit + ATT_CHUNK;
+    const size_t smem = (size_t)(3 * 128 + 32 + 64 * 128 + local + 8) * sizeof(float);
+    AO_REQUIRE(smem <= 160 * 1024, "a cache of %lld positions over %d workgroups per head does not fit the kernel's LDS "
+               "score buffer: use a larger split", (long long)max_seq, nsplit);
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head, (unsigned)nsplit), dim3(ATT_THREADS), smem, st,
+                       (const uint16_t*)qkv_bf16, (const float*)qkv_f32_parts, nparts, (const uint16_t*)freqs_cis_bf16,
+                       pos_dev, (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16, nsplit,
+                       (float*)workspace_f32);
+    AO_LAUNCH_CHECK();
+    if (nsplit > 1) {
+        hipLaunchKernelGGL(attention_merge_kernel, dim3((unsigned)n_head), dim3(128), 0, st, (const float*)workspace_f32,
+                           nsplit, (uint16_t*)out_bf16);
+        AO_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
 extern "C" int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* freqs_cis_bf16, const int32_t* pos_dev,
                                              void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim,
                                              int64_t max_seq, void* out_bf16, void* stream) {
-    AO_REQUIRE(qkv_bf16 && freqs_cis_bf16 && pos_dev && k_cache && v_cache && out_bf16, "null pointer argument");
-    AO_REQUIRE(head_dim == 128, "decode attention kernel is built for head_dim 128, got %d", head_dim);
-    AO_REQUIRE(n_kv > 0 && n_head % n_kv == 0, "n_head=%d must be a multiple of n_kv=%d", n_head, n_kv);
-    AO_REQUIRE(max_seq > 0 && max_seq <= 8192, "max_seq=%lld outside (0, 8192]", (long long)max_seq);
-    const size_t smem = (size_t)(3 * 128 + 32 + 64 * 128 + max_seq + 8) * sizeof(float);
-    hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head), dim3(ATT_THREADS), smem, (hipStream_t)stream,
-                       (const uint16_t*)qkv_bf16, (const float*)nullptr, 0, (const uint16_t*)freqs_cis_bf16, pos_dev,
-                       (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16);
-    AO_LAUNCH_CHECK();
-    return 0;
+    AO_REQUIRE(qkv_bf16, "null pointer argument");
+    return attention_dispatch(qkv_bf16, nullptr, 0, freqs_cis_bf16, pos_dev, k_cache, v_cache, n_head, n_kv, head_dim,
+                              max_seq, 1, nullptr, out_bf16, stream);
 }
 
 extern "C" int ao_amd_llama_decode_attention_parts(const void* qkv_f32_parts, int nparts, const void* freqs_cis_bf16,
                                                    const int32_t* pos_dev, void* k_cache, void* v_cache, int n_head,
                                                    int n_kv, int head_dim, int64_t max_seq, void* out_bf16, void* stream) {
-    AO_REQUIRE(qkv_f32_parts && freqs_cis_bf16 && pos_dev && k_cache && v_cache && out_bf16, "null pointer argument");
+    AO_REQUIRE(qkv_f32_parts, "null pointer argument");
     AO_REQUIRE(nparts >= 1 && nparts <= 8, "number of partial rows %d outside [1, 8]", nparts);
-    AO_REQUIRE(head_dim == 128, "decode attention kernel is built for head_dim 128, got %d", head_dim);
-    AO_REQUIRE(n_kv > 0 && n_head % n_kv == 0, "n_head=%d must be a multiple of n_kv=%d", n_head, n_kv);
-    AO_REQUIRE(max_seq > 0 && max_seq <= 8192, "max_seq=%lld outside (0, 8192]", (long long)max_seq);
-    const size_t smem = (size_t)(3 * 128 + 32 + 64 * 128 + max_seq + 8) * sizeof(float);
-    hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head), dim3(ATT_THREADS), smem, (hipStream_t)stream,
-                       (const uint16_t*)nullptr, (const float*)qkv_f32_parts, nparts, (const uint16_t*)freqs_cis_bf16,
-                       pos_dev, (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16);
-    AO_LAUNCH_CHECK();
-    return 0;
+    return attention_dispatch(nullptr, qkv_f32_parts, nparts, freqs_cis_bf16, pos_dev, k_cache, v_cache, n_head, n_kv,
+                              head_dim, max_seq, 1, nullptr, out_bf16, stream);
+}
+
+extern "C" int ao_amd_llama_decode_attention_split(const void* qkv_bf16, const void* qkv_f32_parts, int nparts,
+                                                   const void* freqs_cis_bf16, const int32_t* pos_dev, void* k_cache,
+                                                   void* v_cache, int n_head, int n_kv, int head_dim, int64_t max_seq,
+                                                   int nsplit, void* workspace_f32, void* out_bf16, void* stream) {
+    AO_REQUIRE((qkv_bf16 != nullptr) != (qkv_f32_parts != nullptr), "pass the fused qkv row either as bf16 or as fp32 parts");
+    AO_REQUIRE(qkv_bf16 || (nparts >= 1 && nparts <= 8), "number of partial rows %d outside [1, 8]", nparts);
+    return attention_dispatch(qkv_bf16, qkv_f32_parts, qkv_bf16 ? 0 : nparts, freqs_cis_bf16, pos_dev, k_cache, v_cache,
+                              n_head, n_kv, head_dim, max_seq, nsplit, workspace_f32, out_bf16, stream);
 }
 
 extern "C" int ao_amd_argmax_bf16(const void* x_bf16, int64_t n, int32_t* out_index, void* stream) {

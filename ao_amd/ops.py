@@ -399,6 +399,14 @@ def _argmax_bf16_cuda(x):
     return out
 
 
+def decode_attention_splits(max_seq: int) -> int:
+    """Workgroups per head of the decode attention for a KV cache of `max_seq` positions: 1 up to 1024 positions
+    (8.5 us at 300, 18 us at 1000 positions), then 4, 8 or 16 so that a workgroup walks at most ~1024 of them."""
+    if max_seq <= 1024:
+        return 1
+    return 4 if max_seq <= 4096 else (8 if max_seq <= 8192 else 16)
+
+
 def _decode_attention_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv):
     require_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache)
     torch._check(qkv.dtype in (torch.bfloat16, torch.float32) and k_cache.dtype is torch.bfloat16
@@ -412,17 +420,31 @@ def _decode_attention_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, 
     row = (n_head + 2 * n_kv) * head_dim
     torch._check(freqs_cis.is_contiguous() and freqs_cis.shape[-2:] == (head_dim // 2, 2), lambda: "bad freqs_cis shape")
     out = torch.empty((1, n_head * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    nparts = 0
     if qkv.dtype is torch.float32:
         # fp32 partial rows of a linear whose K range was split (int4wo_linear_partials): added and rounded in the kernel
         nparts = qkv.numel() // row
         torch._check(qkv.is_contiguous() and qkv.numel() == nparts * row and 1 <= nparts <= 8,
                      lambda: "fp32 qkv must be [parts, 1, (n_head + 2 n_kv) * head_dim] contiguous, 1..8 parts")
+    else:
+        torch._check(qkv.numel() == row and qkv.is_contiguous(),
+                     lambda: "qkv must be the contiguous fused projection of one token")
+    nsplit = decode_attention_splits(max_seq)
+    if nsplit > 1:
+        # long cache: several workgroups per head + a merge launch (the launch shape cannot follow the position, which
+        # lives on the device, so it follows the cache size)
+        work = torch.empty(n_head * nsplit * (head_dim + 2), dtype=torch.float32, device=qkv.device)
+        check(lib().ao_amd_llama_decode_attention_split(None if nparts else qkv.data_ptr(), qkv.data_ptr() if nparts else None,
+                                                        nparts, freqs_cis.data_ptr(), input_pos.data_ptr(),
+                                                        k_cache.data_ptr(), v_cache.data_ptr(), n_head, n_kv, head_dim,
+                                                        max_seq, nsplit, work.data_ptr(), out.data_ptr(),
+                                                        current_stream(qkv.device)))
+        return out
+    if nparts:
         check(lib().ao_amd_llama_decode_attention_parts(qkv.data_ptr(), nparts, freqs_cis.data_ptr(), input_pos.data_ptr(),
                                                         k_cache.data_ptr(), v_cache.data_ptr(), n_head, n_kv, head_dim,
                                                         max_seq, out.data_ptr(), current_stream(qkv.device)))
         return out
-    torch._check(qkv.numel() == row and qkv.is_contiguous(),
-                 lambda: "qkv must be the contiguous fused projection of one token")
     check(lib().ao_amd_llama_decode_attention(qkv.data_ptr(), freqs_cis.data_ptr(), input_pos.data_ptr(),
                                               k_cache.data_ptr(), v_cache.data_ptr(), n_head, n_kv, head_dim, max_seq,
                                               out.data_ptr(), current_stream(qkv.device)))

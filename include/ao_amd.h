@@ -206,7 +206,8 @@ int ao_amd_rmsnorm_bf16(const void* x, const void* weight, int64_t rows, int64_t
 /* One new token, batch 1: rotary embedding of q and k, KV-cache update at *pos_dev, grouped-query attention over
  * positions 0..*pos_dev.  Attention.forward, torchao/_models/llama/model.py:190-211 with apply_rotary_emb :250-266
  * and KVCache.update :85-98.  qkv: [(n_head + 2 n_kv) * head_dim] (fused wqkv output); freqs_cis: [*, head_dim/2, 2]
- * (cos, sin); caches: [n_kv, max_seq, head_dim]; out: [n_head * head_dim].  head_dim must be 128, max_seq <= 8192. */
+ * (cos, sin); caches: [n_kv, max_seq, head_dim]; out: [n_head * head_dim].  head_dim must be 128, max_seq <= 28000 (the
+ * scores of the whole context live in LDS; see the split variant below for more). */
 int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* freqs_cis_bf16, const int32_t* pos_dev,
                                   void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim, int64_t max_seq,
                                   void* out_bf16, void* stream);
@@ -216,6 +217,16 @@ int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* freqs_cis_bf
 int ao_amd_llama_decode_attention_parts(const void* qkv_f32_parts, int nparts, const void* freqs_cis_bf16,
                                         const int32_t* pos_dev, void* k_cache, void* v_cache, int n_head, int n_kv,
                                         int head_dim, int64_t max_seq, void* out_bf16, void* stream);
+
+/* The same step with the context of every head split over `nsplit` (1..16) workgroups that take interleaved 64-position
+ * rows, for long contexts (one workgroup per head walks 8192 positions in ~80 us, eight of them in ~15): partial
+ * (max, sum, output) triples go to `workspace_f32` (n_head * nsplit * 130 floats, caller-owned) and a second, small launch
+ * merges them.  Exactly one of qkv_bf16 / qkv_f32_parts is non-null.  max_seq <= 32768 (scores of one workgroup's share of
+ * the context live in LDS).  No counterpart in the reference, whose attention is F.scaled_dot_product_attention. */
+int ao_amd_llama_decode_attention_split(const void* qkv_bf16, const void* qkv_f32_parts, int nparts,
+                                        const void* freqs_cis_bf16, const int32_t* pos_dev, void* k_cache, void* v_cache,
+                                        int n_head, int n_kv, int head_dim, int64_t max_seq, int nsplit,
+                                        void* workspace_f32, void* out_bf16, void* stream);
 
 /* out_index[0] = index of the largest of n bf16 values (lowest index among equals; NaN counts as largest): the greedy
  * branch of `sample` in the decode harness, torch.argmax over the last position's logits

@@ -212,18 +212,22 @@ def test_rmsnorm_linear_rejects_prefill_shapes():
         ops.int4wo_rmsnorm_linear(make_act(17, K, seed=62).to(dev), nw, 1e-5, packed, qp, g, N)
 
 
-@pytest.mark.parametrize("pos", [0, 5, 130, 511, 512, 700, 1500])
-def test_decode_attention_matches_module_math(pos):
+@pytest.mark.parametrize("pos,S", [(0, 256), (5, 256), (130, 256), (511, 1024), (512, 1024), (700, 1024), (1023, 1024),
+                                   (3, 2048), (700, 2048), (1500, 2048), (2047, 2048), (100, 8192), (5000, 8192),
+                                   (8191, 8192), (12345, 16384)])
+def test_decode_attention_matches_module_math(pos, S):
     """fp32 restatement of Attention.forward for one token (RoPE on interleaved pairs, cache update,
-    GQA softmax attention); tolerance 1e-2 relative L2 (bf16 inputs and output)."""
+    GQA softmax attention); tolerance 1e-2 relative L2 (bf16 inputs and output).  Caches above 1024 positions run
+    with 4, 8 or 16 workgroups per head and the merge launch, whatever the position."""
     from ao_amd import ops
     from ao_amd._models.llama.model import apply_rotary_emb, precompute_freqs_cis
 
     dev = _dev()
     torch.manual_seed(pos)
-    n_head, n_kv, hd, S = 8, 2, 128, (256 if pos < 256 else 2048)   # the kernel walks the cache in chunks of 512
+    n_head, n_kv, hd = 8, 2, 128
+    assert ops.decode_attention_splits(S) == {256: 1, 1024: 1, 2048: 4, 8192: 8, 16384: 16}[S]
     qkv = torch.randn(1, (n_head + 2 * n_kv) * hd).bfloat16().to(dev)
-    freqs = precompute_freqs_cis(2048, hd, 10000, torch.bfloat16, dev)
+    freqs = precompute_freqs_cis(S, hd, 10000, torch.bfloat16, dev)
     k_cache = torch.randn(1, n_kv, S, hd).bfloat16().to(dev)
     v_cache = torch.randn(1, n_kv, S, hd).bfloat16().to(dev)
     kc, vc = k_cache.clone(), v_cache.clone()
@@ -339,13 +343,14 @@ def test_linear_partials_sum_to_the_linear(M, N, K, g, ksplit):
     assert rel_l2(parts_n.sum(0).cpu().numpy(), full_n.cpu().numpy()) <= 1e-3
 
 
-def test_decode_attention_from_partial_rows():
+@pytest.mark.parametrize("S", [64, 4096])
+def test_decode_attention_from_partial_rows(S):
     """fp32 partial qkv rows are added and rounded to bf16 inside the attention kernel: same result as handing it the
     rounded sum."""
     from ao_amd import ops
 
     dev = _dev()
-    n_head, n_kv, hd, S = 8, 2, 128, 64
+    n_head, n_kv, hd = 8, 2, 128
     gen = torch.Generator().manual_seed(5)
     parts = torch.randn(2, 1, (n_head + 2 * n_kv) * hd, generator=gen).to(dev)
     qkv = parts.sum(0).bfloat16()
