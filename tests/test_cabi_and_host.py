@@ -220,3 +220,20 @@ def test_module_swap_host_logic(oracle):
         zpad[:N, :K // g] = bits[:, :, 1].T
         _, q_ref = oracle.int4wo_pack(np.full((Np, Kp), 8, np.int32), spad, zpad, g)
         assert words.shape == q_ref.shape and np.array_equal(words, q_ref)
+
+
+def test_dispatch_rules_are_pure_host_functions():
+    """The shape rules that pick a kernel path need no GPU: prefill two-pass thresholds, context splits of the
+    decode attention, K split of the fused qkv projection."""
+    from ao_amd import ops
+    from ao_amd._models.llama.model import Transformer
+
+    assert ops.int4wo_two_pass(512, 14336, 4096) and not ops.int4wo_two_pass(511, 14336, 4096)
+    assert not ops.int4wo_two_pass(512, 4096, 4096) and ops.int4wo_two_pass(1024, 4096, 4096)
+    assert not ops.int4wo_two_pass(512, 128256, 4096) and ops.int4wo_two_pass(1024, 128256, 4096)
+    assert not ops.int4wo_two_pass(2048, 1024, 4096) and ops.int4wo_two_pass(4096, 1024, 4096)
+    assert [ops.decode_attention_splits(s) for s in (8, 1024, 1025, 4096, 4097, 8192, 8193, 16384)] == [1, 1, 4, 4, 8, 8, 16, 16]
+    assert Transformer.qkv_ksplit(6144) == 2 and Transformer.qkv_ksplit(4096) == 1 and Transformer.qkv_ksplit(2048) == 2
+    assert ops.int4wo_packed_shapes(48, 192, 64) == ((3, 2, 64, 4), (3, 4, 16))
+    with pytest.raises(ValueError):
+        ops.int4wo_packed_shapes(48, 192, 48)
