@@ -199,6 +199,9 @@ class Transformer(nn.Module):
         max_seq_length = find_multiple(max_seq_length, 8)
         self.max_seq_length, self.max_batch_size = max_seq_length, max_batch_size
         dtype = self.output.weight.dtype
+        for name in ("scales", "scales_and_zeros"):  # module-swapped head: the compute dtype is that of its scales
+            if hasattr(self.output, name):
+                dtype = getattr(self.output, name).dtype
         device = self.tok_embeddings.weight.device
         for b in self.layers:
             b.attention.kv_cache = KVCache(max_batch_size, max_seq_length, self.config.n_local_heads,
@@ -223,6 +226,8 @@ class Transformer(nn.Module):
             return None
         kinds, groups = set(), set()
         for lin in self._decode_linears():
+            if not isinstance(lin, nn.Linear):  # module-swapped layers (WeightOnlyInt4Linear, ...) run as modules
+                return None
             w = lin.weight
             if lin.bias is not None or not isinstance(w, AffineQuantizedTensor) or w.dtype is not torch.bfloat16 \
                     or not w.is_cuda:

@@ -1,4 +1,4 @@
-from .GPTQ import Int4WeightOnlyQuantizer, WeightOnlyInt4Linear
+from .GPTQ import Int4WeightOnlyGPTQQuantizer, Int4WeightOnlyQuantizer, WeightOnlyInt4Linear
 from .quant_api import (
     fp6_llm_weight_only,
     int4_weight_only,

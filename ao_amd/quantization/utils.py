@@ -19,6 +19,8 @@ __all__ = [
     "groupwise_affine_quantize_tensor",
     "groupwise_affine_dequantize_tensor",
     "recommended_inductor_config_setter",
+    "unpack_tinygemm_int4pack",
+    "_MultiInput",
 ]
 
 
@@ -97,3 +99,57 @@ def recommended_inductor_config_setter():
     """The reference tunes torch.compile here (:461-476).  This library does not go through inductor:
     kernels are launched directly and decode loops are captured in HIP graphs, so there is nothing to set."""
     return None
+
+
+# Position, inside a 32-wide span of k (two 16-wide k tiles), of nibble p of a tinygemm word held by the lane with
+# t % 4 == 0; lane t adds 2 * (t % 4).  Nibbles 0..3 (low half-word) are the even k of the lane's four pairs, nibbles
+# 4..7 the odd ones, so that `(word >> 4i) & 0x000F000F` is one (k, k + 1) pair.
+_TINYGEMM_NIBBLE_K = (0, 8, 16, 24, 1, 9, 17, 25)
+
+
+def unpack_tinygemm_int4pack(weight_int4pack: torch.Tensor, inner_k_tiles: int) -> torch.Tensor:
+    """The 4-bit codes `[N, K]` (int32, 0..15) of a weight packed by the CUDA build of
+    `aten._convert_weight_to_int4pack` (`[N/8, K/(16*inner_k_tiles), 32, inner_k_tiles/2]` int32), the `weight` entry
+    of state dicts written by the reference's module-swap quantizers (torchao/quantization/GPTQ.py:566-569, :737).
+
+    The layout is the B fragment of `mma.m16n8k16`, as published in PyTorch's int4mm.cu (v2.3): word
+    `[nt][ko][t][j]` belongs to row `8*nt + t//4` and to the two k tiles starting at `16*(ko*inner_k_tiles + 2j)`;
+    its nibbles hold k offsets `2*(t%4) + {0, 8, 16, 24, 1, 9, 17, 25}` in order from the low nibble.  The reference
+    repository holds no packed vectors of this format (the packer lives in PyTorch core), so this restatement is
+    checked against a loop transcription of the same published kernel only.  Words packed by a ROCm build of PyTorch
+    follow a different tile order and are not handled."""
+    assert weight_int4pack.dtype is torch.int32 and weight_int4pack.dim() == 4, "expected the 4-d int32 tinygemm weight"
+    n_tiles, k_outer, lanes, halves = weight_int4pack.shape
+    assert inner_k_tiles in (2, 4, 8) and lanes == 32 and halves * 2 == inner_k_tiles, \
+        f"shape {tuple(weight_int4pack.shape)} is not a tinygemm weight of inner_k_tiles={inner_k_tiles}"
+    dev = weight_int4pack.device
+    shifts = torch.arange(0, 32, 4, device=dev, dtype=torch.int32)
+    nib = (weight_int4pack.unsqueeze(-1) >> shifts) & 0xF  # [nt, ko, t, j, p]
+    nib = nib.reshape(n_tiles, k_outer, 8, 4, halves, 8)  # t -> (row in tile, t % 4)
+    # destination order: [nt, row, ko, j, position in the 32-wide span]
+    nib = nib.permute(0, 2, 1, 4, 3, 5).reshape(n_tiles, 8, k_outer, halves, 32)
+    # source index (t % 4, p) flattened as 8 * (t % 4) + p, for each position of the span
+    src = torch.empty(32, dtype=torch.long)
+    for tc in range(4):
+        for p, koff in enumerate(_TINYGEMM_NIBBLE_K):
+            src[koff + 2 * tc] = 8 * tc + p
+    codes = nib.index_select(-1, src.to(dev))
+    return codes.reshape(n_tiles * 8, k_outer * inner_k_tiles * 16).contiguous()
+
+
+class _MultiInput:
+    """The values one positional argument of a model takes over the calibration samples (reference
+    torchao/quantization/utils.py:106-122)."""
+
+    def __init__(self, inputs):
+        self.values = list(inputs)
+
+    def add_input(self, input):
+        self.values.append(input)
+        return self
+
+    def __getitem__(self, slice):
+        return _MultiInput(self.values[slice])
+
+    def cuda(self):
+        self.values = [v.cuda() if isinstance(v, torch.Tensor) else v for v in self.values]

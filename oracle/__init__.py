@@ -6,6 +6,10 @@ algorithm) plus numpy restatements of the FP6-LLM bit packing.  Only ``tests/``,
 package; the shipped ``ao_amd`` package never does.
 
 bf16 / fp16 tensors are passed as ``numpy.uint16`` bit patterns.
+
+Parity unpinned: ``tinygemm_int4pack`` (layout of aten._convert_weight_to_int4pack on CUDA, published in PyTorch
+core, absent from the reference tree, no vectors).  ``obq_quantize`` is the textbook form of GPTQ's recurrence, a
+mathematical cross-check rather than a restatement of reference code.
 """
 import ctypes
 import os
@@ -336,3 +340,60 @@ def pack_tc_fpx_generic(codes, nbits):
             frags.append(ty)
             used += y
     return np.concatenate(frags).reshape(M, -1)
+
+
+# --- tinygemm int4 weight layout (PARITY UNPINNED) -------------------------------------------------------------
+# aten._convert_weight_to_int4pack lives in PyTorch core (aten/src/ATen/native/cuda/int4mm.cu, v2.3,
+# matrix_to_m16n8k16_Bint4_layout), not in the reference repository, which holds no vectors of this format.  This
+# is a thread-by-thread loop transcription of that published CUDA kernel; nothing available here pins it.
+
+def tinygemm_int4pack(codes, inner_k_tiles):
+    """codes int [N, K] (0..15) -> uint32 [N/8, K/(16*inner_k_tiles), 32, inner_k_tiles/2], one CUDA lane at a time."""
+    codes = np.asarray(codes)
+    N, K = codes.shape
+    assert N % 8 == 0 and K % (inner_k_tiles * 16) == 0 and inner_k_tiles in (2, 4, 8)
+    out = np.zeros((N // 8, K // (inner_k_tiles * 16), 32, inner_k_tiles // 2), np.uint32)
+    for n_tile in range(N // 8):
+        for k_outer in range(K // (inner_k_tiles * 16)):
+            for t in range(32):
+                n0 = n_tile * 8 + t // 4
+                for inner in range(0, inner_k_tiles, 2):
+                    base0 = (k_outer * inner_k_tiles + inner) * 16
+                    base1 = base0 + 16
+                    k0, k4 = base0 + (t % 4) * 2, base1 + (t % 4) * 2
+                    ks = [k0, k0 + 1, k0 + 8, k0 + 9, k4, k4 + 1, k4 + 8, k4 + 9]
+                    v = [int(codes[n0, k]) & 0xF for k in ks]
+                    word = (v[7] << 28) | (v[5] << 24) | (v[3] << 20) | (v[1] << 16) | (v[6] << 12) | (v[4] << 8) \
+                        | (v[2] << 4) | v[0]
+                    out[n_tile, k_outer, t, inner // 2] = word
+    return out
+
+
+# --- GPTQ: textbook column-by-column optimal brain quantization, the form GPTQ's Cholesky recurrence is derived
+# from (Frantar et al. 2022, eq. 2-3).  Float64, one explicit inverse of the remaining Hessian per column; slow and
+# meant for a few dozen columns.  It cross-checks the blocked Cholesky solver of the library, which follows
+# torchao/quantization/GPTQ.py:300-398; the per-column quantizer is passed in.
+
+def obq_quantize(H, W, groupsize, get_qparams, quant_dequant, percdamp=0.01):
+    """H [K, K], W [N, K] float64 -> dequantized weights [N, K] (float64).
+
+    get_qparams(W_group [N, g]) -> qparams at each group start, from the error-compensated weights;
+    quant_dequant(w_col [N], qparams) -> [N] quantized-dequantized column."""
+    H = np.array(H, np.float64)
+    W = np.array(W, np.float64)
+    K = W.shape[1]
+    dead = np.diag(H) == 0
+    H[dead, dead] = 1
+    W[:, dead] = 0
+    H[np.arange(K), np.arange(K)] += percdamp * np.mean(np.diag(H))
+    DQ = np.zeros_like(W)
+    qparams = None
+    for i in range(K):
+        if i % groupsize == 0:
+            qparams = get_qparams(W[:, i:i + groupsize])
+        Hinv = np.linalg.inv(H[i:, i:])  # inverse Hessian of the columns not yet quantized
+        dq = quant_dequant(W[:, i], qparams)
+        DQ[:, i] = dq
+        err = (W[:, i] - dq) / Hinv[0, 0]
+        W[:, i:] -= np.outer(err, Hinv[0, :])
+    return DQ

@@ -184,3 +184,21 @@ def test_constructor_checks():
     biased = nn.Sequential(nn.Linear(256, 64, bias=True)).bfloat16().to(_dev())
     with pytest.raises(AssertionError, match="bias=False"):
         Int4WeightOnlyQuantizer(groupsize=64).quantize(biased)
+
+
+def test_module_swapped_llama_decodes_token_by_token():
+    """A Llama-architecture model whose linears were swapped for `WeightOnlyInt4Linear` modules is not a candidate for
+    the fused decode step (that one reads tensor-subclass weights); it decodes through the modules, eagerly and under
+    graph capture, with the same tokens."""
+    from ao_amd._models.llama.generate import build_random_model, generate
+    from ao_amd.quantization.GPTQ import Int4WeightOnlyQuantizer, WeightOnlyInt4Linear
+
+    print("case module swap llama decode", flush=True)
+    dev = _dev()
+    model = Int4WeightOnlyQuantizer(groupsize=64).quantize(build_random_model("tiny128", dev))
+    assert isinstance(model.output, WeightOnlyInt4Linear)
+    prompt = torch.arange(3, 19, dtype=torch.int, device=dev)
+    eager = generate(model, prompt, 8, greedy=True)
+    assert model.fused_decode_kind() is None
+    graphed = generate(model, prompt, 8, greedy=True, use_graph=True)
+    assert eager.shape == (24,) and torch.equal(eager, graphed)
