@@ -59,6 +59,8 @@ _SIGNATURES = {
     "ao_amd_int8wo_linear": ([_p, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _p, _int, _i64, _p], _int),
     "ao_amd_int8wo_linear_residual": ([_p, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p], _int),
     "ao_amd_int8wo_linear_gated": ([_p, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p], _int),
+    "ao_amd_int8wo_rmsnorm_linear": ([_p, _i64, _i64, _i64, _p, ctypes.c_float, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p], _int),
+    "ao_amd_int8wo_swiglu": ([_p, _i64, _i64, _i64, _p, ctypes.c_float, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p], _int),
     "ao_amd_int8_to_bf16": ([_p, _i64, _i64, _i64, _p, _p], _int),
     "ao_amd_hqq_dequantize": ([_p, _int, _i64, _i64, _p, _p, _i64, _int, _p, _p], _int),
     "ao_amd_rmsnorm_bf16": ([_p, _p, _i64, _i64, ctypes.c_float, _p, _p], _int),

@@ -312,14 +312,17 @@ class Transformer(nn.Module):
         return logits.view(1, 1, cfg.vocab_size)
 
     def _fused_decode_int8(self, idx: Tensor, input_pos: Tensor) -> Tensor:
-        """The same step over int8 weight-only linears: the streaming int8 kernel per linear, the RMSNorm and decode
-        attention kernels, with the residual add and the SiLU(gate) * up product fused into the linear that precedes them."""
+        """The same step over int8 weight-only linears: the streaming int8 kernel per linear and the decode attention
+        kernel, with each RMSNorm fused into the linears it feeds and the residual add and the SiLU(gate) * up product
+        fused into the linear that precedes them; w1 and w3 stream in one launch (5 launches per layer)."""
         from ... import ops
 
         cfg = self.config
 
-        def lin(x, layer, residual=None, gate=None):
+        def lin(x, layer, residual=None, gate=None, norm=None):
             lay = layer.weight.layout_tensor
+            if norm is not None:
+                return ops.int8wo_rmsnorm_linear(x, norm.weight, norm.eps, lay.int_data, lay.scale.reshape(-1), gate)
             if residual is not None:
                 return ops.int8wo_linear_residual(x, lay.int_data, lay.scale.reshape(-1), residual)
             if gate is not None:
@@ -330,13 +333,15 @@ class Transformer(nn.Module):
         pos = input_pos.to(torch.int32) if input_pos.dtype is not torch.int32 else input_pos
         for b in self.layers:
             att, ffn = b.attention, b.feed_forward
-            qkv = lin(ops.rmsnorm(x, b.attention_norm.weight, b.attention_norm.eps), att.wqkv)
+            qkv = lin(x, att.wqkv, norm=b.attention_norm)
             y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
                                            cfg.n_head, cfg.n_local_heads)
             h = lin(y, att.wo, residual=x)
-            hn = ops.rmsnorm(h, b.ffn_norm.weight, b.ffn_norm.eps)
-            x = lin(lin(hn, ffn.w3, gate=lin(hn, ffn.w1)), ffn.w2, residual=h)
-        return lin(ops.rmsnorm(x, self.norm.weight, self.norm.eps), self.output).view(1, 1, cfg.vocab_size)
+            g, u = ffn.w1.weight.layout_tensor, ffn.w3.weight.layout_tensor
+            act = ops.int8wo_swiglu(h, g.int_data, g.scale.reshape(-1), u.int_data, u.scale.reshape(-1),
+                                    b.ffn_norm.weight, b.ffn_norm.eps)
+            x = lin(act, ffn.w2, residual=h)
+        return lin(x, self.output, norm=self.norm).view(1, 1, cfg.vocab_size)
 
     def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None) -> Tensor:
         assert self.freqs_cis is not None, "Caches must be initialized first"

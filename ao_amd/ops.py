@@ -6,6 +6,7 @@ include/ao_amd.h with raw pointers on torch's current stream; there is no CPU im
 a CPU tensor raises.
 """
 import weakref
+from typing import Optional
 
 import torch
 from torch import Tensor
@@ -50,6 +51,8 @@ _LIB.define("int4wo_interleave_pair(Tensor packed_gate, Tensor qparams_gate, Ten
 _LIB.define("int4wo_swiglu_interleaved(Tensor x, Tensor? norm_weight, float eps, Tensor packed_pair, Tensor qparams_pair, int group_size, int N) -> Tensor")
 _LIB.define("int8wo_linear(Tensor x, Tensor w_int8, Tensor scale, Tensor? bias, bool fp32_out) -> Tensor")
 _LIB.define("int8wo_linear_fused(Tensor x, Tensor w_int8, Tensor scale, Tensor other, bool gated) -> Tensor")
+_LIB.define("int8wo_swiglu(Tensor x, Tensor? norm_weight, float eps, Tensor w_gate, Tensor scale_gate, Tensor w_up, Tensor scale_up) -> Tensor")
+_LIB.define("int8wo_rmsnorm_linear(Tensor x, Tensor norm_weight, float eps, Tensor w_int8, Tensor scale, Tensor? gate) -> Tensor")
 _LIB.define("hqq_dequantize(Tensor packed_2xint4, Tensor scales, Tensor zeros, int group_size) -> Tensor")
 _LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
 _LIB.define("argmax_bf16(Tensor x) -> Tensor")
@@ -264,6 +267,58 @@ def _int8wo_linear_fused_cuda(x, w_int8, scale, other, gated):
     fn = lib().ao_amd_int8wo_linear_gated if gated else lib().ao_amd_int8wo_linear_residual
     check(fn(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, w_int8.data_ptr(), w_int8.stride(0), scale.data_ptr(), N,
              other.data_ptr(), other.stride(0) if M > 0 else N, y.data_ptr(), N, current_stream(x.device)))
+    return y
+
+
+def _int8wo_rmsnorm_linear_cuda(x, norm_weight, eps, w_int8, scale, gate):
+    """linear(rmsnorm(x)), or silu(gate) * linear(rmsnorm(x)), in one launch; decode shapes only (the library rejects
+    activations whose rows do not fit a workgroup's LDS)."""
+    require_cuda(x, norm_weight, w_int8, scale, gate)
+    torch._check(x.dim() == 2 and x.dtype is torch.bfloat16, lambda: "input must be a 2d bfloat16 tensor")
+    _check_norm(x, norm_weight)
+    torch._check(w_int8.dim() == 2 and w_int8.dtype is torch.int8 and w_int8.stride(1) == 1,
+                 lambda: "weight must be a 2d int8 tensor with unit inner stride")
+    M, K = x.shape
+    N = w_int8.shape[0]
+    torch._check(w_int8.shape[1] == K, lambda: f"weight in_features {w_int8.shape[1]} != input features {K}")
+    torch._check(scale.dtype is torch.bfloat16 and scale.numel() == N, lambda: "scale must be bfloat16 of size N")
+    if gate is not None:
+        torch._check(gate.dtype is torch.bfloat16 and tuple(gate.shape) == (M, N) and gate.stride(1) == 1,
+                     lambda: "the gate must be a bfloat16 [M, N] tensor with unit inner stride")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    scale = scale.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    check(lib().ao_amd_int8wo_rmsnorm_linear(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, norm_weight.data_ptr(),
+                                             float(eps), w_int8.data_ptr(), w_int8.stride(0), scale.data_ptr(), N,
+                                             None if gate is None else gate.data_ptr(),
+                                             gate.stride(0) if gate is not None and M > 0 else N, y.data_ptr(), N,
+                                             current_stream(x.device)))
+    return y
+
+
+def _int8wo_swiglu_cuda(x, norm_weight, eps, w_gate, scale_gate, w_up, scale_up):
+    """silu(linear(x', w_gate)) * linear(x', w_up) in one launch, x' = rmsnorm(x) when a norm weight is given; decode
+    shapes only."""
+    require_cuda(x, norm_weight, w_gate, scale_gate, w_up, scale_up)
+    torch._check(x.dim() == 2 and x.dtype is torch.bfloat16, lambda: "input must be a 2d bfloat16 tensor")
+    if norm_weight is not None:
+        _check_norm(x, norm_weight)
+    M, K = x.shape
+    N = w_gate.shape[0]
+    for w, sc in ((w_gate, scale_gate), (w_up, scale_up)):
+        torch._check(w.dim() == 2 and w.dtype is torch.int8 and w.stride(1) == 1 and tuple(w.shape) == (N, K),
+                     lambda: "weights must be int8 [N, K] tensors of one shape with unit inner stride")
+        torch._check(sc.dtype is torch.bfloat16 and sc.numel() == N, lambda: "scale must be bfloat16 of size N")
+    torch._check(w_gate.stride(0) == w_up.stride(0), lambda: "both weights must have the same row stride")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    check(lib().ao_amd_int8wo_swiglu(x.data_ptr(), M, K, x.stride(0) if M > 0 else K,
+                                     None if norm_weight is None else norm_weight.data_ptr(), float(eps),
+                                     w_gate.data_ptr(), scale_gate.contiguous().data_ptr(), w_up.data_ptr(),
+                                     scale_up.contiguous().data_ptr(), w_gate.stride(0), N, y.data_ptr(), N,
+                                     current_stream(x.device)))
     return y
 
 
@@ -556,6 +611,8 @@ _LIB.impl("int4wo_interleave_pair", _interleave_pair_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu_interleaved", _swiglu_interleaved_cuda, "CUDA")
 _LIB.impl("int8wo_linear", _int8wo_linear_cuda, "CUDA")
 _LIB.impl("int8wo_linear_fused", _int8wo_linear_fused_cuda, "CUDA")
+_LIB.impl("int8wo_rmsnorm_linear", _int8wo_rmsnorm_linear_cuda, "CUDA")
+_LIB.impl("int8wo_swiglu", _int8wo_swiglu_cuda, "CUDA")
 _LIB.impl("hqq_dequantize", _hqq_dequantize_cuda, "CUDA")
 _LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
 _LIB.impl("llama_decode_attention", _decode_attention_cuda, "CUDA")
@@ -575,7 +632,7 @@ def _no_cpu(name):
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
               "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int4wo_linear_partials", "int4wo_interleave_pair",
-              "int4wo_swiglu_interleaved", "int8wo_linear", "int8wo_linear_fused", "hqq_dequantize", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
+              "int4wo_swiglu_interleaved", "int8wo_linear", "int8wo_linear_fused", "int8wo_rmsnorm_linear", "int8wo_swiglu", "hqq_dequantize", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
               "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
@@ -654,6 +711,16 @@ def _(x, norm_weight, eps, packed_pair, qparams_pair, group_size, N):
 
 @torch.library.register_fake("torchao::int8wo_linear_fused")
 def _(x, w_int8, scale, other, gated):
+    return x.new_empty((x.shape[0], w_int8.shape[0]), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::int8wo_swiglu")
+def _(x, norm_weight, eps, w_gate, scale_gate, w_up, scale_up):
+    return x.new_empty((x.shape[0], w_gate.shape[0]), dtype=torch.bfloat16)
+
+
+@torch.library.register_fake("torchao::int8wo_rmsnorm_linear")
+def _(x, norm_weight, eps, w_int8, scale, gate):
     return x.new_empty((x.shape[0], w_int8.shape[0]), dtype=torch.bfloat16)
 
 
@@ -803,6 +870,18 @@ def hqq_dequantize(packed_2xint4: Tensor, scales: Tensor, zeros: Tensor, group_s
 def int8wo_linear_residual(x: Tensor, w_int8: Tensor, scale: Tensor, residual: Tensor) -> Tensor:
     """bf16(int8wo_linear(x)) + residual in one launch."""
     return torch.ops.torchao.int8wo_linear_fused.default(x, w_int8, scale, residual, False)
+
+
+def int8wo_swiglu(x: Tensor, w_gate: Tensor, scale_gate: Tensor, w_up: Tensor, scale_up: Tensor,
+                  norm_weight: Optional[Tensor] = None, eps: float = 0.0) -> Tensor:
+    """silu(int8wo_linear(x', w_gate)) * int8wo_linear(x', w_up) in one launch, x' = rmsnorm(x) with a norm weight."""
+    return torch.ops.torchao.int8wo_swiglu.default(x, norm_weight, eps, w_gate, scale_gate, w_up, scale_up)
+
+
+def int8wo_rmsnorm_linear(x: Tensor, norm_weight: Tensor, eps: float, w_int8: Tensor, scale: Tensor,
+                          gate: Optional[Tensor] = None) -> Tensor:
+    """int8wo_linear(rmsnorm(x)) in one launch, optionally times silu(gate); for the few rows of a decode step."""
+    return torch.ops.torchao.int8wo_rmsnorm_linear.default(x, norm_weight, eps, w_int8, scale, gate)
 
 
 def int8wo_linear_gated(x: Tensor, w_int8: Tensor, scale: Tensor, gate: Tensor) -> Tensor:

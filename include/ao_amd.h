@@ -193,6 +193,23 @@ int ao_amd_int8wo_linear_gated(const void* x_bf16, int64_t M, int64_t K, int64_t
                                const void* scale_bf16, int64_t N, const void* gate_bf16, int64_t ldgate, void* y_bf16,
                                int64_t ldy, void* stream);
 
+/* linear(rmsnorm(x)) in one launch for the decode step: y = bf16(bf16(rmsnorm(x) @ bf16(Wq)^T) * scale), with
+ * rmsnorm(x) = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * norm_weight) (RMSNorm.forward followed by the linear it feeds,
+ * torchao/_models/llama/model.py:232-244, :160-163, :209-214).  gate_bf16 may be null; when given the `_gated`
+ * epilogue above applies.  Only for activations whose (at most 16) rows fit the workgroup's LDS: M * K * 2 bytes at
+ * most 64 KB; other shapes are rejected.  norm_weight 16-byte aligned, bf16 [K]. */
+int ao_amd_int8wo_rmsnorm_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* norm_weight_bf16,
+                                 float eps, const void* w_int8, int64_t ldw, const void* scale_bf16, int64_t N,
+                                 const void* gate_bf16, int64_t ldgate, void* y_bf16, int64_t ldy, void* stream);
+
+/* SwiGLU over two int8 weights in one launch: y = bf16(silu(g)) * u with g = linear(x', w_gate), u = linear(x', w_up),
+ * each rounded as ao_amd_int8wo_linear rounds it, and x' = rmsnorm(x) when norm_weight_bf16 is given, else x
+ * (F.silu(self.w1(x)) * self.w3(x), FeedForward.forward, torchao/_models/llama/model.py:209-214).  Both weights int8
+ * [N, K] with the same row stride ldw, 16-byte aligned.  Same LDS limit as ao_amd_int8wo_rmsnorm_linear. */
+int ao_amd_int8wo_swiglu(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* norm_weight_bf16, float eps,
+                         const void* w_gate_int8, const void* scale_gate_bf16, const void* w_up_int8,
+                         const void* scale_up_bf16, int64_t ldw, int64_t N, void* y_bf16, int64_t ldy, void* stream);
+
 /* bf16 copy of the int8 codes (`w_int8.to(x.dtype)` of the same formula) for prefill-sized batches: the caller then
  * runs a plain bf16 GEMM on it and multiplies by the scale.  K a multiple of 16, 16-byte aligned rows. */
 int ao_amd_int8_to_bf16(const void* w_int8, int64_t N, int64_t K, int64_t ldw, void* out_bf16, void* stream);

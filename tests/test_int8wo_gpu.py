@@ -148,3 +148,67 @@ def test_fused_epilogues_match_the_module_chain(M):
     got = ops.int8wo_linear_gated(x, q, s, other).float().cpu().numpy()
     want = (torch.nn.functional.silu(other) * y).float().cpu().numpy()
     assert np.count_nonzero(got != want) <= 0.002 * got.size + 1 and rel_l2(got, want) <= 1e-3
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 512, 1024), (3, 512, 1024), (16, 256, 2048), (1, 6144, 4096), (1, 4096, 14336),
+                                   (1, 1000, 4096), (2, 8208, 4096)])
+def test_fused_rmsnorm_matches_the_separate_kernels(M, N, K):
+    """RMSNorm applied while the activation rows are staged in LDS: the normalized rows are those of the stand-alone
+    RMSNorm kernel unless the two sums of squares (different summation orders) round apart, so the linear is compared
+    with a tolerance of a few bf16 steps on few elements; with and without the SiLU(gate) epilogue."""
+    from ao_amd import ops
+
+    print(f"case int8 fused norm M={M} N={N} K={K}", flush=True)
+    dev = _dev()
+    gen = torch.Generator().manual_seed(M * 7 + N)
+    q = torch.randint(-127, 128, (N, K), generator=gen, dtype=torch.int8).to(dev)
+    s = (torch.rand(N, generator=gen) * 1e-3 + 1e-4).bfloat16().to(dev)
+    x = (make_act(M, K, seed=80 + M) * 3).to(dev)
+    nw = (1 + 0.1 * torch.randn(K, generator=gen)).bfloat16().to(dev)
+    gate = make_act(M, N, seed=81).to(dev)
+    xn = ops.rmsnorm(x, nw, 1e-5)
+    want = ops.int8wo_linear(xn, q, s).float().cpu().numpy()
+    got = ops.int8wo_rmsnorm_linear(x, nw, 1e-5, q, s).float().cpu().numpy()
+    assert rel_l2(got, want) <= 2e-3 and np.count_nonzero(got != want) <= 0.02 * got.size + 1
+    want_g = ops.int8wo_linear_gated(xn, q, s, gate).float().cpu().numpy()
+    got_g = ops.int8wo_rmsnorm_linear(x, nw, 1e-5, q, s, gate).float().cpu().numpy()
+    assert rel_l2(got_g, want_g) <= 2e-3 and np.count_nonzero(got_g != want_g) <= 0.02 * got_g.size + 1
+
+
+def test_fused_rmsnorm_rejects_rows_that_do_not_fit_lds():
+    from ao_amd import ops
+    from ao_amd._lib import AoAmdError
+
+    dev = _dev()
+    q = torch.zeros(256, 4096, dtype=torch.int8, device=dev)
+    s = torch.ones(256, dtype=torch.bfloat16, device=dev)
+    nw = torch.ones(4096, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(AoAmdError, match="fit in LDS"):
+        ops.int8wo_rmsnorm_linear(torch.zeros(16, 4096, dtype=torch.bfloat16, device=dev), nw, 1e-5, q, s)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 512, 1024), (4, 1000, 2048), (1, 14336, 4096), (16, 256, 1024)])
+@pytest.mark.parametrize("with_norm", [False, True])
+def test_two_weight_swiglu_matches_the_gated_chain(M, N, K, with_norm):
+    """One launch over w1 and w3 against linear -> gated linear: every rounding is the same, so equality but for
+    elements where the accumulation order of a sum sitting on a bf16 boundary differs (none expected: same order)."""
+    from ao_amd import ops
+
+    print(f"case int8 swiglu M={M} N={N} K={K} norm={with_norm}", flush=True)
+    dev = _dev()
+    gen = torch.Generator().manual_seed(M + N + K)
+    qg = torch.randint(-127, 128, (N, K), generator=gen, dtype=torch.int8).to(dev)
+    qu = torch.randint(-127, 128, (N, K), generator=gen, dtype=torch.int8).to(dev)
+    sg = (torch.rand(N, generator=gen) * 1e-3 + 1e-4).bfloat16().to(dev)
+    su = (torch.rand(N, generator=gen) * 1e-3 + 1e-4).bfloat16().to(dev)
+    x = (make_act(M, K, seed=90 + M) * 2).to(dev)
+    nw = (1 + 0.1 * torch.randn(K, generator=gen)).bfloat16().to(dev) if with_norm else None
+    if with_norm:
+        gate = ops.int8wo_rmsnorm_linear(x, nw, 1e-5, qg, sg)
+        want = ops.int8wo_rmsnorm_linear(x, nw, 1e-5, qu, su, gate)
+    else:
+        want = ops.int8wo_linear_gated(x, qu, su, ops.int8wo_linear(x, qg, sg))
+    got = ops.int8wo_swiglu(x, qg, sg, qu, su, nw, 1e-5)
+    assert got.shape == (M, N) and got.dtype is torch.bfloat16
+    g, w = got.float().cpu().numpy(), want.float().cpu().numpy()
+    assert rel_l2(g, w) <= 1e-3 and np.count_nonzero(g != w) <= 0.01 * g.size + 1
