@@ -12,7 +12,7 @@ from typing import Optional
 
 import torch
 
-from ...quantization import int4_weight_only, int8_weight_only, quantize
+from ...quantization import fp6_llm_weight_only, int4_weight_only, int8_weight_only, quantize
 from ...utils import get_model_size_in_bytes
 from .model import Transformer, prepare_inputs_for_model
 
@@ -158,7 +158,8 @@ def random_init_(model: torch.nn.Module, std: float = 0.02, seed: int = 1234) ->
 
 def build_random_model(name: str, device, quantization: Optional[str] = None, seed: int = 1234) -> Transformer:
     """Random-init bf16 model on `device`, optionally quantized ("int4wo-<group>" or "int8wo", the names of the
-    reference's generate.py:199-215)."""
+    reference's generate.py:199-215; "fp6": FP6-LLM e3m2 weights on an fp16 model, the flow of
+    torchao/prototype/quant_llm/README.md:9-20)."""
     prev = torch.get_default_dtype()
     torch.set_default_dtype(torch.bfloat16)
     try:
@@ -170,6 +171,9 @@ def build_random_model(name: str, device, quantization: Optional[str] = None, se
     model.eval()
     if quantization == "int8wo":
         quantize(model, int8_weight_only())
+    elif quantization == "fp6":
+        model = model.half()
+        quantize(model, fp6_llm_weight_only())
     elif quantization:
         assert quantization.startswith("int4wo-"), f"unsupported quantization {quantization}"
         group = int(quantization.split("-")[-1])

@@ -202,6 +202,9 @@ class Transformer(nn.Module):
         for name in ("scales", "scales_and_zeros"):  # module-swapped head: the compute dtype is that of its scales
             if hasattr(self.output, name):
                 dtype = getattr(self.output, name).dtype
+        w_scale = getattr(self.output.weight, "scale", None)  # FPx weight subclass: reports float32, computes in fp16
+        if torch.is_tensor(w_scale) and dtype is torch.float32:
+            dtype = w_scale.dtype
         device = self.tok_embeddings.weight.device
         for b in self.layers:
             b.attention.kv_cache = KVCache(max_batch_size, max_seq_length, self.config.n_local_heads,

@@ -406,8 +406,9 @@ def main():
                     help="build the model, run one pass of the roofline leg and a copy kernel of known size, no decode "
                          "loop: the command to put under rocprofv3 --pmc")
     ap.add_argument("--quantization", default=None,
-                    help="int4wo-<group> (default: int4wo-<--group>, the headline configuration) or int8wo: the decode "
-                         "loop of the reference's other weight-only configuration, reported without the int4 roofline leg")
+                    help="int4wo-<group> (default: int4wo-<--group>, the headline configuration), int8wo or fp6 (e3m2 on an "
+                         "fp16 model): the decode loop of the reference's other weight-only configurations, reported "
+                         "without the int4 roofline leg")
     ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6", "int8"), default=None,
                     help="instead of the decode benchmark, print one line per kernel case of the named sweep")
     args = ap.parse_args()
@@ -473,7 +474,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": "fp16" if quant == "fp6" else "bf16",
         "data": "synthetic",
         "config": {
             "workload": (f"{args.model}-architecture random-init (weights ~N(0,0.02), seed 1234), {quant} on every "

@@ -416,3 +416,28 @@ def test_single_row_many_row_blocks_one_hot_is_exact(oracle):
         x[0, k] = 1.0
         y = ops.int4wo_linear(x.to(dev), packed, qp, g, N, None, True).cpu().numpy()
         assert np.array_equal(y[0], dq[:, k]), k
+
+
+def test_fp6_model_decodes_eagerly_and_under_graph_capture():
+    """FP6-LLM e3m2 weights on an fp16 Llama-architecture model (the flow of torchao/prototype/quant_llm/README.md:9-20):
+    the KV cache takes the model's fp16, the module-by-module decode gives the same tokens eagerly and from a HIP graph,
+    and the logits stay close to the fp16 model's."""
+    from ao_amd._models.llama.generate import build_random_model, generate
+    from ao_amd.prototype.quant_llm import QuantLlmLinearWeight
+
+    dev = _dev()
+    model = build_random_model("tiny128", dev, "fp6")
+    ref = build_random_model("tiny128", dev).half()
+    assert isinstance(model.output.weight, QuantLlmLinearWeight) and model.tok_embeddings.weight.dtype is torch.float16
+    prompt = torch.randint(0, model.config.vocab_size, (12,), device=dev, dtype=torch.int)
+    with torch.no_grad():
+        for m in (model, ref):
+            m.setup_caches(1, 64)
+        assert model.layers[0].attention.kv_cache.k_cache.dtype is torch.float16
+        assert model.fused_decode_kind() is None
+        pos = torch.arange(12, device=dev)
+        got, want = model(prompt.view(1, -1), pos).float(), ref(prompt.view(1, -1), pos).float()
+    assert rel_l2(got.cpu().numpy(), want.cpu().numpy()) <= 0.15
+    a = generate(model, prompt, 8, use_graph=True, greedy=True)
+    b = generate(model, prompt, 8, use_graph=False, greedy=True)
+    assert torch.equal(a, b)
