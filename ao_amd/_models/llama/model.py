@@ -218,14 +218,18 @@ class Transformer(nn.Module):
                                                                  b.feed_forward.w3, b.feed_forward.w2)]
 
     def fused_decode_kind(self) -> Optional[str]:
-        """"int4" / "int8" when a batch-1 single-token step can run on the HIP decode path, else None.  int4: every
-        linear an int4 weight in the gfx950 layout with one group size; int8: every linear a per-channel int8
-        weight in the plain layout with in_features a multiple of 128; in both cases bf16 everywhere, head_dim 128,
-        caches set up for batch 1."""
+        """"int4" / "int8" / "fp6" when a batch-1 single-token step can run on the HIP decode path, else None.  int4:
+        every linear an int4 weight in the gfx950 layout with one group size; int8: every linear a per-channel int8
+        weight in the plain layout with in_features a multiple of 128, both with bf16 everywhere; fp6: every linear an
+        FPx weight on an fp16 model; in all cases head_dim 128 and caches set up for batch 1."""
         from ...dtypes.affine_quantized_tensor import AffineQuantizedTensor, Gfx950WaveTiledAQTLayout, PlainAQTLayout
 
         if self.freqs_cis is None or self.max_batch_size != 1 or self.config.head_dim != 128 \
-                or self.max_seq_length > 16384 or self.tok_embeddings.weight.dtype is not torch.bfloat16:
+                or self.max_seq_length > 16384:
+            return None
+        if self.tok_embeddings.weight.dtype is torch.float16:
+            return "fp6" if self._fp6_decode_ready() else None
+        if self.tok_embeddings.weight.dtype is not torch.bfloat16:
             return None
         kinds, groups = set(), set()
         for lin in self._decode_linears():
@@ -248,6 +252,15 @@ class Transformer(nn.Module):
         if kinds == {"int4"} and len(groups) == 1 and self.config.intermediate_size % 16 == 0:
             return "int4"
         return "int8" if kinds == {"int8"} else None
+
+    def _fp6_decode_ready(self) -> bool:
+        from ...prototype.quant_llm import QuantLlmLinearWeight
+
+        for lin in self._decode_linears():
+            if not isinstance(lin, nn.Linear) or lin.bias is not None or not isinstance(lin.weight, QuantLlmLinearWeight) \
+                    or not lin.weight.fpx_data.is_cuda or lin.weight.scale.dtype is not torch.float16:
+                return False
+        return self.freqs_cis.dtype is torch.float16
 
     def fused_decode_ready(self) -> bool:
         return self.fused_decode_kind() is not None
@@ -346,6 +359,33 @@ class Transformer(nn.Module):
             x = lin(act, ffn.w2, residual=h)
         return lin(x, self.output, norm=self.norm).view(1, 1, cfg.vocab_size)
 
+    def _fused_decode_fp6(self, idx: Tensor, input_pos: Tensor) -> Tensor:
+        """The same step over FPx weights on an fp16 model: the fp6 GEMV per linear with the residual add and the
+        SiLU(gate) * up product in its epilogue, and the fp16 instances of the RMSNorm and decode attention kernels
+        (8 launches per layer)."""
+        from ... import ops
+
+        cfg = self.config
+
+        def lin(x, layer, residual=None, gate=None):
+            w = layer.weight
+            if residual is None and gate is None:
+                return ops.fp6_linear_native(w.ebits, w.mbits, x, w.native(), w.scale)
+            return ops.fp6_linear_native_fused(w.ebits, w.mbits, x, w.native(), w.scale,
+                                               residual if gate is None else gate, gate is not None)
+
+        x = self.tok_embeddings(idx).view(1, cfg.dim)
+        pos = input_pos.to(torch.int32) if input_pos.dtype is not torch.int32 else input_pos
+        for b in self.layers:
+            att, ffn = b.attention, b.feed_forward
+            qkv = lin(ops.rmsnorm(x, b.attention_norm.weight, b.attention_norm.eps), att.wqkv)
+            y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
+                                           cfg.n_head, cfg.n_local_heads)
+            h = lin(y, att.wo, residual=x)
+            hn = ops.rmsnorm(h, b.ffn_norm.weight, b.ffn_norm.eps)
+            x = lin(lin(hn, ffn.w3, gate=lin(hn, ffn.w1)), ffn.w2, residual=h)
+        return lin(ops.rmsnorm(x, self.norm.weight, self.norm.eps), self.output).view(1, 1, cfg.vocab_size)
+
     def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None) -> Tensor:
         assert self.freqs_cis is not None, "Caches must be initialized first"
         if self.use_fused_decode and idx.numel() == 1 and input_pos is not None and input_pos.numel() == 1:
@@ -354,6 +394,8 @@ class Transformer(nn.Module):
                 return self._fused_decode(idx, input_pos)
             if kind == "int8":
                 return self._fused_decode_int8(idx, input_pos)
+            if kind == "fp6":
+                return self._fused_decode_fp6(idx, input_pos)
         mask = self.causal_mask[None, None, input_pos]
         freqs_cis = self.freqs_cis[input_pos]
         x = self.tok_embeddings(idx)

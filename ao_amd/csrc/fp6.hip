@@ -236,7 +236,9 @@ template <int WAVES, bool E3M2>
 __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
                                                                  const uint32_t* __restrict__ native,
                                                                  const uint16_t* __restrict__ scale, int64_t N, int64_t Kp,
-                                                                 uint16_t* __restrict__ out) {
+                                                                 uint16_t* __restrict__ out,
+                                                                 const uint16_t* __restrict__ residual,
+                                                                 const uint16_t* __restrict__ gate) {
     __shared__ float red[WAVES][4][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -323,7 +325,16 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* 
 #pragma unroll
             for (int w = 0; w < WAVES; ++w) s += red[w][i][lane];
             const int64_t m = m0 + 4 * qd + i;
-            if (m < M && n < N) out[m * N + n] = f32_to_f16_bits(s);
+            if (m < M && n < N) {
+                // the module's next elementwise op on the fp16 result, fused: h + linear(...) or silu(gate) * linear(...)
+                float v = s;
+                if (residual) v = f16_bits_to_f32(f32_to_f16_bits(v)) + f16_bits_to_f32(residual[m * N + n]);
+                if (gate) {
+                    const float gt = f16_bits_to_f32(gate[m * N + n]);
+                    v = f16_bits_to_f32(f32_to_f16_bits(gt / (1.0f + expf(-gt)))) * f16_bits_to_f32(f32_to_f16_bits(v));
+                }
+                out[m * N + n] = f32_to_f16_bits(v);
+            }
         }
     }
 }
@@ -525,9 +536,13 @@ extern "C" int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, int nbits
     return 0;
 }
 
-extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native,
-                                 const void* scale_f16, int64_t N, int ebits, int mbits, void* out_f16, void* stream) {
+static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
+                               int64_t N, int ebits, int mbits, const void* residual_f16, const void* gate_f16,
+                               void* out_f16, void* stream) {
     AO_REQUIRE(x_f16 && weights_native && scale_f16 && out_f16, "null pointer argument");
+    AO_REQUIRE(!(residual_f16 && gate_f16), "residual and gate epilogues are exclusive");
+    AO_REQUIRE(!(residual_f16 || gate_f16) || M <= 16, "the fused epilogues exist for at most 16 activation rows, got %lld",
+               (long long)M);
     if (int rc = check_fp6_format(ebits, mbits)) return rc;
     AO_REQUIRE(K % 64 == 0, "Expected in_features to be a multiple of 64, but received %lld", (long long)K);
     AO_REQUIRE(N > 0 && N % 16 == 0, "out_features must be a positive multiple of 16, got %lld", (long long)N);
@@ -544,10 +559,12 @@ extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const 
     const uint32_t* nat = (const uint32_t*)weights_native;
     const uint16_t* sc = (const uint16_t*)scale_f16;
     uint16_t* o = (uint16_t*)out_f16;
+    const uint16_t* res = (const uint16_t*)residual_f16;
+    const uint16_t* gt = (const uint16_t*)gate_f16;
     hipEvent_t ev0 = g_prof_start, ev1 = g_prof_stop;  // optional per-kernel timing, see common.h
     g_prof_start = g_prof_stop = nullptr;
     // tiled kernel: 128 x 128 workgroup tiles when they give at least one workgroup per CU, else 64 x 64
-    if (M > 16 && K % 128 == 0) {
+    if (M > 16 && K % 128 == 0 && !res && !gt) {
         // ... and 32 x 64 tiles when even those leave CUs idle
         const bool big = ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
         const bool tiny = !big && ((RB + 3) / 4) * ((M + 63) / 64) < 192;
@@ -568,9 +585,9 @@ extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const 
     }
 #define AO_FP6_LAUNCH(W)                                                                                                 \
     if (ebits == 3)                                                                                                      \
-        hipExtLaunchKernelGGL((fp6_linear_kernel<W, true>), grid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o); \
+        hipExtLaunchKernelGGL((fp6_linear_kernel<W, true>), grid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o, res, gt); \
     else                                                                                                                 \
-        hipExtLaunchKernelGGL((fp6_linear_kernel<W, false>), grid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o)
+        hipExtLaunchKernelGGL((fp6_linear_kernel<W, false>), grid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o, res, gt)
     switch (waves) {
         case 1: AO_FP6_LAUNCH(1); break;
         case 2: AO_FP6_LAUNCH(2); break;
@@ -581,4 +598,17 @@ extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const 
 #undef AO_FP6_LAUNCH
     AO_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native,
+                                 const void* scale_f16, int64_t N, int ebits, int mbits, void* out_f16, void* stream) {
+    return fp6_linear_dispatch(x_f16, M, K, weights_native, scale_f16, N, ebits, mbits, nullptr, nullptr, out_f16, stream);
+}
+
+extern "C" int ao_amd_fp6_linear_fused(const void* x_f16, int64_t M, int64_t K, const void* weights_native,
+                                       const void* scale_f16, int64_t N, int ebits, int mbits, const void* residual_f16,
+                                       const void* gate_f16, void* out_f16, void* stream) {
+    AO_REQUIRE((residual_f16 != nullptr) != (gate_f16 != nullptr), "pass exactly one of residual and gate");
+    return fp6_linear_dispatch(x_f16, M, K, weights_native, scale_f16, N, ebits, mbits, residual_f16, gate_f16, out_f16,
+                               stream);
 }

@@ -9,10 +9,28 @@
 
 namespace ao {
 
-// out = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * w ), statistics in fp32.  One workgroup per row.
+// The 16-bit element type of the activations, weights and caches: bf16 (the int4 / int8 models) or fp16 (the FP6 model,
+// whose linear takes fp16 activations).  Conversions of single values and of the two halves of a packed dword, and the
+// rounding an op writing that dtype applies.
+struct ElemBf16 {
+    static __device__ __forceinline__ float lo(uint32_t u) { return __uint_as_float(u << 16); }
+    static __device__ __forceinline__ float hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+    static __device__ __forceinline__ float from_bits(uint16_t b) { return bf16_bits_to_f32(b); }
+    static __device__ __forceinline__ uint16_t to_bits(float f) { return f32_to_bf16_bits(f); }
+    static __device__ __forceinline__ float rne(float f) { return rne_bf16(f); }
+};
+struct ElemF16 {
+    static __device__ __forceinline__ float lo(uint32_t u) { return f16_bits_to_f32((uint16_t)(u & 0xffffu)); }
+    static __device__ __forceinline__ float hi(uint32_t u) { return f16_bits_to_f32((uint16_t)(u >> 16)); }
+    static __device__ __forceinline__ float from_bits(uint16_t b) { return f16_bits_to_f32(b); }
+    static __device__ __forceinline__ uint16_t to_bits(float f) { return f32_to_f16_bits(f); }
+    static __device__ __forceinline__ float rne(float f) { return f16_bits_to_f32(f32_to_f16_bits(f)); }
+};
+
+// out = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * w ), statistics in fp32 (or fp16 throughout).  One workgroup per row.
 // VEC: dim is a multiple of 8 and the rows are 16-byte aligned; every thread then issues all of its
 // 16-byte loads (up to 4 chunks, dim <= 8192) before the first use so the row is read in one round trip.
-template <bool VEC>
+template <bool VEC, class E>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                        int64_t dim, float eps, uint16_t* __restrict__ out) {
     __shared__ float part[4];
@@ -38,7 +56,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
             const uint32_t u[4] = {xv[c].x, xv[c].y, xv[c].z, xv[c].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float lo = __uint_as_float(u[j] << 16), hi = __uint_as_float(u[j] & 0xffff0000u);
+                const float lo = E::lo(u[j]), hi = E::hi(u[j]);
                 ss += lo * lo + hi * hi;
             }
         }
@@ -55,9 +73,9 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
                 uint32_t o[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const float lo = rne_bf16(__uint_as_float(u[j] << 16) * r) * __uint_as_float(g[j] << 16);
-                    const float hi = rne_bf16(__uint_as_float(u[j] & 0xffff0000u) * r) * __uint_as_float(g[j] & 0xffff0000u);
-                    o[j] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+                    const float lo = E::rne(E::lo(u[j]) * r) * E::lo(g[j]);
+                    const float hi = E::rne(E::hi(u[j]) * r) * E::hi(g[j]);
+                    o[j] = (uint32_t)E::to_bits(lo) | ((uint32_t)E::to_bits(hi) << 16);
                 }
                 reinterpret_cast<uint4*>(out + row * dim)[idx] = make_uint4(o[0], o[1], o[2], o[3]);
             }
@@ -65,7 +83,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
         return;
     }
     for (int64_t i = threadIdx.x; i < dim; i += 256) {
-        float v = bf16_bits_to_f32(xr[i]);
+        float v = E::from_bits(xr[i]);
         ss += v * v;
     }
     ss = wave_sum(ss);
@@ -74,8 +92,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
     const float mean = (part[0] + part[1] + part[2] + part[3]) / (float)dim;
     const float r = rsqrtf(mean + eps);
     for (int64_t i = threadIdx.x; i < dim; i += 256) {
-        float v = rne_bf16(bf16_bits_to_f32(xr[i]) * r);
-        out[row * dim + i] = f32_to_bf16_bits(v * bf16_bits_to_f32(w[i]));
+        float v = E::rne(E::from_bits(xr[i]) * r);
+        out[row * dim + i] = E::to_bits(v * E::from_bits(w[i]));
     }
 }
 
@@ -94,6 +112,7 @@ constexpr int ATT_THREADS = 1024;
 constexpr int ATT_U = 8;                 // passes per chunk
 constexpr int ATT_CHUNK = 64 * ATT_U;    // positions per chunk
 
+template <class E>
 __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uint16_t* __restrict__ qkv,
                                                                         const float* __restrict__ qkv_parts, int nparts,
                                                                         const uint16_t* __restrict__ freqs,
@@ -133,7 +152,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
         if (nparts == 0) return qkv[i];
         float t = qkv_parts[i];
         for (int p = 1; p < nparts; ++p) t += qkv_parts[p * qkv_len + i];
-        return f32_to_bf16_bits(t);
+        return E::to_bits(t);
     };
     const int64_t qp = (int64_t)h * HD, kp = (int64_t)(n_head + hk) * HD, vp = (int64_t)(n_head + n_kv + hk) * HD;
     uint16_t* kc = k_cache + (int64_t)hk * S * HD;
@@ -157,21 +176,21 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     if (tid < 128) {
         const int which = tid >> 6, i = tid & 63;   // 0: q, 1: k
         const int64_t src = which ? kp : qp;
-        const float x0 = bf16_bits_to_f32(qkv_at(src + 2 * i)), x1 = bf16_bits_to_f32(qkv_at(src + 2 * i + 1));
-        const float c = bf16_bits_to_f32(freqs[((int64_t)pos * 64 + i) * 2]);
-        const float sn = bf16_bits_to_f32(freqs[((int64_t)pos * 64 + i) * 2 + 1]);
-        const float o0 = rne_bf16(x0 * c - x1 * sn), o1 = rne_bf16(x1 * c + x0 * sn);
+        const float x0 = E::from_bits(qkv_at(src + 2 * i)), x1 = E::from_bits(qkv_at(src + 2 * i + 1));
+        const float c = E::from_bits(freqs[((int64_t)pos * 64 + i) * 2]);
+        const float sn = E::from_bits(freqs[((int64_t)pos * 64 + i) * 2 + 1]);
+        const float o0 = E::rne(x0 * c - x1 * sn), o1 = E::rne(x1 * c + x0 * sn);
         float* dst = which ? knew_s : q_s;
         dst[2 * i] = o0;
         dst[2 * i + 1] = o1;
         if (which && (h % rep) == 0 && z == 0) {
-            kc[(int64_t)pos * HD + 2 * i] = f32_to_bf16_bits(o0);
-            kc[(int64_t)pos * HD + 2 * i + 1] = f32_to_bf16_bits(o1);
+            kc[(int64_t)pos * HD + 2 * i] = E::to_bits(o0);
+            kc[(int64_t)pos * HD + 2 * i + 1] = E::to_bits(o1);
         }
     } else if (tid < 256) {
         const int i = tid - 128;
         const uint16_t v = qkv_at(vp + i);
-        vnew_s[i] = bf16_bits_to_f32(v);
+        vnew_s[i] = E::from_bits(v);
         if ((h % rep) == 0 && z == 0) vc[(int64_t)pos * HD + i] = v;
     }
     __syncthreads();
@@ -204,8 +223,8 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    d += qreg[2 * j] * __uint_as_float(w4[j] << 16);
-                    d += qreg[2 * j + 1] * __uint_as_float(w4[j] & 0xffff0000u);
+                    d += qreg[2 * j] * E::lo(w4[j]);
+                    d += qreg[2 * j + 1] * E::hi(w4[j]);
                 }
             }
             d = row16_sum(d);
@@ -260,8 +279,8 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
                     const uint32_t w4[4] = {rawv[u].x, rawv[u].y, rawv[u].z, rawv[u].w};
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        oacc[2 * j] += p * __uint_as_float(w4[j] << 16);
-                        oacc[2 * j + 1] += p * __uint_as_float(w4[j] & 0xffff0000u);
+                        oacc[2 * j] += p * E::lo(w4[j]);
+                        oacc[2 * j + 1] += p * E::hi(w4[j]);
                     }
                 }
             }
@@ -279,7 +298,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
 #pragma unroll 16
         for (int w = 0; w < 64; ++w) o += po[w * HD + tid];
         if (nsplit == 1) {
-            out[(int64_t)h * HD + tid] = f32_to_bf16_bits(o * inv);
+            out[(int64_t)h * HD + tid] = E::to_bits(o * inv);
         } else {
             float* dst = part + ((int64_t)h * nsplit + z) * (HD + 2);
             dst[2 + tid] = o;
@@ -289,6 +308,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
 }
 
 // Combines the `nsplit` partial results of one head: out = sum_z e^(m_z - M) o_z / sum_z e^(m_z - M) l_z, M = max_z m_z.
+template <class E>
 __global__ __launch_bounds__(128) void attention_merge_kernel(const float* __restrict__ part, int nsplit,
                                                               uint16_t* __restrict__ out) {
     constexpr int HD = 128;
@@ -303,7 +323,7 @@ __global__ __launch_bounds__(128) void attention_merge_kernel(const float* __res
         L += w * p[z * (HD + 2) + 1];
         o += w * p[z * (HD + 2) + 2 + d];
     }
-    out[(int64_t)h * HD + d] = f32_to_bf16_bits(o / L);
+    out[(int64_t)h * HD + d] = E::to_bits(o / L);
 }
 
 // Index of the largest of n bf16 values (the lowest such index; a NaN counts as larger than any number), for
@@ -387,26 +407,37 @@ __global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __res
 
 using namespace ao;
 
-extern "C" int ao_amd_rmsnorm_bf16(const void* x, const void* weight, int64_t rows, int64_t dim, float eps, void* out,
-                                   void* stream) {
+template <class E>
+static int rmsnorm_dispatch(const void* x, const void* weight, int64_t rows, int64_t dim, float eps, void* out, void* stream) {
     AO_REQUIRE(x && weight && out, "null pointer argument");
     AO_REQUIRE(rows >= 0 && dim > 0, "bad shape rows=%lld dim=%lld", (long long)rows, (long long)dim);
     if (rows == 0) return 0;
     const bool vec = (dim % 8 == 0) && dim <= 8192 &&
                      (((uintptr_t)x | (uintptr_t)weight | (uintptr_t)out) & 15) == 0;
     if (vec)
-        hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream,
+        hipLaunchKernelGGL((rmsnorm_kernel<true, E>), dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream,
                            (const uint16_t*)x, (const uint16_t*)weight, dim, eps, (uint16_t*)out);
     else
-        hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream,
+        hipLaunchKernelGGL((rmsnorm_kernel<false, E>), dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream,
                            (const uint16_t*)x, (const uint16_t*)weight, dim, eps, (uint16_t*)out);
     AO_LAUNCH_CHECK();
     return 0;
 }
 
+extern "C" int ao_amd_rmsnorm_bf16(const void* x, const void* weight, int64_t rows, int64_t dim, float eps, void* out,
+                                   void* stream) {
+    return rmsnorm_dispatch<ElemBf16>(x, weight, rows, dim, eps, out, stream);
+}
+
+extern "C" int ao_amd_rmsnorm_f16(const void* x, const void* weight, int64_t rows, int64_t dim, float eps, void* out,
+                                  void* stream) {
+    return rmsnorm_dispatch<ElemF16>(x, weight, rows, dim, eps, out, stream);
+}
+
 static int attention_dispatch(const void* qkv_bf16, const void* qkv_f32_parts, int nparts, const void* freqs_cis_bf16,
                               const int32_t* pos_dev, void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim,
-                              int64_t max_seq, int nsplit, void* workspace_f32, void* out_bf16, void* stream) {
+                              int64_t max_seq, int nsplit, void* workspace_f32, void* out_bf16, void* stream,
+                              bool f16 = false) {
     AO_REQUIRE((qkv_bf16 || qkv_f32_parts) && freqs_cis_bf16 && pos_dev && k_cache && v_cache && out_bf16,
                "null pointer argument");
     AO_REQUIRE(head_dim == 128, "decode attention kernel is built for head_dim 128, got %d", head_dim);
@@ -420,14 +451,25 @@ static int attention_dispatch(const void* qkv_bf16, const void* qkv_f32_parts, i
     AO_REQUIRE(smem <= 160 * 1024, "a cache of %lld positions over %d workgroups per head does not fit the kernel's LDS "
                "score buffer: use a larger split", (long long)max_seq, nsplit);
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)n_head, (unsigned)nsplit), dim3(ATT_THREADS), smem, st,
-                       (const uint16_t*)qkv_bf16, (const float*)qkv_f32_parts, nparts, (const uint16_t*)freqs_cis_bf16,
-                       pos_dev, (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16, nsplit,
-                       (float*)workspace_f32);
+    const dim3 grid((unsigned)n_head, (unsigned)nsplit);
+    if (f16)
+        hipLaunchKernelGGL(decode_attention_kernel<ElemF16>, grid, dim3(ATT_THREADS), smem, st, (const uint16_t*)qkv_bf16,
+                           (const float*)qkv_f32_parts, nparts, (const uint16_t*)freqs_cis_bf16, pos_dev,
+                           (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16, nsplit,
+                           (float*)workspace_f32);
+    else
+        hipLaunchKernelGGL(decode_attention_kernel<ElemBf16>, grid, dim3(ATT_THREADS), smem, st, (const uint16_t*)qkv_bf16,
+                           (const float*)qkv_f32_parts, nparts, (const uint16_t*)freqs_cis_bf16, pos_dev,
+                           (uint16_t*)k_cache, (uint16_t*)v_cache, n_head, n_kv, max_seq, (uint16_t*)out_bf16, nsplit,
+                           (float*)workspace_f32);
     AO_LAUNCH_CHECK();
     if (nsplit > 1) {
-        hipLaunchKernelGGL(attention_merge_kernel, dim3((unsigned)n_head), dim3(128), 0, st, (const float*)workspace_f32,
-                           nsplit, (uint16_t*)out_bf16);
+        if (f16)
+            hipLaunchKernelGGL(attention_merge_kernel<ElemF16>, dim3((unsigned)n_head), dim3(128), 0, st,
+                               (const float*)workspace_f32, nsplit, (uint16_t*)out_bf16);
+        else
+            hipLaunchKernelGGL(attention_merge_kernel<ElemBf16>, dim3((unsigned)n_head), dim3(128), 0, st,
+                               (const float*)workspace_f32, nsplit, (uint16_t*)out_bf16);
         AO_LAUNCH_CHECK();
     }
     return 0;
@@ -458,6 +500,15 @@ extern "C" int ao_amd_llama_decode_attention_split(const void* qkv_bf16, const v
     AO_REQUIRE(qkv_bf16 || (nparts >= 1 && nparts <= 8), "number of partial rows %d outside [1, 8]", nparts);
     return attention_dispatch(qkv_bf16, qkv_f32_parts, qkv_bf16 ? 0 : nparts, freqs_cis_bf16, pos_dev, k_cache, v_cache,
                               n_head, n_kv, head_dim, max_seq, nsplit, workspace_f32, out_bf16, stream);
+}
+
+extern "C" int ao_amd_llama_decode_attention_f16(const void* qkv_f16, const void* freqs_cis_f16, const int32_t* pos_dev,
+                                                 void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim,
+                                                 int64_t max_seq, int nsplit, void* workspace_f32, void* out_f16,
+                                                 void* stream) {
+    AO_REQUIRE(qkv_f16, "null pointer argument");
+    return attention_dispatch(qkv_f16, nullptr, 0, freqs_cis_f16, pos_dev, k_cache, v_cache, n_head, n_kv, head_dim, max_seq,
+                              nsplit, workspace_f32, out_f16, stream, true);
 }
 
 extern "C" int ao_amd_argmax_bf16(const void* x_bf16, int64_t n, int32_t* out_index, void* stream) {

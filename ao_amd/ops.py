@@ -63,6 +63,7 @@ _LIB.define("fp6_quantize_pack(Tensor w, int ebits, int mbits) -> (Tensor, Tenso
 _LIB.define("fp6_dequantize(Tensor fpx_data, Tensor? scale, int ebits, int mbits) -> Tensor")
 _LIB.define("fp6_repack(Tensor fpx_data, int nbits=6) -> Tensor")
 _LIB.define("fp6_linear_native(int ebits, int mbits, Tensor x, Tensor native, Tensor scale) -> Tensor")
+_LIB.define("fp6_linear_native_fused(int ebits, int mbits, Tensor x, Tensor native, Tensor scale, Tensor other, bool gated) -> Tensor")
 
 
 # Activation rows from which the int4 linear dequantizes the weight once and calls the library bf16 GEMM.
@@ -435,12 +436,14 @@ def _hqq_dequantize_cuda(packed_2xint4, scales, zeros, group_size):
 
 def _rmsnorm_cuda(x, weight, eps):
     require_cuda(x, weight)
-    torch._check(x.dtype is torch.bfloat16 and weight.dtype is torch.bfloat16, lambda: "rmsnorm needs bfloat16 tensors")
+    torch._check(x.dtype in (torch.bfloat16, torch.float16) and weight.dtype is x.dtype,
+                 lambda: "rmsnorm needs bfloat16 or float16 tensors of one dtype")
     dim = x.shape[-1]
     torch._check(weight.numel() == dim, lambda: "weight size does not match the last dimension")
     xc = x.contiguous()
     out = torch.empty_like(xc)
-    check(lib().ao_amd_rmsnorm_bf16(xc.data_ptr(), weight.contiguous().data_ptr(), xc.numel() // dim, dim, float(eps),
+    fn = lib().ao_amd_rmsnorm_bf16 if x.dtype is torch.bfloat16 else lib().ao_amd_rmsnorm_f16
+    check(fn(xc.data_ptr(), weight.contiguous().data_ptr(), xc.numel() // dim, dim, float(eps),
                                     out.data_ptr(), current_stream(x.device)))
     return out
 
@@ -462,8 +465,32 @@ def decode_attention_splits(max_seq: int) -> int:
     return 4 if max_seq <= 4096 else (8 if max_seq <= 8192 else 16)
 
 
+def _decode_attention_f16_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv):
+    """The fp16 instance of the decode attention (FP6 model): every tensor float16."""
+    torch._check(k_cache.dtype is torch.float16 and v_cache.dtype is torch.float16 and freqs_cis.dtype is torch.float16,
+                 lambda: "float16 decode attention needs float16 caches and freqs_cis")
+    torch._check(input_pos.dtype is torch.int32 and input_pos.numel() == 1, lambda: "input_pos must be one int32")
+    torch._check(k_cache.dim() == 4 and k_cache.shape[0] == 1 and k_cache.shape[1] == n_kv and k_cache.is_contiguous()
+                 and v_cache.shape == k_cache.shape and v_cache.is_contiguous(),
+                 lambda: "caches must be contiguous [1, n_kv, max_seq, head_dim]")
+    head_dim, max_seq = k_cache.shape[3], k_cache.shape[2]
+    torch._check(freqs_cis.is_contiguous() and freqs_cis.shape[-2:] == (head_dim // 2, 2), lambda: "bad freqs_cis shape")
+    torch._check(qkv.numel() == (n_head + 2 * n_kv) * head_dim and qkv.is_contiguous(),
+                 lambda: "qkv must be the contiguous fused projection of one token")
+    out = torch.empty((1, n_head * head_dim), dtype=torch.float16, device=qkv.device)
+    nsplit = decode_attention_splits(max_seq)
+    work = torch.empty(n_head * nsplit * (head_dim + 2), dtype=torch.float32, device=qkv.device) if nsplit > 1 else None
+    check(lib().ao_amd_llama_decode_attention_f16(qkv.data_ptr(), freqs_cis.data_ptr(), input_pos.data_ptr(),
+                                                  k_cache.data_ptr(), v_cache.data_ptr(), n_head, n_kv, head_dim, max_seq,
+                                                  nsplit, None if work is None else work.data_ptr(), out.data_ptr(),
+                                                  current_stream(qkv.device)))
+    return out
+
+
 def _decode_attention_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv):
     require_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache)
+    if qkv.dtype is torch.float16:
+        return _decode_attention_f16_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, n_kv)
     torch._check(qkv.dtype in (torch.bfloat16, torch.float32) and k_cache.dtype is torch.bfloat16
                  and v_cache.dtype is torch.bfloat16 and freqs_cis.dtype is torch.bfloat16,
                  lambda: "decode attention needs bfloat16 tensors (or fp32 partial rows for qkv)")
@@ -572,6 +599,24 @@ def _fp6_linear_native_cuda(ebits, mbits, x, native, scale):
     return out
 
 
+def _fp6_linear_native_fused_cuda(ebits, mbits, x, native, scale, other, gated):
+    """fp16(linear) + other (gated = False) or silu(other) * fp16(linear) (gated = True) in one launch; at most 16 rows."""
+    require_cuda(x, native, scale, other)
+    _check_fp6_format(ebits, mbits)
+    torch._check(x.dim() == 2 and x.dtype is torch.float16, lambda: "input must be a 2d FP16 tensor")
+    torch._check(scale.dim() == 1 and scale.dtype is torch.float16, lambda: "scale must be a 1d FP16 tensor")
+    M, K = x.shape
+    N = scale.shape[0]
+    torch._check(native.dtype is torch.int32 and native.numel() == _fp6_native_numel(N, K), lambda: "Dimensions mismatched")
+    torch._check(other.dtype is torch.float16 and tuple(other.shape) == (M, N) and other.is_contiguous(),
+                 lambda: "the fused operand must be a contiguous FP16 [M, N] tensor")
+    out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    check(lib().ao_amd_fp6_linear_fused(x.contiguous().data_ptr(), M, K, native.data_ptr(), scale.contiguous().data_ptr(), N,
+                                        ebits, mbits, None if gated else other.data_ptr(),
+                                        other.data_ptr() if gated else None, out.data_ptr(), current_stream(x.device)))
+    return out
+
+
 # quant_llm_linear takes the TC-FPx bytes on every call (torchao/ops.py:15-37); the kernel wants the native
 # order, so the repack is cached per weight tensor object (weak reference) and version counter.  A new tensor
 # object, even one that reuses a freed address, never hits a stale entry.
@@ -601,6 +646,7 @@ _LIB.impl("fp6_quantize_pack", _fp6_quantize_pack_cuda, "CUDA")
 _LIB.impl("fp6_dequantize", _fp6_dequantize_cuda, "CUDA")
 _LIB.impl("fp6_repack", _fp6_repack_cuda, "CUDA")
 _LIB.impl("fp6_linear_native", _fp6_linear_native_cuda, "CUDA")
+_LIB.impl("fp6_linear_native_fused", _fp6_linear_native_fused_cuda, "CUDA")
 _LIB.impl("quant_llm_linear", _quant_llm_linear_cuda, "CUDA")
 _LIB.impl("int4wo_linear_residual", _linear_residual_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu", _swiglu_cuda, "CUDA")
@@ -633,7 +679,7 @@ def _no_cpu(name):
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
               "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int4wo_linear_partials", "int4wo_interleave_pair",
               "int4wo_swiglu_interleaved", "int8wo_linear", "int8wo_linear_fused", "int8wo_rmsnorm_linear", "int8wo_swiglu", "hqq_dequantize", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
-              "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native"):
+              "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native", "fp6_linear_native_fused"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
 
@@ -781,6 +827,11 @@ def _(fpx_data, nbits=6):
     return fpx_data.new_empty((_fp6_native_numel(fpx_data.shape[0], fpx_data.shape[1] // nbits * 8),), dtype=torch.int32)
 
 
+@torch.library.register_fake("torchao::fp6_linear_native_fused")
+def _(ebits, mbits, x, native, scale, other, gated):
+    return x.new_empty((x.shape[0], scale.shape[0]), dtype=torch.float16)
+
+
 @torch.library.register_fake("torchao::fp6_linear_native")
 def _(ebits, mbits, x, native, scale):
     return x.new_empty((x.shape[0], scale.shape[0]))
@@ -815,6 +866,12 @@ def fp6_repack(fpx_data: Tensor, nbits: int = 6) -> Tensor:
 def fp6_linear_native(ebits: int, mbits: int, x: Tensor, native: Tensor, scale: Tensor) -> Tensor:
     """x fp16 [M,K] @ W^T with W given in the native tile order -> fp16 [M,N]."""
     return torch.ops.torchao.fp6_linear_native.default(ebits, mbits, x, native, scale)
+
+
+def fp6_linear_native_fused(ebits: int, mbits: int, x: Tensor, native: Tensor, scale: Tensor, other: Tensor,
+                            gated: bool) -> Tensor:
+    """fp16(fp6 linear) + other, or silu(other) * fp16(fp6 linear) when gated; at most 16 rows, one launch."""
+    return torch.ops.torchao.fp6_linear_native_fused.default(ebits, mbits, x, native, scale, other, gated)
 
 
 def int4wo_linear_residual(x, packed, qparams, group_size, N, residual, bias=None):
@@ -890,7 +947,7 @@ def int8wo_linear_gated(x: Tensor, w_int8: Tensor, scale: Tensor, gate: Tensor) 
 
 
 def rmsnorm(x, weight, eps: float):
-    """RMSNorm over the last dimension of a bf16 tensor."""
+    """RMSNorm over the last dimension of a bf16 or fp16 tensor."""
     return torch.ops.torchao.rmsnorm.default(x, weight, eps)
 
 

@@ -245,6 +245,14 @@ int ao_amd_llama_decode_attention_split(const void* qkv_bf16, const void* qkv_f3
                                         int n_head, int n_kv, int head_dim, int64_t max_seq, int nsplit,
                                         void* workspace_f32, void* out_bf16, void* stream);
 
+/* The same two harness kernels over fp16 activations, weights and caches, for the FP6 model (whose linear takes fp16):
+ * RMSNorm.forward and Attention.forward as above, every rounding to fp16 instead of bf16.  The attention entry takes
+ * the context split directly (nsplit = 1 and a null workspace for short caches). */
+int ao_amd_rmsnorm_f16(const void* x, const void* weight, int64_t rows, int64_t dim, float eps, void* out, void* stream);
+int ao_amd_llama_decode_attention_f16(const void* qkv_f16, const void* freqs_cis_f16, const int32_t* pos_dev, void* k_cache,
+                                      void* v_cache, int n_head, int n_kv, int head_dim, int64_t max_seq, int nsplit,
+                                      void* workspace_f32, void* out_f16, void* stream);
+
 /* out_index[0] = index of the largest of n bf16 values (lowest index among equals; NaN counts as largest): the greedy
  * branch of `sample` in the decode harness, torch.argmax over the last position's logits
  * (torchao/_models/llama/generate.py:34-53 samples from the same logits row). */
@@ -283,6 +291,14 @@ int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, int nbits, void* nat
  * torchao/csrc/cuda/fp6_llm/fp6_linear.cu:139-196.  `weights_native` is the output of ao_amd_fp6_repack. */
 int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
                       int64_t N, int ebits, int mbits, void* out_f16, void* stream);
+
+/* The same linear for at most 16 activation rows with the module's next elementwise op on its fp16 result fused into the
+ * epilogue (exactly one of the two operands, fp16 [M, N], is non-null): out = fp16(linear) + residual (h + attention(...),
+ * h + feed_forward(...), TransformerBlock.forward, torchao/_models/llama/model.py:160-163) or
+ * out = fp16(silu(gate)) * fp16(linear) (F.silu(self.w1(x)) * self.w3(x), FeedForward.forward, :209-214). */
+int ao_amd_fp6_linear_fused(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
+                            int64_t N, int ebits, int mbits, const void* residual_f16, const void* gate_f16, void* out_f16,
+                            void* stream);
 
 /* Measurement aid (no counterpart in the reference): arm a (hipEvent_t start, hipEvent_t stop) pair on the
  * calling thread; the next linear launch (int4wo or fp6) records its kernel's own begin / end timestamps into

@@ -420,8 +420,9 @@ def test_single_row_many_row_blocks_one_hot_is_exact(oracle):
 
 def test_fp6_model_decodes_eagerly_and_under_graph_capture():
     """FP6-LLM e3m2 weights on an fp16 Llama-architecture model (the flow of torchao/prototype/quant_llm/README.md:9-20):
-    the KV cache takes the model's fp16, the module-by-module decode gives the same tokens eagerly and from a HIP graph,
-    and the logits stay close to the fp16 model's."""
+    the KV cache takes the model's fp16; the fused fp16 decode step (fp6 GEMVs with fused epilogues, fp16 RMSNorm and
+    attention kernels) against the module-by-module forward; the same tokens eagerly and from a HIP graph; logits close
+    to the fp16 model's."""
     from ao_amd._models.llama.generate import build_random_model, generate
     from ao_amd.prototype.quant_llm import QuantLlmLinearWeight
 
@@ -434,10 +435,60 @@ def test_fp6_model_decodes_eagerly_and_under_graph_capture():
         for m in (model, ref):
             m.setup_caches(1, 64)
         assert model.layers[0].attention.kv_cache.k_cache.dtype is torch.float16
-        assert model.fused_decode_kind() is None
+        assert model.fused_decode_kind() == "fp6" and ref.fused_decode_kind() is None
         pos = torch.arange(12, device=dev)
         got, want = model(prompt.view(1, -1), pos).float(), ref(prompt.view(1, -1), pos).float()
-    assert rel_l2(got.cpu().numpy(), want.cpu().numpy()) <= 0.15
+        assert rel_l2(got.cpu().numpy(), want.cpu().numpy()) <= 0.15
+        tok = torch.tensor([[7]], device=dev, dtype=torch.int)
+        p = torch.tensor([12], device=dev, dtype=torch.int)
+        model.use_fused_decode = False
+        unfused = model(tok, p).float()
+        k_unfused = model.layers[1].attention.kv_cache.k_cache[0, :, 12].clone()
+        model.use_fused_decode = True
+        fused = model(tok, p).float()
+        assert torch.equal(model.layers[1].attention.kv_cache.k_cache[0, :, 12], k_unfused) or rel_l2(
+            model.layers[1].attention.kv_cache.k_cache[0, :, 12].float().cpu().numpy(), k_unfused.float().cpu().numpy()) <= 5e-3
+    assert rel_l2(fused.cpu().numpy(), unfused.cpu().numpy()) <= 2e-2
     a = generate(model, prompt, 8, use_graph=True, greedy=True)
     b = generate(model, prompt, 8, use_graph=False, greedy=True)
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 4096), (3, 512), (2, 1000)])
+def test_rmsnorm_fp16_matches_the_module_formula(rows, dim):
+    """bit for bit `(x.float() * rsqrt(mean(x^2) + eps)).half() * w` (RMSNorm.forward on an fp16 model), up to elements
+    where the kernel's sum of squares (another order) moves the scale by an fp32 ulp."""
+    from ao_amd import ops
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(rows + dim)
+    x = (torch.randn(rows, dim, generator=g) * 2).half().to(dev)
+    w = (1 + 0.1 * torch.randn(dim, generator=g)).half().to(dev)
+    xf = x.float()
+    want = (xf * torch.rsqrt(torch.mean(xf * xf, dim=-1, keepdim=True) + 1e-5)).half() * w
+    got = ops.rmsnorm(x, w, 1e-5)
+    assert got.dtype is torch.float16 and got.shape == want.shape
+    diff = (got != want).sum().item()
+    assert diff <= 0.002 * got.numel() + 1 and rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 1e-3
+
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+def test_fp6_fused_epilogues_match_the_module_chain(M):
+    from ao_amd import ops
+
+    dev = _dev()
+    N, K = 256, 512
+    g = torch.Generator().manual_seed(M)
+    w = (torch.randn(N, K, generator=g) * 0.05).half().to(dev)
+    data, scale = ops.fp6_quantize_pack(w, 3, 2)
+    native = ops.fp6_repack(data, 6)
+    x = torch.randn(M, K, generator=g).half().to(dev)
+    other = torch.randn(M, N, generator=g).half().to(dev)
+    y = ops.fp6_linear_native(3, 2, x, native, scale)
+    assert torch.equal(ops.fp6_linear_native_fused(3, 2, x, native, scale, other, False), other + y)
+    got = ops.fp6_linear_native_fused(3, 2, x, native, scale, other, True).float().cpu().numpy()
+    want = (torch.nn.functional.silu(other) * y).float().cpu().numpy()
+    assert np.count_nonzero(got != want) <= 0.002 * got.size + 1 and rel_l2(got, want) <= 1e-3
+    with pytest.raises(Exception, match="at most 16"):
+        ops.fp6_linear_native_fused(3, 2, torch.zeros(17, K, dtype=torch.float16, device=dev), native, scale,
+                                    torch.zeros(17, N, dtype=torch.float16, device=dev), False)
