@@ -360,31 +360,32 @@ class Transformer(nn.Module):
         return lin(x, self.output, norm=self.norm).view(1, 1, cfg.vocab_size)
 
     def _fused_decode_fp6(self, idx: Tensor, input_pos: Tensor) -> Tensor:
-        """The same step over FPx weights on an fp16 model: the fp6 GEMV per linear with the residual add and the
-        SiLU(gate) * up product in its epilogue, and the fp16 instances of the RMSNorm and decode attention kernels
-        (8 launches per layer)."""
+        """The same step over FPx weights on an fp16 model: the fp6 GEMV per linear with each RMSNorm fused into the
+        staging of the linear it feeds, the residual add in the epilogue, w1 and w3 in one launch with the
+        SiLU(gate) * up product, and the fp16 instance of the decode attention kernel (5 launches per layer)."""
         from ... import ops
 
         cfg = self.config
 
-        def lin(x, layer, residual=None, gate=None):
+        def lin(x, layer, residual=None, norm=None):
             w = layer.weight
-            if residual is None and gate is None:
-                return ops.fp6_linear_native(w.ebits, w.mbits, x, w.native(), w.scale)
-            return ops.fp6_linear_native_fused(w.ebits, w.mbits, x, w.native(), w.scale,
-                                               residual if gate is None else gate, gate is not None)
+            if norm is not None:
+                return ops.fp6_rmsnorm_linear(w.ebits, w.mbits, x, norm.weight, norm.eps, w.native(), w.scale)
+            return ops.fp6_linear_native_fused(w.ebits, w.mbits, x, w.native(), w.scale, residual, False)
 
         x = self.tok_embeddings(idx).view(1, cfg.dim)
         pos = input_pos.to(torch.int32) if input_pos.dtype is not torch.int32 else input_pos
         for b in self.layers:
             att, ffn = b.attention, b.feed_forward
-            qkv = lin(ops.rmsnorm(x, b.attention_norm.weight, b.attention_norm.eps), att.wqkv)
+            qkv = lin(x, att.wqkv, norm=b.attention_norm)
             y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
                                            cfg.n_head, cfg.n_local_heads)
             h = lin(y, att.wo, residual=x)
-            hn = ops.rmsnorm(h, b.ffn_norm.weight, b.ffn_norm.eps)
-            x = lin(lin(hn, ffn.w3, gate=lin(hn, ffn.w1)), ffn.w2, residual=h)
-        return lin(ops.rmsnorm(x, self.norm.weight, self.norm.eps), self.output).view(1, 1, cfg.vocab_size)
+            g, u = ffn.w1.weight, ffn.w3.weight
+            act = ops.fp6_swiglu(g.ebits, g.mbits, h, g.native(), g.scale, u.native(), u.scale, b.ffn_norm.weight,
+                                 b.ffn_norm.eps)
+            x = lin(act, ffn.w2, residual=h)
+        return lin(x, self.output, norm=self.norm).view(1, 1, cfg.vocab_size)
 
     def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None) -> Tensor:
         assert self.freqs_cis is not None, "Caches must be initialized first"

@@ -339,6 +339,234 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* 
     }
 }
 
+// ---------------------------------------------------------------- skinny path (at most 16 rows staged in LDS)
+// The decode shapes.  The workgroup copies its activation rows into LDS once (zero-filled to the tile boundary,
+// optionally through RMSNorm), so the tile loop touches global memory for weights only, and the weight stream runs
+// through a ring of D tile buffers: inline-asm loads with explicit vmcnt waits keep D - 1 tiles in flight per wave (the
+// compiler does not keep a count across such a ring and would drain it before every tile).  The waits have no register
+// operands; the one consumer of loaded registers is the asm volatile conversion below, and volatile blocks keep their
+// program order.  DUAL streams two weights (w1, w3) against the one staged block for SwiGLU in one launch.
+struct Fp6GemvArgs {
+    const uint16_t* x; int64_t M, K, Kp;
+    const uint32_t* native; const uint16_t* scale; int64_t N;
+    uint16_t* out;
+    const uint16_t* residual;   // out = fp16(linear) + residual, or null
+    const uint16_t* gate;       // out = fp16(silu(gate)) * fp16(linear), or null
+    const uint16_t* norm_w; float norm_eps;   // RMSNorm weight [K] applied while staging, or null
+    const uint32_t* native_up; const uint16_t* scale_up;  // DUAL: second weight of the same shape and its scales
+};
+
+typedef uint32_t u32x4v_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2v_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ u32x4v_t fp6_stream_lo(const void* sbase, uint32_t voff) {
+    u32x4v_t v;
+    asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    return v;
+}
+__device__ __forceinline__ u32x2v_t fp6_stream_hi(const void* sbase, uint32_t voff) {
+    u32x2v_t v;
+    asm volatile("global_load_dwordx2 %0, %1, %2 offset:1024 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    return v;
+}
+template <int COUNT>
+__device__ __forceinline__ void fp6_stream_wait() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(COUNT) : "memory");
+}
+template <bool E3M2>
+__device__ __forceinline__ f16x32_t fp6_convert_ordered(const u32x6_t& packed) {
+    f16x32_t v;
+    if (E3M2) asm volatile("v_cvt_scalef32_pk32_f16_bf6 %0, %1, 1.0" : "=&v"(v) : "v"(packed));
+    else asm volatile("v_cvt_scalef32_pk32_f16_fp6 %0, %1, 1.0" : "=&v"(v) : "v"(packed));
+    return v;
+}
+
+template <int WAVES, bool E3M2, bool DUAL>
+__global__ __launch_bounds__(WAVES * 64) void fp6_gemv_kernel(const Fp6GemvArgs a) {
+    __shared__ float red[DUAL ? 2 : 1][WAVES][4][64];
+    extern __shared__ __align__(16) uint16_t xs[];  // [rows][Kp] fp16
+    __shared__ __align__(16) uint4 zero_s[4];
+    __shared__ float norm_part[WAVES];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, qd = lane >> 4;
+    const int64_t rb = blockIdx.x, m0 = (int64_t)blockIdx.y * 16;
+    const int KB = (int)(a.Kp / 128);
+    const char* tiles = reinterpret_cast<const char*>(a.native + rb * KB * 384);
+    const char* tiles_up = reinterpret_cast<const char*>((DUAL ? a.native_up : a.native) + rb * KB * 384);
+    const uint32_t vlo = lane * 16, vhi = lane * 8;
+    union { uint16_t h; _Float16 f; } sc, sc_up;
+    sc.h = a.scale[rb * 16 + r];
+    sc_up.h = DUAL ? a.scale_up[rb * 16 + r] : sc.h;
+    const f16x2_t sc2 = {sc.f, sc.f}, sc2_up = {sc_up.f, sc_up.f};
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc_up = {0.f, 0.f, 0.f, 0.f};
+
+    const bool xact = (m0 + r) < a.M;
+    const char* xs_lane = xact ? reinterpret_cast<const char*>(xs + (int64_t)r * a.Kp + qd * 32)
+                               : reinterpret_cast<const char*>(zero_s);
+    const int xs_step = xact ? 256 : 0;  // bytes per K tile
+
+    constexpr int D = 4;
+    constexpr int LPT = DUAL ? 4 : 2;  // loads per tile
+    struct Buf { u32x4v_t lo; u32x2v_t hi; };
+    Buf buf[D], buf_up[D];  // (a ring per weight: one struct holding both made the compiler split it into bytes)
+    const int nt = wave < KB ? (KB - wave + WAVES - 1) / WAVES : 0;
+    auto load_w = [&](int slot, int kb) {
+        buf[slot].lo = fp6_stream_lo(tiles + (int64_t)kb * 1536, vlo);
+        buf[slot].hi = fp6_stream_hi(tiles + (int64_t)kb * 1536, vhi);
+        if (DUAL) {
+            buf_up[slot].lo = fp6_stream_lo(tiles_up + (int64_t)kb * 1536, vlo);
+            buf_up[slot].hi = fp6_stream_hi(tiles_up + (int64_t)kb * 1536, vhi);
+        }
+    };
+    auto wait_w = [&](int younger) {
+        if (younger >= 3) fp6_stream_wait<3 * LPT>();
+        else if (younger == 2) fp6_stream_wait<2 * LPT>();
+        else if (younger == 1) fp6_stream_wait<LPT>();
+        else fp6_stream_wait<0>();
+    };
+    auto mma_tile = [&](const u32x4v_t& lo, const u32x2v_t& hi, const f16x2_t& s2, int kb, f32x4_t& c) {
+        const u32x6_t packed = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y};
+        const f16x32_t v = fp6_convert_ordered<E3M2>(packed);
+        const uint4* xl = reinterpret_cast<const uint4*>(xs_lane + (int64_t)kb * xs_step);
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            union { f16x2_t p[4]; f16x8_t v; } w;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f16x2_t pr = {v[sl * 8 + 2 * j], v[sl * 8 + 2 * j + 1]};
+                w.p[j] = pr * s2;  // fp16(fp6 * scale), the one rounding of the reference kernel
+            }
+            union { uint4 q; f16x8_t v; } xa;
+            xa.q = xl[sl];
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa.v, w.v, c, 0, 0, 0);
+        }
+    };
+    auto compute_tile = [&](int slot, int kb) {
+        mma_tile(buf[slot].lo, buf[slot].hi, sc2, kb, acc);
+        if (DUAL) mma_tile(buf_up[slot].lo, buf_up[slot].hi, sc2_up, kb, acc_up);
+    };
+    // always D - 1 tiles' worth of requests (a wave with fewer tiles asks for its last one again), on their way while
+    // the activations are staged
+#pragma unroll
+    for (int j = 0; j < D - 1; ++j) load_w(j, (nt > 0 ? wave : 0) + (j < nt ? j : (nt > 0 ? nt - 1 : 0)) * WAVES);
+
+    {
+        constexpr int T = WAVES * 64;
+        const int tid = threadIdx.x;
+        if (tid < 4) zero_s[tid] = make_uint4(0, 0, 0, 0);
+        const int rows = (int)((a.M - m0) < 16 ? (a.M - m0) : 16);
+        const int chunks = (int)(a.K / 8), chunks_p = (int)(a.Kp / 8);
+        const uint4* nrow_w = reinterpret_cast<const uint4*>(a.norm_w);
+        auto halves = [](uint32_t u, float& lo, float& hi) {
+            lo = f16_bits_to_f32((uint16_t)(u & 0xffffu));
+            hi = f16_bits_to_f32((uint16_t)(u >> 16));
+        };
+        for (int rr = 0; rr < rows; ++rr) {
+            const uint4* xrow = reinterpret_cast<const uint4*>(a.x + (m0 + rr) * a.K);
+            uint4* orow = reinterpret_cast<uint4*>(xs) + (int64_t)rr * chunks_p;
+            for (int c = chunks + tid; c < chunks_p; c += T) orow[c] = make_uint4(0, 0, 0, 0);
+            if (a.norm_w == nullptr) {
+                for (int c = tid; c < chunks; c += T) orow[c] = xrow[c];
+            } else {
+                float ss = 0.f;
+                for (int c = tid; c < chunks; c += T) {
+                    const uint4 v = xrow[c];
+                    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        float lo, hi;
+                        halves(u[j], lo, hi);
+                        ss += lo * lo + hi * hi;
+                    }
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) norm_part[wave] = ss;
+                __syncthreads();
+                float tot = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) tot += norm_part[w];
+                const float rs = rsqrtf(tot / (float)a.K + a.norm_eps);
+                // RMSNorm of one chunk (torchao/_models/llama/model.py:232-244) on fp16: fp16(fp16(x * rs) * w)
+                for (int c = tid; c < chunks; c += T) {
+                    const uint4 v = xrow[c], g = nrow_w[c];
+                    const uint32_t u[4] = {v.x, v.y, v.z, v.w}, gw[4] = {g.x, g.y, g.z, g.w};
+                    uint32_t o[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        float lo, hi, glo, ghi;
+                        halves(u[j], lo, hi);
+                        halves(gw[j], glo, ghi);
+                        const float olo = f16_bits_to_f32(f32_to_f16_bits(lo * rs)) * glo;
+                        const float ohi = f16_bits_to_f32(f32_to_f16_bits(hi * rs)) * ghi;
+                        o[j] = (uint32_t)f32_to_f16_bits(olo) | ((uint32_t)f32_to_f16_bits(ohi) << 16);
+                    }
+                    orow[c] = make_uint4(o[0], o[1], o[2], o[3]);
+                }
+                if (rr + 1 < rows) __syncthreads();  // norm_part is rewritten for the next row
+            }
+        }
+        __syncthreads();
+    }
+
+    auto younger = [&](int i, int ahead) { return (nt - 1 - i) < ahead ? (nt - 1 - i) : ahead; };
+    int i0 = 0;
+    // steady state: every tile of the group has a tile D - 1 ahead to request; constant wait counts
+    for (; i0 + 2 * D - 1 <= nt; i0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            load_w((j + D - 1) % D, wave + (i0 + j + D - 1) * WAVES);
+            wait_w(D - 1);
+            compute_tile(j, wave + (i0 + j) * WAVES);
+        }
+    }
+    for (; i0 < nt; i0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            const int i = i0 + j;
+            if (i < nt) {
+                if (i + D - 1 < nt) load_w((j + D - 1) % D, wave + (i + D - 1) * WAVES);
+                wait_w(younger(i, D - 1));
+                compute_tile(j, wave + i * WAVES);
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // duplicate requests of a short wave
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        red[0][wave][i][lane] = acc[i];
+        if (DUAL) red[DUAL ? 1 : 0][wave][i][lane] = acc_up[i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int64_t n = rb * 16 + r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float s = 0.f, s_up = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                s += red[0][w][i][lane];
+                if (DUAL) s_up += red[DUAL ? 1 : 0][w][i][lane];
+            }
+            const int64_t m = m0 + 4 * qd + i;
+            if (m < a.M && n < a.N) {
+                float v = s;
+                if (DUAL) {
+                    const float gt = f16_bits_to_f32(f32_to_f16_bits(s));
+                    v = f16_bits_to_f32(f32_to_f16_bits(gt / (1.0f + expf(-gt)))) * f16_bits_to_f32(f32_to_f16_bits(s_up));
+                }
+                if (a.residual) v = f16_bits_to_f32(f32_to_f16_bits(v)) + f16_bits_to_f32(a.residual[m * a.N + n]);
+                if (a.gate) {
+                    const float gt = f16_bits_to_f32(a.gate[m * a.N + n]);
+                    v = f16_bits_to_f32(f32_to_f16_bits(gt / (1.0f + expf(-gt)))) * f16_bits_to_f32(f32_to_f16_bits(v));
+                }
+                a.out[m * a.N + n] = f32_to_f16_bits(v);
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- GEMM path (M > 16)
 // Workgroup tile: 128 activation rows x 128 weight rows, K walked in 128-wide tiles; the same skeleton as the int4
 // GEMM.  Each of the 4 waves owns two 16-row weight blocks: it loads their native tiles (24 bytes per lane) straight
@@ -536,9 +764,22 @@ extern "C" int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, int nbits
     return 0;
 }
 
+template <bool E3M2, bool DUAL>
+static void launch_fp6_gemv(int waves, dim3 grid, size_t smem, hipStream_t st, hipEvent_t ev0, hipEvent_t ev1,
+                            const Fp6GemvArgs& a) {
+    switch (waves) {
+        case 1: hipExtLaunchKernelGGL((fp6_gemv_kernel<1, E3M2, DUAL>), grid, dim3(64), smem, st, ev0, ev1, 0, a); break;
+        case 2: hipExtLaunchKernelGGL((fp6_gemv_kernel<2, E3M2, DUAL>), grid, dim3(128), smem, st, ev0, ev1, 0, a); break;
+        case 4: hipExtLaunchKernelGGL((fp6_gemv_kernel<4, E3M2, DUAL>), grid, dim3(256), smem, st, ev0, ev1, 0, a); break;
+        case 8: hipExtLaunchKernelGGL((fp6_gemv_kernel<8, E3M2, DUAL>), grid, dim3(512), smem, st, ev0, ev1, 0, a); break;
+        default: hipExtLaunchKernelGGL((fp6_gemv_kernel<16, E3M2, DUAL>), grid, dim3(1024), smem, st, ev0, ev1, 0, a); break;
+    }
+}
+
 static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
                                int64_t N, int ebits, int mbits, const void* residual_f16, const void* gate_f16,
-                               void* out_f16, void* stream) {
+                               void* out_f16, void* stream, const void* norm_weight_f16 = nullptr, float norm_eps = 0.f,
+                               const void* native_up = nullptr, const void* scale_up_f16 = nullptr) {
     AO_REQUIRE(x_f16 && weights_native && scale_f16 && out_f16, "null pointer argument");
     AO_REQUIRE(!(residual_f16 && gate_f16), "residual and gate epilogues are exclusive");
     AO_REQUIRE(!(residual_f16 || gate_f16) || M <= 16, "the fused epilogues exist for at most 16 activation rows, got %lld",
@@ -564,6 +805,31 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
     hipEvent_t ev0 = g_prof_start, ev1 = g_prof_stop;  // optional per-kernel timing, see common.h
     g_prof_start = g_prof_stop = nullptr;
     // tiled kernel: 128 x 128 workgroup tiles when they give at least one workgroup per CU, else 64 x 64
+    // few rows: staged in LDS (at most 64 KB, and no more per wave than keeps several workgroups on a CU); worth the
+    // pass over the rows and the barrier once a wave has 4 or more K tiles to stream
+    const bool need_lds = norm_weight_f16 || native_up;
+    const int64_t xbytes = (M < 16 ? M : 16) * Kp * 2;
+    if (need_lds)
+        while (waves < 16 && xbytes > (int64_t)waves * 16 * 1024) waves *= 2;
+    const bool fits = M <= 16 && xbytes <= 64 * 1024 && xbytes <= (int64_t)waves * 16 * 1024;
+    AO_REQUIRE(!need_lds || (fits && (((uintptr_t)norm_weight_f16) & 15) == 0 && (((uintptr_t)native_up) & 15) == 0),
+               "the fused RMSNorm and the two-weight SwiGLU need at most 16 activation rows that fit in LDS (M=%lld K=%lld) "
+               "and 16-byte aligned operands", (long long)M, (long long)K);
+    AO_REQUIRE(!native_up || (scale_up_f16 && !res && !gt), "the two-weight SwiGLU takes the second weight's scales and no "
+               "other epilogue");
+    if (fits && (need_lds || KB >= 4 * waves)) {
+        Fp6GemvArgs a{xx, M, K, Kp, nat, sc, N, o, res, gt, (const uint16_t*)norm_weight_f16, norm_eps,
+                      (const uint32_t*)native_up, (const uint16_t*)scale_up_f16};
+        if (ebits == 3) {
+            if (native_up) launch_fp6_gemv<true, true>(waves, grid, (size_t)xbytes, st, ev0, ev1, a);
+            else launch_fp6_gemv<true, false>(waves, grid, (size_t)xbytes, st, ev0, ev1, a);
+        } else {
+            if (native_up) launch_fp6_gemv<false, true>(waves, grid, (size_t)xbytes, st, ev0, ev1, a);
+            else launch_fp6_gemv<false, false>(waves, grid, (size_t)xbytes, st, ev0, ev1, a);
+        }
+        AO_LAUNCH_CHECK();
+        return 0;
+    }
     if (M > 16 && K % 128 == 0 && !res && !gt) {
         // ... and 32 x 64 tiles when even those leave CUs idle
         const bool big = ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
@@ -611,4 +877,20 @@ extern "C" int ao_amd_fp6_linear_fused(const void* x_f16, int64_t M, int64_t K, 
     AO_REQUIRE((residual_f16 != nullptr) != (gate_f16 != nullptr), "pass exactly one of residual and gate");
     return fp6_linear_dispatch(x_f16, M, K, weights_native, scale_f16, N, ebits, mbits, residual_f16, gate_f16, out_f16,
                                stream);
+}
+
+extern "C" int ao_amd_fp6_rmsnorm_linear(const void* x_f16, int64_t M, int64_t K, const void* norm_weight_f16, float eps,
+                                         const void* weights_native, const void* scale_f16, int64_t N, int ebits, int mbits,
+                                         void* out_f16, void* stream) {
+    AO_REQUIRE(norm_weight_f16, "null pointer argument");
+    return fp6_linear_dispatch(x_f16, M, K, weights_native, scale_f16, N, ebits, mbits, nullptr, nullptr, out_f16, stream,
+                               norm_weight_f16, eps);
+}
+
+extern "C" int ao_amd_fp6_swiglu(const void* x_f16, int64_t M, int64_t K, const void* norm_weight_f16, float eps,
+                                 const void* native_gate, const void* scale_gate_f16, const void* native_up,
+                                 const void* scale_up_f16, int64_t N, int ebits, int mbits, void* out_f16, void* stream) {
+    AO_REQUIRE(native_up && scale_up_f16, "null pointer argument");
+    return fp6_linear_dispatch(x_f16, M, K, native_gate, scale_gate_f16, N, ebits, mbits, nullptr, nullptr, out_f16, stream,
+                               norm_weight_f16, eps, native_up, scale_up_f16);
 }

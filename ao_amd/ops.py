@@ -63,6 +63,8 @@ _LIB.define("fp6_quantize_pack(Tensor w, int ebits, int mbits) -> (Tensor, Tenso
 _LIB.define("fp6_dequantize(Tensor fpx_data, Tensor? scale, int ebits, int mbits) -> Tensor")
 _LIB.define("fp6_repack(Tensor fpx_data, int nbits=6) -> Tensor")
 _LIB.define("fp6_linear_native(int ebits, int mbits, Tensor x, Tensor native, Tensor scale) -> Tensor")
+_LIB.define("fp6_rmsnorm_linear(int ebits, int mbits, Tensor x, Tensor norm_weight, float eps, Tensor native, Tensor scale) -> Tensor")
+_LIB.define("fp6_swiglu(int ebits, int mbits, Tensor x, Tensor? norm_weight, float eps, Tensor native_gate, Tensor scale_gate, Tensor native_up, Tensor scale_up) -> Tensor")
 _LIB.define("fp6_linear_native_fused(int ebits, int mbits, Tensor x, Tensor native, Tensor scale, Tensor other, bool gated) -> Tensor")
 
 
@@ -617,6 +619,45 @@ def _fp6_linear_native_fused_cuda(ebits, mbits, x, native, scale, other, gated):
     return out
 
 
+def _check_fp6_decode_operands(x, native, scale, norm_weight):
+    torch._check(x.dim() == 2 and x.dtype is torch.float16, lambda: "input must be a 2d FP16 tensor")
+    torch._check(scale.dim() == 1 and scale.dtype is torch.float16, lambda: "scale must be a 1d FP16 tensor")
+    M, K = x.shape
+    N = scale.shape[0]
+    torch._check(native.dtype is torch.int32 and native.numel() == _fp6_native_numel(N, K), lambda: "Dimensions mismatched")
+    if norm_weight is not None:
+        torch._check(norm_weight.dtype is torch.float16 and norm_weight.numel() == K and norm_weight.is_contiguous(),
+                     lambda: "norm weight must be a contiguous FP16 vector of the input's row length")
+    return M, K, N
+
+
+def _fp6_rmsnorm_linear_cuda(ebits, mbits, x, norm_weight, eps, native, scale):
+    """fp6 linear of rmsnorm(x) in one launch; decode shapes only."""
+    require_cuda(x, norm_weight, native, scale)
+    _check_fp6_format(ebits, mbits)
+    M, K, N = _check_fp6_decode_operands(x, native, scale, norm_weight)
+    out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    check(lib().ao_amd_fp6_rmsnorm_linear(x.contiguous().data_ptr(), M, K, norm_weight.data_ptr(), float(eps),
+                                          native.data_ptr(), scale.contiguous().data_ptr(), N, ebits, mbits, out.data_ptr(),
+                                          current_stream(x.device)))
+    return out
+
+
+def _fp6_swiglu_cuda(ebits, mbits, x, norm_weight, eps, native_gate, scale_gate, native_up, scale_up):
+    """silu(linear_gate(x')) * linear_up(x') in one launch, x' = rmsnorm(x) with a norm weight; decode shapes only."""
+    require_cuda(x, norm_weight, native_gate, scale_gate, native_up, scale_up)
+    _check_fp6_format(ebits, mbits)
+    M, K, N = _check_fp6_decode_operands(x, native_gate, scale_gate, norm_weight)
+    _check_fp6_decode_operands(x, native_up, scale_up, None)
+    torch._check(scale_up.shape[0] == N, lambda: "both weights must have the same shape")
+    out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    check(lib().ao_amd_fp6_swiglu(x.contiguous().data_ptr(), M, K, None if norm_weight is None else norm_weight.data_ptr(),
+                                  float(eps), native_gate.data_ptr(), scale_gate.contiguous().data_ptr(),
+                                  native_up.data_ptr(), scale_up.contiguous().data_ptr(), N, ebits, mbits, out.data_ptr(),
+                                  current_stream(x.device)))
+    return out
+
+
 # quant_llm_linear takes the TC-FPx bytes on every call (torchao/ops.py:15-37); the kernel wants the native
 # order, so the repack is cached per weight tensor object (weak reference) and version counter.  A new tensor
 # object, even one that reuses a freed address, never hits a stale entry.
@@ -647,6 +688,8 @@ _LIB.impl("fp6_dequantize", _fp6_dequantize_cuda, "CUDA")
 _LIB.impl("fp6_repack", _fp6_repack_cuda, "CUDA")
 _LIB.impl("fp6_linear_native", _fp6_linear_native_cuda, "CUDA")
 _LIB.impl("fp6_linear_native_fused", _fp6_linear_native_fused_cuda, "CUDA")
+_LIB.impl("fp6_rmsnorm_linear", _fp6_rmsnorm_linear_cuda, "CUDA")
+_LIB.impl("fp6_swiglu", _fp6_swiglu_cuda, "CUDA")
 _LIB.impl("quant_llm_linear", _quant_llm_linear_cuda, "CUDA")
 _LIB.impl("int4wo_linear_residual", _linear_residual_cuda, "CUDA")
 _LIB.impl("int4wo_swiglu", _swiglu_cuda, "CUDA")
@@ -679,7 +722,8 @@ def _no_cpu(name):
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
               "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int4wo_linear_partials", "int4wo_interleave_pair",
               "int4wo_swiglu_interleaved", "int8wo_linear", "int8wo_linear_fused", "int8wo_rmsnorm_linear", "int8wo_swiglu", "hqq_dequantize", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
-              "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native", "fp6_linear_native_fused"):
+              "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native", "fp6_linear_native_fused", "fp6_rmsnorm_linear",
+              "fp6_swiglu"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
 
 
@@ -827,6 +871,16 @@ def _(fpx_data, nbits=6):
     return fpx_data.new_empty((_fp6_native_numel(fpx_data.shape[0], fpx_data.shape[1] // nbits * 8),), dtype=torch.int32)
 
 
+@torch.library.register_fake("torchao::fp6_rmsnorm_linear")
+def _(ebits, mbits, x, norm_weight, eps, native, scale):
+    return x.new_empty((x.shape[0], scale.shape[0]), dtype=torch.float16)
+
+
+@torch.library.register_fake("torchao::fp6_swiglu")
+def _(ebits, mbits, x, norm_weight, eps, native_gate, scale_gate, native_up, scale_up):
+    return x.new_empty((x.shape[0], scale_gate.shape[0]), dtype=torch.float16)
+
+
 @torch.library.register_fake("torchao::fp6_linear_native_fused")
 def _(ebits, mbits, x, native, scale, other, gated):
     return x.new_empty((x.shape[0], scale.shape[0]), dtype=torch.float16)
@@ -866,6 +920,19 @@ def fp6_repack(fpx_data: Tensor, nbits: int = 6) -> Tensor:
 def fp6_linear_native(ebits: int, mbits: int, x: Tensor, native: Tensor, scale: Tensor) -> Tensor:
     """x fp16 [M,K] @ W^T with W given in the native tile order -> fp16 [M,N]."""
     return torch.ops.torchao.fp6_linear_native.default(ebits, mbits, x, native, scale)
+
+
+def fp6_rmsnorm_linear(ebits: int, mbits: int, x: Tensor, norm_weight: Tensor, eps: float, native: Tensor,
+                       scale: Tensor) -> Tensor:
+    """fp6 linear of rmsnorm(x) in one launch (at most 16 rows)."""
+    return torch.ops.torchao.fp6_rmsnorm_linear.default(ebits, mbits, x, norm_weight, eps, native, scale)
+
+
+def fp6_swiglu(ebits: int, mbits: int, x: Tensor, native_gate: Tensor, scale_gate: Tensor, native_up: Tensor,
+               scale_up: Tensor, norm_weight: Optional[Tensor] = None, eps: float = 0.0) -> Tensor:
+    """silu(fp6 linear_gate(x')) * fp6 linear_up(x') in one launch, x' = rmsnorm(x) with a norm weight (at most 16 rows)."""
+    return torch.ops.torchao.fp6_swiglu.default(ebits, mbits, x, norm_weight, eps, native_gate, scale_gate, native_up,
+                                                scale_up)
 
 
 def fp6_linear_native_fused(ebits: int, mbits: int, x: Tensor, native: Tensor, scale: Tensor, other: Tensor,

@@ -300,6 +300,18 @@ int ao_amd_fp6_linear_fused(const void* x_f16, int64_t M, int64_t K, const void*
                             int64_t N, int ebits, int mbits, const void* residual_f16, const void* gate_f16, void* out_f16,
                             void* stream);
 
+/* Decode-step fusions over the same linear, for at most 16 activation rows that fit a workgroup's LDS (M * K * 2 bytes at
+ * most 64 KB): `_rmsnorm_linear` = linear(rmsnorm(x)) with rmsnorm(x) = fp16(fp16(x * rsqrt(mean(x^2) + eps)) * norm_weight)
+ * (RMSNorm.forward then the linear it feeds, torchao/_models/llama/model.py:232-244); `_swiglu` =
+ * fp16(silu(linear_gate(x'))) * linear_up(x') over two weights of one shape in one launch, x' = rmsnorm(x) when
+ * norm_weight_f16 is given, else x (FeedForward.forward, :209-214). */
+int ao_amd_fp6_rmsnorm_linear(const void* x_f16, int64_t M, int64_t K, const void* norm_weight_f16, float eps,
+                              const void* weights_native, const void* scale_f16, int64_t N, int ebits, int mbits,
+                              void* out_f16, void* stream);
+int ao_amd_fp6_swiglu(const void* x_f16, int64_t M, int64_t K, const void* norm_weight_f16, float eps,
+                      const void* native_gate, const void* scale_gate_f16, const void* native_up, const void* scale_up_f16,
+                      int64_t N, int ebits, int mbits, void* out_f16, void* stream);
+
 /* Measurement aid (no counterpart in the reference): arm a (hipEvent_t start, hipEvent_t stop) pair on the
  * calling thread; the next linear launch (int4wo or fp6) records its kernel's own begin / end timestamps into
  * the pair and disarms, so hipEventElapsedTime(start, stop) is the kernel duration free of launch gaps.

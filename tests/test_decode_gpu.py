@@ -492,3 +492,41 @@ def test_fp6_fused_epilogues_match_the_module_chain(M):
     with pytest.raises(Exception, match="at most 16"):
         ops.fp6_linear_native_fused(3, 2, torch.zeros(17, K, dtype=torch.float16, device=dev), native, scale,
                                     torch.zeros(17, N, dtype=torch.float16, device=dev), False)
+
+
+@pytest.mark.parametrize("M,N,K,fmt", [(1, 256, 512, (3, 2)), (1, 4096, 4096, (3, 2)), (1, 1024, 14336, (3, 2)),
+                                       (4, 512, 1024, (2, 3)), (16, 256, 1024, (3, 2)), (2, 256, 192, (2, 2)),
+                                       (1, 14336, 4096, (3, 1))])
+def test_fp6_staged_gemv_fusions_match_the_separate_kernels(M, N, K, fmt):
+    """The LDS-staged fp6 GEMV (weights streamed through asm-issued loads with explicit waits): plain linear identical
+    to the fp16 matmul on the dequantized weight within the kernel tolerance, fused RMSNorm against the fp16 RMSNorm
+    kernel + linear, two-weight SwiGLU against linear -> gated linear (same roundings: equal but for a few elements
+    where the norm's sum of squares rounds apart)."""
+    from ao_amd import ops
+
+    print(f"case fp6 staged M={M} N={N} K={K} fmt={fmt}", flush=True)
+    dev = _dev()
+    e, m = fmt
+    g = torch.Generator().manual_seed(M + N + K)
+    wg = (torch.randn(N, K, generator=g) * 0.05).half().to(dev)
+    wu = (torch.randn(N, K, generator=g) * 0.05).half().to(dev)
+    dg, sg = ops.fp6_quantize_pack(wg, e, m)
+    du, su = ops.fp6_quantize_pack(wu, e, m)
+    ng, nu = ops.fp6_repack(dg, 1 + e + m), ops.fp6_repack(du, 1 + e + m)
+    x = torch.randn(M, K, generator=g).half().to(dev)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).half().to(dev)
+    y = ops.fp6_linear_native(e, m, x, ng, sg)
+    ref = x.float() @ ops.fp6_dequantize(dg, sg, e, m).float().t()
+    assert rel_l2(y.float().cpu().numpy(), ref.cpu().numpy()) <= 1e-3
+    xn = ops.rmsnorm(x, nw, 1e-5)
+    want = ops.fp6_linear_native(e, m, xn, ng, sg).float().cpu().numpy()
+    got = ops.fp6_rmsnorm_linear(e, m, x, nw, 1e-5, ng, sg).float().cpu().numpy()
+    assert rel_l2(got, want) <= 2e-3 and np.count_nonzero(got != want) <= 0.02 * got.size + 1
+    want2 = ops.fp6_linear_native_fused(e, m, x, nu, su, y, True)
+    got2 = ops.fp6_swiglu(e, m, x, ng, sg, nu, su)
+    g2, w2 = got2.float().cpu().numpy(), want2.float().cpu().numpy()
+    assert rel_l2(g2, w2) <= 1e-3 and np.count_nonzero(g2 != w2) <= 0.002 * g2.size + 1
+    want3 = ops.fp6_linear_native_fused(e, m, xn, nu, su, ops.fp6_linear_native(e, m, xn, ng, sg), True)
+    got3 = ops.fp6_swiglu(e, m, x, ng, sg, nu, su, nw, 1e-5)
+    g3, w3 = got3.float().cpu().numpy(), want3.float().cpu().numpy()
+    assert rel_l2(g3, w3) <= 2e-3 and np.count_nonzero(g3 != w3) <= 0.02 * g3.size + 1
