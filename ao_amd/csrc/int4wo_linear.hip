@@ -194,6 +194,12 @@ struct LinearArgs {
                                                        // stores its fp32 partial sums at y + z * M * ldy (the consumer adds them)
     int pair8;                                         // GEMV only: rows 0-7 of every 16-row block are gate rows, rows 8-15
                                                        // the matching up rows; y[m, 8*rb + r] = silu(gate) * up, N = output rows
+    // GEMV only, derived on the host so that the 16 waves a CU starts at once do not each spend scalar issue slots on
+    // 64-bit divisions and shifts before their first load: K tiles, K tiles per blockIdx.z, bytes of one row block's
+    // packed codes and qparams, 16-byte chunks per activation row
+    int kb_total, kb_per_split;
+    uint32_t block_bytes, qblock_bytes;
+    int chunks_per_row;
 };
 
 __device__ __forceinline__ float silu_bf16(float a) {
@@ -454,9 +460,9 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, qd = lane >> 4;
-    const int64_t rb = blockIdx.x;
+    const uint32_t rb = blockIdx.x;
     const int64_t m0 = (int64_t)blockIdx.y * 16;
-    const int KB = (int)(a.Kp / 128);
+    const int KB = a.kb_total;
     const uint32_t magic = 0x43004300u;
     const bool sel_lane = qd == (r >> 2);
     const uint32_t one_bits = (r & 1) ? 0x3F800000u : 0x00003F80u;
@@ -466,10 +472,11 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     const u32x4_t sel_b = {0u, 0u, s_even, s_odd};
 
     // scalar bases of this row block's streams; per-lane offsets never change
-    const char* wbase = reinterpret_cast<const char*>(a.packed) + rb * KB * 1024;
-    const char* wbase2 = reinterpret_cast<const char*>(DUAL ? a.packed2 : a.packed) + rb * KB * 1024;
-    const char* qbase = reinterpret_cast<const char*>(a.qparams) + rb * (a.Kp / G) * 64;
-    const char* qbase2 = reinterpret_cast<const char*>(DUAL ? a.qparams2 : a.qparams) + rb * (a.Kp / G) * 64;
+    const uint64_t woffs = (uint64_t)rb * a.block_bytes, qoffs = (uint64_t)rb * a.qblock_bytes;
+    const char* wbase = reinterpret_cast<const char*>(a.packed) + woffs;
+    const char* wbase2 = reinterpret_cast<const char*>(DUAL ? a.packed2 : a.packed) + woffs;
+    const char* qbase = reinterpret_cast<const char*>(a.qparams) + qoffs;
+    const char* qbase2 = reinterpret_cast<const char*>(DUAL ? a.qparams2 : a.qparams) + qoffs;
     const uint32_t woff = lane * 16;
     // group of (tile kb, quarter qd) = (kb*128 + qd*32) / G = tile part + lane part for every G in {32..256}
     const uint32_t qoff = (uint32_t)(r + (G < 128 ? (qd * 32 / G) * 16 : 0)) * 4;
@@ -549,7 +556,7 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     }
     // K tiles of this workgroup: all of them, or the blockIdx.z-th run when K is split across workgroups;
     // tiles of this wave: kb = kb0 + i*WAVES, i = 0..nt-1; tile i lives in buf[i % D]
-    const int kbs = (KB + a.ksplit - 1) / a.ksplit;
+    const int kbs = a.kb_per_split;
     const int kbeg = (int)blockIdx.z * kbs;
     const int kcnt = KB - kbeg < kbs ? (KB - kbeg > 0 ? KB - kbeg : 0) : kbs;
     const int kb0 = kbeg + wave;
@@ -561,7 +568,7 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     constexpr int T = WAVES * 64;
     const int tid = threadIdx.x;
     const int rows = (int)((a.M - m0) < 16 ? (a.M - m0) : 16);
-    const int chunks_per_row = (int)(a.Kp / 8);
+    const int chunks_per_row = a.chunks_per_row;
     const bool fast_stage = rows == 1 && chunks_per_row <= 2 * T;
     // The early loads are unconditional (indices clamped into the row, the norm weight replaced by the row itself
     // when there is none) and so is the wait below: a register that an asm load is still filling must reach its
@@ -944,7 +951,7 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
                (long long)n_out);
     AO_REQUIRE(!residual_bf16 || ldres >= N, "residual row stride %lld smaller than N=%lld", (long long)ldres, (long long)N);
     AO_REQUIRE((((uintptr_t)packed) & 15) == 0 && (((uintptr_t)packed2) & 15) == 0, "packed buffer must be 16-byte aligned");
-    AO_REQUIRE(Kp / 128 < (1 << 23), "in_features too large: K=%lld", (long long)K);
+    AO_REQUIRE(Kp / 128 < (1 << 21), "in_features too large: K=%lld", (long long)K);
     if (M == 0) return 0;
     const bool dual = packed2 != nullptr;
     AO_REQUIRE(!dual || qparams2, "null pointer argument");
@@ -975,7 +982,9 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     LinearArgs a{(const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams,
                  (const uint4*)packed2, (const uint32_t*)qparams2, n_out, Kp, (const uint16_t*)bias_bf16,
                  (const uint16_t*)residual_bf16, ldres, y, y_dtype == AO_F32, ldy,
-                 (const uint16_t*)norm_weight_bf16, norm_eps, ksplit, pair8 ? 1 : 0};
+                 (const uint16_t*)norm_weight_bf16, norm_eps, ksplit, pair8 ? 1 : 0,
+                 (int)KB_all, (int)((KB_all + ksplit - 1) / ksplit), (uint32_t)(KB_all * 1024), (uint32_t)(Kp / g * 64),
+                 (int)(Kp / 8)};
     hipStream_t st = (hipStream_t)stream;
     // the fused RMSNorm lives in the activation staging of the GEMV kernel only
     AO_REQUIRE(!norm_weight_bf16 || (xmode == X_LDS && M <= 16 && (((uintptr_t)norm_weight_bf16) & 15) == 0),
