@@ -49,6 +49,7 @@ _SIGNATURES = {
     "ao_amd_fp6_linear": ([_p, _i64, _i64, _p, _p, _i64, _int, _int, _p, _p], _int),
     "ao_amd_fp6_rmsnorm_linear": ([_p, _i64, _i64, _p, ctypes.c_float, _p, _p, _i64, _int, _int, _p, _p], _int),
     "ao_amd_fp6_swiglu": ([_p, _i64, _i64, _p, ctypes.c_float, _p, _p, _p, _p, _i64, _int, _int, _p, _p], _int),
+    "ao_amd_fp6_native_to_f16": ([_p, _p, _i64, _i64, _int, _int, _p, _p], _int),
     "ao_amd_fp6_linear_fused": ([_p, _i64, _i64, _p, _p, _i64, _int, _int, _p, _p, _p, _p], _int),
     "ao_amd_rmsnorm_f16": ([_p, _p, _i64, _i64, ctypes.c_float, _p, _p], _int),
     "ao_amd_llama_decode_attention_f16": ([_p, _p, _p, _p, _p, _int, _int, _int, _i64, _int, _p, _p, _p], _int),

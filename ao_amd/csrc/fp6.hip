@@ -339,6 +339,44 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* 
     }
 }
 
+// ---------------------------------------------------------------- native tiles -> fp16 matrix
+// W[N,K] fp16 = fp16(fpx value * scale), the dequantization of the linear kernels as a pass of its own, for batches
+// large enough that the library fp16 GEMM on the converted weight beats the fused kernel.  One wave per 16-row x 128-k
+// tile: 24 bytes in, 64 bytes out per lane (the four quarter-lanes of a row write 256 contiguous bytes).
+template <bool E3M2>
+__global__ __launch_bounds__(256) void fp6_native_to_f16_kernel(const uint32_t* __restrict__ native,
+                                                                 const uint16_t* __restrict__ scale, int64_t N, int64_t K,
+                                                                 int64_t KB, uint16_t* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tile >= (N / 16) * KB) return;
+    const int64_t rb = tile / KB, kb = tile - rb * KB;
+    const int r = lane & 15, qd = lane >> 4;
+    const uint32_t* t = native + tile * 384;
+    const uint4 lo = reinterpret_cast<const uint4*>(t)[lane];
+    const uint2 hi = reinterpret_cast<const uint2*>(t + 256)[lane];
+    union { uint16_t h; _Float16 f; } sc;
+    sc.h = scale[rb * 16 + r];
+    const f16x2_t sc2 = {sc.f, sc.f};
+    const u32x6_t packed = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y};
+    f16x32_t v;
+    if (E3M2) v = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(packed, 1.0f);
+    else v = __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(packed, 1.0f);
+    const int64_t k0 = kb * 128 + qd * 32;
+    if (k0 >= K) return;  // K is a multiple of 64: the last tile may be half padding
+    uint16_t* dst = out + (rb * 16 + r) * K + k0;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+        union { f16x2_t p[4]; uint4 q; } w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const f16x2_t pr = {v[sl * 8 + 2 * j], v[sl * 8 + 2 * j + 1]};
+            w.p[j] = pr * sc2;
+        }
+        reinterpret_cast<uint4*>(dst)[sl] = w.q;
+    }
+}
+
 // ---------------------------------------------------------------- skinny path (at most 16 rows staged in LDS)
 // The decode shapes.  The workgroup copies its activation rows into LDS once (zero-filled to the tile boundary,
 // optionally through RMSNorm), so the tile loop touches global memory for weights only, and the weight stream runs
@@ -893,4 +931,24 @@ extern "C" int ao_amd_fp6_swiglu(const void* x_f16, int64_t M, int64_t K, const 
     AO_REQUIRE(native_up && scale_up_f16, "null pointer argument");
     return fp6_linear_dispatch(x_f16, M, K, native_gate, scale_gate_f16, N, ebits, mbits, nullptr, nullptr, out_f16, stream,
                                norm_weight_f16, eps, native_up, scale_up_f16);
+}
+
+extern "C" int ao_amd_fp6_native_to_f16(const void* weights_native, const void* scale_f16, int64_t N, int64_t K, int ebits,
+                                        int mbits, void* out_f16, void* stream) {
+    AO_REQUIRE(weights_native && scale_f16 && out_f16, "null pointer argument");
+    if (int rc = check_fp6_format(ebits, mbits)) return rc;
+    AO_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 64 == 0, "need out_features a multiple of 16 and in_features a multiple "
+               "of 64, got (%lld, %lld)", (long long)N, (long long)K);
+    AO_REQUIRE((((uintptr_t)weights_native) & 15) == 0 && (((uintptr_t)out_f16) & 15) == 0, "buffers must be 16-byte aligned");
+    const int64_t KB = round_up(K, 128) / 128, tiles = (N / 16) * KB;
+    AO_REQUIRE((tiles + 3) / 4 <= 0x7fffffff, "weight too large for one launch");
+    const dim3 grid((unsigned)((tiles + 3) / 4));
+    if (ebits == 3)
+        hipLaunchKernelGGL(fp6_native_to_f16_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream,
+                           (const uint32_t*)weights_native, (const uint16_t*)scale_f16, N, K, KB, (uint16_t*)out_f16);
+    else
+        hipLaunchKernelGGL(fp6_native_to_f16_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream,
+                           (const uint32_t*)weights_native, (const uint16_t*)scale_f16, N, K, KB, (uint16_t*)out_f16);
+    AO_LAUNCH_CHECK();
+    return 0;
 }

@@ -75,6 +75,7 @@ TWO_PASS_MIN_M = 512
 
 
 INT8_TWO_PASS_MIN_M = 128
+FP6_TWO_PASS_MIN_M = 1024
 
 
 def int4wo_two_pass(M: int, N: int, K: int) -> bool:
@@ -595,6 +596,14 @@ def _fp6_linear_native_cuda(ebits, mbits, x, native, scale):
     M, K = x.shape
     N = scale.shape[0]
     torch._check(native.dtype is torch.int32 and native.numel() == _fp6_native_numel(N, K), lambda: "Dimensions mismatched")
+    if M >= FP6_TWO_PASS_MIN_M:
+        # prefill-sized batch: the weight as an fp16 matrix (HIP kernel, the same fp16(fpx * scale) values the fused
+        # kernel multiplies) and the library fp16 GEMM; the fused kernel tops out near 0.95 PFLOP/s, the library GEMM
+        # at 1.3-1.5, and the conversion costs about as much as 300 activation rows
+        w16 = torch.empty((N, K), dtype=torch.float16, device=x.device)
+        check(lib().ao_amd_fp6_native_to_f16(native.data_ptr(), scale.contiguous().data_ptr(), N, K, ebits, mbits,
+                                             w16.data_ptr(), current_stream(x.device)))
+        return torch.nn.functional.linear(x, w16)
     out = torch.empty((M, N), dtype=torch.float16, device=x.device)
     check(lib().ao_amd_fp6_linear(x.contiguous().data_ptr(), M, K, native.data_ptr(), scale.contiguous().data_ptr(), N,
                                   ebits, mbits, out.data_ptr(), current_stream(x.device)))

@@ -300,6 +300,12 @@ int ao_amd_fp6_linear_fused(const void* x_f16, int64_t M, int64_t K, const void*
                             int64_t N, int ebits, int mbits, const void* residual_f16, const void* gate_f16, void* out_f16,
                             void* stream);
 
+/* W[N,K] fp16 = fp16(fpx value * scale) from the native tiles: the dequantization inside ao_amd_fp6_linear as a pass of
+ * its own (the values of the reference's dequantization, utils_parallel_dequant.cuh:47-59), for prefill-sized batches: the
+ * host then runs the library fp16 GEMM on it (from 1024 activation rows on the fused kernel is the slower of the two). */
+int ao_amd_fp6_native_to_f16(const void* weights_native, const void* scale_f16, int64_t N, int64_t K, int ebits, int mbits,
+                             void* out_f16, void* stream);
+
 /* Decode-step fusions over the same linear, for at most 16 activation rows that fit a workgroup's LDS (M * K * 2 bytes at
  * most 64 KB): `_rmsnorm_linear` = linear(rmsnorm(x)) with rmsnorm(x) = fp16(fp16(x * rsqrt(mean(x^2) + eps)) * norm_weight)
  * (RMSNorm.forward then the linear it feeds, torchao/_models/llama/model.py:232-244); `_swiglu` =

@@ -160,3 +160,36 @@ def test_weight_subclass_and_api(oracle):
     dq = m[0].weight.dequantize(torch.float32).cpu().numpy()
     ref = oracle.fpx_to_f32(codes, 3, 2) * scale.view(np.float16).astype(np.float32)[:, None]
     assert np.array_equal(dq, ref)
+
+
+@pytest.mark.parametrize("fmt,shape", [((3, 2), (256, 1024)), ((3, 2), (512, 192)), ((2, 3), (320, 256)), ((2, 2), (128, 320)),
+                                       ((3, 1), (64, 128))])
+def test_native_to_fp16_is_the_scaled_weight_and_feeds_the_two_pass_linear(oracle, fmt, shape):
+    """Prefill path: the native tiles converted to an fp16 matrix are bit for bit fp16(fpx value * scale) (oracle codes
+    and scales, one fp16 multiply each, zero rows / ragged last K tile included), and the op's result from 1024 rows on
+    (library GEMM on that matrix) stays within the op's tolerance of the oracle."""
+    from ao_amd import _lib, ops
+
+    e, m = fmt
+    N, K = shape
+    print(f"case fp6 two-pass fmt={fmt} N={N} K={K}", flush=True)
+    dev = _dev()
+    g = torch.Generator().manual_seed(N + K + e)
+    w = (torch.randn(N, K, generator=g) * 0.05).half()
+    w[3] = 0
+    data, scale = ops.fp6_quantize_pack(w.to(dev), e, m)
+    native = ops.fp6_repack(data, 1 + e + m)
+    w16 = torch.empty((N, K), dtype=torch.float16, device=dev)
+    _lib.check(_lib.lib().ao_amd_fp6_native_to_f16(native.data_ptr(), scale.data_ptr(), N, K, e, m, w16.data_ptr(),
+                                                   _lib.current_stream(dev)))
+    values = ops.fp6_dequantize(data, None, e, m)              # exact fpx values (fp32), unscaled
+    want = (values.half() * scale.view(-1, 1))                  # one fp16 multiply, as the kernels do
+    assert np.array_equal(bits16(w16), bits16(want))
+    M = ops.FP6_TWO_PASS_MIN_M
+    x = (torch.rand(M, K, generator=g) + 0.5).half().to(dev)
+    y = ops.fp6_linear_native(e, m, x, native, scale).float().cpu().numpy()
+    ref = (x.double() @ want.double().t()).cpu().numpy()
+    ref16 = ref.astype(np.float16).astype(np.float32)
+    assert rel_l2(y, ref16) <= 1e-3
+    y_small = ops.fp6_linear_native(e, m, x[:64], native, scale).float().cpu().numpy()   # fused kernel, same rows
+    assert rel_l2(y[:64], y_small) <= 1e-3
