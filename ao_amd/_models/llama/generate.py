@@ -37,7 +37,7 @@ def sample(logits, temperature: float = 1.0, top_k: Optional[int] = None, greedy
     """Next token from the last position's logits.  greedy=True is argmax (no random numbers)."""
     if greedy:
         last = logits[0, -1]
-        if last.is_cuda and last.dtype is torch.bfloat16 and last.is_contiguous():
+        if last.is_cuda and last.dtype in (torch.bfloat16, torch.float16) and last.is_contiguous():
             from ... import ops
 
             return ops.argmax_bf16(last), None

@@ -18,6 +18,7 @@ struct ElemBf16 {
     static __device__ __forceinline__ float from_bits(uint16_t b) { return bf16_bits_to_f32(b); }
     static __device__ __forceinline__ uint16_t to_bits(float f) { return f32_to_bf16_bits(f); }
     static __device__ __forceinline__ float rne(float f) { return rne_bf16(f); }
+    static constexpr uint32_t kNegInf2 = 0xff80ff80u;  // two -inf
 };
 struct ElemF16 {
     static __device__ __forceinline__ float lo(uint32_t u) { return f16_bits_to_f32((uint16_t)(u & 0xffffu)); }
@@ -25,6 +26,7 @@ struct ElemF16 {
     static __device__ __forceinline__ float from_bits(uint16_t b) { return f16_bits_to_f32(b); }
     static __device__ __forceinline__ uint16_t to_bits(float f) { return f32_to_f16_bits(f); }
     static __device__ __forceinline__ float rne(float f) { return f16_bits_to_f32(f32_to_f16_bits(f)); }
+    static constexpr uint32_t kNegInf2 = 0xfc00fc00u;  // two -inf
 };
 
 // out = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * w ), statistics in fp32 (or fp16 throughout).  One workgroup per row.
@@ -331,7 +333,8 @@ __global__ __launch_bounds__(128) void attention_merge_kernel(const float* __res
 // thread requests all of its 16-byte chunks (up to 16: n <= 131072 elements in one round trip) before the first
 // comparison.  A thread meets its elements in increasing index order, so "strictly greater" keeps the lowest
 // index; NaNs only raise a flag in the hot loop and are located by a second pass in the rare case that one exists.
-__global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __restrict__ x, int64_t n,
+template <class E>
+__global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* __restrict__ x, int64_t n,
                                                             int32_t* __restrict__ out) {
     __shared__ float bv_s[16];
     __shared__ int32_t bi_s[16];
@@ -350,7 +353,7 @@ __global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __res
 #pragma unroll
             for (int j = 0; j < MAXC; ++j) {
                 const int64_t c = c0 + (int64_t)j * 1024 + tid;
-                raw[j] = make_uint4(0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u);  // -inf
+                raw[j] = make_uint4(E::kNegInf2, E::kNegInf2, E::kNegInf2, E::kNegInf2);  // -inf
                 if (c < nchunk) raw[j] = reinterpret_cast<const uint4*>(x)[c];
             }
 #pragma unroll
@@ -359,7 +362,7 @@ __global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __res
                 const uint32_t u[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const float lo = __uint_as_float(u[e] << 16), hi = __uint_as_float(u[e] & 0xffff0000u);
+                    const float lo = E::lo(u[e]), hi = E::hi(u[e]);
                     any_nan |= (lo != lo) | (hi != hi);
                     if (lo > best) { best = lo; besti = base + 2 * e; }
                     if (hi > best) { best = hi; besti = base + 2 * e + 1; }
@@ -368,7 +371,7 @@ __global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __res
         }
     }
     for (int64_t i = (vec ? nchunk * 8 : 0) + tid; i < n; i += 1024) {
-        const float v = bf16_bits_to_f32(x[i]);
+        const float v = E::from_bits(x[i]);
         any_nan |= v != v;
         if (v > best) { best = v; besti = (int32_t)i; }
     }
@@ -390,7 +393,7 @@ __global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t* __res
     if (__syncthreads_or(any_nan)) {
         // rare path: the answer is the first NaN
         for (int64_t i = tid; i < n; i += 1024) {
-            const float v = bf16_bits_to_f32(x[i]);
+            const float v = E::from_bits(x[i]);
             if (v != v) { atomicMin(&nan_s, (int)i); break; }
         }
         __syncthreads();
@@ -514,7 +517,16 @@ extern "C" int ao_amd_llama_decode_attention_f16(const void* qkv_f16, const void
 extern "C" int ao_amd_argmax_bf16(const void* x_bf16, int64_t n, int32_t* out_index, void* stream) {
     AO_REQUIRE(x_bf16 && out_index, "null pointer argument");
     AO_REQUIRE(n > 0 && n < (int64_t)1 << 31, "argmax over n=%lld elements is outside (0, 2^31)", (long long)n);
-    hipLaunchKernelGGL(argmax_bf16_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint16_t*)x_bf16, n,
+    hipLaunchKernelGGL(argmax_kernel<ElemBf16>, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint16_t*)x_bf16, n,
+                       out_index);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_argmax_f16(const void* x_f16, int64_t n, int32_t* out_index, void* stream) {
+    AO_REQUIRE(x_f16 && out_index, "null pointer argument");
+    AO_REQUIRE(n > 0 && n < (int64_t)1 << 31, "argmax over n=%lld elements is outside (0, 2^31)", (long long)n);
+    hipLaunchKernelGGL(argmax_kernel<ElemF16>, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint16_t*)x_f16, n,
                        out_index);
     AO_LAUNCH_CHECK();
     return 0;

@@ -453,10 +453,11 @@ def _rmsnorm_cuda(x, weight, eps):
 
 def _argmax_bf16_cuda(x):
     require_cuda(x)
-    torch._check(x.dtype is torch.bfloat16 and x.dim() == 1 and x.is_contiguous() and x.numel() > 0,
-                 lambda: "argmax_bf16 needs a non-empty contiguous 1d bfloat16 tensor")
+    torch._check(x.dtype in (torch.bfloat16, torch.float16) and x.dim() == 1 and x.is_contiguous() and x.numel() > 0,
+                 lambda: "argmax_bf16 needs a non-empty contiguous 1d bfloat16 (or float16) tensor")
     out = torch.empty(1, dtype=torch.int32, device=x.device)
-    check(lib().ao_amd_argmax_bf16(x.data_ptr(), x.numel(), out.data_ptr(), current_stream(x.device)))
+    fn = lib().ao_amd_argmax_bf16 if x.dtype is torch.bfloat16 else lib().ao_amd_argmax_f16
+    check(fn(x.data_ptr(), x.numel(), out.data_ptr(), current_stream(x.device)))
     return out
 
 

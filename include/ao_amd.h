@@ -257,6 +257,8 @@ int ao_amd_llama_decode_attention_f16(const void* qkv_f16, const void* freqs_cis
  * branch of `sample` in the decode harness, torch.argmax over the last position's logits
  * (torchao/_models/llama/generate.py:34-53 samples from the same logits row). */
 int ao_amd_argmax_bf16(const void* x_bf16, int64_t n, int32_t* out_index, void* stream);
+/* The same over n fp16 values (the logits of an FP6 / fp16 model). */
+int ao_amd_argmax_f16(const void* x_f16, int64_t n, int32_t* out_index, void* stream);
 
 /* ---------------------------------------------------------------- FP6-LLM (Quant-LLM FPx, e3m2 / e2m2 ...)
  * Interchange format = the reference's TC-FPx bytes, bit for bit. */

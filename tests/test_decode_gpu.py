@@ -250,13 +250,14 @@ def test_decode_attention_matches_module_math(pos, S):
     assert rel_l2(out.float().cpu().numpy(), ref) <= 1e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n", [1, 7, 8, 1000, 128256])
-def test_argmax_bf16(n):
+def test_argmax_bf16(n, dtype):
     from ao_amd import ops
 
     dev = _dev()
     g = torch.Generator().manual_seed(n)
-    x = torch.randn(n, generator=g).bfloat16()
+    x = torch.randn(n, generator=g).to(dtype)
     if n >= 1000:
         x[n // 3] = x[n - 5] = x.max() + 1   # a tie: the lower index wins
     out = ops.argmax_bf16(x.to(dev))
@@ -268,7 +269,7 @@ def test_argmax_bf16(n):
         x[n - 2] = float("nan")   # a NaN counts as the largest value, like torch.argmax
         x[n // 2] = float("nan")
         assert int(ops.argmax_bf16(x.to(dev)).item()) == n // 2
-        assert int(ops.argmax_bf16(torch.full((n,), float("-inf")).bfloat16().to(dev)).item()) == 0
+        assert int(ops.argmax_bf16(torch.full((n,), float("-inf")).to(dtype).to(dev)).item()) == 0
 
 
 def test_fused_decode_step_matches_module_path():
