@@ -72,6 +72,7 @@ _SIGNATURES = {
     "ao_amd_rmsnorm_bf16": ([_p, _p, _i64, _i64, ctypes.c_float, _p, _p], _int),
     "ao_amd_argmax_bf16": ([_p, _i64, _p, _p], _int),
     "ao_amd_argmax_f16": ([_p, _i64, _p, _p], _int),
+    "ao_amd_llama_decode_advance": ([_p, _int, _i64, _p, _p, _p, _p], _int),
     "ao_amd_llama_decode_attention": ([_p, _p, _p, _p, _p, _int, _int, _int, _i64, _p, _p], _int),
 }
 

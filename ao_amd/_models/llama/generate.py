@@ -71,7 +71,17 @@ class GraphedDecoder:
         self.graph = None
 
     def _step(self):
-        nxt, _ = decode_one_token(self.model, self.token, self.pos, **self.sampling_kwargs)
+        if self.sampling_kwargs.get("greedy") and self.token.is_cuda:
+            last = self.model(self.token, self.pos)[0, -1]
+            if last.dtype in (torch.bfloat16, torch.float16) and last.is_contiguous():
+                from ... import ops
+
+                # argmax, next input token and position in one launch
+                ops.decode_advance_(last, self.next_token, self.token, self.pos)
+                return
+            nxt = torch.argmax(last, dim=-1, keepdim=True).to(dtype=torch.int)
+        else:
+            nxt, _ = decode_one_token(self.model, self.token, self.pos, **self.sampling_kwargs)
         self.next_token.copy_(nxt.view(-1))
         self.token.copy_(nxt.view(1, 1))
         self.pos.add_(1)

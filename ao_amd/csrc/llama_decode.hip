@@ -335,7 +335,15 @@ __global__ __launch_bounds__(128) void attention_merge_kernel(const float* __res
 // index; NaNs only raise a flag in the hot loop and are located by a second pass in the rare case that one exists.
 template <class E>
 __global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* __restrict__ x, int64_t n,
-                                                            int32_t* __restrict__ out) {
+                                                            int32_t* __restrict__ out, int32_t* __restrict__ token,
+                                                            int32_t* __restrict__ pos) {
+    // `token` / `pos` (null or the decode loop's device-side state): the chosen index also becomes the next step's
+    // input token and the position advances by one, which saves the loop three small launches per token
+    auto publish = [&](int32_t idx) {
+        out[0] = idx;
+        if (token) token[0] = idx;
+        if (pos) pos[0] += 1;
+    };
     __shared__ float bv_s[16];
     __shared__ int32_t bi_s[16];
     __shared__ int nan_s;
@@ -397,12 +405,12 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* __restrict
             if (v != v) { atomicMin(&nan_s, (int)i); break; }
         }
         __syncthreads();
-        if (tid == 0) out[0] = nan_s;
+        if (tid == 0) publish(nan_s);
         return;
     }
     if (tid == 0) {
         for (int w = 1; w < 16; ++w) merge(bv_s[w], bi_s[w]);
-        out[0] = besti == 0x7fffffff ? 0 : besti;
+        publish(besti == 0x7fffffff ? 0 : besti);
     }
 }
 
@@ -518,7 +526,7 @@ extern "C" int ao_amd_argmax_bf16(const void* x_bf16, int64_t n, int32_t* out_in
     AO_REQUIRE(x_bf16 && out_index, "null pointer argument");
     AO_REQUIRE(n > 0 && n < (int64_t)1 << 31, "argmax over n=%lld elements is outside (0, 2^31)", (long long)n);
     hipLaunchKernelGGL(argmax_kernel<ElemBf16>, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint16_t*)x_bf16, n,
-                       out_index);
+                       out_index, (int32_t*)nullptr, (int32_t*)nullptr);
     AO_LAUNCH_CHECK();
     return 0;
 }
@@ -527,7 +535,21 @@ extern "C" int ao_amd_argmax_f16(const void* x_f16, int64_t n, int32_t* out_inde
     AO_REQUIRE(x_f16 && out_index, "null pointer argument");
     AO_REQUIRE(n > 0 && n < (int64_t)1 << 31, "argmax over n=%lld elements is outside (0, 2^31)", (long long)n);
     hipLaunchKernelGGL(argmax_kernel<ElemF16>, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint16_t*)x_f16, n,
-                       out_index);
+                       out_index, (int32_t*)nullptr, (int32_t*)nullptr);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_llama_decode_advance(const void* logits, int is_f16, int64_t n, int32_t* next_token, int32_t* token,
+                                           int32_t* pos, void* stream) {
+    AO_REQUIRE(logits && next_token && token && pos, "null pointer argument");
+    AO_REQUIRE(n > 0 && n < (int64_t)1 << 31, "argmax over n=%lld elements is outside (0, 2^31)", (long long)n);
+    if (is_f16)
+        hipLaunchKernelGGL(argmax_kernel<ElemF16>, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint16_t*)logits, n,
+                           next_token, token, pos);
+    else
+        hipLaunchKernelGGL(argmax_kernel<ElemBf16>, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint16_t*)logits, n,
+                           next_token, token, pos);
     AO_LAUNCH_CHECK();
     return 0;
 }

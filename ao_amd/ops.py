@@ -20,6 +20,7 @@ __all__ = [
     "fp6_dequantize",
     "fp6_repack",
     "fp6_linear_native",
+    "decode_advance_",
     "int4wo_linear_residual",
     "int4wo_swiglu",
     "int4wo_rmsnorm_linear",
@@ -449,6 +450,20 @@ def _rmsnorm_cuda(x, weight, eps):
     check(fn(xc.data_ptr(), weight.contiguous().data_ptr(), xc.numel() // dim, dim, float(eps),
                                     out.data_ptr(), current_stream(x.device)))
     return out
+
+
+def decode_advance_(logits_row: Tensor, next_token: Tensor, token: Tensor, pos: Tensor) -> None:
+    """In place, one launch: next_token[0] = token[0] = argmax(logits_row), pos[0] += 1 (greedy sampling plus the decode
+    loop's bookkeeping on its device-side state).  logits_row: contiguous 1d bf16 / fp16; the others one int32 each."""
+    require_cuda(logits_row, next_token, token, pos)
+    torch._check(logits_row.dtype in (torch.bfloat16, torch.float16) and logits_row.dim() == 1
+                 and logits_row.is_contiguous() and logits_row.numel() > 0,
+                 lambda: "logits must be a non-empty contiguous 1d bfloat16 or float16 tensor")
+    for t in (next_token, token, pos):
+        torch._check(t.dtype is torch.int32 and t.numel() == 1, lambda: "state cells must hold one int32 each")
+    check(lib().ao_amd_llama_decode_advance(logits_row.data_ptr(), int(logits_row.dtype is torch.float16),
+                                            logits_row.numel(), next_token.data_ptr(), token.data_ptr(), pos.data_ptr(),
+                                            current_stream(logits_row.device)))
 
 
 def _argmax_bf16_cuda(x):

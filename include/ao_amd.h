@@ -260,6 +260,13 @@ int ao_amd_argmax_bf16(const void* x_bf16, int64_t n, int32_t* out_index, void* 
 /* The same over n fp16 values (the logits of an FP6 / fp16 model). */
 int ao_amd_argmax_f16(const void* x_f16, int64_t n, int32_t* out_index, void* stream);
 
+/* Greedy sampling and the bookkeeping of one decode step in one launch: next_token[0] = token[0] = argmax(logits[0..n)),
+ * pos[0] += 1 (decode_one_token + the loop's `input_pos += 1; cur_token = next_token`,
+ * torchao/_models/llama/generate.py:58-77, on device-side state so that the step can live in a HIP graph).
+ * logits bf16 (is_f16 = 0) or fp16; the three int32 cells are distinct device addresses. */
+int ao_amd_llama_decode_advance(const void* logits, int is_f16, int64_t n, int32_t* next_token, int32_t* token,
+                                int32_t* pos, void* stream);
+
 /* ---------------------------------------------------------------- FP6-LLM (Quant-LLM FPx, e3m2 / e2m2 ...)
  * Interchange format = the reference's TC-FPx bytes, bit for bit. */
 
