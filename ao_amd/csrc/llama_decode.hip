@@ -137,7 +137,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int sub = lane >> 4, l16 = lane & 15;
     const int rg = wave * 4 + sub;  // row group 0..63
-    const int pos = pos_ptr[0];
+    const int pos = __builtin_amdgcn_readfirstlane(pos_ptr[0]);  // uniform: branches on it are scalar
     const int T = pos + 1;
     // Long contexts: `nsplit` workgroups per head (blockIdx.y = z) take the 64-position rows z, z + nsplit, ... of
     // the context, so that any context length spreads evenly over them; each leaves (max, sum, unnormalised output) in
@@ -146,6 +146,12 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     const int z = blockIdx.y;
     auto tpos = [&](int ridx) { return (ridx * nsplit + z) * 64 + rg; };
     const int nchunk = (T + ATT_CHUNK * nsplit - 1) / (ATT_CHUNK * nsplit);  // chunk iterations of this workgroup
+    // rows of this workgroup that hold a position < T: a prefix of its rows; the others are skipped as a whole
+    const int rows_total = (T + 63) / 64;
+    const int npass = rows_total > z ? (rows_total - z + nsplit - 1) / nsplit : 0;
+    // a row's cached positions are read without a bounds branch: positions >= pos (never used: the new token's k / v
+    // come from qkv, later ones are masked) read the last cached row instead
+    const int last_cached = pos > 0 ? pos - 1 : 0;
 
     // element i of the fused qkv row: a bf16 value, or the bf16 rounding of the sum of `nparts` fp32 partial rows
     // (a linear whose K range was split across workgroups leaves the last add to its consumer)
@@ -165,10 +171,10 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     uint4 rawk[U], rawv[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        const int t = tpos(u);
         rawk[u] = make_uint4(0, 0, 0, 0);
         rawv[u] = make_uint4(0, 0, 0, 0);
-        if (t < pos) {
+        if (u < npass) {
+            const int t = tpos(u) < last_cached ? tpos(u) : last_cached;
             rawk[u] = *reinterpret_cast<const uint4*>(kc + (int64_t)t * HD + l16 * 8);
             rawv[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)t * HD + l16 * 8);
         }
@@ -209,13 +215,15 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
         if (c > 0) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int t = tpos(c * U + u);
-                rawk[u] = make_uint4(0, 0, 0, 0);
-                if (t < pos) rawk[u] = *reinterpret_cast<const uint4*>(kc + (int64_t)t * HD + l16 * 8);
+                if (c * U + u < npass) {
+                    const int t = tpos(c * U + u) < last_cached ? tpos(c * U + u) : last_cached;
+                    rawk[u] = *reinterpret_cast<const uint4*>(kc + (int64_t)t * HD + l16 * 8);
+                }
             }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
+            if (c * U + u >= npass) break;
             const int t = tpos(c * U + u);
             const uint32_t w4[4] = {rawk[u].x, rawk[u].y, rawk[u].z, rawk[u].w};
             float d = 0.f;
@@ -243,7 +251,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     for (int w = 1; w < 16; ++w) gmax = fmaxf(gmax, red[w]);
     const float gsub = gmax == -INFINITY ? 0.f : gmax;  // a workgroup without positions (split mode, short context)
     float lsum = 0.f;
-    for (int li = tid; li < nchunk * ATT_CHUNK; li += ATT_THREADS) {
+    for (int li = tid; li < npass * 64; li += ATT_THREADS) {
         const float p = expf(sc[li] - gsub);
         sc[li] = p;
         lsum += p;
@@ -264,13 +272,15 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
         if (c > 0) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int t = tpos(c * U + u);
-                rawv[u] = make_uint4(0, 0, 0, 0);
-                if (t < pos) rawv[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)t * HD + l16 * 8);
+                if (c * U + u < npass) {
+                    const int t = tpos(c * U + u) < last_cached ? tpos(c * U + u) : last_cached;
+                    rawv[u] = *reinterpret_cast<const uint4*>(vc + (int64_t)t * HD + l16 * 8);
+                }
             }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
+            if (c * U + u >= npass) break;
             const int t = tpos(c * U + u);
             if (t < T) {
                 const float p = sc[(c * U + u) * 64 + rg];
