@@ -1,5 +1,7 @@
 from .GPTQ import Int4WeightOnlyGPTQQuantizer, Int4WeightOnlyQuantizer, WeightOnlyInt4Linear
 from .quant_api import (
+    change_linear_weights_to_int4_woqtensors,
+    change_linear_weights_to_int8_woqtensors,
     fp6_llm_weight_only,
     int4_weight_only,
     int8_weight_only,

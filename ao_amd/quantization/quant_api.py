@@ -12,6 +12,7 @@ import torch
 from .quant_primitives import MappingType, ZeroPointDomain
 
 __all__ = ["quantize", "quantize_", "int4_weight_only", "int8_weight_only", "fp6_llm_weight_only",
+           "change_linear_weights_to_int4_woqtensors", "change_linear_weights_to_int8_woqtensors",
            "quant_llm_fpx_weight_only"]
 
 
@@ -108,3 +109,17 @@ def quant_llm_fpx_weight_only(ebits: int, mbits: int):
 
 def fp6_llm_weight_only():
     return quant_llm_fpx_weight_only(3, 2)
+
+
+def change_linear_weights_to_int4_woqtensors(model, groupsize=128, inner_k_tiles=8, filter_fn=None):
+    """Legacy entry point (reference quant_api.py:119-141, which refuses to run on PyTorch >= 2.4): every linear weight
+    becomes a groupwise int4 weight-only tensor, in place.  The legacy `Int4WeightOnlyQuantizedLinearWeight` subclass
+    (subclass.py:394-601) computes the same codes and qparams through the same helpers; here the call maps to
+    `quantize_(model, int4_weight_only(groupsize, inner_k_tiles))`."""
+    quantize_(model, int4_weight_only(group_size=groupsize, inner_k_tiles=inner_k_tiles), filter_fn)
+
+
+def change_linear_weights_to_int8_woqtensors(model, filter_fn=None, **kwargs):
+    """Legacy entry point (reference quant_api.py:103-117): per-channel int8 weight-only on every linear, in place;
+    maps to `quantize_(model, int8_weight_only())`."""
+    quantize_(model, int8_weight_only(), filter_fn)

@@ -212,3 +212,25 @@ def test_two_weight_swiglu_matches_the_gated_chain(M, N, K, with_norm):
     assert got.shape == (M, N) and got.dtype is torch.bfloat16
     g, w = got.float().cpu().numpy(), want.float().cpu().numpy()
     assert rel_l2(g, w) <= 1e-3 and np.count_nonzero(g != w) <= 0.01 * g.size + 1
+
+
+def test_legacy_entry_points_map_to_quantize():
+    """change_linear_weights_to_int{4,8}_woqtensors (reference quant_api.py:103-141) give the same weights as
+    quantize_ with the matching constructor."""
+    import copy
+
+    from ao_amd import int4_weight_only, int8_weight_only, quantize_
+    from ao_amd.quantization import change_linear_weights_to_int4_woqtensors, change_linear_weights_to_int8_woqtensors
+
+    dev = _dev()
+    torch.manual_seed(1)
+    base = torch.nn.Sequential(torch.nn.Linear(256, 128, bias=False)).to(dev).bfloat16()
+    x = torch.randn(3, 256, device=dev).bfloat16()
+    for legacy, modern in ((lambda m: change_linear_weights_to_int4_woqtensors(m, groupsize=64),
+                            lambda m: quantize_(m, int4_weight_only(group_size=64))),
+                           (change_linear_weights_to_int8_woqtensors, lambda m: quantize_(m, int8_weight_only()))):
+        a, b = copy.deepcopy(base), copy.deepcopy(base)
+        legacy(a)
+        modern(b)
+        with torch.no_grad():
+            assert type(a[0].weight) is type(b[0].weight) and torch.equal(a(x), b(x))
