@@ -107,12 +107,53 @@ __device__ __forceinline__ uint32_t tc_fpx_code(const uint8_t* __restrict__ tc, 
 }
 
 // ---------------------------------------------------------------- quantize + pack (to_scaled_tc_fpx)
-// One workgroup per 64-row block.  Pass 1: row amax -> fp32 scale (amax clamped at 1e-12, divided by the largest
-// normal).  Pass 2, per 16-column slice: 1024 codes into LDS, then the threads assemble the bytes of the high
-// plane (FP6: one byte of the 2-bit plane per thread; FP5: one byte of the 1-bit plane per thread of the first
-// two waves) and two bytes of the 4-bit plane of that slice.
+// The row scale is amax clamped at 1e-12 and divided by the largest normal, in fp32; the codes are fpx(w / scale).
+// A workgroup packs a run of 16-column slices of one 64-row block: per slice 1024 codes go into LDS, then the threads
+// assemble the bytes of the high plane (FP6: one byte of the 2-bit plane per thread; FP5: one byte of the 1-bit plane
+// per thread of the first two waves) and two bytes of the 4-bit plane of that slice.
+//
+// 16-bit inputs run as three launches so that the packing spreads over the whole chip: fp6_row_amax_kernel leaves each
+// row's amax (exact in the input dtype: 16 bits) in the scale output, the pack kernel (AMAX_GIVEN, blockIdx.y = run of
+// slices) derives the fp32 scale from it, fp6_scale_finalize_kernel replaces it by the fp16 scale.  fp32 inputs (amax
+// does not fit the 16-bit cell) keep the one-launch form: one workgroup per 64-row block computes the scales itself.
+__global__ __launch_bounds__(256) void fp6_row_amax_kernel(const void* __restrict__ w, int w_dtype, int64_t N, int64_t K,
+                                                            uint16_t* __restrict__ amax_out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= N) return;
+    float amax = 0.f;
+    bool has_nan = false;
+    for (int64_t c = lane; c < K; c += 64) {
+        const float v = fabsf(load_f(w, w_dtype, row * K + c));
+        if (v != v) has_nan = true;
+        amax = fmaxf(amax, v);
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+        has_nan |= (bool)__shfl_xor((int)has_nan, o, 64);
+    }
+    if (lane == 0)
+        amax_out[row] = has_nan ? (w_dtype == AO_BF16 ? 0x7fc0 : 0x7e00)
+                                : (w_dtype == AO_BF16 ? f32_to_bf16_bits(amax) : f32_to_f16_bits(amax));
+}
+
+__device__ __forceinline__ float fp6_scale_of_amax(float amax, float max_normal) {
+    // a NaN amax stays NaN through the clamp (the comparison is false) and the division
+    return __fdiv_rn(amax < 1e-12f ? 1e-12f : amax, max_normal);
+}
+
+__global__ __launch_bounds__(256) void fp6_scale_finalize_kernel(uint16_t* __restrict__ scale, int64_t N, int w_dtype,
+                                                                  float max_normal) {
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= N) return;
+    const float amax = w_dtype == AO_BF16 ? bf16_bits_to_f32(scale[row]) : f16_bits_to_f32(scale[row]);
+    scale[row] = f32_to_f16_bits(fp6_scale_of_amax(amax, max_normal));
+}
+
+template <bool AMAX_GIVEN, int ebits, int mbits>  // the format as constants: the cast's masks and bounds fold away
 __global__ __launch_bounds__(256) void fp6_quantize_pack_kernel(const void* __restrict__ w, int w_dtype, int64_t N,
-                                                                 int64_t K, int ebits, int mbits,
+                                                                 int64_t K, int64_t slices_per_wg,
                                                                  uint8_t* __restrict__ out, uint16_t* __restrict__ scale_out) {
     __shared__ float scale_s[64];
     __shared__ uint8_t codes_s[64][17];
@@ -121,7 +162,13 @@ __global__ __launch_bounds__(256) void fp6_quantize_pack_kernel(const void* __re
     const int exp_bias = (1 << (ebits - 1)) - 1;
     const float max_normal = __uint_as_float((uint32_t)(((1 << ebits) - 1) - exp_bias + 127) << 23) *
                              ((float)((1 << (mbits + 1)) - 1) / (float)(1 << mbits));
-    for (int rr = wave * 16; rr < wave * 16 + 16; ++rr) {
+    if (AMAX_GIVEN) {
+        if (tid < 64) {
+            const uint16_t bits = scale_out[a * 64 + tid];
+            scale_s[tid] = fp6_scale_of_amax(w_dtype == AO_BF16 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits), max_normal);
+        }
+    }
+    for (int rr = wave * 16; rr < wave * 16 + 16 && !AMAX_GIVEN; ++rr) {
         const int64_t row = a * 64 + rr;
         float amax = 0.f;
         bool has_nan = false;
@@ -147,7 +194,9 @@ __global__ __launch_bounds__(256) void fp6_quantize_pack_kernel(const void* __re
     uint8_t* p2 = out;
     uint8_t* p4 = out + (nbits == 6 ? N * K / 4 : N * K / 8);
     const int64_t E = K >> 4;
-    for (int64_t e = 0; e < E; ++e) {
+    const int64_t e_begin = (int64_t)blockIdx.y * slices_per_wg;
+    const int64_t e_end = e_begin + slices_per_wg < E ? e_begin + slices_per_wg : E;
+    for (int64_t e = e_begin; e < e_end; ++e) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int idx = tid + j * 256, rr = idx >> 4, cc = idx & 15;
@@ -764,8 +813,42 @@ extern "C" int ao_amd_fp6_quantize_pack(const void* w, int w_dtype, int64_t N, i
     AO_REQUIRE(N > 0 && K > 0 && N % 64 == 0 && K % 64 == 0,
                "TC-FPx packing needs out_features and in_features to be multiples of 64, got (%lld, %lld)", (long long)N,
                (long long)K);
-    hipLaunchKernelGGL(fp6_quantize_pack_kernel, dim3((unsigned)(N / 64)), dim3(256), 0, (hipStream_t)stream, w, w_dtype, N,
-                       K, ebits, mbits, (uint8_t*)out_tc, (uint16_t*)out_scale_f16);
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t E = K / 16;
+    if (w_dtype == AO_BF16 || w_dtype == AO_F16) {
+        // enough workgroups for the chip: about 2048, each with a run of 16-column slices of one 64-row block
+        int64_t splits = (2048 + N / 64 - 1) / (N / 64);
+        if (splits > E) splits = E;
+        if (splits > 65535) splits = 65535;
+        const int64_t per_wg = (E + splits - 1) / splits;
+        splits = (E + per_wg - 1) / per_wg;
+        const int exp_bias = (1 << (ebits - 1)) - 1;
+        union { uint32_t u; float f; } top;
+        top.u = (uint32_t)(((1 << ebits) - 1) - exp_bias + 127) << 23;
+        const float max_normal = top.f * ((float)((1 << (mbits + 1)) - 1) / (float)(1 << mbits));
+        hipLaunchKernelGGL(fp6_row_amax_kernel, dim3((unsigned)((N + 3) / 4)), dim3(256), 0, st, w, w_dtype, N, K,
+                           (uint16_t*)out_scale_f16);
+        const dim3 grid((unsigned)(N / 64), (unsigned)splits);
+#define AO_FP6_PACK(EB, MB)                                                                                              \
+    hipLaunchKernelGGL((fp6_quantize_pack_kernel<true, EB, MB>), grid, dim3(256), 0, st, w, w_dtype, N, K, per_wg,       \
+                       (uint8_t*)out_tc, (uint16_t*)out_scale_f16)
+        if (ebits == 3 && mbits == 2) AO_FP6_PACK(3, 2);
+        else if (ebits == 2 && mbits == 3) AO_FP6_PACK(2, 3);
+        else if (ebits == 2 && mbits == 2) AO_FP6_PACK(2, 2);
+        else AO_FP6_PACK(3, 1);
+#undef AO_FP6_PACK
+        hipLaunchKernelGGL(fp6_scale_finalize_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, st,
+                           (uint16_t*)out_scale_f16, N, w_dtype, max_normal);
+    } else {
+#define AO_FP6_PACK(EB, MB)                                                                                              \
+    hipLaunchKernelGGL((fp6_quantize_pack_kernel<false, EB, MB>), dim3((unsigned)(N / 64)), dim3(256), 0, st, w, w_dtype, N,  \
+                       K, E, (uint8_t*)out_tc, (uint16_t*)out_scale_f16)
+        if (ebits == 3 && mbits == 2) AO_FP6_PACK(3, 2);
+        else if (ebits == 2 && mbits == 3) AO_FP6_PACK(2, 3);
+        else if (ebits == 2 && mbits == 2) AO_FP6_PACK(2, 2);
+        else AO_FP6_PACK(3, 1);
+#undef AO_FP6_PACK
+    }
     AO_LAUNCH_CHECK();
     return 0;
 }
