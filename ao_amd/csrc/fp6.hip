@@ -932,6 +932,9 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
     const int64_t xbytes = (M < 16 ? M : 16) * Kp * 2;
     if (need_lds)
         while (waves < 16 && xbytes > (int64_t)waves * 16 * 1024) waves *= 2;
+    // a wave count that leaves each wave at least 4 K tiles keeps the staged path worth its barrier
+    if (!need_lds && M <= 16)
+        while (waves > 4 && KB < 4 * waves && xbytes <= (int64_t)(waves / 2) * 16 * 1024) waves /= 2;
     const bool fits = M <= 16 && xbytes <= 64 * 1024 && xbytes <= (int64_t)waves * 16 * 1024;
     AO_REQUIRE(!need_lds || (fits && (((uintptr_t)norm_weight_f16) & 15) == 0 && (((uintptr_t)native_up) & 15) == 0),
                "the fused RMSNorm and the two-weight SwiGLU need at most 16 activation rows that fit in LDS (M=%lld K=%lld) "
