@@ -967,6 +967,9 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // a single activation row is staged fastest when the workgroup's threads cover it with two 16-byte chunks each
     if (M == 1)
         while (waves < 16 && (int64_t)waves * 128 < Kp / 8 && waves * 2 <= KB) waves *= 2;
+    // ... but not with fewer than 4 K tiles per wave while the row still fits two chunks per thread
+    if (M == 1)
+        while (waves > 4 && KB < 4 * waves && (int64_t)(waves / 2) * 128 >= Kp / 8) waves /= 2;
     const bool aligned = (K == Kp) && ((ldx & 7) == 0) && ((((uintptr_t)x_bf16) & 15) == 0);
     const int64_t rows = M < 16 ? M : 16;
     const size_t xbytes = (size_t)rows * (size_t)Kp * 2;
