@@ -123,10 +123,26 @@ __global__ __launch_bounds__(256) void fp6_row_amax_kernel(const void* __restric
     if (row >= N) return;
     float amax = 0.f;
     bool has_nan = false;
-    for (int64_t c = lane; c < K; c += 64) {
-        const float v = fabsf(load_f(w, w_dtype, row * K + c));
-        if (v != v) has_nan = true;
-        amax = fmaxf(amax, v);
+    const uint16_t* wrow = reinterpret_cast<const uint16_t*>(w) + row * K;
+    if ((((uintptr_t)wrow) & 15) == 0) {
+        // 16-byte loads: K is a multiple of 64, so a row is a whole number of 8-element chunks
+        for (int64_t c = lane; c < K / 8; c += 64) {
+            const uint4 q = reinterpret_cast<const uint4*>(wrow)[c];
+            const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float lo = fabsf(w_dtype == AO_BF16 ? __uint_as_float(u[j] << 16) : f16_bits_to_f32((uint16_t)(u[j] & 0xffffu)));
+                const float hi = fabsf(w_dtype == AO_BF16 ? __uint_as_float(u[j] & 0xffff0000u) : f16_bits_to_f32((uint16_t)(u[j] >> 16)));
+                has_nan |= (lo != lo) | (hi != hi);
+                amax = fmaxf(amax, fmaxf(lo, hi));
+            }
+        }
+    } else {
+        for (int64_t c = lane; c < K; c += 64) {
+            const float v = fabsf(load_f(w, w_dtype, row * K + c));
+            if (v != v) has_nan = true;
+            amax = fmaxf(amax, v);
+        }
     }
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) {
