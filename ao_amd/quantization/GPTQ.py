@@ -89,6 +89,10 @@ class WeightOnlyInt4Linear(nn.Module):
     in_features: int
     out_features: int
     weight: torch.Tensor
+    # which PyTorch build packed the `weight` of a reference-format state dict given to load_state_dict: "cuda" or
+    # "rocm" (the two write different words into the same shape; see unpack_tinygemm_int4pack).  Set it on the class
+    # or on a module before loading.
+    tinygemm_packed_by: str = "cuda"
 
     def __init__(self, in_features: int, out_features: int, bias=False, device=None, dtype=None,
                  groupsize: int = 128, inner_k_tiles: int = 8) -> None:
@@ -130,7 +134,7 @@ class WeightOnlyInt4Linear(nn.Module):
         if w is not None and w.dim() == 4 and tuple(w.shape) == tinygemm_shape and tuple(w.shape) != tuple(self.weight.shape):
             sz = state_dict.get(prefix + "scales_and_zeros", self.scales_and_zeros)
             dev = self.weight.device
-            codes = unpack_tinygemm_int4pack(w.to(dev), self.inner_k_tiles)
+            codes = unpack_tinygemm_int4pack(w.to(dev), self.inner_k_tiles, self.tinygemm_packed_by)
             scales = sz[:, :, 0].t().contiguous().to(device=dev, dtype=torch.bfloat16)
             zeros = sz[:, :, 1].t().contiguous().to(device=dev, dtype=torch.bfloat16)
             state_dict[key], _ = torch.ops.torchao.int4wo_pack(codes, scales, zeros, self.groupsize)

@@ -107,32 +107,56 @@ def recommended_inductor_config_setter():
 _TINYGEMM_NIBBLE_K = (0, 8, 16, 24, 1, 9, 17, 25)
 
 
-def unpack_tinygemm_int4pack(weight_int4pack: torch.Tensor, inner_k_tiles: int) -> torch.Tensor:
-    """The 4-bit codes `[N, K]` (int32, 0..15) of a weight packed by the CUDA build of
-    `aten._convert_weight_to_int4pack` (`[N/8, K/(16*inner_k_tiles), 32, inner_k_tiles/2]` int32), the `weight` entry
-    of state dicts written by the reference's module-swap quantizers (torchao/quantization/GPTQ.py:566-569, :737).
+# The same for a word packed by a ROCm build: the packed tensor, read flat, is [N/16, K/(16*inner_k_tiles), 64,
+# inner_k_tiles/2] (one 64-lane wavefront per 16 rows); the lane with t // 16 == 0 holds these positions of the 32-wide
+# span and lane t adds 4 * (t // 16).
+_TINYGEMM_NIBBLE_K_ROCM = (0, 2, 16, 18, 1, 3, 17, 19)
 
-    The layout is the B fragment of `mma.m16n8k16`, as published in PyTorch's int4mm.cu (v2.3): word
+
+def unpack_tinygemm_int4pack(weight_int4pack: torch.Tensor, inner_k_tiles: int, packed_by: str = "cuda") -> torch.Tensor:
+    """The 4-bit codes `[N, K]` (int32, 0..15) of a weight packed by `aten._convert_weight_to_int4pack`
+    (`[N/8, K/(16*inner_k_tiles), 32, inner_k_tiles/2]` int32), the `weight` entry of state dicts written by the
+    reference's module-swap quantizers (torchao/quantization/GPTQ.py:566-569, :737).  The words depend on the
+    PyTorch build that packed them:
+
+    `packed_by="cuda"`: the B fragment of `mma.m16n8k16`, as published in PyTorch's int4mm.cu (v2.3): word
     `[nt][ko][t][j]` belongs to row `8*nt + t//4` and to the two k tiles starting at `16*(ko*inner_k_tiles + 2j)`;
     its nibbles hold k offsets `2*(t%4) + {0, 8, 16, 24, 1, 9, 17, 25}` in order from the low nibble.  The reference
     repository holds no packed vectors of this format (the packer lives in PyTorch core), so this restatement is
-    checked against a loop transcription of the same published kernel only.  Words packed by a ROCm build of PyTorch
-    follow a different tile order and are not handled."""
+    checked against a loop transcription of the same published kernel only.
+
+    `packed_by="rocm"`: what the same operator of a PyTorch-ROCm build writes on a 64-lane device.  The tensor has
+    the same shape but, read flat, is `[N/16][ko][t in 0..63][j]`: the word belongs to row `16*nt + t%16` and to the
+    32-wide span of k starting at `16*inner_k_tiles*ko + 32*j`; its nibbles hold k offsets
+    `4*(t//16) + {0, 2, 16, 18, 1, 3, 17, 19}`.  This one is checked on the GPU against the operator itself."""
     assert weight_int4pack.dtype is torch.int32 and weight_int4pack.dim() == 4, "expected the 4-d int32 tinygemm weight"
     n_tiles, k_outer, lanes, halves = weight_int4pack.shape
     assert inner_k_tiles in (2, 4, 8) and lanes == 32 and halves * 2 == inner_k_tiles, \
         f"shape {tuple(weight_int4pack.shape)} is not a tinygemm weight of inner_k_tiles={inner_k_tiles}"
+    if packed_by not in ("cuda", "rocm"):
+        raise ValueError(f"packed_by must be 'cuda' or 'rocm', got {packed_by!r}")
     dev = weight_int4pack.device
     shifts = torch.arange(0, 32, 4, device=dev, dtype=torch.int32)
-    nib = (weight_int4pack.unsqueeze(-1) >> shifts) & 0xF  # [nt, ko, t, j, p]
-    nib = nib.reshape(n_tiles, k_outer, 8, 4, halves, 8)  # t -> (row in tile, t % 4)
-    # destination order: [nt, row, ko, j, position in the 32-wide span]
-    nib = nib.permute(0, 2, 1, 4, 3, 5).reshape(n_tiles, 8, k_outer, halves, 32)
-    # source index (t % 4, p) flattened as 8 * (t % 4) + p, for each position of the span
     src = torch.empty(32, dtype=torch.long)
-    for tc in range(4):
-        for p, koff in enumerate(_TINYGEMM_NIBBLE_K):
-            src[koff + 2 * tc] = 8 * tc + p
+    if packed_by == "cuda":
+        rows, lane_groups, lane_step, nibble_k = 8, 4, 2, _TINYGEMM_NIBBLE_K
+        words = weight_int4pack
+    else:
+        assert n_tiles % 2 == 0, "a ROCm-packed tinygemm weight has a multiple of 16 rows"
+        rows, lane_groups, lane_step, nibble_k = 16, 4, 4, _TINYGEMM_NIBBLE_K_ROCM
+        words = weight_int4pack.reshape(n_tiles // 2, k_outer, 64, halves)
+    nib = (words.unsqueeze(-1) >> shifts) & 0xF  # [nt, ko, t, j, p]
+    if packed_by == "cuda":
+        nib = nib.reshape(-1, k_outer, rows, lane_groups, halves, 8)  # t -> (row in tile, t % 4)
+        nib = nib.permute(0, 2, 1, 4, 3, 5)
+    else:
+        nib = nib.reshape(-1, k_outer, lane_groups, rows, halves, 8)  # t -> (t // 16, row in tile)
+        nib = nib.permute(0, 3, 1, 4, 2, 5)
+    # now [nt, row, ko, j, lane group, p]; gather (lane group, p) into the 32 positions of the span
+    nib = nib.reshape(-1, rows, k_outer, halves, 32)
+    for lg in range(lane_groups):
+        for p, koff in enumerate(nibble_k):
+            src[koff + lane_step * lg] = 8 * lg + p
     codes = nib.index_select(-1, src.to(dev))
     return codes.reshape(n_tiles * 8, k_outer * inner_k_tiles * 16).contiguous()
 

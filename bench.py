@@ -279,7 +279,7 @@ def _time_linear(L, launch, iters, armed=True):
 def sweep(kind, iters=100):
     """Per-kernel lines for the shapes of the other benchmark configurations: int4 GEMV (M in 1, 4; g in 64, 128),
     int4 GEMM (M in 16 .. 2048, g=64), the FP6 e3m2 linear (M in 1, 16, 128, 512) and the int8 weight-only linear
-    (M in 1, 4, 16); one JSON line per case."""
+    (M in 1, 4, 16); one JSON line per case.  `tinygemm` times PyTorch's own int4 matmul operator beside this library's."""
     import torch
 
     from ao_amd import _lib
@@ -388,6 +388,64 @@ def sweep(kind, iters=100):
                                   "GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
                                   "TFLOPs": round(tfs, 2), "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
             del wq
+    elif kind == "tinygemm":
+        # The operator the reference's int4 weight-only linear dispatches to (torchao/dtypes/affine_quantized_tensor.py:631 ->
+        # aten._weight_int4pack_mm), as this PyTorch-ROCm build implements it, beside torch.ops.torchao.int4wo_linear
+        # on the same codes and qparams.  Both run from a replayed HIP graph of one launch per weight copy, so the
+        # figure is device time per launch with cold weights and no host dispatch in it.
+        from ao_amd import ops
+        from ao_amd.quantization.utils import groupwise_affine_quantize_tensor
+
+        def replayed_us(fn, n, reps):
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                for i in range(n):
+                    fn(i)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    for i in range(n):
+                        fn(i)
+            for _ in range(2):
+                graph.replay()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                graph.replay()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) * 1e3 / (reps * n)
+
+        g = 64
+        for N, K in [(4096, 4096), (6144, 4096), (14336, 4096), (4096, 14336), (128256, 4096)]:
+            w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).bfloat16()
+            codes, sz = groupwise_affine_quantize_tensor(w, 4, g)
+            try:
+                theirs = torch.ops.aten._convert_weight_to_int4pack(
+                    ((codes[:, ::2] << 4) | codes[:, 1::2]).to(torch.uint8), 8)
+            except (RuntimeError, NotImplementedError) as e:
+                sys.exit(f"aten._convert_weight_to_int4pack is not available on this device: {e}")
+            mine, mine_q = ops.int4wo_pack(codes, sz[:, :, 0].t().contiguous(), sz[:, :, 1].t().contiguous(), g)
+            copies = max(2, -(-SWEEP_ROTATE_BYTES // (N * K // 2)))
+            theirs_c, sz_c = [theirs.clone() for _ in range(copies)], [sz.clone() for _ in range(copies)]
+            mine_c, mine_qc = [mine.clone() for _ in range(copies)], [mine_q.clone() for _ in range(copies)]
+            for M in (1, 4, 16, 512, 2048):
+                if M * N >= 1 << 28:
+                    continue
+                x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
+                reps = 20 if M <= 16 else 2
+                t_us = replayed_us(lambda i: torch.ops.aten._weight_int4pack_mm(x, theirs_c[i % copies], g,
+                                                                                 sz_c[i % copies]), copies, reps)
+                m_us = replayed_us(lambda i: ops.int4wo_linear(x, mine_c[i % copies], mine_qc[i % copies], g, N),
+                                   copies, reps)
+                y_t = torch.ops.aten._weight_int4pack_mm(x, theirs, g, sz).float()
+                y_m = ops.int4wo_linear(x, mine, mine_q, g, N).float()
+                print(json.dumps({"N": N, "K": K, "M": M, "group": g, "aten_weight_int4pack_mm_us": round(t_us, 2),
+                                  "int4wo_linear_us": round(m_us, 2), "speedup": round(t_us / m_us, 2),
+                                  "rel_l2_between_outputs": float(f"{float((y_t - y_m).norm() / y_m.norm()):.3e}")}),
+                      flush=True)
+            del w, codes, theirs_c, sz_c, mine_c, mine_qc
     else:
         sys.exit(f"unknown sweep {kind}")
 
@@ -409,7 +467,7 @@ def main():
                     help="int4wo-<group> (default: int4wo-<--group>, the headline configuration), int8wo or fp6 (e3m2 on an "
                          "fp16 model): the decode loop of the reference's other weight-only configurations, reported "
                          "without the int4 roofline leg")
-    ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6", "int8"), default=None,
+    ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6", "int8", "tinygemm"), default=None,
                     help="instead of the decode benchmark, print one line per kernel case of the named sweep")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -369,6 +369,33 @@ def tinygemm_int4pack(codes, inner_k_tiles):
     return out
 
 
+def tinygemm_int4pack_rocm(codes, inner_k_tiles):
+    """codes int [N, K] (0..15) -> uint32 [N/8, K/(16*inner_k_tiles), 32, inner_k_tiles/2] as the ROCm build of
+    aten._convert_weight_to_int4pack fills it on a 64-lane device, one lane at a time: the buffer is, read flat,
+    [N/16][K/(16*inner_k_tiles)][64 lanes][inner_k_tiles/2]; lane t of a tile owns row t % 16 and, in each 32-wide
+    span of k, the offsets 4*(t//16) + {0, 1, 2, 3} and 16 + the same, even ones in the low half-word.  Pinned by
+    tests/test_gptq_gpu.py against the operator of the installed PyTorch (bit for bit, inner_k_tiles 2, 4, 8)."""
+    codes = np.asarray(codes)
+    N, K = codes.shape
+    assert N % 16 == 0 and K % (inner_k_tiles * 16) == 0 and inner_k_tiles in (2, 4, 8)
+    k_outer = K // (inner_k_tiles * 16)
+    out = np.zeros((N // 16, k_outer, 64, inner_k_tiles // 2), np.uint32)
+    for n_tile in range(N // 16):
+        for ko in range(k_outer):
+            for t in range(64):
+                row = n_tile * 16 + t % 16
+                for j in range(inner_k_tiles // 2):
+                    base = ko * inner_k_tiles * 16 + 32 * j + 4 * (t // 16)
+                    word = 0
+                    for half, first in ((0, base), (1, base + 16)):
+                        for i in range(4):
+                            # even offsets go to nibbles 0..3, odd ones to nibbles 4..7, in (base, base+16) pairs
+                            nibble = (i % 2) * 4 + (i // 2) + 2 * half
+                            word |= (int(codes[row, first + i]) & 0xF) << (4 * nibble)
+                    out[n_tile, ko, t, j] = word
+    return out.reshape(N // 8, k_outer, 32, inner_k_tiles // 2)
+
+
 # --- GPTQ: textbook column-by-column optimal brain quantization, the form GPTQ's Cholesky recurrence is derived
 # from (Frantar et al. 2022, eq. 2-3).  Float64, one explicit inverse of the remaining Hessian per column; slow and
 # meant for a few dozen columns.  It cross-checks the blocked Cholesky solver of the library, which follows

@@ -196,3 +196,38 @@ def test_tinygemm_word_is_four_k_pairs_under_the_half_word_mask():
         for i, off in enumerate((0, 8, 16, 24)):
             pair = (word >> (4 * i)) & 0x000F000F
             assert pair & 0xF == codes[row, k0 + off] and pair >> 16 == codes[row, k0 + off + 1]
+
+
+def _rocm_fixture():
+    import os
+    return np.load(os.path.join(os.path.dirname(__file__), "golden", "tinygemm_rocm_int4pack.npz"))
+
+
+@pytest.mark.parametrize("inner_k_tiles", [2, 4, 8])
+def test_rocm_tinygemm_layout_matches_the_words_pytorch_rocm_wrote(inner_k_tiles):
+    # golden/tinygemm_rocm_int4pack.npz holds what aten._convert_weight_to_int4pack of PyTorch-ROCm wrote on gfx950
+    # (tests/golden/make_tinygemm_rocm.py); the oracle's lane-by-lane restatement and the library's unpacker must
+    # both agree with it
+    fx = _rocm_fixture()
+    codes, words = fx["codes"], fx[f"packed_ikt{inner_k_tiles}"]
+    np.testing.assert_array_equal(oracle.tinygemm_int4pack_rocm(codes, inner_k_tiles).view(np.int32), words)
+    got = unpack_tinygemm_int4pack(torch.from_numpy(words), inner_k_tiles, packed_by="rocm")
+    np.testing.assert_array_equal(got.numpy(), codes)
+    # and the CUDA layout is a different one: the unpacker of one must not read the other
+    assert not np.array_equal(unpack_tinygemm_int4pack(torch.from_numpy(words), inner_k_tiles).numpy(), codes)
+
+
+def test_pytorch_int4_matmul_rounds_once_where_dequantize_rounds_twice():
+    # The fixture's aten._weight_int4pack_mm output is reproduced bit for bit by w = bf16((q-8)*s + z) (one rounding)
+    # with fp32 accumulation; the reference's dequantize (torchao/quantization/quant_primitives.py:265-274), which the
+    # linear of this library follows, rounds the product first, and lands within a few 1e-3 of it.
+    fx = _rocm_fixture()
+    bf = lambda name: torch.from_numpy(fx[name]).view(torch.bfloat16).double().numpy()
+    rb = lambda a: torch.from_numpy(np.asarray(a, np.float32)).bfloat16().double().numpy()
+    s, z = np.repeat(bf("scales_bits").T, 64, 1), np.repeat(bf("zeros_bits").T, 64, 1)
+    q, x, y = fx["codes"].astype(np.float64) - 8.0, bf("x_bits"), bf("mm_bits")
+    once = rb(x @ rb(q * s + z).T)
+    twice = x @ rb(rb(q * s) + z).T
+    np.testing.assert_array_equal(once, y)
+    rel = np.linalg.norm(twice - y) / np.linalg.norm(twice)
+    assert 1e-4 < rel < 5e-3
