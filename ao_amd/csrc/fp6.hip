@@ -20,6 +20,8 @@ typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x32_t __attribute__((ext_vector_type(32)));
 typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4v_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2v_t __attribute__((ext_vector_type(2)));
 
 // ---------------------------------------------------------------- scalar casts
 // fp32 -> FPx code in the low 1+ebits+mbits bits: round to nearest even, saturate to the largest normal, no
@@ -295,45 +297,69 @@ __global__ __launch_bounds__(256) void fp6_repack_kernel(const uint8_t* __restri
 // ---------------------------------------------------------------- linear
 // out[M,N] fp16 = x[M,K] fp16 @ W^T, W = fp16(fp6 * scale), fp32 accumulation (quant_llm_linear,
 // torchao/csrc/cuda/fp6_llm/fp6_linear.cu:139-196 with the dequantization of utils_parallel_dequant.cuh:47-59).
-// One workgroup per 16-row block; WAVES waves take the 128-wide K tiles round-robin, double-buffered;
-// blockIdx.y selects a chunk of 16 activation rows.  E3M2: e3m2 codes, otherwise e2m3.
-template <int WAVES, bool E3M2>
+// One workgroup per RBW consecutive 16-row blocks; WAVES waves take the 128-wide K tiles round-robin, double-buffered,
+// and multiply each activation tile they load against the RBW weight tiles of that k (with 16 activation rows a
+// wave reads 4 KiB of activations per 1.5 KiB weight tile, so sharing them over row blocks is what keeps the cache
+// traffic below the weight stream).  blockIdx.y selects a chunk of 16 activation rows.  E3M2: e3m2 codes, otherwise
+// e2m3.  The host launches RBW > 1 only when N / 16 is a multiple of it.
+template <int WAVES, bool E3M2, int RBW>
 __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
                                                                  const uint32_t* __restrict__ native,
                                                                  const uint16_t* __restrict__ scale, int64_t N, int64_t Kp,
                                                                  uint16_t* __restrict__ out,
                                                                  const uint16_t* __restrict__ residual,
                                                                  const uint16_t* __restrict__ gate) {
-    __shared__ float red[WAVES][4][64];
+    __shared__ float red[RBW][WAVES][4][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, qd = lane >> 4;
-    const int64_t rb = blockIdx.x, m0 = (int64_t)blockIdx.y * 16;
+    const int64_t rb0 = (int64_t)blockIdx.x * RBW, m0 = (int64_t)blockIdx.y * 16;
     const int KB = (int)(Kp / 128);
-    const uint32_t* tiles = native + rb * KB * 384;
+    const uint32_t* tiles = native + rb0 * KB * 384;
     const bool xact = (m0 + r) < M;
     const uint16_t* xp = x + (xact ? (m0 + r) : 0) * K + qd * 32;
-    union { uint16_t h; _Float16 f; } sc;
-    sc.h = scale[rb * 16 + r];
-    const f16x2_t sc2 = {sc.f, sc.f};
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    // Tile buffers hold native vectors, not HIP's uint4 / uint2 structs: a struct load is a memcpy into the buffer,
+    // which then stays in memory (scratch or LDS) instead of registers once it holds more than one row block.
+    f16x2_t sc2_0, sc2_1, sc2_2, sc2_3;
+    f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
+    auto row_scale = [&](int j) {
+        union { uint16_t h; _Float16 f; } sc;
+        sc.h = scale[(rb0 + j) * 16 + r];
+        return f16x2_t{sc.f, sc.f};
+    };
+    sc2_0 = row_scale(0);
+    sc2_1 = RBW > 1 ? row_scale(1) : sc2_0;
+    sc2_2 = RBW > 2 ? row_scale(2) : sc2_0;
+    sc2_3 = RBW > 3 ? row_scale(3) : sc2_0;
 
-    struct Buf { uint4 lo; uint2 hi; uint4 x[4]; };
-    auto load_tile = [&](Buf& b, int kb) {
+    struct Buf { u32x6_t w0, w1, w2, w3; u32x4v_t x[4]; };
+    // the 24 bytes of a lane: 16 from the first kilobyte of the tile, 8 from its last 512 bytes; joined by shuffles
+    // right at the load (an element-wise initializer, or a widening shuffle of a buffer member, goes through memory)
+    auto load_w = [&](const uint32_t* t) __attribute__((always_inline)) {
+        const u32x4v_t lo = reinterpret_cast<const u32x4v_t*>(t)[lane];
+        const u32x2v_t hi = reinterpret_cast<const u32x2v_t*>(t + 256)[lane];
+        return __builtin_shufflevector(lo, __builtin_shufflevector(hi, hi, 0, 1, -1, -1), 0, 1, 2, 3, 4, 5);
+    };
+    auto load_tile = [&](Buf& b, int kb) __attribute__((always_inline)) {
         const uint32_t* t = tiles + (int64_t)kb * 384;
-        b.lo = reinterpret_cast<const uint4*>(t)[lane];
-        b.hi = reinterpret_cast<const uint2*>(t + 256)[lane];
+        const int64_t next = (int64_t)KB * 384;  // same k tile of the next row block
+        b.w0 = load_w(t);
+        if (RBW > 1) b.w1 = load_w(t + next);
+        if (RBW > 2) {
+            b.w2 = load_w(t + 2 * next);
+            b.w3 = load_w(t + 3 * next);
+        }
         if (xact) {
             const int64_t k0 = (int64_t)kb * 128 + qd * 32;
             if (k0 + 32 <= K) {
-                const uint4* xv = reinterpret_cast<const uint4*>(xp + (int64_t)kb * 128);
+                const u32x4v_t* xv = reinterpret_cast<const u32x4v_t*>(xp + (int64_t)kb * 128);
 #pragma unroll
                 for (int sl = 0; sl < 4; ++sl) b.x[sl] = xv[sl];
             } else {
 #pragma unroll
                 for (int sl = 0; sl < 4; ++sl) {
-                    union { uint4 q; uint16_t h[8]; } u;
-                    u.q = make_uint4(0, 0, 0, 0);
+                    union { u32x4v_t q; uint16_t h[8]; } u;
+                    u.q = u32x4v_t{0, 0, 0, 0};
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
                         if (k0 + sl * 8 + e < K) u.h[e] = xp[(int64_t)kb * 128 + sl * 8 + e];
@@ -342,8 +368,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* 
             }
         }
     };
-    auto compute_tile = [&](const Buf& b) {
-        const u32x6_t packed = {b.lo.x, b.lo.y, b.lo.z, b.lo.w, b.hi.x, b.hi.y};
+    auto block_mfma = [&](const u32x6_t& packed, const f16x2_t sc2, const Buf& b, f32x4_t& acc)
+        __attribute__((always_inline)) {
         f16x32_t v;
         if (E3M2) v = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(packed, 1.0f);
         else v = __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(packed, 1.0f);
@@ -351,21 +377,29 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* 
         for (int sl = 0; sl < 4; ++sl) {
             union { f16x2_t p[4]; f16x8_t v; } w;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const f16x2_t pr = {v[sl * 8 + 2 * j], v[sl * 8 + 2 * j + 1]};
-                w.p[j] = pr * sc2;  // v_pk_mul_f16: fp16(fp6 * scale), the one rounding of the reference kernel
+            for (int e = 0; e < 4; ++e) {
+                const f16x2_t pr = {v[sl * 8 + 2 * e], v[sl * 8 + 2 * e + 1]};
+                w.p[e] = pr * sc2;  // v_pk_mul_f16: fp16(fp6 * scale), the one rounding of the reference kernel
             }
-            union { uint4 q; f16x8_t v; } xa;
+            union { u32x4v_t q; f16x8_t v; } xa;
             xa.q = b.x[sl];
             acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa.v, w.v, acc, 0, 0, 0);
+        }
+    };
+    auto compute_tile = [&](const Buf& b) __attribute__((always_inline)) {
+        block_mfma(b.w0, sc2_0, b, acc0);
+        if (RBW > 1) block_mfma(b.w1, sc2_1, b, acc1);
+        if (RBW > 2) {
+            block_mfma(b.w2, sc2_2, b, acc2);
+            block_mfma(b.w3, sc2_3, b, acc3);
         }
     };
 
     Buf b0, b1;
 #pragma unroll
     for (int sl = 0; sl < 4; ++sl) {
-        b0.x[sl] = make_uint4(0, 0, 0, 0);
-        b1.x[sl] = make_uint4(0, 0, 0, 0);
+        b0.x[sl] = u32x4v_t{0, 0, 0, 0};
+        b1.x[sl] = u32x4v_t{0, 0, 0, 0};
     }
     int kb = wave;
     if (kb < KB) load_tile(b0, kb);
@@ -380,15 +414,23 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* 
         kb = kb2;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][i][lane] = acc[i];
+    for (int i = 0; i < 4; ++i) {
+        red[0][wave][i][lane] = acc0[i];
+        if (RBW > 1) red[1][wave][i][lane] = acc1[i];
+        if (RBW > 2) {
+            red[2][wave][i][lane] = acc2[i];
+            red[3][wave][i][lane] = acc3[i];
+        }
+    }
     __syncthreads();
-    if (wave == 0) {
-        const int64_t n = rb * 16 + r;
+    // wave j (and j + WAVES, ...) sums and stores row block j
+    for (int j = wave; j < RBW; j += WAVES) {
+        const int64_t n = (rb0 + j) * 16 + r;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float s = 0.f;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) s += red[w][i][lane];
+            for (int w = 0; w < WAVES; ++w) s += red[j][w][i][lane];
             const int64_t m = m0 + 4 * qd + i;
             if (m < M && n < N) {
                 // the module's next elementwise op on the fp16 result, fused: h + linear(...) or silu(gate) * linear(...)
@@ -459,8 +501,6 @@ struct Fp6GemvArgs {
     const uint32_t* native_up; const uint16_t* scale_up;  // DUAL: second weight of the same shape and its scales
 };
 
-typedef uint32_t u32x4v_t __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2v_t __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ u32x4v_t fp6_stream_lo(const void* sbase, uint32_t voff) {
     u32x4v_t v;
@@ -913,6 +953,16 @@ static void launch_fp6_gemv(int waves, dim3 grid, size_t smem, hipStream_t st, h
     }
 }
 
+// Row blocks a wave of fp6_linear_kernel takes per activation tile: 1 below 4 activation rows (the weight stream
+// dominates), else the largest of 4, 2 that divides the row-block count and leaves 192 or more workgroups (with 128
+// on the 256 CUs the launch was measured slower than one row block per wave).
+static int fp6_row_blocks_per_wave(int64_t M, int64_t RB, int64_t mchunks) {
+    if (M < 4) return 1;
+    for (int rbw = 4; rbw > 1; rbw /= 2)
+        if (RB % rbw == 0 && (RB / rbw) * mchunks >= 192) return rbw;
+    return 1;
+}
+
 static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
                                int64_t N, int ebits, int mbits, const void* residual_f16, const void* gate_f16,
                                void* out_f16, void* stream, const void* norm_weight_f16 = nullptr, float norm_eps = 0.f,
@@ -957,7 +1007,10 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
                "and 16-byte aligned operands", (long long)M, (long long)K);
     AO_REQUIRE(!native_up || (scale_up_f16 && !res && !gt), "the two-weight SwiGLU takes the second weight's scales and no "
                "other epilogue");
-    if (fits && (need_lds || KB >= 4 * waves)) {
+    // (with four row blocks per activation tile in registers the rows need no staging: 12.7 / 12.9 us against 13.1 /
+    // 17.4 us staged at 4 / 8 rows on 14336 x 4096; 16 rows, which never fit, 13.9 against 21.8 us)
+    const bool shared_tiles = !need_lds && M >= 4 && fp6_row_blocks_per_wave(M, RB, mchunks) == 4;
+    if (fits && !shared_tiles && (need_lds || KB >= 4 * waves)) {
         Fp6GemvArgs a{xx, M, K, Kp, nat, sc, N, o, res, gt, (const uint16_t*)norm_weight_f16, norm_eps,
                       (const uint32_t*)native_up, (const uint16_t*)scale_up_f16};
         if (ebits == 3) {
@@ -989,18 +1042,33 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
         AO_LAUNCH_CHECK();
         return 0;
     }
-#define AO_FP6_LAUNCH(W)                                                                                                 \
+#define AO_FP6_LAUNCH(W, R)                                                                                              \
     if (ebits == 3)                                                                                                      \
-        hipExtLaunchKernelGGL((fp6_linear_kernel<W, true>), grid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o, res, gt); \
+        hipExtLaunchKernelGGL((fp6_linear_kernel<W, true, R>), lgrid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o, res, gt); \
     else                                                                                                                 \
-        hipExtLaunchKernelGGL((fp6_linear_kernel<W, false>), grid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o, res, gt)
-    switch (waves) {
-        case 1: AO_FP6_LAUNCH(1); break;
-        case 2: AO_FP6_LAUNCH(2); break;
-        case 4: AO_FP6_LAUNCH(4); break;
-        case 8: AO_FP6_LAUNCH(8); break;
-        default: AO_FP6_LAUNCH(16); break;
+        hipExtLaunchKernelGGL((fp6_linear_kernel<W, false, R>), lgrid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, Kp, o, res, gt)
+#define AO_FP6_LAUNCH_WAVES(R, WMAX)                                                                                     \
+    switch (waves) {                                                                                                     \
+        case 1: AO_FP6_LAUNCH(1, R); break;                                                                              \
+        case 2: AO_FP6_LAUNCH(2, R); break;                                                                              \
+        case 4: AO_FP6_LAUNCH(4, R); break;                                                                              \
+        case 8: AO_FP6_LAUNCH(8, R); break;                                                                              \
+        default: AO_FP6_LAUNCH(WMAX, R); break;                                                                          \
     }
+    // With 4 or more activation rows a wave reads more activation than weight bytes per tile: let it take 2 or 4 row
+    // blocks per activation tile while that leaves at least 128 workgroups, and size the K split for that grid.
+    const int rbw = fp6_row_blocks_per_wave(M, RB, mchunks);
+    if (rbw > 1) {
+        // (16 waves of 4 row blocks would not fit the 128 registers a lane of a 1024-thread workgroup has)
+        const int wmax = rbw == 4 ? 8 : 16;
+        waves = 1;
+        while (waves < wmax && (RB / rbw) * mchunks * waves * 2 <= 4096 + (RB / rbw) * mchunks && waves * 2 <= KB) waves *= 2;
+    }
+    dim3 lgrid((unsigned)(RB / rbw), (unsigned)mchunks);
+    if (rbw == 4) { AO_FP6_LAUNCH_WAVES(4, 8) }
+    else if (rbw == 2) { AO_FP6_LAUNCH_WAVES(2, 16) }
+    else { AO_FP6_LAUNCH_WAVES(1, 16) }
+#undef AO_FP6_LAUNCH_WAVES
 #undef AO_FP6_LAUNCH
     AO_LAUNCH_CHECK();
     return 0;

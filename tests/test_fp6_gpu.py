@@ -85,6 +85,26 @@ def test_linear_matches_oracle(oracle, shape, M):
     assert rel.mean() < 1e-3
 
 
+@pytest.mark.parametrize("N,K,M", [(14336, 1024, 16), (14336, 512, 8), (6144, 576, 5), (3072, 320, 40), (2048, 192, 100), (4096, 4096, 16)])
+def test_linear_with_shared_activation_tiles_matches_oracle(oracle, N, K, M):
+    """Sizes at which a wave of the few-row kernel multiplies one activation tile against 4 or 2 row blocks (4 or more
+    activation rows, 192 or more workgroups left), with whole and half last K tiles and more than one 16-row chunk."""
+    from ao_amd import ops
+
+    print(f"case fp6 linear shared activation tiles N={N} K={K} M={M}", flush=True)
+    dev = _dev()
+    g = torch.Generator().manual_seed(N + K + M)
+    x = (torch.rand(M, K, generator=g) + 0.5).half()
+    packed = torch.randint(0, 256, (N, K // 8 * 6), dtype=torch.uint8, generator=g)
+    scale = (torch.rand(N, generator=g) + 0.5).half()
+    y = ops.quant_llm_linear(3, 2, x.to(dev), packed.to(dev), scale.to(dev), 1).float().cpu().numpy()
+    codes = oracle.unpack_tc_fp6(packed.numpy(), N, K)
+    y_ref16 = oracle.fpx_linear(bits16(x), codes, bits16(scale), 3, 2).astype(np.float16).astype(np.float32)
+    assert rel_l2(y, y_ref16) <= 1e-3
+    rel = np.abs(y - y_ref16) / np.maximum(np.abs(y_ref16), 1e-6)
+    assert rel.mean() < 1e-3
+
+
 def test_e2m3_format(oracle):
     from ao_amd import ops
 
