@@ -715,10 +715,11 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_gemv_kernel(const Fp6GemvArgs 
 // GEMM.  Each of the 4 waves owns two 16-row weight blocks: it loads their native tiles (24 bytes per lane) straight
 // into registers, converts them once (one v_cvt_scalef32_pk32 + 16 v_pk_mul_f16 per block and tile) and multiplies
 // them against the eight 16-row activation blocks of the tile (64 MFMAs per wave and tile).  The activation tile is
-// double-buffered in LDS (row stride 272 bytes), fetched two tiles ahead into registers; every load is
-// unconditional (rows past M alias the last row, tiles past the end repeat the last tile) so that the compiler's
-// vmcnt waits stay exact.
-template <bool E3M2, int NBW, int MBLK>
+// double-buffered in LDS (row stride 272 bytes); weights and activations are fetched PF tiles ahead into rings of
+// registers (a small tile computes for far less than a memory latency, so its loop is as fast as its loads are
+// deep; the activation ring may be shorter, XD tiles, where registers are short); every load is unconditional (rows past M alias the last row, tiles past the end repeat the last tile) so
+// that the compiler's vmcnt waits stay exact.
+template <bool E3M2, int NBW, int MBLK, int PF, int XD>
 __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
                                                            const uint32_t* __restrict__ native,
                                                            const uint16_t* __restrict__ scale, int64_t N,
@@ -744,27 +745,31 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
         const int64_t m = m0 + xrow + 16 * j;
         xrow_ptr[j] = x + (m < M ? m : M - 1) * K + xchunk * 8;
     }
-    u32x4_t xr[XCH];
-    auto load_x = [&](int kb) {
+    static_assert(PF >= 2 && PF % 2 == 0, "the ring of prefetched tiles alternates between the two LDS buffers");
+    static_assert(PF % XD == 0, "a round of the weight ring is a whole number of rounds of the activation ring");
+    u32x4_t xr[XD][XCH];
+    auto load_x = [&](u32x4_t (&dst)[XCH], int kb) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < XCH; ++j) xr[j] = *reinterpret_cast<const u32x4_t*>(xrow_ptr[j] + (int64_t)kb * 128);
+        for (int j = 0; j < XCH; ++j) dst[j] = *reinterpret_cast<const u32x4_t*>(xrow_ptr[j] + (int64_t)kb * 128);
     };
-    auto store_x = [&](int buf) {
+    auto store_x = [&](int buf, const u32x4_t (&src)[XCH]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < XCH; ++j)
-            *reinterpret_cast<u32x4_t*>(xs_all[buf] + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
+            *reinterpret_cast<u32x4_t*>(xs_all[buf] + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = src[j];
     };
 
-    struct WBuf { u32x4_t lo0, lo1; u32x2_t hi0, hi1; };
+    // the 24 bytes of a lane per tile, joined into the conversion's operand right at the load
+    struct WBuf { u32x6_t w0, w1; };
     const uint32_t* t0 = native + (has0 ? nb0 : 0) * KB * 384;
     const uint32_t* t1 = native + (has1 ? nb0 + 1 : 0) * KB * 384;
-    auto load_w = [&](WBuf& b, int kb) {
-        b.lo0 = reinterpret_cast<const u32x4_t*>(t0 + (int64_t)kb * 384)[lane];
-        b.hi0 = reinterpret_cast<const u32x2_t*>(t0 + (int64_t)kb * 384 + 256)[lane];
-        if (NBW > 1) {
-            b.lo1 = reinterpret_cast<const u32x4_t*>(t1 + (int64_t)kb * 384)[lane];
-            b.hi1 = reinterpret_cast<const u32x2_t*>(t1 + (int64_t)kb * 384 + 256)[lane];
-        }
+    auto load_w6 = [&](const uint32_t* t) __attribute__((always_inline)) {
+        const u32x4_t lo = reinterpret_cast<const u32x4_t*>(t)[lane];
+        const u32x2_t hi = reinterpret_cast<const u32x2_t*>(t + 256)[lane];
+        return __builtin_shufflevector(lo, __builtin_shufflevector(hi, hi, 0, 1, -1, -1), 0, 1, 2, 3, 4, 5);
+    };
+    auto load_w = [&](WBuf& b, int kb) __attribute__((always_inline)) {
+        b.w0 = load_w6(t0 + (int64_t)kb * 384);
+        if (NBW > 1) b.w1 = load_w6(t1 + (int64_t)kb * 384);
     };
     union { uint16_t h; _Float16 f; } s0, s1;
     s0.h = scale[(has0 ? nb0 : 0) * 16 + r];
@@ -777,17 +782,16 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
         acc0[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         acc1[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
-    auto convert = [&](const u32x4_t& lo, const u32x2_t& hi) {
-        const u32x6_t packed = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y};
+    auto convert = [&](const u32x6_t& packed) __attribute__((always_inline)) {
         if (E3M2) return __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(packed, 1.0f);
         return __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(packed, 1.0f);
     };
-    auto compute = [&](const WBuf& b, int buf) {
+    auto compute = [&](const WBuf& b, int buf) __attribute__((always_inline)) {
         const uint16_t* xs = xs_all[buf];
-        const f16x32_t v0 = convert(b.lo0, b.hi0), v1 = NBW > 1 ? convert(b.lo1, b.hi1) : v0;
+        const f16x32_t v0 = convert(b.w0), v1 = NBW > 1 ? convert(b.w1) : v0;
         union XFrag { uint4 q; f16x8_t v; };
         XFrag xa[2][MBLK];
-        auto read_frags = [&](int sl, XFrag* dst) {
+        auto read_frags = [&](int sl, XFrag* dst) __attribute__((always_inline)) {
 #pragma unroll
             for (int mb = 0; mb < MBLK; ++mb)
                 dst[mb].q = *reinterpret_cast<const uint4*>(xs + (mb * 16 + r) * XSTRIDE + qd * 32 + sl * 8);
@@ -813,27 +817,35 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
         }
     };
 
-    WBuf b0, b1;
+    // Weight tile t lives in ring slot t % PF, its activations in slot t % XD until they move to LDS buffer t & 1.
+    // Iteration `cur` stages the activations of tile cur + 1 into the other LDS buffer (free since the barrier that
+    // ended iteration cur - 1), refills that slot with tile cur + 1 + XD, computes tile cur and refills its weight
+    // slot with tile cur + PF.
+    WBuf wb[PF];
     const int last = KB - 1;
-    load_x(0);
-    load_w(b0, 0);
-    store_x(0);
-    load_x(1 < last ? 1 : last);
-    load_w(b1, 1 < last ? 1 : last);
-    __syncthreads();
-    for (int kb = 0; kb + 1 < KB; kb += 2) {
-        store_x(1);
-        load_x(kb + 2 < last ? kb + 2 : last);
-        compute(b0, 0);
-        load_w(b0, kb + 2 < last ? kb + 2 : last);
-        __syncthreads();
-        store_x(0);
-        load_x(kb + 3 < last ? kb + 3 : last);
-        compute(b1, 1);
-        load_w(b1, kb + 3 < last ? kb + 3 : last);
-        __syncthreads();
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+        if (j < XD) load_x(xr[j], j < last ? j : last);
+        load_w(wb[j], j < last ? j : last);
     }
-    if (KB & 1) compute(b0, 0);
+    store_x(0, xr[0]);
+    load_x(xr[0], XD < last ? XD : last);
+    __syncthreads();
+    auto stage = [&](int cur, int j) __attribute__((always_inline)) {  // j = cur % PF, a constant after unrolling
+        store_x((j + 1) & 1, xr[(j + 1) % XD]);
+        load_x(xr[(j + 1) % XD], cur + 1 + XD < last ? cur + 1 + XD : last);
+        compute(wb[j], j & 1);
+        load_w(wb[j], cur + PF < last ? cur + PF : last);
+        __syncthreads();
+    };
+    int kb = 0;
+    for (; kb + PF <= KB; kb += PF) {  // whole rounds of the ring, branch-free inside
+#pragma unroll
+        for (int j = 0; j < PF; ++j) stage(kb + j, j);
+    }
+#pragma unroll
+    for (int j = 0; j < PF - 1; ++j)
+        if (kb + j < KB) stage(kb + j, j);  // uniform over the workgroup
 
     // acc[mb][i] = C[m = m0 + 16*mb + 4*qd + i][n = 16*nb + r]
 #pragma unroll
@@ -1031,13 +1043,13 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
                    big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64));
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
         if (ebits == 3) {
-            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 2, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
-            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 2>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
-            else hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 2, 8, 2, 1>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 2, 8, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            else hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 4, 4, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
         } else {
-            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 2, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
-            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 2>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
-            else hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 2, 8, 2, 1>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 2, 8, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            else hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 4, 4, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
         }
         AO_LAUNCH_CHECK();
         return 0;
