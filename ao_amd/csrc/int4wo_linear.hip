@@ -862,6 +862,142 @@ __global__ __launch_bounds__(256, 2) void int4wo_gemm_kernel(const LinearArgs a)
     }
 }
 
+// The 64-weight-row GEMM tile for batches that give the plain GEMM about one wave per SIMD: there the K loop of a
+// tile is a chain of dependent dequantize + MFMA steps that nothing overlaps.  KP groups of 4 waves share a workgroup
+// tile and take the K tiles round-robin (group p: tiles p, p + KP, ...), each with its own pair of LDS activation
+// buffers; their partial accumulators meet in LDS (in the activation buffers, idle by then) and group 0 stores.
+// Every group runs the same number of iterations, so the barriers stay uniform: a group whose last tile does not
+// exist loads the last real tile again and skips the arithmetic.
+template <int G, int MBLK, int KP>
+__global__ __launch_bounds__(256 * KP) void int4wo_gemm_ksplit_kernel(const LinearArgs a) {
+    constexpr int BM = 16 * MBLK, XSTRIDE = 136;  // bf16 elements per LDS row
+    constexpr int XCH = BM / 16;                  // 16-byte activation chunks per thread and K tile
+    __shared__ __align__(16) uint16_t xs_all[KP][2][BM * XSTRIDE];
+    static_assert((KP - 1) * 4 * MBLK * 4 * 64 * 4 <= KP * 2 * BM * XSTRIDE * 2, "partial sums fit the activation buffers");
+    const int tid = threadIdx.x & 255, lane = tid & 63;
+    const int part = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);
+    const int wave = __builtin_amdgcn_readfirstlane((threadIdx.x >> 6) & 3);
+    const int r = lane & 15, qd = lane >> 4;
+    const int KB = (int)(a.Kp / 128);
+    const int IT = (KB + KP - 1) / KP;  // iterations of every group
+    const int64_t nblocks = (a.N + 15) / 16;
+    const int64_t nb0 = (int64_t)blockIdx.x * 4 + wave;
+    const bool has0 = nb0 < nblocks;
+    const int64_t m0 = (int64_t)blockIdx.y * BM;
+    const uint32_t magic = 0x43004300u, one_lo = 0x00003F80u, one_hi = 0x3F800000u;
+    auto tile = [&](int i) __attribute__((always_inline)) {
+        const int kb = part + KP * i;
+        return kb < KB ? kb : KB - 1;
+    };
+
+    const int xrow = tid >> 4, xchunk = tid & 15;
+    u32x4_t xr[XCH];
+    const uint16_t* xrow_ptr[XCH];
+#pragma unroll
+    for (int j = 0; j < XCH; ++j) {
+        const int64_t m = m0 + xrow + 16 * j;
+        xrow_ptr[j] = a.x + (m < a.M ? m : a.M - 1) * a.ldx + xchunk * 8;
+    }
+    auto load_x = [&](int kb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < XCH; ++j) xr[j] = *reinterpret_cast<const u32x4_t*>(xrow_ptr[j] + (int64_t)kb * 128);
+    };
+    auto store_x = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < XCH; ++j)
+            *reinterpret_cast<u32x4_t*>(xs_all[part][buf] + (xrow + 16 * j) * XSTRIDE + xchunk * 8) = xr[j];
+    };
+
+    struct WBuf { u32x4_t w0; uint32_t q0; };
+    const uint4* wp0 = a.packed + (has0 ? nb0 : 0) * KB * 64 + lane;
+    const uint32_t* qp0 = a.qparams + (has0 ? nb0 : 0) * (a.Kp / G) * 16 + r;
+    auto load_w = [&](WBuf& b, int kb) __attribute__((always_inline)) {
+        b.w0 = *reinterpret_cast<const u32x4_t*>(wp0 + (int64_t)kb * 64);
+        b.q0 = qp0[((kb * 128 + qd * 32) / G) * 16];
+    };
+
+    f32x4_t acc0[MBLK];
+#pragma unroll
+    for (int mb = 0; mb < MBLK; ++mb) acc0[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const WBuf& b, int buf) __attribute__((always_inline)) {
+        const uint16_t* xs = xs_all[part][buf];
+        const GroupConst g0 = make_group(b.q0);
+        const uint32_t w0[4] = {b.w0.x, b.w0.y, b.w0.z, b.w0.w};
+        union XFrag { uint4 q; bf16x8_t v; };
+        XFrag xa[2][MBLK];
+        auto read_frags = [&](int sl, XFrag* dst) __attribute__((always_inline)) {
+#pragma unroll
+            for (int mb = 0; mb < MBLK; ++mb)
+                dst[mb].q = *reinterpret_cast<const uint4*>(xs + (mb * 16 + r) * XSTRIDE + qd * 32 + sl * 8);
+        };
+        read_frags(0, xa[0]);
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            if (sl + 1 < 4) read_frags(sl + 1, xa[(sl + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            const bf16x8_t bw0 = dequant8(w0[sl], g0, magic, one_lo, one_hi);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int mb = 0; mb < MBLK; ++mb)
+                acc0[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[sl & 1][mb].v, bw0, acc0[mb], 0, 0, 0);
+        }
+    };
+
+    WBuf b0, b1;
+    load_x(tile(0));
+    load_w(b0, tile(0));
+    store_x(0);
+    load_x(tile(1));
+    load_w(b1, tile(1));
+    __syncthreads();
+    for (int i = 0; i + 1 < IT; i += 2) {
+        store_x(1);
+        load_x(tile(i + 2));
+        if (part + KP * i < KB) compute(b0, 0);
+        load_w(b0, tile(i + 2));
+        __syncthreads();
+        store_x(0);
+        load_x(tile(i + 3));
+        if (part + KP * (i + 1) < KB) compute(b1, 1);
+        load_w(b1, tile(i + 3));
+        __syncthreads();
+    }
+    if ((IT & 1) && part + KP * (IT - 1) < KB) compute(b0, 0);
+
+    // partial sums of groups 1.. -> LDS -> group 0
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(&xs_all[0][0][0]);
+    if (part > 0) {
+#pragma unroll
+        for (int mb = 0; mb < MBLK; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[((((part - 1) * 4 + wave) * MBLK + mb) * 4 + i) * 64 + lane] = acc0[mb][i];
+    }
+    __syncthreads();
+    if (part > 0 || !has0) return;
+#pragma unroll
+    for (int p = 1; p < KP; ++p)
+#pragma unroll
+        for (int mb = 0; mb < MBLK; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc0[mb][i] += red[((((p - 1) * 4 + wave) * MBLK + mb) * 4 + i) * 64 + lane];
+    // acc[mb][i] = C[m = m0 + 16*mb + 4*qd + i][n = 16*nb + r]
+    const int64_t n = nb0 * 16 + r;
+    if (n >= a.N) return;
+    const float bv = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.f;
+#pragma unroll
+    for (int mb = 0; mb < MBLK; ++mb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t m = m0 + mb * 16 + 4 * qd + i;
+            if (m < a.M) {
+                const float v = acc0[mb][i] + bv;
+                if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = v;
+                else ((uint16_t*)a.y)[m * a.ldy + n] = f32_to_bf16_bits(v);
+            }
+        }
+}
+
 template <typename Kernel>
 static void launch_timed(Kernel kernel, dim3 grid, dim3 block, size_t smem, hipStream_t st, const LinearArgs& a) {
     if (g_prof_start && g_prof_stop) {
@@ -1014,9 +1150,13 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
         dim3 ggrid(big ? (unsigned)((RB + 7) / 8) : (unsigned)((RB + 3) / 4),
                    big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64));
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
-#define AO_GEMM_LAUNCH(GG)                                                                        \
-    if (big) launch_timed(int4wo_gemm_kernel<GG, 2, 8>, ggrid, dim3(256), 0, st, a);              \
-    else if (tiny) launch_timed(int4wo_gemm_kernel<GG, 1, 2>, ggrid, dim3(256), 0, st, a);        \
+        // the small tiles split their K loop over 4 groups of waves once each group has 2 or more K tiles
+        const bool ksplit_tiles = !big && KB_all >= 8;
+#define AO_GEMM_LAUNCH(GG)                                                                                     \
+    if (big) launch_timed(int4wo_gemm_kernel<GG, 2, 8>, ggrid, dim3(256), 0, st, a);                           \
+    else if (tiny && ksplit_tiles) launch_timed(int4wo_gemm_ksplit_kernel<GG, 2, 4>, ggrid, dim3(1024), 0, st, a); \
+    else if (tiny) launch_timed(int4wo_gemm_kernel<GG, 1, 2>, ggrid, dim3(256), 0, st, a);                     \
+    else if (ksplit_tiles) launch_timed(int4wo_gemm_ksplit_kernel<GG, 4, 4>, ggrid, dim3(1024), 0, st, a);     \
     else launch_timed(int4wo_gemm_kernel<GG, 1, 4>, ggrid, dim3(256), 0, st, a)
         switch (g) {
             case 32: AO_GEMM_LAUNCH(32); break;
