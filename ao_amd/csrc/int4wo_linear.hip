@@ -1150,8 +1150,10 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
         dim3 ggrid(big ? (unsigned)((RB + 7) / 8) : (unsigned)((RB + 3) / 4),
                    big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64));
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
-        // the small tiles split their K loop over 4 groups of waves once each group has 2 or more K tiles
-        const bool ksplit_tiles = !big && KB_all >= 8;
+        // the small tiles split their K loop over 4 groups of waves: the 32-row tiles (at most one workgroup per CU) once
+        // each group has 2 or more K tiles; the 64-row tiles (192 or more workgroups, which already overlap each other)
+        // from 64 K tiles on (K = 14336, 512 rows: -4 %; K = 4096: +4 % and therefore not split)
+        const bool ksplit_tiles = !big && KB_all >= (tiny ? 8 : 64);
 #define AO_GEMM_LAUNCH(GG)                                                                                     \
     if (big) launch_timed(int4wo_gemm_kernel<GG, 2, 8>, ggrid, dim3(256), 0, st, a);                           \
     else if (tiny && ksplit_tiles) launch_timed(int4wo_gemm_ksplit_kernel<GG, 2, 4>, ggrid, dim3(1024), 0, st, a); \

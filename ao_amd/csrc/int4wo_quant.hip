@@ -34,6 +34,46 @@ struct QParamArgs {
     void* zp;
 };
 
+// scale and zero point of one block from its min / max: quant_primitives.py:338-367
+__device__ __forceinline__ void finish_qparams(const QParamArgs& a, float mn, float mx, int has_nan, int64_t blk) {
+    const int dt = a.in_dtype;
+    if (has_nan) { mn = NAN; mx = NAN; }   // torch.amin / amax propagate NaN
+
+    const float range = (float)(double)(a.qmax - a.qmin);
+    const float half_range = (float)((double)(a.qmax - a.qmin) / 2.0);
+    const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
+    const float epsv = rd(dt, a.eps < 0.f ? dtype_eps_dev(dt) : a.eps);
+
+    float mn_neg = mn, mx_pos = mx;
+    if (a.preserve_zero) {  // :338-340
+        mn_neg = mn < 0.f ? mn : (mn != mn ? mn : 0.f);
+        mx_pos = mx > 0.f ? mx : (mx != mx ? mx : 0.f);
+    }
+    float scale, zp;
+    if (a.mapping == AO_MAP_SYMMETRIC) {  // :345-353
+        float neg = rd(dt, -mn_neg);
+        mx_pos = neg > mx_pos ? neg : mx_pos;
+        scale = rd(dt, __fdiv_rn(mx_pos, half_range));
+        zp = rd(dt, (float)(int)((double)(a.qmax + a.qmin + 1) / 2.0));
+    } else {
+        float d = rd(dt, mx_pos - mn_neg);  // :355
+        scale = rd(dt, __fdiv_rn(d, range));
+        if (a.preserve_zero) {  // :356-358
+            float q = rd(dt, __fdiv_rn(mn_neg, scale));
+            q = rd(dt, __builtin_rintf(q));
+            zp = rd(dt, (float)a.qmin - q);
+            float lo = rd(dt, (float)a.qmin), hi = rd(dt, (float)a.qmax);
+            zp = zp < lo ? lo : (zp > hi ? hi : zp);
+        } else {  // :360-362
+            float q = rd(dt, scale * mid);
+            zp = rd(dt, mn_neg + q);
+        }
+    }
+    if (!(scale >= epsv) && scale == scale) scale = epsv;  // clamp(min=eps) :365
+    store_f(a.scale, a.scale_dtype, blk, scale);
+    store_f(a.zp, a.zp_dtype, blk, zp);
+}
+
 template <int TPB>
 __global__ __launch_bounds__(256) void choose_qparams_kernel(QParamArgs a) {
     constexpr int BLOCKS_PER_WG = 256 / TPB;
@@ -75,41 +115,48 @@ __global__ __launch_bounds__(256) void choose_qparams_kernel(QParamArgs a) {
         has_nan = red_nan[0] | red_nan[1] | red_nan[2] | red_nan[3];
     }
     if (!active || t != 0) return;
-    if (has_nan) { mn = NAN; mx = NAN; }   // torch.amin / amax propagate NaN
+    finish_qparams(a, mn, mx, has_nan, blk);
+}
 
-    const float range = (float)(double)(a.qmax - a.qmin);
-    const float half_range = (float)((double)(a.qmax - a.qmin) / 2.0);
-    const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
-    const float epsv = rd(dt, a.eps < 0.f ? dtype_eps_dev(dt) : a.eps);
-
-    float mn_neg = mn, mx_pos = mx;
-    if (a.preserve_zero) {  // :338-340
-        mn_neg = mn < 0.f ? mn : (mn != mn ? mn : 0.f);
-        mx_pos = mx > 0.f ? mx : (mx != mx ? mx : 0.f);
-    }
-    float scale, zp;
-    if (a.mapping == AO_MAP_SYMMETRIC) {  // :345-353
-        float neg = rd(dt, -mn_neg);
-        mx_pos = neg > mx_pos ? neg : mx_pos;
-        scale = rd(dt, __fdiv_rn(mx_pos, half_range));
-        zp = rd(dt, (float)(int)((double)(a.qmax + a.qmin + 1) / 2.0));
+// Row groups (bN == 1) whose length is 8 * TPG, TPG a power of two up to 64: a thread reads eight consecutive
+// elements with one 16-byte (32-byte for fp32) load, TPG neighbouring lanes reduce with shuffles, the first of them
+// finishes the group.  Index arithmetic once per eight elements.
+__global__ __launch_bounds__(256) void choose_qparams_vec8_kernel(QParamArgs a, uint32_t chunks, uint32_t tpg, uint32_t GK) {
+    const uint32_t ci = blockIdx.x * 256u + threadIdx.x;
+    const bool active = ci < chunks;
+    const uint32_t cc = active ? ci : chunks - 1;
+    const uint32_t blk = cc / tpg, part = cc % tpg;
+    const uint32_t r = blk / GK, gk = blk % GK;
+    const int64_t off = (int64_t)r * a.ld + (int64_t)gk * a.bK + part * 8;
+    float x[8];
+    if (a.in_dtype == AO_F32) {
+        const float4 v0 = *reinterpret_cast<const float4*>((const float*)a.in + off);
+        const float4 v1 = *reinterpret_cast<const float4*>((const float*)a.in + off + 4);
+        x[0] = v0.x; x[1] = v0.y; x[2] = v0.z; x[3] = v0.w; x[4] = v1.x; x[5] = v1.y; x[6] = v1.z; x[7] = v1.w;
     } else {
-        float d = rd(dt, mx_pos - mn_neg);  // :355
-        scale = rd(dt, __fdiv_rn(d, range));
-        if (a.preserve_zero) {  // :356-358
-            float q = rd(dt, __fdiv_rn(mn_neg, scale));
-            q = rd(dt, __builtin_rintf(q));
-            zp = rd(dt, (float)a.qmin - q);
-            float lo = rd(dt, (float)a.qmin), hi = rd(dt, (float)a.qmax);
-            zp = zp < lo ? lo : (zp > hi ? hi : zp);
-        } else {  // :360-362
-            float q = rd(dt, scale * mid);
-            zp = rd(dt, mn_neg + q);
+        const uint4 v = *reinterpret_cast<const uint4*>((const uint16_t*)a.in + off);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint16_t lo = (uint16_t)(w[j] & 0xffffu), hi = (uint16_t)(w[j] >> 16);
+            x[2 * j] = a.in_dtype == AO_BF16 ? bf16_bits_to_f32(lo) : f16_bits_to_f32(lo);
+            x[2 * j + 1] = a.in_dtype == AO_BF16 ? bf16_bits_to_f32(hi) : f16_bits_to_f32(hi);
         }
     }
-    if (!(scale >= epsv) && scale == scale) scale = epsv;  // clamp(min=eps) :365
-    store_f(a.scale, a.scale_dtype, blk, scale);
-    store_f(a.zp, a.zp_dtype, blk, zp);
+    float mn = INFINITY, mx = -INFINITY;
+    int has_nan = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        if (x[j] != x[j]) has_nan = 1;
+        mn = fminf(mn, x[j]);
+        mx = fmaxf(mx, x[j]);
+    }
+    for (uint32_t o = tpg >> 1; o >= 1; o >>= 1) {
+        mn = fminf(mn, __shfl_xor(mn, (int)o, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, (int)o, 64));
+        has_nan |= __shfl_xor(has_nan, (int)o, 64);
+    }
+    if (active && part == 0) finish_qparams(a, mn, mx, has_nan, blk);
 }
 
 // ---------------------------------------------------------------- quantize_affine / dequantize_affine (elementwise)
@@ -127,6 +174,32 @@ struct QuantArgs {
     int out_dtype;
 };
 
+// one element of quantize_affine (z is ignored when there is no zero point): quant_primitives.py:179-206
+__device__ __forceinline__ int64_t quantize_elem(const QuantArgs& a, float x, float s, float z) {
+    float q;
+    if (a.zp_domain == AO_ZP_INT) {  // :191-194
+        float inv = rd(a.scale_dtype, __fdiv_rn(1.0f, s));
+        int dt1 = promote(a.in_dtype, a.scale_dtype);
+        float t = rd(dt1, x * inv);
+        t = rd(dt1, __builtin_rintf(t));
+        if (a.zp) t = rd(promote(dt1, a.zp_dtype), t + z);
+        q = t;
+    } else {  // :195-203
+        const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
+        int dtm = promote(a.zp_dtype, a.scale_dtype);
+        float sm = rd(a.scale_dtype, s * mid);
+        float mv = rd(dtm, z - sm);
+        int dt1 = promote(a.in_dtype, dtm);
+        float t = rd(dt1, x - mv);
+        t = rd(promote(dt1, a.scale_dtype), __fdiv_rn(t, s));
+        q = __builtin_rintf(t);
+    }
+    if (q < (float)a.qmin) q = (float)a.qmin;
+    if (q > (float)a.qmax) q = (float)a.qmax;
+    if (q != q) q = 0.f;
+    return (int64_t)q;
+}
+
 // torchao/quantization/quant_primitives.py:134-206
 __global__ __launch_bounds__(256) void quantize_affine_kernel(QuantArgs a) {
     const int64_t total = a.N * a.K;
@@ -136,29 +209,8 @@ __global__ __launch_bounds__(256) void quantize_affine_kernel(QuantArgs a) {
         const int64_t g = (r / a.bN) * GK + c / a.bK;
         const float x = load_f(a.in, a.in_dtype, r * a.ld + c);
         const float s = load_f(a.scale, a.scale_dtype, g);
-        float q;
-        if (a.zp_domain == AO_ZP_INT) {  // :191-194
-            float inv = rd(a.scale_dtype, __fdiv_rn(1.0f, s));
-            int dt1 = promote(a.in_dtype, a.scale_dtype);
-            float t = rd(dt1, x * inv);
-            t = rd(dt1, __builtin_rintf(t));
-            if (a.zp) t = rd(promote(dt1, a.zp_dtype), t + load_f(a.zp, a.zp_dtype, g));
-            q = t;
-        } else {  // :195-203
-            const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
-            const float z = load_f(a.zp, a.zp_dtype, g);
-            int dtm = promote(a.zp_dtype, a.scale_dtype);
-            float sm = rd(a.scale_dtype, s * mid);
-            float mv = rd(dtm, z - sm);
-            int dt1 = promote(a.in_dtype, dtm);
-            float t = rd(dt1, x - mv);
-            t = rd(promote(dt1, a.scale_dtype), __fdiv_rn(t, s));
-            q = __builtin_rintf(t);
-        }
-        if (q < (float)a.qmin) q = (float)a.qmin;
-        if (q > (float)a.qmax) q = (float)a.qmax;
-        if (q != q) q = 0.f;
-        const int64_t qi = (int64_t)q;
+        const float z = a.zp ? load_f(a.zp, a.zp_dtype, g) : 0.f;
+        const int64_t qi = quantize_elem(a, x, s, z);
         switch (a.out_dtype) {
             case AO_I32: ((int32_t*)a.out)[i] = (int32_t)qi; break;
             case AO_I64: ((int64_t*)a.out)[i] = qi; break;
@@ -166,6 +218,75 @@ __global__ __launch_bounds__(256) void quantize_affine_kernel(QuantArgs a) {
             default: ((uint8_t*)a.out)[i] = (uint8_t)qi; break;
         }
     }
+}
+
+// Eight consecutive elements of one row per thread; they share a block when bK is a multiple of 8, so the index
+// arithmetic and the scale / zero point loads happen once per eight elements, the input arrives as one 16-byte
+// (fp32: two) load and the codes leave as 16-byte (int8: 8-byte) stores.
+__device__ __forceinline__ void load8_float(const void* p, int dtype, int64_t off, float* x) {
+    if (dtype == AO_F32) {
+        const float4 v0 = *reinterpret_cast<const float4*>((const float*)p + off);
+        const float4 v1 = *reinterpret_cast<const float4*>((const float*)p + off + 4);
+        x[0] = v0.x; x[1] = v0.y; x[2] = v0.z; x[3] = v0.w; x[4] = v1.x; x[5] = v1.y; x[6] = v1.z; x[7] = v1.w;
+    } else {
+        const uint4 v = *reinterpret_cast<const uint4*>((const uint16_t*)p + off);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint16_t lo = (uint16_t)(w[j] & 0xffffu), hi = (uint16_t)(w[j] >> 16);
+            x[2 * j] = dtype == AO_BF16 ? bf16_bits_to_f32(lo) : f16_bits_to_f32(lo);
+            x[2 * j + 1] = dtype == AO_BF16 ? bf16_bits_to_f32(hi) : f16_bits_to_f32(hi);
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a, uint32_t chunks, uint32_t K8) {
+    const uint32_t ci = blockIdx.x * 256u + threadIdx.x;
+    if (ci >= chunks) return;
+    const uint32_t r = ci / K8, c = (ci % K8) * 8u;
+    const int64_t g = (int64_t)(r / (uint32_t)a.bN) * (a.K / a.bK) + c / (uint32_t)a.bK;
+    float x[8];
+    load8_float(a.in, a.in_dtype, (int64_t)r * a.ld + c, x);
+    const float s = load_f(a.scale, a.scale_dtype, g);
+    const float z = a.zp ? load_f(a.zp, a.zp_dtype, g) : 0.f;
+    int64_t q[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) q[j] = quantize_elem(a, x[j], s, z);
+    const int64_t o = (int64_t)r * a.K + c;
+    if (a.out_dtype == AO_I32) {
+        int4* dst = reinterpret_cast<int4*>((int32_t*)a.out + o);
+        dst[0] = make_int4((int)q[0], (int)q[1], (int)q[2], (int)q[3]);
+        dst[1] = make_int4((int)q[4], (int)q[5], (int)q[6], (int)q[7]);
+    } else if (a.out_dtype == AO_I64) {
+        longlong2* dst = reinterpret_cast<longlong2*>((int64_t*)a.out + o);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[j] = make_longlong2(q[2 * j], q[2 * j + 1]);
+    } else {  // int8 and uint8 codes have the same low byte
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            lo |= ((uint32_t)q[j] & 0xffu) << (8 * j);
+            hi |= ((uint32_t)q[4 + j] & 0xffu) << (8 * j);
+        }
+        *reinterpret_cast<uint2*>((uint8_t*)a.out + o) = make_uint2(lo, hi);
+    }
+}
+
+// one element of dequantize_affine: quant_primitives.py:257-274
+__device__ __forceinline__ float dequantize_elem(const QuantArgs& a, int64_t q, float s, int64_t zi, float zf) {
+    float v;
+    if (a.zp_domain == AO_ZP_INT) {  // :257-264
+        int32_t d = (int32_t)q;
+        if (a.zp) d -= (int32_t)zi;
+        v = rd(a.out_dtype, (float)d);
+        v = rd(a.out_dtype, v * s);
+    } else {  // :265-274
+        const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
+        v = rd(a.out_dtype, (float)q - mid);
+        v = rd(a.out_dtype, v * s);
+        if (a.zp) v = rd(a.out_dtype, v + zf);
+    }
+    return v;
 }
 
 // torchao/quantization/quant_primitives.py:208-276
@@ -177,19 +298,57 @@ __global__ __launch_bounds__(256) void dequantize_affine_kernel(QuantArgs a) {
         const int64_t g = (r / a.bN) * GK + c / a.bK;
         const int64_t q = load_i(a.in, a.in_dtype, i);
         const float s = load_f(a.scale, a.scale_dtype, g);
-        float v;
-        if (a.zp_domain == AO_ZP_INT) {  // :257-264
-            int32_t d = (int32_t)q;
-            if (a.zp) d -= (int32_t)load_i(a.zp, a.zp_dtype, g);
-            v = rd(a.out_dtype, (float)d);
-            v = rd(a.out_dtype, v * s);
-        } else {  // :265-274
-            const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
-            v = rd(a.out_dtype, (float)q - mid);
-            v = rd(a.out_dtype, v * s);
-            if (a.zp) v = rd(a.out_dtype, v + load_f(a.zp, a.zp_dtype, g));
+        const int64_t zi = a.zp && a.zp_domain == AO_ZP_INT ? load_i(a.zp, a.zp_dtype, g) : 0;
+        const float zf = a.zp && a.zp_domain != AO_ZP_INT ? load_f(a.zp, a.zp_dtype, g) : 0.f;
+        store_f(a.out, a.out_dtype, i, dequantize_elem(a, q, s, zi, zf));
+    }
+}
+
+// Eight consecutive codes of one row per thread, as in quantize_affine_vec8_kernel.
+__global__ __launch_bounds__(256) void dequantize_affine_vec8_kernel(QuantArgs a, uint32_t chunks, uint32_t K8) {
+    const uint32_t ci = blockIdx.x * 256u + threadIdx.x;
+    if (ci >= chunks) return;
+    const uint32_t r = ci / K8, c = (ci % K8) * 8u;
+    const int64_t g = (int64_t)(r / (uint32_t)a.bN) * (a.K / a.bK) + c / (uint32_t)a.bK;
+    const int64_t o = (int64_t)r * a.K + c;
+    int64_t q[8];
+    if (a.in_dtype == AO_I32) {
+        const int4 v0 = *reinterpret_cast<const int4*>((const int32_t*)a.in + o);
+        const int4 v1 = *reinterpret_cast<const int4*>((const int32_t*)a.in + o + 4);
+        q[0] = v0.x; q[1] = v0.y; q[2] = v0.z; q[3] = v0.w; q[4] = v1.x; q[5] = v1.y; q[6] = v1.z; q[7] = v1.w;
+    } else if (a.in_dtype == AO_I64) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const longlong2 v = *reinterpret_cast<const longlong2*>((const int64_t*)a.in + o + 2 * j);
+            q[2 * j] = v.x; q[2 * j + 1] = v.y;
         }
-        store_f(a.out, a.out_dtype, i, v);
+    } else {
+        const uint2 v = *reinterpret_cast<const uint2*>((const uint8_t*)a.in + o);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t b = ((j < 4 ? v.x : v.y) >> (8 * (j & 3))) & 0xffu;
+            q[j] = a.in_dtype == AO_I8 ? (int64_t)(int8_t)b : (int64_t)b;
+        }
+    }
+    const float s = load_f(a.scale, a.scale_dtype, g);
+    const int64_t zi = a.zp && a.zp_domain == AO_ZP_INT ? load_i(a.zp, a.zp_dtype, g) : 0;
+    const float zf = a.zp && a.zp_domain != AO_ZP_INT ? load_f(a.zp, a.zp_dtype, g) : 0.f;
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = dequantize_elem(a, q[j], s, zi, zf);
+    if (a.out_dtype == AO_F32) {
+        float4* dst = reinterpret_cast<float4*>((float*)a.out + o);
+        dst[0] = make_float4(v[0], v[1], v[2], v[3]);
+        dst[1] = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = a.out_dtype == AO_BF16 ? f32_to_bf16_bits(v[2 * j]) : f32_to_f16_bits(v[2 * j]);
+            const uint32_t hi = a.out_dtype == AO_BF16 ? f32_to_bf16_bits(v[2 * j + 1]) : f32_to_f16_bits(v[2 * j + 1]);
+            w[j] = (lo & 0xffffu) | (hi << 16);
+        }
+        *reinterpret_cast<uint4*>((uint16_t*)a.out + o) = make_uint4(w[0], w[1], w[2], w[3]);
     }
 }
 
@@ -506,13 +665,27 @@ extern "C" int ao_amd_choose_qparams_affine(const void* in, int in_dtype, int64_
                  scale_dtype, zp_dtype, scale, zero_point};
     const int64_t nblocks = (N / bN) * (K / bK);
     hipStream_t st = (hipStream_t)stream;
-    if (bN * bK <= 2048) {
+    const int64_t tpg = bK / 8;
+    const bool vec8 = bN == 1 && bK % 8 == 0 && tpg <= 64 && (tpg & (tpg - 1)) == 0 && ld % 8 == 0 &&
+                      (uintptr_t)in % 16 == 0 && N * (K / 8) < (int64_t)0xffffff00u;
+    if (vec8) {
+        const uint32_t chunks = (uint32_t)(N * (K / 8));
+        hipLaunchKernelGGL(choose_qparams_vec8_kernel, dim3((chunks + 255u) / 256u), dim3(256), 0, st, a, chunks,
+                           (uint32_t)tpg, (uint32_t)(K / bK));
+    } else if (bN * bK <= 2048) {
         hipLaunchKernelGGL(choose_qparams_kernel<64>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, a);
     } else {
         hipLaunchKernelGGL(choose_qparams_kernel<256>, dim3((unsigned)nblocks), dim3(256), 0, st, a);
     }
     AO_LAUNCH_CHECK();
     return 0;
+}
+
+// quantize_affine / dequantize_affine take eight elements per thread when a run of eight never crosses a block or a
+// row and every vector access is 16-byte aligned
+static bool elementwise_vec8(int64_t N, int64_t K, int64_t ld, int64_t bN, int64_t bK, const void* in, const void* out) {
+    return K % 8 == 0 && bK % 8 == 0 && ld % 8 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+           bN < ((int64_t)1 << 31) && N * (K / 8) < (int64_t)0xffffff00u;
 }
 
 static unsigned elementwise_grid(int64_t total) {
@@ -534,7 +707,13 @@ extern "C" int ao_amd_quantize_affine(const void* in, int in_dtype, int64_t N, i
     if (int rc = check_block(N, K, bN, bK)) return rc;
     AO_REQUIRE(ld >= K, "row stride %lld smaller than K=%lld", (long long)ld, (long long)K);
     QuantArgs a{in, in_dtype, N, K, ld, bN, bK, scale, scale_dtype, zero_point, zp_dtype, qmin, qmax, zp_domain, out, out_dtype};
-    hipLaunchKernelGGL(quantize_affine_kernel, dim3(elementwise_grid(N * K)), dim3(256), 0, (hipStream_t)stream, a);
+    if (elementwise_vec8(N, K, ld, bN, bK, in, out)) {
+        const uint32_t chunks = (uint32_t)(N * (K / 8));
+        hipLaunchKernelGGL(quantize_affine_vec8_kernel, dim3((chunks + 255u) / 256u), dim3(256), 0, (hipStream_t)stream, a,
+                           chunks, (uint32_t)(K / 8));
+    } else {
+        hipLaunchKernelGGL(quantize_affine_kernel, dim3(elementwise_grid(N * K)), dim3(256), 0, (hipStream_t)stream, a);
+    }
     AO_LAUNCH_CHECK();
     return 0;
 }
@@ -549,7 +728,13 @@ extern "C" int ao_amd_dequantize_affine(const void* in, int in_dtype, int64_t N,
     AO_REQUIRE(zp_domain == AO_ZP_INT || zp_domain == AO_ZP_FLOAT, "Unexpected zero point domain: %d", zp_domain);
     if (int rc = check_block(N, K, bN, bK)) return rc;
     QuantArgs a{in, in_dtype, N, K, K, bN, bK, scale, scale_dtype, zero_point, zp_dtype, qmin, qmax, zp_domain, out, out_dtype};
-    hipLaunchKernelGGL(dequantize_affine_kernel, dim3(elementwise_grid(N * K)), dim3(256), 0, (hipStream_t)stream, a);
+    if (elementwise_vec8(N, K, K, bN, bK, in, out)) {
+        const uint32_t chunks = (uint32_t)(N * (K / 8));
+        hipLaunchKernelGGL(dequantize_affine_vec8_kernel, dim3((chunks + 255u) / 256u), dim3(256), 0, (hipStream_t)stream,
+                           a, chunks, (uint32_t)(K / 8));
+    } else {
+        hipLaunchKernelGGL(dequantize_affine_kernel, dim3(elementwise_grid(N * K)), dim3(256), 0, (hipStream_t)stream, a);
+    }
     AO_LAUNCH_CHECK();
     return 0;
 }

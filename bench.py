@@ -446,6 +446,41 @@ def sweep(kind, iters=100):
                                   "rel_l2_between_outputs": float(f"{float((y_t - y_m).norm() / y_m.norm()):.3e}")}),
                       flush=True)
             del w, codes, theirs_c, sz_c, mine_c, mine_qc
+    elif kind == "quantize":
+        # the one-time quantize side at its reference call (quant_api.py:376-385: asymmetric, (1, g) blocks, int32 codes
+        # in 0..15, bf16 scale and zero point in the float domain): the three primitives and the fused quantize + pack
+        for N, K, g in [(4096, 4096, 128), (4096, 4096, 64), (14336, 4096, 64), (4096, 14336, 64)]:
+            copies = max(2, -(-SWEEP_ROTATE_BYTES // (N * K * 2)))
+            w = (torch.randn(copies, N, K, device=dev, generator=gen) * 0.02).bfloat16()
+            scale = torch.empty(N, K // g, dtype=torch.bfloat16, device=dev)
+            zero = torch.empty_like(scale)
+            codes = torch.empty(copies, N, K, dtype=torch.int32, device=dev)
+            deq = torch.empty(N, K, dtype=torch.bfloat16, device=dev)
+            _, _, pb, qb = _lib.packed_shape(N, K, g)
+            packed = torch.empty(pb // 4, dtype=torch.int32, device=dev)
+            qp = torch.empty(qb // 4, dtype=torch.int32, device=dev)
+            BF16, I32, ASYM, ZP_FLOAT = 1, 3, 1, 1
+            qparam_bytes = 4 * N * K // g
+            steps = [
+                ("choose_qparams_affine", N * K * 2 + qparam_bytes, lambda i: _lib.check(L.ao_amd_choose_qparams_affine(
+                    w[i % copies].data_ptr(), BF16, N, K, K, 1, g, ASYM, 0, 15, 1e-6, 0, ZP_FLOAT, BF16, BF16,
+                    scale.data_ptr(), zero.data_ptr(), st))),
+                ("quantize_affine", N * K * 6 + qparam_bytes, lambda i: _lib.check(L.ao_amd_quantize_affine(
+                    w[i % copies].data_ptr(), BF16, N, K, K, 1, g, scale.data_ptr(), BF16, zero.data_ptr(), BF16, 0, 15,
+                    ZP_FLOAT, codes[i % copies].data_ptr(), I32, st))),
+                ("dequantize_affine", N * K * 6 + qparam_bytes, lambda i: _lib.check(L.ao_amd_dequantize_affine(
+                    codes[i % copies].data_ptr(), I32, N, K, 1, g, scale.data_ptr(), BF16, zero.data_ptr(), BF16, 0, 15,
+                    ZP_FLOAT, deq.data_ptr(), BF16, st))),
+                ("int4wo_quantize_pack", N * K * 2 + N * K // 2 + qparam_bytes, lambda i: _lib.check(
+                    L.ao_amd_int4wo_quantize_pack(w[i % copies].data_ptr(), N, K, K, g, packed.data_ptr(), qp.data_ptr(),
+                                                  st))),
+            ]
+            for name, nbytes, launch in steps:
+                us = _time_linear(L, launch, iters, armed=False)
+                print(json.dumps({"kernel": name, "N": N, "K": K, "group": g, "us": round(us, 2),
+                                  "GBs": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / 8000.0, 4)}),
+                      flush=True)
+            del w, codes
     else:
         sys.exit(f"unknown sweep {kind}")
 
@@ -467,7 +502,7 @@ def main():
                     help="int4wo-<group> (default: int4wo-<--group>, the headline configuration), int8wo or fp6 (e3m2 on an "
                          "fp16 model): the decode loop of the reference's other weight-only configurations, reported "
                          "without the int4 roofline leg")
-    ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6", "int8", "tinygemm"), default=None,
+    ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6", "int8", "tinygemm", "quantize"), default=None,
                     help="instead of the decode benchmark, print one line per kernel case of the named sweep")
     args = ap.parse_args()
     if args.gpus != 1:
