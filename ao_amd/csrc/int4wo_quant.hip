@@ -175,29 +175,35 @@ struct QuantArgs {
 };
 
 // one element of quantize_affine (z is ignored when there is no zero point): quant_primitives.py:179-206
+// Intermediate roundings use the hardware bf16 converter: it differs from the software rounding only in the payload of a
+// NaN, and a NaN code becomes 0 below.  SMALL: the clamp range lies within +-2^24, so the 32-bit float -> int conversion
+// gives the same code as the 64-bit sequence.
+__device__ __forceinline__ float rd_nan_free(int dtype, float v) { return dtype == AO_BF16 ? hw_rne_bf16(v) : rd(dtype, v); }
+
+template <bool SMALL>
 __device__ __forceinline__ int64_t quantize_elem(const QuantArgs& a, float x, float s, float z) {
     float q;
     if (a.zp_domain == AO_ZP_INT) {  // :191-194
-        float inv = rd(a.scale_dtype, __fdiv_rn(1.0f, s));
+        float inv = rd_nan_free(a.scale_dtype, __fdiv_rn(1.0f, s));
         int dt1 = promote(a.in_dtype, a.scale_dtype);
-        float t = rd(dt1, x * inv);
-        t = rd(dt1, __builtin_rintf(t));
-        if (a.zp) t = rd(promote(dt1, a.zp_dtype), t + z);
+        float t = rd_nan_free(dt1, x * inv);
+        t = rd_nan_free(dt1, __builtin_rintf(t));
+        if (a.zp) t = rd_nan_free(promote(dt1, a.zp_dtype), t + z);
         q = t;
     } else {  // :195-203
         const float mid = (float)((double)(a.qmax + a.qmin + 1) / 2.0);
         int dtm = promote(a.zp_dtype, a.scale_dtype);
-        float sm = rd(a.scale_dtype, s * mid);
-        float mv = rd(dtm, z - sm);
+        float sm = rd_nan_free(a.scale_dtype, s * mid);
+        float mv = rd_nan_free(dtm, z - sm);
         int dt1 = promote(a.in_dtype, dtm);
-        float t = rd(dt1, x - mv);
-        t = rd(promote(dt1, a.scale_dtype), __fdiv_rn(t, s));
+        float t = rd_nan_free(dt1, x - mv);
+        t = rd_nan_free(promote(dt1, a.scale_dtype), __fdiv_rn(t, s));
         q = __builtin_rintf(t);
     }
     if (q < (float)a.qmin) q = (float)a.qmin;
     if (q > (float)a.qmax) q = (float)a.qmax;
     if (q != q) q = 0.f;
-    return (int64_t)q;
+    return SMALL ? (int64_t)(int32_t)q : (int64_t)q;
 }
 
 // torchao/quantization/quant_primitives.py:134-206
@@ -210,7 +216,7 @@ __global__ __launch_bounds__(256) void quantize_affine_kernel(QuantArgs a) {
         const float x = load_f(a.in, a.in_dtype, r * a.ld + c);
         const float s = load_f(a.scale, a.scale_dtype, g);
         const float z = a.zp ? load_f(a.zp, a.zp_dtype, g) : 0.f;
-        const int64_t qi = quantize_elem(a, x, s, z);
+        const int64_t qi = quantize_elem<false>(a, x, s, z);
         switch (a.out_dtype) {
             case AO_I32: ((int32_t*)a.out)[i] = (int32_t)qi; break;
             case AO_I64: ((int64_t*)a.out)[i] = qi; break;
@@ -250,8 +256,13 @@ __global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a, 
     const float s = load_f(a.scale, a.scale_dtype, g);
     const float z = a.zp ? load_f(a.zp, a.zp_dtype, g) : 0.f;
     int64_t q[8];
+    if (a.qmin >= -(1 << 24) && a.qmax <= (1 << 24)) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) q[j] = quantize_elem(a, x[j], s, z);
+        for (int j = 0; j < 8; ++j) q[j] = quantize_elem<true>(a, x[j], s, z);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) q[j] = quantize_elem<false>(a, x[j], s, z);
+    }
     const int64_t o = (int64_t)r * a.K + c;
     if (a.out_dtype == AO_I32) {
         int4* dst = reinterpret_cast<int4*>((int32_t*)a.out + o);
@@ -273,7 +284,8 @@ __global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a, 
 }
 
 // one element of dequantize_affine: quant_primitives.py:257-274
-__device__ __forceinline__ float dequantize_elem(const QuantArgs& a, int64_t q, float s, int64_t zi, float zf) {
+template <typename QInt>  // int64_t, or int32_t for codes that were stored in 32 bits or fewer (cheaper int -> float)
+__device__ __forceinline__ float dequantize_elem(const QuantArgs& a, QInt q, float s, int64_t zi, float zf) {
     float v;
     if (a.zp_domain == AO_ZP_INT) {  // :257-264
         int32_t d = (int32_t)q;
@@ -300,7 +312,7 @@ __global__ __launch_bounds__(256) void dequantize_affine_kernel(QuantArgs a) {
         const float s = load_f(a.scale, a.scale_dtype, g);
         const int64_t zi = a.zp && a.zp_domain == AO_ZP_INT ? load_i(a.zp, a.zp_dtype, g) : 0;
         const float zf = a.zp && a.zp_domain != AO_ZP_INT ? load_f(a.zp, a.zp_dtype, g) : 0.f;
-        store_f(a.out, a.out_dtype, i, dequantize_elem(a, q, s, zi, zf));
+        store_f(a.out, a.out_dtype, i, dequantize_elem<int64_t>(a, q, s, zi, zf));
     }
 }
 
@@ -335,7 +347,9 @@ __global__ __launch_bounds__(256) void dequantize_affine_vec8_kernel(QuantArgs a
     const float zf = a.zp && a.zp_domain != AO_ZP_INT ? load_f(a.zp, a.zp_dtype, g) : 0.f;
     float v[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = dequantize_elem(a, q[j], s, zi, zf);
+    for (int j = 0; j < 8; ++j)
+        v[j] = a.in_dtype == AO_I64 ? dequantize_elem<int64_t>(a, q[j], s, zi, zf)
+                                    : dequantize_elem<int32_t>(a, (int32_t)q[j], s, zi, zf);
     if (a.out_dtype == AO_F32) {
         float4* dst = reinterpret_cast<float4*>((float*)a.out + o);
         dst[0] = make_float4(v[0], v[1], v[2], v[3]);
