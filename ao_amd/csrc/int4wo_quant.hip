@@ -118,39 +118,50 @@ __global__ __launch_bounds__(256) void choose_qparams_kernel(QParamArgs a) {
     finish_qparams(a, mn, mx, has_nan, blk);
 }
 
-// Row groups (bN == 1) whose length is 8 * TPG, TPG a power of two up to 64: a thread reads eight consecutive
-// elements with one 16-byte (32-byte for fp32) load, TPG neighbouring lanes reduce with shuffles, the first of them
-// finishes the group.  Index arithmetic once per eight elements.
-__global__ __launch_bounds__(256) void choose_qparams_vec8_kernel(QParamArgs a, uint32_t chunks, uint32_t tpg, uint32_t GK) {
-    const uint32_t ci = blockIdx.x * 256u + threadIdx.x;
-    const bool active = ci < chunks;
-    const uint32_t cc = active ? ci : chunks - 1;
-    const uint32_t blk = cc / tpg, part = cc % tpg;
-    const uint32_t r = blk / GK, gk = blk % GK;
-    const int64_t off = (int64_t)r * a.ld + (int64_t)gk * a.bK + part * 8;
-    float x[8];
-    if (a.in_dtype == AO_F32) {
-        const float4 v0 = *reinterpret_cast<const float4*>((const float*)a.in + off);
-        const float4 v1 = *reinterpret_cast<const float4*>((const float*)a.in + off + 4);
+// eight consecutive elements of a floating dtype as fp32: one 16-byte load (two for fp32)
+__device__ __forceinline__ void load8_float(const void* p, int dtype, int64_t off, float* x) {
+    if (dtype == AO_F32) {
+        const float4 v0 = *reinterpret_cast<const float4*>((const float*)p + off);
+        const float4 v1 = *reinterpret_cast<const float4*>((const float*)p + off + 4);
         x[0] = v0.x; x[1] = v0.y; x[2] = v0.z; x[3] = v0.w; x[4] = v1.x; x[5] = v1.y; x[6] = v1.z; x[7] = v1.w;
     } else {
-        const uint4 v = *reinterpret_cast<const uint4*>((const uint16_t*)a.in + off);
+        const uint4 v = *reinterpret_cast<const uint4*>((const uint16_t*)p + off);
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const uint16_t lo = (uint16_t)(w[j] & 0xffffu), hi = (uint16_t)(w[j] >> 16);
-            x[2 * j] = a.in_dtype == AO_BF16 ? bf16_bits_to_f32(lo) : f16_bits_to_f32(lo);
-            x[2 * j + 1] = a.in_dtype == AO_BF16 ? bf16_bits_to_f32(hi) : f16_bits_to_f32(hi);
+            x[2 * j] = dtype == AO_BF16 ? bf16_bits_to_f32(lo) : f16_bits_to_f32(lo);
+            x[2 * j + 1] = dtype == AO_BF16 ? bf16_bits_to_f32(hi) : f16_bits_to_f32(hi);
         }
     }
+}
+
+// Row groups (bN == 1) whose length is 8 * CH * TPG, TPG a power of two up to 64: a thread reads CH runs of eight
+// consecutive elements (CH = 4: 32 elements, 64 contiguous bytes of a 16-bit dtype) with 16-byte loads, TPG neighbouring
+// lanes reduce with shuffles and the first of them finishes the group.  The finish (divisions, roundings) runs once per
+// wave whatever the number of lanes that need it, so the more elements a lane covers the less it weighs: 32 per lane
+// whenever the group length allows.
+template <int CH>
+__global__ __launch_bounds__(256) void choose_qparams_vec8_kernel(QParamArgs a, uint32_t units, uint32_t tpg, uint32_t GK) {
+    const uint32_t ui = blockIdx.x * 256u + threadIdx.x;
+    const bool active = ui < units;
+    const uint32_t uu = active ? ui : units - 1;
+    const uint32_t blk = uu / tpg, part = uu % tpg;
+    const uint32_t r = blk / GK, gk = blk % GK;
+    const int64_t off = (int64_t)r * a.ld + (int64_t)gk * a.bK + part * (8 * CH);
+    float x[CH][8];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) load8_float(a.in, a.in_dtype, off + 8 * c, x[c]);
     float mn = INFINITY, mx = -INFINITY;
     int has_nan = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        if (x[j] != x[j]) has_nan = 1;
-        mn = fminf(mn, x[j]);
-        mx = fmaxf(mx, x[j]);
-    }
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (x[c][j] != x[c][j]) has_nan = 1;
+            mn = fminf(mn, x[c][j]);
+            mx = fmaxf(mx, x[c][j]);
+        }
     for (uint32_t o = tpg >> 1; o >= 1; o >>= 1) {
         mn = fminf(mn, __shfl_xor(mn, (int)o, 64));
         mx = fmaxf(mx, __shfl_xor(mx, (int)o, 64));
@@ -229,22 +240,6 @@ __global__ __launch_bounds__(256) void quantize_affine_kernel(QuantArgs a) {
 // Eight consecutive elements of one row per thread; they share a block when bK is a multiple of 8, so the index
 // arithmetic and the scale / zero point loads happen once per eight elements, the input arrives as one 16-byte
 // (fp32: two) load and the codes leave as 16-byte (int8: 8-byte) stores.
-__device__ __forceinline__ void load8_float(const void* p, int dtype, int64_t off, float* x) {
-    if (dtype == AO_F32) {
-        const float4 v0 = *reinterpret_cast<const float4*>((const float*)p + off);
-        const float4 v1 = *reinterpret_cast<const float4*>((const float*)p + off + 4);
-        x[0] = v0.x; x[1] = v0.y; x[2] = v0.z; x[3] = v0.w; x[4] = v1.x; x[5] = v1.y; x[6] = v1.z; x[7] = v1.w;
-    } else {
-        const uint4 v = *reinterpret_cast<const uint4*>((const uint16_t*)p + off);
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint16_t lo = (uint16_t)(w[j] & 0xffffu), hi = (uint16_t)(w[j] >> 16);
-            x[2 * j] = dtype == AO_BF16 ? bf16_bits_to_f32(lo) : f16_bits_to_f32(lo);
-            x[2 * j + 1] = dtype == AO_BF16 ? bf16_bits_to_f32(hi) : f16_bits_to_f32(hi);
-        }
-    }
-}
 
 __global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a, uint32_t chunks, uint32_t K8) {
     const uint32_t ci = blockIdx.x * 256u + threadIdx.x;
@@ -679,13 +674,19 @@ extern "C" int ao_amd_choose_qparams_affine(const void* in, int in_dtype, int64_
                  scale_dtype, zp_dtype, scale, zero_point};
     const int64_t nblocks = (N / bN) * (K / bK);
     hipStream_t st = (hipStream_t)stream;
-    const int64_t tpg = bK / 8;
+    const int ch = bK % 32 == 0 ? 4 : 1;  // runs of eight elements per thread
+    const int64_t tpg = bK / (8 * ch);
     const bool vec8 = bN == 1 && bK % 8 == 0 && tpg <= 64 && (tpg & (tpg - 1)) == 0 && ld % 8 == 0 &&
                       (uintptr_t)in % 16 == 0 && N * (K / 8) < (int64_t)0xffffff00u;
     if (vec8) {
-        const uint32_t chunks = (uint32_t)(N * (K / 8));
-        hipLaunchKernelGGL(choose_qparams_vec8_kernel, dim3((chunks + 255u) / 256u), dim3(256), 0, st, a, chunks,
-                           (uint32_t)tpg, (uint32_t)(K / bK));
+        const uint32_t units = (uint32_t)(N * (K / (8 * ch)));
+        if (ch == 4) {
+            hipLaunchKernelGGL(choose_qparams_vec8_kernel<4>, dim3((units + 255u) / 256u), dim3(256), 0, st, a, units,
+                               (uint32_t)tpg, (uint32_t)(K / bK));
+        } else {
+            hipLaunchKernelGGL(choose_qparams_vec8_kernel<1>, dim3((units + 255u) / 256u), dim3(256), 0, st, a, units,
+                               (uint32_t)tpg, (uint32_t)(K / bK));
+        }
     } else if (bN * bK <= 2048) {
         hipLaunchKernelGGL(choose_qparams_kernel<64>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, a);
     } else {
