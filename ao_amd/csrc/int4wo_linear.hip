@@ -15,6 +15,7 @@
 //   u  = T.lo*1 + T.hi*0 + z  /  T.lo*0 + T.hi*1 + z   fp32 add of the bf16 operands  (2 v_dot2_f32_bf16)
 //   W  = cvt_pk_bf16(u0, u1)                           second rounding                (1 v_cvt_pk_bf16_f32)
 #include "common.h"
+#include "int4wo_linear.h"
 
 namespace ao {
 
@@ -92,7 +93,6 @@ __device__ __forceinline__ bf16x8_t dequant8(uint32_t w, const GroupConst& g, ui
     return out.v;
 }
 
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 // The dequantization of a dword (8 codes) runs as a three-stage software pipeline so that the VALU and the
 // matrix core overlap; each stage is one asm volatile block (volatile blocks keep their program order, which
@@ -181,32 +181,6 @@ __device__ __forceinline__ uint4 load_x8_checked(const uint16_t* __restrict__ x,
     return r.q;
 }
 
-struct LinearArgs {
-    const uint16_t* x; int64_t M, K, ldx;
-    const uint4* packed; const uint32_t* qparams;
-    const uint4* packed2; const uint32_t* qparams2;   // DUAL only
-    int64_t N, Kp;
-    const uint16_t* bias;                              // [N] or null
-    const uint16_t* residual; int64_t ldres;           // [M,N] or null
-    void* y; int y_is_f32; int64_t ldy;
-    const uint16_t* norm_w; float norm_eps;            // GEMV only: RMSNorm weight [K] applied to x while staging, or null
-    int ksplit;                                        // GEMV only: blockIdx.z takes the z-th of `ksplit` contiguous runs of K tiles and
-                                                       // stores its fp32 partial sums at y + z * M * ldy (the consumer adds them)
-    int pair8;                                         // GEMV only: rows 0-7 of every 16-row block are gate rows, rows 8-15
-                                                       // the matching up rows; y[m, 8*rb + r] = silu(gate) * up, N = output rows
-    // GEMV only, derived on the host so that the 16 waves a CU starts at once do not each spend scalar issue slots on
-    // 64-bit divisions and shifts before their first load: K tiles, K tiles per blockIdx.z, bytes of one row block's
-    // packed codes and qparams, 16-byte chunks per activation row
-    int kb_total, kb_per_split;
-    uint32_t block_bytes, qblock_bytes;
-    int chunks_per_row;
-};
-
-__device__ __forceinline__ float silu_bf16(float a) {
-    // F.silu on a bf16 tensor: computed in fp32, result rounded to bf16
-    return hw_rne_bf16(a / (1.0f + expf(-a)));
-}
-
 // How a wave gets its activation fragments (MFMA A operand: row m = lane%16, 8 consecutive k):
 constexpr int X_GLOBAL = 0;   // 16-byte global loads, prefetched with the weight tile (K % 128 == 0, aligned rows)
 constexpr int X_CHECKED = 1;  // element-wise global loads with bounds checks (any K, any alignment)
@@ -225,22 +199,6 @@ struct TileBuf {
 // The compiler cannot keep a precise count across the conditional loads of the register ring and falls back to
 // vmcnt(0), i.e. it would drain every prefetch before each tile.  The wait block takes the loaded registers as
 // in/out operands, so no consumer of them can be scheduled above the wait.
-// scalar base (SGPR pair) + 32-bit per-lane byte offset: the per-tile address update is one scalar add
-__device__ __forceinline__ u32x4_t asm_load_b128_nt(const void* sbase, uint32_t voff) {
-    u32x4_t v;
-    asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
-    return v;
-}
-__device__ __forceinline__ u32x4_t asm_load_b128(const void* sbase, uint32_t voff) {
-    u32x4_t v;
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
-    return v;
-}
-__device__ __forceinline__ uint32_t asm_load_b32(const void* sbase, uint32_t voff) {
-    uint32_t v;
-    asm volatile("global_load_dword %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
-    return v;
-}
 // Wait until at most `younger_tiles` tiles' worth of loads are outstanding (loads return in order, so the
 // tile requested before them has arrived).  The block has no register operands: every consumer of loaded
 // registers is itself an asm volatile block (make_group_asm, first_half), and volatile blocks stay in order.
@@ -1167,6 +1125,11 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
             default: AO_GEMM_LAUNCH(256); break;
         }
 #undef AO_GEMM_LAUNCH
+        AO_LAUNCH_CHECK();
+        return 0;
+    }
+    // one activation row: the kernel built on the 4x4x4 matrix instructions (group size 64 and up, K up to 16384)
+    if (M == 1 && aligned && !dual && launch_int4wo_gemv1(a, g, RB, st)) {
         AO_LAUNCH_CHECK();
         return 0;
     }

@@ -64,3 +64,97 @@ def test_prefetched_registers_are_untouched_until_the_first_wait(tmp_path, sourc
         assert not touched, (name, touched[:4])
         scratch = re.search(r"\.amdhsa_private_segment_fixed_size (\d+)", meta)
         assert scratch is None or int(scratch.group(1)) == 0, (name, scratch.group(0))
+
+
+def test_gemv1_ring_registers_are_untouched_between_their_request_and_the_loop(tmp_path):
+    """int4wo_gemv1_kernel requests seven weight tiles into fixed registers, stages its activations with compiler
+    generated code, then enters the hand-scheduled loop with the requests possibly still in flight.  Checked on the
+    generated ISA of every instantiation:
+      * nothing between the first request and the loop's first instruction names a ring register, and the loop
+        receives the tiles where the requests put them;
+      * the activation registers are not read between their loads and the one explicit wait that covers them;
+      * a wave that skips the loop waits for its requests before any other instruction of that path names a ring register;
+      * every operand the compiler hands the loop lives below the loop's own register range (the loop overwrites
+        its own registers, the accumulator output included, while it still reads its operands);
+      * no scratch memory."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not available")
+    asm = tmp_path / "gemv1.s"
+    subprocess.run([hipcc, *_FLAGS, "-o", str(asm), os.path.join(_ROOT, "ao_amd", "csrc", "int4wo_gemv1.hip")], check=True,
+                   capture_output=True, timeout=600)
+    text = asm.read_text()
+    inc = open(os.path.join(_ROOT, "ao_amd", "csrc", "int4wo_gemv1_loop.inc")).read()
+    depth = int(re.search(r"#define GEMV1_RING_DEPTH (\d+)", inc).group(1))
+    vbase = int(re.search(r"#define GEMV1_VBASE (\d+)", inc).group(1))
+    template = [t.replace("\\n", "").replace("\\t", "").strip()
+                for t in re.findall(r'"((?:[^"\\]|\\.)*)"', inc.split("#define GEMV1_LOOP_ASM", 1)[1])]
+    template = [t for t in template if t]
+    ring = set()
+    for j in range(depth - 1):
+        w = re.search(r'#define GEMV1_W%d "\{v\[(\d+):(\d+)\]\}"' % j, inc)
+        ring.update(range(int(w.group(1)), int(w.group(2)) + 1))
+    kernels = list(re.finditer(r"^(_ZN2ao19int4wo_gemv1_kernelILi\d+ELi\d+ELb[01]EEE\w*): ; @.*?\n(.*?)s_endpgm(.*?)\.end_amdhsa_kernel", text, re.S | re.M))
+    assert len(kernels) == 15
+    for m in kernels:
+        name, body, meta = m.group(1), m.group(2), m.group(3)
+        tp = re.match(r"_ZN2ao19int4wo_gemv1_kernelILi(\d+)ELi(\d+)ELb([01])E", name)
+        xl, norm = int(tp.group(2)), tp.group(3) == "1"
+        lines = [l for l in body.splitlines() if l.strip() and not re.match(r"\s*;(?!;#ASM)", l) and not l.strip().startswith(".") or re.match(r"\.LBB", l.strip())]
+        code = lambda l: l.strip() and not l.strip().startswith((";", "."))
+        first = next(i for i, l in enumerate(lines) if re.search(r"global_load_dwordx4 v\[\d+:\d+\], v\d+, s\[.* nt", l))
+        loop = next(i for i, l in enumerate(lines) if l.strip() == template[0])
+        assert first < loop, name
+        requests = [l for l in lines[first:loop] if "global_load_dword" in l]
+        assert len(requests) == depth - 1, (name, len(requests))
+        got = set()
+        for l in requests:
+            got |= _regs(l.split(",")[0])
+        assert got == ring, (name, sorted(got ^ ring))
+        for i in range(first, loop):
+            if "global_load_dword" not in lines[i]:
+                continue
+            dest = _regs(lines[i].split(",")[0])
+            others = [l.strip() for l in lines[i + 1:loop] if code(l) and _regs(l) & dest]
+            assert not others, (name, lines[i].strip(), others[:4])
+        # activation loads: plain 16-byte loads before the first request, waited for by one vmcnt wait
+        xloads = [i for i, l in enumerate(lines[:first]) if re.search(r"global_load_dwordx4 v\[\d+:\d+\], v\d+, s\[\d+:\d+\]$", l.strip())]
+        assert len(xloads) == xl // 2 + (2 * xl + 2 if norm else xl), (name, len(xloads))
+        wait = next(i for i, l in enumerate(lines) if "s_waitcnt vmcnt(%d)" % (depth - 1) in l)
+        assert xloads[-1] < wait < loop
+        for i in xloads:
+            dest = _regs(lines[i].split(",")[0])
+            early = [l.strip() for l in lines[i + 1:wait] if code(l) and _regs(l) & dest]
+            assert not early, (name, lines[i].strip(), early[:4])
+        # the path around the loop
+        skip = [i for i, l in enumerate(lines) if l.strip() == "s_waitcnt vmcnt(0)" and not loop <= i < loop + len(template)]
+        assert len(skip) == 1, (name, skip)
+        j = skip[0]
+        while not re.match(r"\.LBB\d+_\d+:", lines[j].strip()):
+            j -= 1
+        before = [l.strip() for l in lines[j + 1:skip[0]] if code(l) and _regs(l) & ring]
+        assert not before, (name, before[:4])
+        # operands of the loop
+        actual = [l.strip() for l in lines[loop:loop + len(template)]]
+        assert len(actual) == len(template)
+        operands = {}
+        for t, a in zip(template, actual):
+            if "%[" not in t:
+                assert t == a, (name, t, a)
+                continue
+            pat = re.escape(t)
+            pat = re.sub(r"%\\\[(\w+)\\\]", lambda mm: "(?P<%s_%d>v\\[\\d+:\\d+\\]|v\\d+)" % (mm.group(1), len(operands) + id(mm) % 1000), pat)
+            mm = re.fullmatch(pat, a)
+            assert mm, (name, t, a)
+            for key, val in mm.groupdict().items():
+                operands.setdefault(key.rsplit("_", 1)[0], set()).add(val)
+        assert set(operands) == {"woff", "qaddr", "xaddr", "mask", "sello", "selhi", "bc1", "bc2"}, (name, sorted(operands))
+        used = set()
+        for key, vals in operands.items():
+            assert len(vals) == 1, (name, key, vals)
+            regs = _regs(next(iter(vals)))
+            assert max(regs) < vbase, (name, key, vals)
+            assert not (regs & used), (name, key, vals)
+            used |= regs
+        scratch = re.search(r"\.amdhsa_private_segment_fixed_size (\d+)", meta)
+        assert scratch is None or int(scratch.group(1)) == 0, (name, scratch.group(0))
