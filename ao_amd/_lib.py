@@ -41,6 +41,7 @@ _SIGNATURES = {
     "ao_amd_int4wo_unpack": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _p], _int),
     "ao_amd_int4wo_dequantize": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
     "ao_amd_int4wo_linear": ([_p, _i64, _i64, _i64, _p, _p, _i64, _i64, _p, _p, _int, _i64, _p], _int),
+    "ao_amd_int4wo_linear_plan": ([_i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _int, _int, ctypes.c_char_p, _i64], _int),
     "ao_amd_profile_next_linear": ([_p, _p], _int),
     "ao_amd_fp6_quantize_pack": ([_p, _int, _i64, _i64, _int, _int, _p, _p, _p], _int),
     "ao_amd_fp6_dequantize": ([_p, _p, _i64, _i64, _int, _int, _p, _p], _int),
@@ -132,3 +133,13 @@ def packed_shape(N: int, K: int, g: int):
     out = [ctypes.c_int64() for _ in range(4)]
     check(lib().ao_amd_int4wo_packed_shape(N, K, g, *[ctypes.byref(o) for o in out]))
     return tuple(o.value for o in out)
+
+
+def int4wo_linear_plan(M: int, K: int, N: int, g: int, *, aligned: bool = True, residual: bool = False, norm: bool = False,
+                       dual: bool = False, pair8: bool = False, ksplit: int = 1, y_dtype: int = BF16) -> str:
+    """Name of the kernel instantiation the int4 linear entry points run for this problem (host-side decision only:
+    nothing is launched, no GPU is needed)."""
+    buf = ctypes.create_string_buffer(128)
+    check(lib().ao_amd_int4wo_linear_plan(M, K, N, g, int(aligned), int(residual), int(norm), int(dual), int(pair8), ksplit,
+                                          y_dtype, buf, 128))
+    return buf.value.decode()

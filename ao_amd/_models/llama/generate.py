@@ -69,6 +69,9 @@ class GraphedDecoder:
         self.pos = torch.zeros(1, dtype=torch.int, device=device)
         self.next_token = torch.zeros(1, dtype=torch.int, device=device)
         self.graph = None
+        # host mirror of the device-side position: a replay advances `pos` on the device, where the host cannot see it,
+        # so the bound of the KV cache is enforced here (the attention kernel only degrades to NaN outputs past it)
+        self.host_pos = 0
 
     def _step(self):
         if self.sampling_kwargs.get("greedy") and self.token.is_cuda:
@@ -89,6 +92,9 @@ class GraphedDecoder:
     def capture(self, token: torch.Tensor, pos: int, warmup: int = 2):
         """Capture at position `pos`.  The warm-up and capture steps write KV-cache slots pos..pos+warmup,
         which later real steps overwrite; the static buffers are reset afterwards."""
+        if pos >= self.model.max_seq_length:
+            raise IndexError(f"capture at position {pos} is past the KV cache ({self.model.max_seq_length} positions)")
+        warmup = max(0, min(warmup, self.model.max_seq_length - 1 - pos))  # warm-up steps stay inside the cache too
         self.token.copy_(token.view(1, 1))
         self.pos.fill_(pos)
         side = torch.cuda.Stream()
@@ -105,10 +111,15 @@ class GraphedDecoder:
             self._step()
         self.token.copy_(token.view(1, 1))
         self.pos.fill_(pos)
+        self.host_pos = pos
 
     def step(self) -> torch.Tensor:
         """One decoded token (device tensor, valid until the next step)."""
+        if self.host_pos >= self.model.max_seq_length:
+            raise IndexError(f"decode step at position {self.host_pos} is past the KV cache "
+                             f"({self.model.max_seq_length} positions); call setup_caches with a longer max_seq_length")
         self.graph.replay()
+        self.host_pos += 1
         return self.next_token
 
 
@@ -141,6 +152,9 @@ def generate(model: Transformer, prompt: torch.Tensor, max_new_tokens: int, *, i
     seq = torch.empty(T_new, dtype=prompt.dtype, device=device)
     seq[:T] = prompt.view(-1)
     max_seq_length = min(T_new, model.config.block_size) if not interactive else 350
+    if T_new > max_seq_length:
+        raise ValueError(f"prompt ({T}) + max_new_tokens ({max_new_tokens}) = {T_new} positions do not fit the "
+                         f"{max_seq_length}-position KV cache" + (" of interactive mode" if interactive else " (block_size)"))
     model.setup_caches(max_batch_size=1, max_seq_length=max_seq_length)
     x, input_pos = prepare_inputs_for_model(prompt, max_new_tokens)
     next_token = prefill(model, x, input_pos, **sampling_kwargs).clone()

@@ -53,5 +53,7 @@ __device__ __forceinline__ uint32_t asm_load_b32(const void* sbase, uint32_t vof
 // Single-row GEMV on the 4x4x4 matrix instructions (int4wo_gemv1.hip).  Returns true when it took the launch;
 // false when the shape is outside what it handles (the caller then uses the general kernels).
 bool launch_int4wo_gemv1(const LinearArgs& a, int64_t g, int64_t RB, hipStream_t st);
+// The same decision without a launch: writes the instantiation it would run ("int4wo_gemv1_kernel<waves,xl,norm> wpr=..")
+bool int4wo_gemv1_plan(const LinearArgs& a, int64_t g, int64_t RB, char* out, size_t cap);
 
 }  // namespace ao

@@ -1030,7 +1030,13 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
                            const void* packed2, const void* qparams2, int64_t N, int64_t g, const void* bias_bf16,
                            const void* residual_bf16, int64_t ldres, void* y, int y_dtype, int64_t ldy, void* stream,
                            const void* norm_weight_bf16 = nullptr, float norm_eps = 0.f, bool pair8 = false,
-                           int ksplit = 1) {
+                           int ksplit = 1, char* plan_out = nullptr, size_t plan_cap = 0) {
+    // plan_out: do not launch; write the name of the kernel the arguments select (ao_amd_int4wo_linear_plan)
+#define AO_PLAN(...)                                    \
+    if (plan_out) {                                     \
+        snprintf(plan_out, plan_cap, __VA_ARGS__);      \
+        return 0;                                       \
+    }
     // pair8: `packed` / `qparams` hold 2 * N rows (gate and up rows interleaved in eights), the output has N columns
     const int64_t n_out = N;
     if (pair8) N *= 2;
@@ -1112,6 +1118,9 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
         // each group has 2 or more K tiles; the 64-row tiles (192 or more workgroups, which already overlap each other)
         // from 64 K tiles on (K = 14336, 512 rows: -4 %; K = 4096: +4 % and therefore not split)
         const bool ksplit_tiles = !big && KB_all >= (tiny ? 8 : 64);
+        AO_PLAN("%s<%lld,%d,%d>", (!big && ksplit_tiles) ? "int4wo_gemm_ksplit_kernel" : "int4wo_gemm_kernel", (long long)g,
+                big ? 2 : (tiny && ksplit_tiles ? 2 : (tiny ? 1 : (ksplit_tiles ? 4 : 1))),
+                big ? 8 : (tiny && ksplit_tiles ? 4 : (tiny ? 2 : 4)));
 #define AO_GEMM_LAUNCH(GG)                                                                                     \
     if (big) launch_timed(int4wo_gemm_kernel<GG, 2, 8>, ggrid, dim3(256), 0, st, a);                           \
     else if (tiny && ksplit_tiles) launch_timed(int4wo_gemm_ksplit_kernel<GG, 2, 4>, ggrid, dim3(1024), 0, st, a); \
@@ -1129,10 +1138,18 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
         return 0;
     }
     // one activation row: the kernel built on the 4x4x4 matrix instructions (group size 64 and up, K up to 16384)
-    if (M == 1 && aligned && !dual && launch_int4wo_gemv1(a, g, RB, st)) {
-        AO_LAUNCH_CHECK();
-        return 0;
+    if (M == 1 && aligned && !dual) {
+        char name[96];
+        if (int4wo_gemv1_plan(a, g, RB, name, sizeof(name))) {
+            AO_PLAN("%s", name);
+            launch_int4wo_gemv1(a, g, RB, st);
+            AO_LAUNCH_CHECK();
+            return 0;
+        }
     }
+    AO_PLAN("%s<%lld,%d,%s%d>", xmode == X_LDS ? "int4wo_gemv_kernel" : "int4wo_linear_kernel", (long long)g, waves,
+            xmode == X_LDS ? "" : (xmode == X_GLOBAL ? "X_GLOBAL," : "X_CHECKED,"), dual ? 1 : 0);
+#undef AO_PLAN
     dim3 grid((unsigned)RB, (unsigned)mchunks, (unsigned)ksplit);
     const size_t smem = xmode == X_LDS ? xbytes : 0;
     if (dual) {
@@ -1156,6 +1173,19 @@ extern "C" int ao_amd_profile_next_linear(void* start_event, void* stop_event) {
     g_prof_start = (hipEvent_t)start_event;
     g_prof_stop = (hipEvent_t)stop_event;
     return 0;
+}
+
+extern "C" int ao_amd_int4wo_linear_plan(int64_t M, int64_t K, int64_t N, int64_t g, int aligned, int has_residual,
+                                         int has_norm, int dual, int pair8, int ksplit, int y_dtype, char* out,
+                                         int64_t out_cap) {
+    AO_REQUIRE(out && out_cap > 0, "null pointer argument");
+    // dummy operands: 16-byte aligned (or deliberately odd) addresses that are never dereferenced
+    const void* p = reinterpret_cast<const void*>(aligned ? (uintptr_t)4096 : (uintptr_t)4098);
+    const void* w = reinterpret_cast<const void*>((uintptr_t)8192);
+    out[0] = 0;
+    return linear_dispatch(p, M, K, K, w, w, dual ? w : nullptr, dual ? w : nullptr, N, g, nullptr, has_residual ? w : nullptr,
+                           pair8 ? 2 * N : N, const_cast<void*>(w), y_dtype, N, nullptr, has_norm ? w : nullptr, 1e-5f,
+                           pair8 != 0, ksplit, out, (size_t)out_cap);
 }
 
 extern "C" int ao_amd_int4wo_linear(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed,

@@ -138,6 +138,19 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     const int sub = lane >> 4, l16 = lane & 15;
     const int rg = wave * 4 + sub;  // row group 0..63
     const int pos = __builtin_amdgcn_readfirstlane(pos_ptr[0]);  // uniform: branches on it are scalar
+    // The position lives in device memory (a graphed decode loop advances it there), so the host cannot vouch for it:
+    // a position outside the cache (whose length also bounds the rows of freqs) touches no memory and leaves NaN
+    // outputs, which the next linear propagates to the logits.
+    if (pos < 0 || pos >= S) {
+        const float qnan = __uint_as_float(0x7fc00000u);
+        if (nsplit > 1) {
+            float* dst = part + ((int64_t)blockIdx.x * nsplit + blockIdx.y) * (HD + 2);
+            if (threadIdx.x < HD + 2) dst[threadIdx.x] = qnan;
+        } else if (threadIdx.x < HD) {
+            out[(int64_t)blockIdx.x * HD + threadIdx.x] = E::to_bits(qnan);
+        }
+        return;
+    }
     const int T = pos + 1;
     // Long contexts: `nsplit` workgroups per head (blockIdx.y = z) take the 64-position rows z, z + nsplit, ... of
     // the context, so that any context length spreads evenly over them; each leaves (max, sum, unnormalised output) in

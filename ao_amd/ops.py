@@ -494,6 +494,8 @@ def _decode_attention_f16_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_he
                  lambda: "caches must be contiguous [1, n_kv, max_seq, head_dim]")
     head_dim, max_seq = k_cache.shape[3], k_cache.shape[2]
     torch._check(freqs_cis.is_contiguous() and freqs_cis.shape[-2:] == (head_dim // 2, 2), lambda: "bad freqs_cis shape")
+    torch._check(freqs_cis.shape[0] >= max_seq,
+                 lambda: f"freqs_cis has {freqs_cis.shape[0]} rows for a cache of {max_seq} positions")
     torch._check(qkv.numel() == (n_head + 2 * n_kv) * head_dim and qkv.is_contiguous(),
                  lambda: "qkv must be the contiguous fused projection of one token")
     out = torch.empty((1, n_head * head_dim), dtype=torch.float16, device=qkv.device)
@@ -520,6 +522,8 @@ def _decode_attention_cuda(qkv, freqs_cis, input_pos, k_cache, v_cache, n_head, 
     head_dim, max_seq = k_cache.shape[3], k_cache.shape[2]
     row = (n_head + 2 * n_kv) * head_dim
     torch._check(freqs_cis.is_contiguous() and freqs_cis.shape[-2:] == (head_dim // 2, 2), lambda: "bad freqs_cis shape")
+    torch._check(freqs_cis.shape[0] >= max_seq,
+                 lambda: f"freqs_cis has {freqs_cis.shape[0]} rows for a cache of {max_seq} positions")
     out = torch.empty((1, n_head * head_dim), dtype=torch.bfloat16, device=qkv.device)
     nparts = 0
     if qkv.dtype is torch.float32:

@@ -135,6 +135,15 @@ int ao_amd_int4wo_rmsnorm_swiglu(const void* x_bf16, int64_t M, int64_t K, int64
                                  float eps, const void* packed_gate, const void* qparams_gate, const void* packed_up,
                                  const void* qparams_up, int64_t N, int64_t g, void* y_bf16, int64_t ldy, void* stream);
 
+/* Which kernel instantiation the int4 linear entry points above run for a problem, without launching anything: writes a
+ * name such as "int4wo_gemm_ksplit_kernel<64,4,4>" or "int4wo_gemv1_kernel<4,2,0> wpr=4" to `out`.  `aligned`: K is a
+ * multiple of max(128, g) and the activation rows are 16-byte aligned; the other flags say which fused variant is meant
+ * (residual epilogue, RMSNorm on the activations, two weights, interleaved gate/up weight, K split).  The test suite walks
+ * the dispatch with it so that no instantiation ships without a test that reaches it.  No counterpart in the reference
+ * (its dispatch is `aten::_weight_int4pack_mm`'s own, affine_quantized_tensor.py:631). */
+int ao_amd_int4wo_linear_plan(int64_t M, int64_t K, int64_t N, int64_t g, int aligned, int has_residual, int has_norm,
+                              int dual, int pair8, int ksplit, int y_dtype, char* out, int64_t out_cap);
+
 /* Linear with the K range split over `ksplit` (1..8) groups of workgroups, for weights whose row-block count does not fill
  * the CUs evenly (Llama-3-8B wqkv: 384 row blocks on 256 CUs): y_f32_parts[z][M][ldy] = sum over the z-th run of K tiles
  * of x' W^T in fp32, x' = x or its RMSNorm as in ao_amd_int4wo_rmsnorm_linear.  The consumer adds the parts and rounds
@@ -222,9 +231,10 @@ int ao_amd_rmsnorm_bf16(const void* x, const void* weight, int64_t rows, int64_t
 
 /* One new token, batch 1: rotary embedding of q and k, KV-cache update at *pos_dev, grouped-query attention over
  * positions 0..*pos_dev.  Attention.forward, torchao/_models/llama/model.py:190-211 with apply_rotary_emb :250-266
- * and KVCache.update :85-98.  qkv: [(n_head + 2 n_kv) * head_dim] (fused wqkv output); freqs_cis: [*, head_dim/2, 2]
+ * and KVCache.update :85-98.  qkv: [(n_head + 2 n_kv) * head_dim] (fused wqkv output); freqs_cis: [>= max_seq, head_dim/2, 2]
  * (cos, sin); caches: [n_kv, max_seq, head_dim]; out: [n_head * head_dim].  head_dim must be 128, max_seq <= 28000 (the
- * scores of the whole context live in LDS; see the split variant below for more). */
+ * scores of the whole context live in LDS; see the split variant below for more).  The position is read on the device:
+ * one outside [0, max_seq) touches neither cache nor freqs_cis and yields NaN outputs (the reference's index ops raise). */
 int ao_amd_llama_decode_attention(const void* qkv_bf16, const void* freqs_cis_bf16, const int32_t* pos_dev,
                                   void* k_cache, void* v_cache, int n_head, int n_kv, int head_dim, int64_t max_seq,
                                   void* out_bf16, void* stream);

@@ -237,3 +237,25 @@ def test_dispatch_rules_are_pure_host_functions():
     assert ops.int4wo_packed_shapes(48, 192, 64) == ((3, 2, 64, 4), (3, 4, 16))
     with pytest.raises(ValueError):
         ops.int4wo_packed_shapes(48, 192, 48)
+
+
+def test_decode_loop_refuses_positions_past_the_kv_cache():
+    """The graphed decode loop advances its position on the device; the host mirror must stop it at the end of the
+    cache (the attention kernel itself only degrades to NaN there), and generate() must refuse a request that cannot fit."""
+    from types import SimpleNamespace
+
+    import torch
+
+    from ao_amd._models.llama.generate import GraphedDecoder, generate
+
+    gd = GraphedDecoder(SimpleNamespace(max_seq_length=4), "cpu", greedy=True)
+    gd.host_pos = 4
+    with pytest.raises(IndexError, match="past the KV cache"):
+        gd.step()
+    with pytest.raises(IndexError, match="past the KV cache"):
+        gd.capture(torch.zeros(1, dtype=torch.int), pos=4)
+    model = SimpleNamespace(config=SimpleNamespace(block_size=16))
+    with pytest.raises(ValueError, match="do not fit"):
+        generate(model, torch.zeros(10, dtype=torch.int), 10)
+    with pytest.raises(ValueError, match="interactive"):
+        generate(model, torch.zeros(300, dtype=torch.int), 100, interactive=True)

@@ -531,3 +531,36 @@ def test_fp6_staged_gemv_fusions_match_the_separate_kernels(M, N, K, fmt):
     got3 = ops.fp6_swiglu(e, m, x, ng, sg, nu, su, nw, 1e-5)
     g3, w3 = got3.float().cpu().numpy(), want3.float().cpu().numpy()
     assert rel_l2(g3, w3) <= 2e-3 and np.count_nonzero(g3 != w3) <= 0.02 * g3.size + 1
+
+
+def test_fused_decode_step_on_the_llama3_8b_configuration():
+    """The benchmark's own model (32 layers, dim 4096, 32 / 8 heads, FFN 14336, vocabulary 128256, int4wo-64 on every
+    linear, random weights): one fused decode step against the module-by-module forward on the same cache state, then
+    16 graph-replayed tokens against the eager fused loop."""
+    from ao_amd._models.llama.generate import build_random_model, generate
+
+    dev = _dev()
+    print("case fused decode Llama-3-8B", flush=True)
+    model = build_random_model("Llama-3-8B", dev, "int4wo-64")
+    T = 24
+    prompt = torch.randint(0, model.config.vocab_size, (T,), device=dev, dtype=torch.int)
+    with torch.no_grad():
+        model.setup_caches(1, 64)
+        assert model.fused_decode_ready()
+        model(prompt.view(1, -1), torch.arange(T, device=dev))
+        tok = torch.tensor([[11]], device=dev, dtype=torch.int)
+        p = torch.tensor([T], device=dev, dtype=torch.int)
+        model.use_fused_decode = False
+        ref = model(tok, p).float()
+        model.use_fused_decode = True
+        out = model(tok, p).float()
+    assert out.shape == ref.shape == (1, 1, model.config.vocab_size)
+    err = rel_l2(out.cpu().numpy(), ref.cpu().numpy())
+    print(f"  fused vs module logits rel-L2 = {err:.3e}", flush=True)
+    # the two paths round to bf16 at different places in every layer (norm folded into the linear, SwiGLU in the
+    # epilogue, split attention); with random weights those differences add up like a random walk over the 32 layers:
+    # 1e-2 per layer (the bound the 2-layer test above meets with 3e-2) times sqrt(32)
+    assert err <= 1e-2 * model.config.n_layer ** 0.5, err
+    a = generate(model, prompt, 16, use_graph=True, greedy=True)
+    b = generate(model, prompt, 16, use_graph=False, greedy=True)
+    assert torch.equal(a, b)

@@ -137,3 +137,75 @@ def test_fp6_properties(shape):
         y = ops.quant_llm_linear(3, 2, x, tc, scale)
         for m in range(M):
             assert rel_l2(y[m].float().cpu().numpy(), dq[:, ks[m]].cpu().numpy()) <= 1e-3, (M, m)
+
+
+@pytest.mark.parametrize("M", [128, 512, 2048])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_int4_prefill_gemm_full_size(shape, M):
+    """The prefill configuration (M in {128, 512, 2048}, g = 64) at the real Llama-3-8B shapes, through the C ABI's
+    fused kernel (whatever tile variant the dispatch picks there): one-hot rows bit for bit, random rows against an
+    fp32 matmul on the bit-exact dequantized weight (2e-5 with fp32 output, 1e-3 with bf16 output)."""
+    from ao_amd import _lib, ops
+
+    N, K = shape
+    g = 64
+    if N * M > (1 << 28):
+        pytest.skip("output larger than the launch allows")
+    plan = _lib.int4wo_linear_plan(M, K, N, g)
+    print(f"case int4 prefill full-size N={N} K={K} M={M}: {plan}", flush=True)
+    assert plan.startswith("int4wo_gemm")
+    dev = _dev()
+    w = _weight(N, K, seed=3 + N + M)
+    packed, qp = ops.int4wo_quantize_pack(w, g)
+    dq = ops.int4wo_dequantize(packed, qp, N, K, g)
+    del w
+    L = _lib.lib()
+    st = torch.cuda.current_stream().cuda_stream
+
+    def run(x, fp32):
+        y = torch.empty(M, N, dtype=torch.float32 if fp32 else torch.bfloat16, device=dev)
+        _lib.check(L.ao_amd_int4wo_linear(x.data_ptr(), M, K, K, packed.data_ptr(), qp.data_ptr(), N, g, None, y.data_ptr(),
+                                          _lib.F32 if fp32 else _lib.BF16, N, st))
+        torch.cuda.synchronize()
+        return y
+
+    gen = torch.Generator(device=dev).manual_seed(M)
+    ks = torch.randint(0, K, (M,), device=dev, generator=gen)
+    ks[0], ks[1] = 0, K - 1
+    xh = torch.zeros(M, K, dtype=torch.bfloat16, device=dev)
+    xh[torch.arange(M, device=dev), ks] = 1.0
+    yh = run(xh, True)
+    exact = bool(torch.equal(yh, dq.float().t()[ks]))
+    assert exact
+    del yh, xh
+    x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
+    ref = x.float() @ dq.float().t()
+    y32 = run(x, True)
+    assert float((y32 - ref).norm() / ref.norm()) <= 2e-5
+    del y32
+    y16 = run(x, False)
+    assert float((y16.float() - ref.bfloat16().float()).norm() / ref.norm()) <= 1e-3
+
+
+def test_config1_output_tolerance(oracle):
+    """The CPU-runnable configuration: one bf16 weight [4096, 4096] ~N(0, 0.02), group 128, x [1, 4096] ~N(0, 1): the
+    linear's output against the oracle's dequantize-then-linear with fp32 accumulation, rel-L2 <= 1e-3 (codes, scales
+    and zeros of this configuration are compared bit for bit in test_int4wo_gpu.py)."""
+    from _util import bits16, make_act, make_weight
+    from ao_amd import ops
+
+    N = K = 4096
+    g = 128
+    w = make_weight(N, K, seed=1234, special=False)
+    x = make_act(1, K, seed=4321)
+    codes, scale, zero = oracle.int4wo_quantize(bits16(w), oracle.BF16, g, N, K)
+    dq = oracle.dequantize_affine(codes, oracle.I32, (1, g), scale, oracle.BF16, zero, oracle.BF16, 0, 15, 1, oracle.BF16)
+    y_ref = oracle.linear(bits16(x), oracle.BF16, dq, oracle.BF16)
+    packed, qp = ops.int4wo_quantize_pack(w.to(_dev()), g)
+    y32 = ops.int4wo_linear(x.to(_dev()), packed, qp, g, N, None, True)
+    err = rel_l2(y32.cpu().numpy(), y_ref)
+    print(f"config 1 output rel-L2 = {err:.3e}", flush=True)
+    assert err <= 1e-3
+    y16 = ops.int4wo_linear(x.to(_dev()), packed, qp, g, N, None, False)
+    y_ref16 = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(y_ref))
+    assert rel_l2(y16.float().cpu().numpy(), y_ref16) <= 1e-3
