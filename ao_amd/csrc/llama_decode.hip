@@ -5,6 +5,8 @@
 //   decode attention   torchao/_models/llama/model.py:190-211  (rotary embedding of q and k, KV-cache update at
 //                      input_pos, grouped-query attention of the one new token over positions 0..pos) and
 //                      :260-266 (apply_rotary_emb), :78-98 (KVCache)
+#include <mutex>
+
 #include "common.h"
 
 namespace ao {
@@ -534,6 +536,50 @@ extern "C" int ao_amd_llama_decode_attention_split(const void* qkv_bf16, const v
     AO_REQUIRE(qkv_bf16 || (nparts >= 1 && nparts <= 8), "number of partial rows %d outside [1, 8]", nparts);
     return attention_dispatch(qkv_bf16, qkv_f32_parts, qkv_bf16 ? 0 : nparts, freqs_cis_bf16, pos_dev, k_cache, v_cache,
                               n_head, n_kv, head_dim, max_seq, nsplit, workspace_f32, out_bf16, stream);
+}
+
+// Workspace of the entry point that allocates nothing: (max, sum, output) triples of up to ATT_STATIC_TRIPLES
+// (head, context share) pairs.  Every device the library runs on holds its own copy until the process ends.
+constexpr int ATT_STATIC_TRIPLES = 2048;
+static __device__ __align__(256) float att_static_scratch[ATT_STATIC_TRIPLES * 130];
+
+// Device address of the current device's copy of att_static_scratch (the array's name is only a host-side handle for
+// the symbol): resolved once per device, on the first call with that device current.
+static int att_static_workspace(float** out) {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static float* ptrs[MAX_DEVICES] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    AO_REQUIRE(e == hipSuccess, "hipGetDevice failed: %s", hipGetErrorString(e));
+    AO_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "device index %d outside [0, %d)", dev, MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(att_static_scratch));
+        AO_REQUIRE(e == hipSuccess && p, "hipGetSymbolAddress(att_static_scratch) failed on device %d: %s", dev,
+                   hipGetErrorString(e));
+        ptrs[dev] = (float*)p;
+    }
+    *out = ptrs[dev];
+    return 0;
+}
+
+extern "C" int ao_amd_llama_decode_attention_split_static(const void* qkv_bf16, const void* qkv_f32_parts, int nparts,
+                                                          const void* freqs_cis_bf16, const int32_t* pos_dev,
+                                                          void* k_cache, void* v_cache, int n_head, int n_kv,
+                                                          int head_dim, int64_t max_seq, int nsplit, void* out_bf16,
+                                                          void* stream) {
+    AO_REQUIRE((qkv_bf16 != nullptr) != (qkv_f32_parts != nullptr), "pass the fused qkv row either as bf16 or as fp32 parts");
+    AO_REQUIRE(qkv_bf16 || (nparts >= 1 && nparts <= 8), "number of partial rows %d outside [1, 8]", nparts);
+    AO_REQUIRE(n_head >= 1 && nsplit >= 1 && (int64_t)n_head * nsplit <= ATT_STATIC_TRIPLES,
+               "n_head * nsplit = %lld exceeds the %d (head, context share) pairs of the built-in workspace: use "
+               "ao_amd_llama_decode_attention_split with a workspace of your own",
+               (long long)n_head * nsplit, ATT_STATIC_TRIPLES);
+    float* ws = nullptr;
+    if (int rc = att_static_workspace(&ws)) return rc;
+    return attention_dispatch(qkv_bf16, qkv_f32_parts, qkv_bf16 ? 0 : nparts, freqs_cis_bf16, pos_dev, k_cache, v_cache,
+                              n_head, n_kv, head_dim, max_seq, nsplit, ws, out_bf16, stream);
 }
 
 extern "C" int ao_amd_llama_decode_attention_f16(const void* qkv_f16, const void* freqs_cis_f16, const int32_t* pos_dev,

@@ -255,6 +255,19 @@ int ao_amd_llama_decode_attention_split(const void* qkv_bf16, const void* qkv_f3
                                         int n_head, int n_kv, int head_dim, int64_t max_seq, int nsplit,
                                         void* workspace_f32, void* out_bf16, void* stream);
 
+/* ao_amd_llama_decode_attention_split without the workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops and harnesses that forbid hipMalloc): the partial (max, sum, output)
+ * triples go to a 1 MiB array that is part of the library's device image (one copy per device, held until the process
+ * ends), whose address the first call on a device looks up (hipGetSymbolAddress).  The call itself allocates and frees
+ * nothing.  n_head * nsplit may be at most 2048; anything larger is rejected with an error.  All calls on one device
+ * share the array: calls that overlap in time on the same device (different streams or threads) race, and nothing in it
+ * needs clearing between calls because every launch rewrites every triple it later reads.  Results are bit-identical to
+ * ao_amd_llama_decode_attention_split.  No counterpart in the reference. */
+int ao_amd_llama_decode_attention_split_static(const void* qkv_bf16, const void* qkv_f32_parts, int nparts,
+                                               const void* freqs_cis_bf16, const int32_t* pos_dev, void* k_cache,
+                                               void* v_cache, int n_head, int n_kv, int head_dim, int64_t max_seq,
+                                               int nsplit, void* out_bf16, void* stream);
+
 /* The same two harness kernels over fp16 activations, weights and caches, for the FP6 model (whose linear takes fp16):
  * RMSNorm.forward and Attention.forward as above, every rounding to fp16 instead of bf16.  The attention entry takes
  * the context split directly (nsplit = 1 and a null workspace for short caches). */
