@@ -50,10 +50,95 @@ __device__ __forceinline__ uint32_t asm_load_b32(const void* sbase, uint32_t vof
     return v;
 }
 
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+struct GroupConst {
+    uint32_t s_lo, s_hi;  // packed bf16 (s, 0) and (0, s)
+    float c136;           // -136 * s (exact in fp32)
+    float z;
+};
+__device__ __forceinline__ GroupConst make_group(uint32_t qp) {
+    GroupConst g;
+    g.s_lo = qp & 0xffffu;
+    g.s_hi = qp << 16;
+    g.c136 = -136.0f * __uint_as_float(qp << 16);
+    g.z = __uint_as_float(qp & 0xffff0000u);
+    return g;
+}
+
+// 8 packed codes -> 8 dequantized bf16 in MFMA B-operand order.
+//
+// One asm block, because the instruction order carries the hardware's dependency rules: a VALU
+// instruction may read the result of a v_dot2 only 3 or more issue slots after it, and the compiler
+// does not look inside inline asm to enforce that.  Every dot2 result below is consumed at least 3
+// instructions later; the trailing s_nop keeps a following consumer of the last v_cvt_pk clear too.
+__device__ __forceinline__ bf16x8_t dequant8(uint32_t w, const GroupConst& g, uint32_t magic, uint32_t one_lo,
+                                             uint32_t one_hi) {
+    union { uint32_t u[4]; bf16x8_t v; } out;
+    uint32_t p0, p1, p2, p3;
+    float a0, a1, a2, a3, a4, a5, a6, a7;
+    asm("v_and_or_b32 %[p0], %[w], %[mask], %[magic]\n\t"
+        "v_lshrrev_b32 %[p1], 4, %[w]\n\t"
+        "v_lshrrev_b32 %[p2], 8, %[w]\n\t"
+        "v_lshrrev_b32 %[p3], 12, %[w]\n\t"
+        "v_and_or_b32 %[p1], %[p1], %[mask], %[magic]\n\t"
+        "v_and_or_b32 %[p2], %[p2], %[mask], %[magic]\n\t"
+        "v_and_or_b32 %[p3], %[p3], %[mask], %[magic]\n\t"
+        "v_dot2_f32_bf16 %[a0], %[p0], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a1], %[p0], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a2], %[p1], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a3], %[p1], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a4], %[p2], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a5], %[p2], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a6], %[p3], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[a7], %[p3], %[shi], %[c]\n\t"
+        "v_cvt_pk_bf16_f32 %[p0], %[a0], %[a1]\n\t"
+        "v_cvt_pk_bf16_f32 %[p1], %[a2], %[a3]\n\t"
+        "v_cvt_pk_bf16_f32 %[p2], %[a4], %[a5]\n\t"
+        "v_cvt_pk_bf16_f32 %[p3], %[a6], %[a7]\n\t"
+        "v_dot2_f32_bf16 %[a0], %[p0], %[olo], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a1], %[p0], %[ohi], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a2], %[p1], %[olo], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a3], %[p1], %[ohi], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a4], %[p2], %[olo], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a5], %[p2], %[ohi], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a6], %[p3], %[olo], %[z]\n\t"
+        "v_dot2_f32_bf16 %[a7], %[p3], %[ohi], %[z]\n\t"
+        "v_cvt_pk_bf16_f32 %[o0], %[a0], %[a1]\n\t"
+        "v_cvt_pk_bf16_f32 %[o1], %[a2], %[a3]\n\t"
+        "v_cvt_pk_bf16_f32 %[o2], %[a4], %[a5]\n\t"
+        "v_cvt_pk_bf16_f32 %[o3], %[a6], %[a7]\n\t"
+        "s_nop 1"
+        : [o0] "=&v"(out.u[0]), [o1] "=&v"(out.u[1]), [o2] "=&v"(out.u[2]), [o3] "=&v"(out.u[3]), [p0] "=&v"(p0),
+          [p1] "=&v"(p1), [p2] "=&v"(p2), [p3] "=&v"(p3), [a0] "=&v"(a0), [a1] "=&v"(a1), [a2] "=&v"(a2),
+          [a3] "=&v"(a3), [a4] "=&v"(a4), [a5] "=&v"(a5), [a6] "=&v"(a6), [a7] "=&v"(a7)
+        : [w] "v"(w), [mask] "s"(0x000F000Fu), [magic] "v"(magic), [slo] "v"(g.s_lo), [shi] "v"(g.s_hi),
+          [c] "v"(g.c136), [z] "v"(g.z), [olo] "v"(one_lo), [ohi] "v"(one_hi));
+    return out.v;
+}
+
+template <typename Kernel>
+inline void launch_timed(Kernel kernel, dim3 grid, dim3 block, size_t smem, hipStream_t st, const LinearArgs& a) {
+    if (g_prof_start && g_prof_stop) {
+        hipExtLaunchKernelGGL(kernel, grid, block, smem, st, g_prof_start, g_prof_stop, 0, a);
+        g_prof_start = g_prof_stop = nullptr;
+        return;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, smem, st, a);
+}
+
 // Single-row GEMV on the 4x4x4 matrix instructions (int4wo_gemv1.hip).  Returns true when it took the launch;
 // false when the shape is outside what it handles (the caller then uses the general kernels).
 bool launch_int4wo_gemv1(const LinearArgs& a, int64_t g, int64_t RB, hipStream_t st);
 // The same decision without a launch: writes the instantiation it would run ("int4wo_gemv1_kernel<waves,xl,norm> wpr=..")
 bool int4wo_gemv1_plan(const LinearArgs& a, int64_t g, int64_t RB, char* out, size_t cap);
+
+
+// Prefill GEMM with the weight tile dequantized once per workgroup into LDS (int4wo_gemm.hip); same contract as above.
+bool launch_int4wo_gemm_lds(const LinearArgs& a, int64_t g, hipStream_t st);
+bool int4wo_gemm_lds_plan(const LinearArgs& a, int64_t g, char* out, size_t cap);
 
 }  // namespace ao

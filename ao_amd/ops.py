@@ -69,10 +69,13 @@ _LIB.define("fp6_swiglu(int ebits, int mbits, Tensor x, Tensor? norm_weight, flo
 _LIB.define("fp6_linear_native_fused(int ebits, int mbits, Tensor x, Tensor native, Tensor scale, Tensor other, bool gated) -> Tensor")
 
 
-# Activation rows from which the int4 linear dequantizes the weight once and calls the library bf16 GEMM.
-# Measured crossovers on MI355X (Llama-3-8B shapes, g = 64): 512 rows for the 14336 x 4096 / 4096 x 14336 weights,
-# 1024 for 4096 x 4096 and for a vocabulary-sized weight, never worth it below about 2048 output features.
-TWO_PASS_MIN_M = 512
+# Activation rows from which the int4 linear dequantizes the weight once into a bf16 scratch weight and calls the
+# library bf16 GEMM instead of the fused kernels.  Measured on MI355X (g = 64, fused / two-pass in us): 14336 x 4096:
+# 512 rows 72 / 83, 1024 rows 132 / 128, 2048 rows 247 / 207, 4096 rows 458 / 358; 4096 x 14336: 2048 rows 245 / 213,
+# 4096 rows 388 / 328; 128256 x 4096: 512 rows 481 / 763, 2048 rows 1809 / 1794, 4096 rows 3621 / 3133.  The fused
+# prefill kernel (exact two-rounding dequantization in the shadow of the matrix instructions) holds 0.39 - 0.50 of the
+# dense bf16 peak, the library GEMM 0.54 - 0.62 from 4096 rows on, where the extra pass over the weight no longer shows.
+TWO_PASS_MIN_M = 4096
 
 
 INT8_TWO_PASS_MIN_M = 128
@@ -80,11 +83,8 @@ FP6_TWO_PASS_MIN_M = 1024
 
 
 def int4wo_two_pass(M: int, N: int, K: int) -> bool:
-    if N < 2048:
-        return M >= 8 * TWO_PASS_MIN_M
-    if N > 32768 or N * K < (1 << 25):
-        return M >= 2 * TWO_PASS_MIN_M
-    return M >= TWO_PASS_MIN_M
+    # a narrow weight gives the library GEMM few tiles as well: twice the rows
+    return M >= (2 * TWO_PASS_MIN_M if N < 2048 else TWO_PASS_MIN_M)
 
 
 def int4wo_packed_shapes(N: int, K: int, group_size: int):
@@ -175,11 +175,11 @@ def _linear_cuda(x: Tensor, packed: Tensor, qparams: Tensor, group_size: int, N:
         torch._check(bias.dtype is torch.bfloat16 and bias.numel() == N, lambda: "bias must be bfloat16 of size N")
         bias = bias.contiguous()
     if int4wo_two_pass(M, N, K) and not fp32_out:
-        # Large batches (prefill): dequantize once into a bf16 scratch weight with the HIP kernel, then one plain
-        # bf16 GEMM from the vendor library (hipBLASLt through torch).  A dense library GEMM runs at about twice
-        # the matrix-core utilisation of the fused kernel, whose VALU dequantization is repaid per 128 activation
-        # rows; the extra pass over the weight (N*K*2.5 bytes) costs less than that from about 512 rows on.
-        # This is the reference's own definition of the result: dequantize, then F.linear.
+        # Very large batches: dequantize once into a bf16 scratch weight with the HIP kernel, then one plain bf16 GEMM
+        # from the vendor library (hipBLASLt through torch), which holds a higher share of the matrix peak than the
+        # fused kernel, whose dequantization competes with the matrix instructions for issue slots; from about 4096
+        # rows on that outweighs the extra pass over the weight (N*K*2.5 bytes).  This is the reference's own
+        # definition of the result: dequantize, then F.linear.
         return torch.nn.functional.linear(x, _dequantize_cuda(packed, qparams, N, K, group_size), bias)
     y = torch.empty((M, N), dtype=torch.float32 if fp32_out else torch.bfloat16, device=x.device)
     check(lib().ao_amd_int4wo_linear(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, packed.data_ptr(),

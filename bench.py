@@ -147,7 +147,7 @@ def roofline_leg(model, passes=3):
     achieved = total_bytes / total_us / 1e3  # GB/s
     return {
         "bound": "hbm",
-        "kernel": "ao::int4wo_gemv_kernel (M=1, g=64)",
+        "kernel": "ao::int4wo_gemv1_kernel (M=1, g=64)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
@@ -159,6 +159,10 @@ def roofline_leg(model, passes=3):
                          for j, k in enumerate(("norm_wqkv", "wo_residual", "norm_w1w3_swiglu", "w2_residual"))}
         | {"output": round(best[-1], 2)},
         "traffic": _traffic_from_profile(),
+        # the counters need rocprofv3 --pmc runs of their own: this figure is read from the committed summary of
+        # those runs, it is not measured by this invocation
+        "traffic_source": "profiles/int4wo_gemv_llama3_8b_decode_pmc.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                          "scaled by a copy kernel of known size; not measured in this run)",
     }
 
 
@@ -231,6 +235,7 @@ def cpu_baseline_leg(config, group=64, min_seconds=10.0):
     c1["linear"] = time.perf_counter() - t0
     head_params = config.vocab_size * dim
     per_token = per_layer * config.n_layer + per_layer * head_params / layer_params
+    torch_leg = _torch_cpu_leg(config, group, shapes, layer_params, head_params)
     return {
         "value": round(1.0 / per_token, 4),
         "unit": "tokens/s",
@@ -240,6 +245,44 @@ def cpu_baseline_leg(config, group=64, min_seconds=10.0):
                    f"({layer_params / 1e6:.0f}M weights), {reps} repetitions, {per_layer:.2f} s per layer; scaled to "
                    f"{config.n_layer} layers + vocabulary head"),
         "config0_steps_ms": {k: round(v * 1e3, 1) for k, v in c1.items()},
+        "torch_all_threads": torch_leg,
+    }
+
+
+def _torch_cpu_leg(config, group, shapes, layer_params, head_params, min_seconds=5.0):
+    """The fastest CPU execution of the same linears this image offers, beside the scalar port: torch's own CPU kernel
+    for the op the reference dispatches to (aten._weight_int4pack_mm; its CPU build is _weight_int4pack_mm_for_cpu in
+    this torch), bf16 activations, every thread torch is configured with.  Same (q - 8) * scale + zero weights."""
+    import torch
+
+    if not hasattr(torch.ops.aten, "_weight_int4pack_mm_for_cpu"):
+        return None
+    gen = torch.Generator().manual_seed(1234)
+    prepared = []
+    for N, K in shapes:
+        q = torch.randint(0, 16, (N, K), dtype=torch.int32, generator=gen)
+        packed = torch.ops.aten._convert_weight_to_int4pack_for_cpu(q, 2)
+        sz = torch.stack([torch.rand(K // group, N, generator=gen) * 0.01 + 1e-3,
+                          torch.randn(K // group, N, generator=gen) * 0.01], dim=-1).bfloat16().contiguous()
+        prepared.append((torch.randn(1, K, generator=gen).bfloat16(), packed, sz))
+    for x, packed, sz in prepared:  # warm-up
+        torch.ops.aten._weight_int4pack_mm_for_cpu(x, packed, group, sz)
+    t_layer, reps = 0.0, 0
+    while t_layer < min_seconds and reps < 2000:
+        t0 = time.perf_counter()
+        for x, packed, sz in prepared:
+            torch.ops.aten._weight_int4pack_mm_for_cpu(x, packed, group, sz)
+        t_layer += time.perf_counter() - t0
+        reps += 1
+    per_layer = t_layer / reps
+    per_token = per_layer * config.n_layer + per_layer * head_params / layer_params
+    return {
+        "value": round(1.0 / per_token, 3),
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "torch aten._weight_int4pack_mm_for_cpu (bf16, M=1)",
+        "sample": (f"one transformer layer's five linears, {reps} repetitions, {per_layer * 1e3:.2f} ms per layer; scaled "
+                   f"to {config.n_layer} layers + vocabulary head; linears only, as for the port"),
     }
 
 

@@ -228,10 +228,9 @@ def test_dispatch_rules_are_pure_host_functions():
     from ao_amd import ops
     from ao_amd._models.llama.model import Transformer
 
-    assert ops.int4wo_two_pass(512, 14336, 4096) and not ops.int4wo_two_pass(511, 14336, 4096)
-    assert not ops.int4wo_two_pass(512, 4096, 4096) and ops.int4wo_two_pass(1024, 4096, 4096)
-    assert not ops.int4wo_two_pass(512, 128256, 4096) and ops.int4wo_two_pass(1024, 128256, 4096)
-    assert not ops.int4wo_two_pass(2048, 1024, 4096) and ops.int4wo_two_pass(4096, 1024, 4096)
+    assert ops.int4wo_two_pass(4096, 14336, 4096) and not ops.int4wo_two_pass(4095, 14336, 4096)
+    assert not ops.int4wo_two_pass(2048, 4096, 4096) and ops.int4wo_two_pass(4096, 128256, 4096)
+    assert not ops.int4wo_two_pass(4096, 1024, 4096) and ops.int4wo_two_pass(8192, 1024, 4096)
     assert [ops.decode_attention_splits(s) for s in (8, 1024, 1025, 4096, 4097, 8192, 8193, 16384)] == [1, 1, 4, 4, 8, 8, 16, 16]
     assert Transformer.qkv_ksplit(6144) == 2 and Transformer.qkv_ksplit(4096) == 1 and Transformer.qkv_ksplit(2048) == 2
     assert ops.int4wo_packed_shapes(48, 192, 64) == ((3, 2, 64, 4), (3, 4, 16))

@@ -46,18 +46,27 @@ def test_dispatch_walk_finds_every_kernel_family():
     plans = _walk()
     families = {n.split("<")[0] for n in plans}
     assert families == {"int4wo_gemv1_kernel", "int4wo_gemv_kernel", "int4wo_linear_kernel", "int4wo_gemm_kernel",
-                        "int4wo_gemm_ksplit_kernel"}
+                        "int4wo_gemm_ksplit_kernel", "int4wo_gemm_lds_kernel"}
     # the tile variants of the matrix-core kernels and both K-split forms
     for g in GROUPS:
         for tile in ("int4wo_gemm_kernel<%d,2,8>", "int4wo_gemm_kernel<%d,1,4>", "int4wo_gemm_kernel<%d,1,2>",
-                     "int4wo_gemm_ksplit_kernel<%d,4,4>", "int4wo_gemm_ksplit_kernel<%d,2,4>"):
+                     "int4wo_gemm_ksplit_kernel<%d,4,4>", "int4wo_gemm_ksplit_kernel<%d,2,4>",
+                     "int4wo_gemm_lds_kernel<%d,1>", "int4wo_gemm_lds_kernel<%d,2>"):
             assert tile % g in plans, tile % g
     # the single-row kernel: exactly the instantiations that int4wo_gemv1.hip compiles (waves, chunks per lane, norm)
     gemv1 = {n.split(" ")[0] for n in plans if n.startswith("int4wo_gemv1_kernel<")}
     want = {"int4wo_gemv1_kernel<%d,2,%d>" % (w, nm) for w in (4, 8, 16) for nm in (0, 1)}
     want |= {"int4wo_gemv1_kernel<4,4,0>", "int4wo_gemv1_kernel<4,4,1>", "int4wo_gemv1_kernel<8,4,0>", "int4wo_gemv1_kernel<4,8,0>"}
     assert gemv1 == want, sorted(gemv1 ^ want)
-    assert len(plans) >= 60
+    # the prefill kernel takes a problem only when its 256-row tiles fill most of the chip
+    from ao_amd import _lib
+
+    assert _lib.int4wo_linear_plan(2048, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel<64,2>")
+    assert _lib.int4wo_linear_plan(512, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
+    assert _lib.int4wo_linear_plan(2048, 14336, 4096, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
+    assert not _lib.int4wo_linear_plan(512, 14336, 4096, 64).startswith("int4wo_gemm_lds_kernel")   # 64 tiles
+    assert not _lib.int4wo_linear_plan(300, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel")   # 212 of 512 tile rows empty
+    assert len(plans) >= 68
 
 
 def _cases():

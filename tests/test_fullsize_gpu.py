@@ -209,3 +209,56 @@ def test_config1_output_tolerance(oracle):
     y16 = ops.int4wo_linear(x.to(_dev()), packed, qp, g, N, None, False)
     y_ref16 = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(y_ref))
     assert rel_l2(y16.float().cpu().numpy(), y_ref16) <= 1e-3
+
+
+@pytest.mark.parametrize("M,N,K,g,bias,fp32", [(2048, 14336, 4096, 64, False, False), (1000, 14336, 4096, 128, True, False),
+                                               (2048, 6100, 1024, 64, True, False), (1792, 4096, 2048, 32, False, True),
+                                               (2048, 4096, 14336, 256, True, False)])
+def test_prefill_gemm_tiles_edges_and_repeated_launches(cabi, M, N, K, g, bias, fp32):
+    """The 256-row prefill kernel (activations through LDS-direct loads, weights dequantized between the matrix
+    instructions): every output element is written (the output starts as NaN), ragged M and N, bias, both output
+    types, and the same launch three times in a row with LDS of every CU overwritten in between by another kernel, so
+    that a read that runs ahead of its data cannot find the previous launch's identical bytes there."""
+    print(f"case prefill gemm M={M} N={N} K={K} g={g} bias={bias} fp32={fp32}", flush=True)
+    dev = torch.device("cuda:0")
+    L = cabi.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    assert cabi.int4wo_linear_plan(M, K, N, g).startswith("int4wo_gemm_lds_kernel")
+    gen = torch.Generator(device=dev).manual_seed(M + N + K)
+    w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).bfloat16()
+    _, _, pb, qb = cabi.packed_shape(N, K, g)
+    packed = torch.empty(pb // 4, dtype=torch.int32, device=dev)
+    qp = torch.empty(qb // 4, dtype=torch.int32, device=dev)
+    cabi.check(L.ao_amd_int4wo_quantize_pack(w.data_ptr(), N, K, K, g, packed.data_ptr(), qp.data_ptr(), st))
+    dq = torch.empty(N, K, dtype=torch.bfloat16, device=dev)
+    cabi.check(L.ao_amd_int4wo_dequantize(packed.data_ptr(), qp.data_ptr(), N, K, g, dq.data_ptr(), st))
+    del w
+    b = (torch.randn(N, device=dev, generator=gen) * 0.1).bfloat16() if bias else None
+    x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
+    ref = x.float() @ dq.float().t()
+    if bias:
+        ref += b.float()
+    y = torch.empty(M, N, dtype=torch.float32 if fp32 else torch.bfloat16, device=dev)
+    for rep in range(3):
+        y.fill_(float("nan"))
+        # a kernel that fills LDS with other data: the fp16 RMSNorm over many rows uses every CU
+        junk = torch.randn(4096, 4096, device=dev).half()
+        torch.nn.functional.layer_norm(junk, (4096,))
+        cabi.check(L.ao_amd_int4wo_linear(x.data_ptr(), M, K, K, packed.data_ptr(), qp.data_ptr(), N, g,
+                                          None if b is None else b.data_ptr(), y.data_ptr(), cabi.F32 if fp32 else cabi.BF16, N, st))
+        torch.cuda.synchronize()
+        finite = bool(torch.isfinite(y.float()).all())
+        want = ref if fp32 else ref.bfloat16().float()
+        err = float((y.float() - want).norm() / ref.norm())
+        print(f"  launch {rep}: finite {finite} rel_l2 {err:.2e}", flush=True)
+        assert finite and err <= (2e-5 if fp32 else 1e-3)
+    # one-hot rows: the kernel's dequantization, bit for bit
+    ks = torch.randint(0, K, (M,), device=dev, generator=gen)
+    xh = torch.zeros(M, K, dtype=torch.bfloat16, device=dev)
+    xh[torch.arange(M, device=dev), ks] = 1.0
+    yh = torch.empty(M, N, dtype=torch.float32, device=dev)
+    cabi.check(L.ao_amd_int4wo_linear(xh.data_ptr(), M, K, K, packed.data_ptr(), qp.data_ptr(), N, g, None, yh.data_ptr(),
+                                      cabi.F32, N, st))
+    torch.cuda.synchronize()
+    exact = bool(torch.equal(yh, dq.float().t()[ks]))
+    assert exact

@@ -223,7 +223,7 @@ def test_linear_gemm_path(cabi, oracle, case, g):
 
 @pytest.mark.parametrize("case", [(272, 1024, 512, 64, True), (1040, 2048, 700, 128, False), (48, 192, 600, 32, True)])
 def test_linear_op_prefill_two_pass(oracle, case, monkeypatch):
-    """From 512 activation rows on (large weights) the op dequantizes the weight once (tiled HIP kernel, bit-exact
+    """From 4096 activation rows on the op dequantizes the weight once (tiled HIP kernel, bit-exact
     against the oracle's dequantize_affine) and calls the library bf16 GEMM: same tolerance against the oracle as
     the fused kernel, and close to the fused kernel's own result."""
     from ao_amd import ops
@@ -257,10 +257,9 @@ def test_linear_op_prefill_two_pass(oracle, case, monkeypatch):
 def test_two_pass_rule():
     from ao_amd import ops
 
-    assert ops.int4wo_two_pass(512, 14336, 4096) and ops.int4wo_two_pass(512, 4096, 14336)
-    assert not ops.int4wo_two_pass(512, 4096, 4096) and ops.int4wo_two_pass(1024, 4096, 4096)
-    assert not ops.int4wo_two_pass(512, 128256, 4096) and ops.int4wo_two_pass(1024, 128256, 4096)
-    assert not ops.int4wo_two_pass(2048, 1024, 4096) and not ops.int4wo_two_pass(511, 14336, 4096)
+    assert ops.int4wo_two_pass(4096, 14336, 4096) and ops.int4wo_two_pass(4096, 4096, 14336)
+    assert not ops.int4wo_two_pass(2048, 14336, 4096) and not ops.int4wo_two_pass(2048, 128256, 4096)
+    assert not ops.int4wo_two_pass(4096, 1024, 4096) and ops.int4wo_two_pass(8192, 1024, 4096)
 
 
 def test_linear_rejects_bad_arguments(cabi):

@@ -158,3 +158,54 @@ def test_gemv1_ring_registers_are_untouched_between_their_request_and_the_loop(t
             used |= regs
         scratch = re.search(r"\.amdhsa_private_segment_fixed_size (\d+)", meta)
         assert scratch is None or int(scratch.group(1)) == 0, (name, scratch.group(0))
+
+
+def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched(tmp_path):
+    """int4wo_gemm_lds_kernel issues every load of its K loop as an asm statement and waits for them with explicit
+    s_waitcnt vmcnt(0) statements; the compiler neither counts those loads nor knows that their target registers are
+    being filled.  Checked on the generated ISA of every instantiation:
+      * between a weight load and the next vmcnt(0) wait (following the loop's back edge once) no instruction reads or
+        writes the load's target registers, so a copy of stale contents or a reuse of a register under a load in flight
+        (the epilogue's, after the last, unused requests of the loop) cannot happen;
+      * the K loop carries the 16 LDS-direct activation requests and the weight requests (a chunk and its scale / zero per
+        32-row block) of its two steps;
+      * no scratch access inside the K loop, every matrix instruction accumulates in accumulation registers."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not available")
+    asm = tmp_path / "gemm.s"
+    subprocess.run([hipcc, *_FLAGS, "-o", str(asm), os.path.join(_ROOT, "ao_amd", "csrc", "int4wo_gemm.hip")], check=True,
+                   capture_output=True, timeout=900)
+    text = asm.read_text()
+    kernels = list(re.finditer(r"^(_ZN2ao22int4wo_gemm_lds_kernelILi(\d+)ELi([12])EEEvNS_10LinearArgsEiii): ; @.*?\n(.*?)s_endpgm(.*?)\.end_amdhsa_kernel",
+                               text, re.S | re.M))
+    assert len(kernels) == 8
+    for m in kernels:
+        name, nt, body, meta = m.group(1), int(m.group(3)), m.group(4), m.group(5)
+        lines = [l.strip() for l in body.splitlines()]
+        lines = [l for l in lines if l and not l.startswith(";") and not (l.startswith(".") and not l.startswith(".LBB"))]
+        labels = {re.match(r"(\.LBB\d+_\d+):", l).group(1): i for i, l in enumerate(lines) if re.match(r"\.LBB\d+_\d+:", l)}
+        back = {}
+        for i, l in enumerate(lines):
+            b = re.match(r"s_c?branch\w* (\.LBB\d+_\d+)", l)
+            if b and labels.get(b.group(1), i) < i:
+                back[i] = labels[b.group(1)]
+        assert len(back) == 1, (name, back)           # the K loop is the only loop
+        (loop_end, loop_head), = back.items()
+        loads = [i for i, l in enumerate(lines) if re.match(r"global_load_dword(x4)? v", l)]
+        assert sum(1 for i in loads if loop_head < i < loop_end) == 2 * nt * 2, name   # chunk + qparams per block, two steps
+        assert sum(1 for l in lines[loop_head:loop_end] if l.startswith("global_load_lds_dwordx4")) == 16, name
+        for i in loads:
+            dest = _regs(lines[i].split(",")[0])
+            j, jumped = i + 1, False
+            while j < len(lines) and lines[j] != "s_waitcnt vmcnt(0)":
+                touched = not lines[j].startswith((".LBB", "s_", "global_load")) and _regs(lines[j]) & dest
+                assert not touched, (name, lines[i], lines[j])
+                if j == loop_end and not jumped:
+                    j, jumped = loop_head, True
+                    continue
+                j += 1
+            assert j < len(lines), (name, lines[i])
+        # values the epilogue needs may be parked in scratch around the loop, never inside it
+        assert not [l for l in lines[loop_head:loop_end] if l.startswith("scratch_")], name
+        assert len(re.findall(r"v_mfma_f32_32x32x16_bf16 a\[", body)) >= 64 * nt, name
