@@ -124,13 +124,14 @@ struct TileBuf {
     uint4 x[4];   // activations for the same 32 k (zero for rows >= M)
 };
 
-// Weight-stream loads of the X_LDS path are issued from inline asm and waited for with explicit vmcnt counts.
-// The compiler cannot keep a precise count across the conditional loads of the register ring and falls back to
-// vmcnt(0), i.e. it would drain every prefetch before each tile.  The wait block takes the loaded registers as
-// in/out operands, so no consumer of them can be scheduled above the wait.
-// Wait until at most `younger_tiles` tiles' worth of loads are outstanding (loads return in order, so the
-// tile requested before them has arrived).  The block has no register operands: every consumer of loaded
-// registers is itself an asm volatile block (make_group_asm, first_half), and volatile blocks stay in order.
+// Weight-stream loads of the X_LDS path are issued from inline asm and waited for with explicit vmcnt counts
+// (the compiler cannot keep a precise count across the conditional loads of the register ring and would fall back
+// to vmcnt(0), draining every prefetch before each tile).
+// wait_tiles: wait until at most `younger_tiles` tiles' worth of loads are outstanding (loads return in order, so
+// the tile requested before them has arrived).  The wait has NO register operands: a tied in/out operand made the
+// compiler copy the register that is still being filled into the operand's register before the wait.  What keeps
+// consumers behind the wait instead: every consumer of loaded registers is itself an asm volatile block
+// (make_group_asm, first_half), and volatile blocks keep their program order.
 template <int LPT>
 __device__ __forceinline__ void wait_tiles(int younger_tiles) {
     if (younger_tiles >= 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LPT) : "memory");
@@ -472,6 +473,10 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     // count below is a constant; later waits only ever wait for more than they need because of it
 #pragma unroll
     for (int j = 0; j < D - 1; ++j) load_tile(buf[j], (nt > 0 ? kb0 : 0) + (j < nt ? j : (nt > 0 ? nt - 1 : 0)) * WAVES);
+    // Unlike wait_tiles, this one wait names the activation registers as tied operands, which is what orders their
+    // compiler-generated consumers (the staging code below) behind it.  A tied operand is only safe because the loads
+    // and the wait sit in the same straight-line code, where the register allocator has no reason to move the values
+    // in between (behind a branch it copied them: see above); the ISA lint of the staged kernels checks that it did not.
     asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(xv0), "+v"(xv1), "+v"(nv0), "+v"(nv1) : [n] "n"((D - 1) * LPT) : "memory");
     {
         __shared__ float norm_part[WAVES];

@@ -250,40 +250,61 @@ def cpu_baseline_leg(config, group=64, min_seconds=10.0):
 
 
 def _torch_cpu_leg(config, group, shapes, layer_params, head_params, min_seconds=5.0):
-    """The fastest CPU execution of the same linears this image offers, beside the scalar port: torch's own CPU kernel
-    for the op the reference dispatches to (aten._weight_int4pack_mm; its CPU build is _weight_int4pack_mm_for_cpu in
-    this torch), bf16 activations, every thread torch is configured with.  Same (q - 8) * scale + zero weights."""
+    """The same linears on the host with torch's own CPU kernels and every thread torch is configured with, beside the
+    scalar port.  `value`: the reference's CPU route for a quantized weight, op by op in bf16 as its tensor subclass
+    does it (dequantize_affine: (q - 8) * scale, + zero, then F.linear; torchao/dtypes/affine_quantized_tensor.py:
+    dequantize() fallback of _quantized_linear_op).  `aten_int4pack_mm`: the fused CPU kernel of the operator the
+    reference dispatches to on a GPU (aten._weight_int4pack_mm; its CPU build is _weight_int4pack_mm_for_cpu here),
+    the fastest CPU execution of these linears this image offers."""
     import torch
+    import torch.nn.functional as F
 
-    if not hasattr(torch.ops.aten, "_weight_int4pack_mm_for_cpu"):
-        return None
     gen = torch.Generator().manual_seed(1234)
     prepared = []
     for N, K in shapes:
         q = torch.randint(0, 16, (N, K), dtype=torch.int32, generator=gen)
-        packed = torch.ops.aten._convert_weight_to_int4pack_for_cpu(q, 2)
-        sz = torch.stack([torch.rand(K // group, N, generator=gen) * 0.01 + 1e-3,
-                          torch.randn(K // group, N, generator=gen) * 0.01], dim=-1).bfloat16().contiguous()
-        prepared.append((torch.randn(1, K, generator=gen).bfloat16(), packed, sz))
-    for x, packed, sz in prepared:  # warm-up
-        torch.ops.aten._weight_int4pack_mm_for_cpu(x, packed, group, sz)
-    t_layer, reps = 0.0, 0
-    while t_layer < min_seconds and reps < 2000:
-        t0 = time.perf_counter()
-        for x, packed, sz in prepared:
-            torch.ops.aten._weight_int4pack_mm_for_cpu(x, packed, group, sz)
-        t_layer += time.perf_counter() - t0
-        reps += 1
-    per_layer = t_layer / reps
-    per_token = per_layer * config.n_layer + per_layer * head_params / layer_params
-    return {
-        "value": round(1.0 / per_token, 3),
+        scale = (torch.rand(N, K // group, generator=gen) * 0.01 + 1e-3).bfloat16()
+        zero = (torch.randn(N, K // group, generator=gen) * 0.01).bfloat16()
+        prepared.append((torch.randn(1, K, generator=gen).bfloat16(), q, scale, zero))
+
+    def eager_layer():
+        for x, q, scale, zero in prepared:
+            N, K = q.shape
+            w = ((q.view(N, K // group, group) - 8).to(torch.bfloat16) * scale.unsqueeze(-1) + zero.unsqueeze(-1)).view(N, K)
+            F.linear(x, w)
+
+    def timed(fn, max_reps):
+        fn()
+        total, reps = 0.0, 0
+        while total < min_seconds and reps < max_reps:
+            t0 = time.perf_counter()
+            fn()
+            total += time.perf_counter() - t0
+            reps += 1
+        return total / reps, reps
+
+    scale_up = config.n_layer + head_params / layer_params
+    per_layer, reps = timed(eager_layer, 50)
+    out = {
+        "value": round(1.0 / (per_layer * scale_up), 4),
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
-        "kind": "torch aten._weight_int4pack_mm_for_cpu (bf16, M=1)",
-        "sample": (f"one transformer layer's five linears, {reps} repetitions, {per_layer * 1e3:.2f} ms per layer; scaled "
+        "kind": "torch eager dequantize (q - 8) * scale + zero in bf16, then F.linear (M=1)",
+        "sample": (f"one transformer layer's five linears, {reps} repetitions, {per_layer * 1e3:.1f} ms per layer; scaled "
                    f"to {config.n_layer} layers + vocabulary head; linears only, as for the port"),
     }
+    if hasattr(torch.ops.aten, "_weight_int4pack_mm_for_cpu"):
+        packed = [(x, torch.ops.aten._convert_weight_to_int4pack_for_cpu(q, 2),
+                   torch.stack([scale.t(), zero.t()], dim=-1).contiguous()) for x, q, scale, zero in prepared]
+
+        def fused_layer():
+            for x, p, sz in packed:
+                torch.ops.aten._weight_int4pack_mm_for_cpu(x, p, group, sz)
+
+        per_layer_f, reps_f = timed(fused_layer, 2000)
+        out["aten_int4pack_mm"] = {"value": round(1.0 / (per_layer_f * scale_up), 3), "unit": "tokens/s",
+                                   "sample": f"{reps_f} repetitions, {per_layer_f * 1e3:.2f} ms per layer"}
+    return out
 
 
 MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 MFMA, published
