@@ -73,5 +73,34 @@ def build(verbose: bool = False, obj_dir: str = None, only_stale: bool = False) 
     return LIB_PATH
 
 
+TORCH_BINDING_PATH = os.path.join(LIB_DIR, "libao_amd_torch.so")
+
+
+def build_torch_binding(verbose: bool = False) -> str:
+    """Compiles csrc/torch_binding/*.cpp (the C++ torch.library registration a torchao maintainer would add) against
+    the installed libtorch and links it to libao_amd.so.  Host code only: hipcc is used as the C++ compiler so that the
+    HIP headers of ATen resolve, no device code is generated.  The Python package does not load the result (it
+    registers the same operators itself); tests load it in a process of its own."""
+    import torch
+
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    tdir = os.path.dirname(torch.__file__)
+    srcs = sorted(glob.glob(os.path.join(CSRC, "torch_binding", "*.cpp")))
+    tmp = TORCH_BINDING_PATH + ".tmp"
+    cmd = [hipcc, "-O2", "-std=c++17", "-fPIC", "-shared", "-w", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DHIPBLAS_V2",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-I", os.path.join(tdir, "include"), "-I", os.path.join(tdir, "include", "torch", "csrc", "api", "include"),
+           "-I", os.path.join(_HERE, "..", "include"), "-I", os.path.join(os.path.dirname(os.path.dirname(os.path.realpath(hipcc))), "include"),
+           "-x", "c++", *srcs, "-o", tmp,
+           "-L", os.path.join(tdir, "lib"), "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip",
+           "-L", LIB_DIR, "-lao_amd", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    os.replace(tmp, TORCH_BINDING_PATH)
+    return TORCH_BINDING_PATH
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_torch_binding(verbose=True))

@@ -258,3 +258,21 @@ def test_decode_loop_refuses_positions_past_the_kv_cache():
         generate(model, torch.zeros(10, dtype=torch.int), 10)
     with pytest.raises(ValueError, match="interactive"):
         generate(model, torch.zeros(300, dtype=torch.int), 100, interactive=True)
+
+
+def test_torchao_alias_package_resolves_to_this_library():
+    """`import torchao` from the repository root gives the reference's import paths for this path (torchao/__init__.py:
+    31-41): the modules are the ao_amd modules themselves."""
+    import ao_amd
+    import torchao
+    from torchao.dtypes import AffineQuantizedTensor
+    from torchao.prototype.quant_llm import QuantLlmLinearWeight  # noqa: F401
+    from torchao.quantization import int4_weight_only, quantize_
+    from torchao.quantization.quant_api import quantize_ as quantize_again
+
+    assert torchao.quantization is ao_amd.quantization and quantize_ is quantize_again is ao_amd.quantize_
+    assert int4_weight_only is ao_amd.int4_weight_only and AffineQuantizedTensor is ao_amd.dtypes.AffineQuantizedTensor
+    assert torchao.ops.quant_llm_linear is ao_amd.ops.quant_llm_linear
+    import torchao._models.llama.model as m
+
+    assert m is ao_amd._models.llama.model
