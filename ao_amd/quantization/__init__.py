@@ -16,6 +16,7 @@ from .quant_primitives import (
     dequantize_affine,
     quantize_affine,
 )
+from .subclass import Int4WeightOnlyQuantizedLinearWeight
 from .unified import Quantizer, TwoStepQuantizer
 from .utils import (
     compute_error,

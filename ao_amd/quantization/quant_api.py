@@ -112,11 +112,21 @@ def fp6_llm_weight_only():
 
 
 def change_linear_weights_to_int4_woqtensors(model, groupsize=128, inner_k_tiles=8, filter_fn=None):
-    """Legacy entry point (reference quant_api.py:119-141, which refuses to run on PyTorch >= 2.4): every linear weight
-    becomes a groupwise int4 weight-only tensor, in place.  The legacy `Int4WeightOnlyQuantizedLinearWeight` subclass
-    (subclass.py:394-601) computes the same codes and qparams through the same helpers; here the call maps to
-    `quantize_(model, int4_weight_only(groupsize, inner_k_tiles))`."""
-    quantize_(model, int4_weight_only(group_size=groupsize, inner_k_tiles=inner_k_tiles), filter_fn)
+    """Legacy entry point (reference quant_api.py:119-141): every linear weight becomes the legacy
+    `Int4WeightOnlyQuantizedLinearWeight` tensor subclass (subclass.py:394-601), in place.  The reference refuses
+    to run it on PyTorch >= 2.4 in favour of `quantize_`; it works here on any version."""
+    from .subclass import Int4WeightOnlyQuantizedLinearWeight
+
+    def is_plain_linear(mod, *args):
+        return _is_linear(mod, *args) and not isinstance(mod.weight, Int4WeightOnlyQuantizedLinearWeight)
+
+    def swap(lin):
+        lin.weight = torch.nn.Parameter(
+            Int4WeightOnlyQuantizedLinearWeight.from_float(lin.weight, groupsize=groupsize, inner_k_tiles=inner_k_tiles),
+            requires_grad=False)
+        return lin
+
+    _replace_with_custom_fn_if_matches_filter(model, swap, is_plain_linear if filter_fn is None else filter_fn)
 
 
 def change_linear_weights_to_int8_woqtensors(model, filter_fn=None, **kwargs):

@@ -251,3 +251,87 @@ def test_device_moves_follow_the_reference():
     again = lin.weight.to(_dev())
     same = bool(torch.equal(again.dequantize(), lin.weight.dequantize()))
     assert again.is_cuda and same
+
+
+# ---------------------------------------------------------------- the legacy subclass (reference subclass.py:394-601)
+def _sqnr(a, b):
+    return float(20 * torch.log10(a.float().norm() / (a.float() - b.float()).norm()))
+
+
+@pytest.mark.parametrize("groupsize,inner_k_tiles", [(128, 8), (256, 4), (64, 2), (32, 8)])
+@pytest.mark.parametrize("shape", [(16, 1024, 16), (1, 1024, 8), (256, 1024, 13), (5, 200, 48)])
+def test_legacy_int4_subclass_matches_the_oracle(oracle, shape, groupsize, inner_k_tiles):
+    """Int4WeightOnlyQuantizedLinearWeight.from_float: the reference's own checks (dequantize and its transpose above
+    15 dB SQNR, linear close to the float linear: test_integration.py:590-660, shapes of :621-657) and, beyond them,
+    the bits: scales_and_zeros and the dequantized weight equal the oracle's tinygemm quantizer, the linear is within
+    1e-3 of the oracle linear on those weights."""
+    from ao_amd.quantization import Int4WeightOnlyQuantizedLinearWeight
+
+    m, k, n = shape
+    print(f"case legacy subclass m={m} k={k} n={n} g={groupsize} ikt={inner_k_tiles}", flush=True)
+    torch.manual_seed(n + k + groupsize)
+    lin = nn.Linear(k, n).bfloat16()   # nn.Linear's own (uniform) init, as in the reference's test
+    w, bias = lin.weight.detach().clone(), lin.bias.detach().clone()
+    lin = lin.to(_dev())
+    lin.weight = nn.Parameter(Int4WeightOnlyQuantizedLinearWeight.from_float(lin.weight, groupsize, inner_k_tiles), requires_grad=False)
+    wq = lin.weight
+    assert isinstance(wq, Int4WeightOnlyQuantizedLinearWeight) and wq.shape == (n, k) and wq.dtype is torch.bfloat16
+    codes, scale, zero, dq = _oracle(oracle, w, groupsize)
+    kg = (k + groupsize - 1) // groupsize * groupsize
+    assert wq.scales_and_zeros.shape == (kg // groupsize, n, 2)
+    qp = wq.q_params()
+    # [N, K/g, 1] each, as the reference's unpack_tinygemm_scales_and_zeros returns them
+    same_q = (np.array_equal(bits16(qp["q_scales"].reshape(n, -1).contiguous()), scale)
+              and np.array_equal(bits16(qp["q_zero_points"].reshape(n, -1).contiguous()), zero))
+    assert same_q
+    d = wq.dequantize()
+    same_dq = np.array_equal(bits16(d), dq[:, :k])
+    assert same_dq and d.shape == (n, k)
+    same_t = bool(torch.equal(wq.t().dequantize(), d.t()))
+    assert same_t and wq.t().shape == (k, n)
+    assert _sqnr(w.to(_dev()), d) > 15 and _sqnr(w.t().to(_dev()), wq.t().dequantize()) > 15
+    x = make_act(m, k, seed=m)
+    with torch.no_grad():
+        y = lin(x.to(_dev()))
+        y_mm = torch.addmm(bias.to(_dev()), x.to(_dev()), wq.t())
+    y_ref = _ref_linear(oracle, x, dq, k, bias)
+    err = rel_l2(y.float().cpu().numpy(), oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(y_ref.astype(np.float32))))
+    same_mm = bool(torch.equal(y_mm, y))
+    assert err <= TOL and same_mm, (err, same_mm)
+
+
+def test_legacy_entry_point_swaps_every_linear_and_round_trips_through_a_state_dict():
+    """change_linear_weights_to_int4_woqtensors (reference quant_api.py:119-141) + the save / load flow of the subclass
+    tests (test_integration.py:945-1027): state_dict -> quantized meta-device skeleton -> load_state_dict(assign=True)"""
+    import ao_amd
+    from ao_amd.quantization import Int4WeightOnlyQuantizedLinearWeight, change_linear_weights_to_int4_woqtensors
+
+    def make(seed):
+        torch.manual_seed(seed)
+        return nn.Sequential(nn.Linear(256, 512), nn.ReLU(), nn.Linear(512, 64)).bfloat16()
+
+    model = make(5).to(_dev())
+    change_linear_weights_to_int4_woqtensors(model, groupsize=64)
+    assert all(isinstance(m.weight, Int4WeightOnlyQuantizedLinearWeight) for m in model if isinstance(m, nn.Linear))
+    x = make_act(7, 256, seed=1).to(_dev())
+    with torch.no_grad():
+        ref = model(x)
+    buf = io.BytesIO()
+    torch.save(model.state_dict(), buf)
+    buf.seek(0)
+    state = torch.load(buf, weights_only=False)   # a file this test wrote itself
+    skeleton = make(99).to(_dev())   # other weights: the loaded state must replace them
+    change_linear_weights_to_int4_woqtensors(skeleton, groupsize=64)
+    with torch.no_grad():
+        differs = not bool(torch.equal(skeleton(x), ref))
+    skeleton.load_state_dict(state, assign=True)
+    with torch.no_grad():
+        out = skeleton(x)
+    same = bool(torch.equal(out, ref))
+    assert differs and same
+    # already-converted weights are left alone by a second call
+    change_linear_weights_to_int4_woqtensors(model, groupsize=64)
+    with torch.no_grad():
+        again = model(x)
+    assert bool(torch.equal(again, ref))
+    del ao_amd
