@@ -1,12 +1,19 @@
 """Mixed matmul over HQQ-format int4 weights (reference torchao/prototype/hqq/mixed_mm.py).
 
-The reference fuses the dequantization into a Triton GEMM.  Here the weight is dequantized by a HIP kernel into a
-matrix of the activation dtype, op by op as the reference's kernel does ((q - zero) * scale, kernels.py:318-358), and
-multiplied by the vendor GEMM; forward and transposed products share the one dequantized matrix.
+The reference fuses the dequantization into a Triton GEMM.  Here the forward product of up to 8 activation rows (the
+decode case the kernel exists for; `ops.hqq_mixed_mm_small` takes up to 16) runs a fused HIP kernel that streams the packed codes once; more rows, and the
+transposed product, dequantize the weight with a HIP kernel into a matrix of the activation dtype, op by op as the
+reference's kernel does ((q - zero) * scale, kernels.py:318-358), and call the vendor GEMM on it.
 """
 import torch
 
 from ... import ops
+
+
+# activation rows up to which the forward product runs the fused kernel (measured on MI355X, kernels only: 4096 x 4096 at
+# 1-4 rows 11 + 4 us against 12 + 16 us for dequantize + library GEMM, 8 rows 16 + 4 against 12 + 16; at 16 rows the
+# fused kernel's per-row FMAs make it the slower of the two on wide weights)
+FUSED_MAX_ROWS = 8
 
 
 def pack_2xint4(t):
@@ -36,6 +43,8 @@ def mixed_mm(a, b, scales, zeros, group_size, transposed=False, acc_dtype=None, 
         assert a.shape[1] == b.shape[0] * 2, "incompatible dimensions"
     else:
         assert a.shape[1] == b.shape[1], "transpose requires (M x N) x (K x N), where reduction dim is N"
+    if not transposed and 1 <= a.shape[0] <= FUSED_MAX_ROWS and b.shape[1] % 4 == 0:
+        return ops.hqq_mixed_mm_small(a, b, scales, zeros, group_size)
     w = ops.hqq_dequantize(b, scales, zeros, group_size)  # [K, N]
     return torch.matmul(a, w.t() if transposed else w)
 

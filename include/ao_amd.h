@@ -179,6 +179,18 @@ int ao_amd_int4wo_swiglu_interleaved(const void* x_bf16, int64_t M, int64_t K, i
 int ao_amd_hqq_dequantize(const void* packed_2xint4, int is_signed, int64_t K, int64_t N, const void* scales,
                           const void* zeros, int64_t group_size, int dtype, void* out, void* stream);
 
+/* The forward product of the same Triton kernel for 1 to 16 activation rows, fused (torchao/prototype/hqq/kernels.py:
+ * 162-388, triton_mixed_mm(a, b, scales, zeros, group_size), mixed_mm.py:38-176): y[M,N] = a[M,K] @ W[K,N] with W as
+ * above (every weight rounded twice to `dtype` exactly as ao_amd_hqq_dequantize rounds it), fp32 accumulation, y in
+ * `dtype`, row stride N.  a: `dtype` [M, K] with row stride lda (even, rows 4-byte aligned); N a multiple of 4, packed
+ * codes 4-byte and scales / zeros 8-byte aligned.  K is cut into slices whose fp32 partial sums go through `workspace`
+ * (ao_amd_hqq_mixed_mm_workspace gives its size; caller-owned, device memory).  More rows, or the transposed product,
+ * take ao_amd_hqq_dequantize and a library GEMM. */
+int ao_amd_hqq_mixed_mm_workspace(int64_t M, int64_t K, int64_t N, int64_t* bytes);
+int ao_amd_hqq_mixed_mm(const void* a, int64_t M, int64_t K, int64_t lda, const void* packed_2xint4, int is_signed, int64_t N,
+                        const void* scales, const void* zeros, int64_t group_size, int dtype, void* workspace,
+                        int64_t workspace_bytes, void* y, void* stream);
+
 /* ---------------------------------------------------------------- int8 weight-only linear
  * y[M,N] = bf16( bf16(x[M,K] @ bf16(w)^T) * scale[N] ) (+ bias, rounded to bf16 again): the per-channel int8
  * weight-only branch of _quantized_linear_op, torchao/dtypes/affine_quantized_tensor.py:641-665

@@ -140,3 +140,64 @@ def test_converter_module_runs_hqq_weights_on_the_int4_kernels(oracle, g):
 
     with pytest.raises(ImportError, match="hqq"):
         HQQLinearTorchWeightOnlyInt4(torch.nn.Linear(K, N, bias=False), cfg, initialize=True)
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,g", [(1, 4096, 4096, 64), (3, 1000, 512, 128), (8, 11008, 4096, 64), (16, 256, 2048, 32), (5, 64, 128, 128)])
+def test_fused_small_m_product_matches_the_dequantized_matmul(oracle, M, N, K, g, dtype, signed):
+    """The fused forward kernel (1-16 rows): within 1e-3 relative L2 of the fp32-accumulated product with the oracle's
+    dequantized weight (rounded to the output dtype), and exactly the dequantized weight on one-hot rows: the kernel
+    rounds every weight as ao_amd_hqq_dequantize does.  N = 1000 and 64 leave lanes and whole waves without columns."""
+    from ao_amd import ops
+    from ao_amd.prototype.hqq import mixed_mm, pack_2xint4
+
+    print(f"case hqq fused M={M} N={N} K={K} g={g} {dtype} signed={signed}", flush=True)
+    dev = _dev()
+    W_q, scale, zero = _hqq_like(N, K, g, dtype, seed=M + N + g, signed=signed)
+    packed = pack_2xint4(W_q.T.contiguous()).to(dev)
+    s, z = scale.T.contiguous().to(dev), zero.T.contiguous().to(dev)
+    code = oracle.BF16 if dtype is torch.bfloat16 else oracle.F16
+    w_ref = oracle.hqq_dequantize(packed.cpu().numpy(), bits16(s.cpu()), bits16(z.cpu()), g, code)   # [K, N] bits
+    w_f32 = (oracle.bf16_bits_to_f32(w_ref) if dtype is torch.bfloat16 else w_ref.view(np.float16).astype(np.float32))
+    x = torch.randn(M, K, dtype=dtype, generator=torch.Generator().manual_seed(3)).to(dev)
+    y = ops.hqq_mixed_mm_small(x, packed, s, z, g)
+    assert y.shape == (M, N) and y.dtype is dtype
+    ref = x.float().cpu().numpy().astype(np.float64) @ w_f32.astype(np.float64)
+    ref_r = torch.from_numpy(ref).to(dtype).float().numpy()
+    err = rel_l2(y.float().cpu().numpy(), ref_r)
+    assert err <= 1e-3, err
+    # the module-level entry point takes the fused kernel up to FUSED_MAX_ROWS rows, the two-pass route beyond
+    from ao_amd.prototype.hqq.mixed_mm import FUSED_MAX_ROWS
+    if N % 16 == 0 or M <= FUSED_MAX_ROWS:
+        y2 = mixed_mm(x, packed, s, z, g)
+        if M <= FUSED_MAX_ROWS:
+            same = bool(torch.equal(y, y2))
+            assert same
+        else:
+            err2 = rel_l2(y2.float().cpu().numpy(), ref_r)
+            assert err2 <= 2e-3, err2
+    # one-hot rows read single weights back, bit for bit
+    ks = torch.randint(0, K, (M,), generator=torch.Generator().manual_seed(4))
+    ks[0], ks[-1] = 0, K - 1
+    xh = torch.zeros(M, K, dtype=dtype)
+    xh[torch.arange(M), ks] = 1.0
+    yh = ops.hqq_mixed_mm_small(xh.to(dev), packed, s, z, g)
+    want = torch.from_numpy(w_ref[ks.numpy()].astype(np.int16)).view(dtype)
+    exact = bool(torch.equal(yh.cpu(), want))
+    assert exact
+
+
+def test_fused_product_limits():
+    from ao_amd import ops
+    from ao_amd.prototype.hqq import mixed_mm, pack_2xint4
+
+    dev = _dev()
+    W_q, scale, zero = _hqq_like(64, 128, 64, torch.float16, seed=1)
+    b = pack_2xint4(W_q.T.contiguous()).to(dev)
+    s, z = scale.T.contiguous().to(dev), zero.T.contiguous().to(dev)
+    with pytest.raises(RuntimeError, match="1 to 16 rows"):
+        ops.hqq_mixed_mm_small(torch.randn(17, 128, dtype=torch.float16, device=dev), b, s, z, 64)
+    # 17 rows go the two-pass way through the module-level entry point
+    y = mixed_mm(torch.randn(17, 128, dtype=torch.float16, device=dev), b, s, z, 64)
+    assert y.shape == (17, 64)
