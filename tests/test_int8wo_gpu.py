@@ -215,22 +215,26 @@ def test_two_weight_swiglu_matches_the_gated_chain(M, N, K, with_norm):
 
 
 def test_legacy_entry_points_map_to_quantize():
-    """change_linear_weights_to_int{4,8}_woqtensors (reference quant_api.py:103-141) give the same weights as
-    quantize_ with the matching constructor."""
+    """change_linear_weights_to_int{4,8}_woqtensors (reference quant_api.py:103-141) compute what quantize_ with the
+    matching constructor computes; the int4 one installs the legacy subclass (reference subclass.py:394), the int8 one
+    the same tensor class as quantize_."""
     import copy
 
     from ao_amd import int4_weight_only, int8_weight_only, quantize_
-    from ao_amd.quantization import change_linear_weights_to_int4_woqtensors, change_linear_weights_to_int8_woqtensors
+    from ao_amd.quantization import (Int4WeightOnlyQuantizedLinearWeight, change_linear_weights_to_int4_woqtensors,
+                                     change_linear_weights_to_int8_woqtensors)
 
     dev = _dev()
     torch.manual_seed(1)
     base = torch.nn.Sequential(torch.nn.Linear(256, 128, bias=False)).to(dev).bfloat16()
     x = torch.randn(3, 256, device=dev).bfloat16()
-    for legacy, modern in ((lambda m: change_linear_weights_to_int4_woqtensors(m, groupsize=64),
-                            lambda m: quantize_(m, int4_weight_only(group_size=64))),
-                           (change_linear_weights_to_int8_woqtensors, lambda m: quantize_(m, int8_weight_only()))):
+    for legacy, modern, cls in ((lambda m: change_linear_weights_to_int4_woqtensors(m, groupsize=64),
+                                 lambda m: quantize_(m, int4_weight_only(group_size=64)), Int4WeightOnlyQuantizedLinearWeight),
+                                (change_linear_weights_to_int8_woqtensors, lambda m: quantize_(m, int8_weight_only()), None)):
         a, b = copy.deepcopy(base), copy.deepcopy(base)
         legacy(a)
         modern(b)
+        same_class = type(a[0].weight) is (type(b[0].weight) if cls is None else cls)
         with torch.no_grad():
-            assert type(a[0].weight) is type(b[0].weight) and torch.equal(a(x), b(x))
+            same_output = torch.equal(a(x), b(x))
+        assert same_class and same_output
