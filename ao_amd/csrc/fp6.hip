@@ -161,12 +161,15 @@ __device__ __forceinline__ float fp6_scale_of_amax(float amax, float max_normal)
     return __fdiv_rn(amax < 1e-12f ? 1e-12f : amax, max_normal);
 }
 
+// the fp16 scale as torch's conversion leaves it: any NaN becomes the default one
+__device__ __forceinline__ uint16_t fp6_scale_bits(float s) { return s != s ? (uint16_t)0x7e00 : f32_to_f16_bits(s); }
+
 __global__ __launch_bounds__(256) void fp6_scale_finalize_kernel(uint16_t* __restrict__ scale, int64_t N, int w_dtype,
                                                                   float max_normal) {
     const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (row >= N) return;
     const float amax = w_dtype == AO_BF16 ? bf16_bits_to_f32(scale[row]) : f16_bits_to_f32(scale[row]);
-    scale[row] = f32_to_f16_bits(fp6_scale_of_amax(amax, max_normal));
+    scale[row] = fp6_scale_bits(fp6_scale_of_amax(amax, max_normal));
 }
 
 template <bool AMAX_GIVEN, int ebits, int mbits>  // the format as constants: the cast's masks and bounds fold away
@@ -204,7 +207,7 @@ __global__ __launch_bounds__(256) void fp6_quantize_pack_kernel(const void* __re
             float s = has_nan ? NAN : (amax < 1e-12f ? 1e-12f : amax);
             s = __fdiv_rn(s, max_normal);
             scale_s[rr] = s;
-            scale_out[row] = f32_to_f16_bits(s);
+            scale_out[row] = fp6_scale_bits(s);
         }
     }
     __syncthreads();
@@ -253,6 +256,246 @@ __global__ __launch_bounds__(256) void fp6_quantize_pack_kernel(const void* __re
             }
         }
         __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------- quantize + pack, 16-bit inputs, FP6: one pass
+// A row group is (64-row block a, half i1, DQ consecutive d): the 4 DQ rows 64 a + 32 i1 + 8 j + d (j = 0..3) over all
+// of K; a workgroup takes one row group after the other.  Thread t owns d = d0 + t % DQ and the 16-column slices
+// e = t / DQ + (THREADS / DQ) i; it loads its 4 x 16 values per slice once (two 16-byte loads a row), keeps them in
+// registers over the row maximum (a workgroup reduction), quantizes them and stores the slice's 16 bytes of the 2-bit
+// plane and 2 x 16 bytes of the 4-bit plane: exactly the bytes the TC layout holds for (a, e, i1, d); DQ neighbouring
+// lanes write 16 DQ consecutive bytes.  The weight is read from memory once, nothing goes through LDS but the row
+// maxima.  (Measured, 14336 x 4096: with one d per workgroup the 16-byte stores, 256 bytes apart, take 24 of 58 us;
+// with two, 32-byte pieces, the kernel runs in 36 us.)
+//
+// The quotient w / scale, correctly rounded as torch's division: with r = RN(1 / s), q0 = RN(w r) and two rounds of
+// e = fma(-q, s, w), q = fma(e, r, q) end at RN(w / s) (Markstein; after the first round q is a faithful rounding of
+// the quotient, which the theorem needs).  The residuals stay exact while s is far from the ends of the fp32 range;
+// rows whose scale is outside [1e-20, 1e20] or not a number take the division instruction sequence and the bitwise cast.
+//
+// The cast: e3m2 is bf8 (e5m2) and e2m3 is fp8 (e4m3) with fewer exponent values, and after scaling by 2^-12 (2^-6)
+// their subnormal ranges coincide too, so v_cvt_pk_bf8_f32 (fp8) of the scaled quotient is the FP6 code with three
+// zero bits in the middle: byte = sign << 7 | code & 31 (checked against the bitwise cast over every fp32 value up to
+// the largest normal).  The scaling is folded into s (a power of two: every rounding stays where it was).  The
+// conversion drops the sign of a zero result's quotient only if the quotient was computed unsigned, so the sign bits
+// are taken from the inputs.  Bytes of 4 consecutive columns sit in one register; the planes are assembled 4 bytes at
+// a time with masks and byte permutes.
+//
+// The 16 row groups of a 64-row block write interleaved 16-byte pieces of the same lines, so they go to workgroups of one
+// XCD (ids 8 apart share an XCD) that run at the same time: that XCD's L2 merges the pieces before they go to memory.
+__device__ __forceinline__ float fp6_div_by_row(float x, float s, float r) {
+    float q = __fmul_rn(x, r);
+    float e = __fmaf_rn(-q, s, x);
+    q = __fmaf_rn(e, r, q);
+    e = __fmaf_rn(-q, s, x);
+    return __fmaf_rn(e, r, q);
+}
+
+// the bytes of four values the long way: division instruction sequence and bitwise cast (rows whose scale is out of
+// the shortcut's range); a real call, so that the rare path does not bloat the loop
+__device__ __attribute__((noinline)) uint32_t fp6_bytes_by_division(float x0, float x1, float x2, float x3, float s,
+                                                                    int ebits, int mbits) {
+    const float x[4] = {x0, x1, x2, x3};
+    uint32_t dw = 0u;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const uint32_t code = f32_to_fpx(__fdiv_rn(x[v], s), ebits, mbits);
+        dw |= ((code & 31u) | ((code & 32u) << 2)) << (8 * v);
+    }
+    return dw;
+}
+
+// One row group's share of a thread: TASKS slices of 4 rows x 16 values, as loaded
+template <int TASKS>
+struct Fp6RowsRaw {
+    u32x4v_t v[TASKS][4][2];
+};
+
+template <bool BF16IN, bool E3M2, int TASKS, int THREADS, int DQ>
+__global__ __launch_bounds__(THREADS) void fp6_quantize_pack_rows_kernel(const uint16_t* __restrict__ w, int64_t N, int64_t K,
+                                                                          uint8_t* __restrict__ out,
+                                                                          uint16_t* __restrict__ scale_out) {
+    constexpr int ebits = E3M2 ? 3 : 2, mbits = E3M2 ? 2 : 3;
+    constexpr int SHIFT = E3M2 ? 12 : 6;   // min normal of bf8 / fp8 over min normal of the FP6 format
+    constexpr int WAVES = THREADS / 64;
+    constexpr int SUBS = 16 / DQ, ESTEP = THREADS / DQ;   // row groups per 64-row block, slices per pass of the workgroup
+    __shared__ uint32_t red[2][WAVES][DQ][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int dq = tid % DQ, el = tid / DQ;
+    const int64_t G = N >> 6, E = K >> 4;
+    // Row groups in the order an XCD takes them: XCD x (workgroup id % 8) owns the 64-row blocks a = x, x + 8, ...,
+    // 16 groups each; its workgroups walk that list with a stride of their number, so the ones that run together are
+    // in the same block.
+    const int xcd = blockIdx.x & 7;
+    const int64_t stride = gridDim.x >> 3, first = blockIdx.x >> 3;
+    const int64_t total = ((G - xcd + 7) >> 3) * SUBS;   // groups of this XCD
+    const int exp_bias = (1 << (ebits - 1)) - 1;
+    const float max_normal = __uint_as_float((uint32_t)(((1 << ebits) - 1) - exp_bias + 127) << 23) *
+                             ((float)((1 << (mbits + 1)) - 1) / (float)(1 << mbits));
+    uint8_t* const p2 = out;
+    uint8_t* const p4 = out + N * K / 4;
+
+    // group l of the list: block a = 8 (l / SUBS) + xcd, half i1 and d = DQ (l % (SUBS / 2)) + dq
+    auto d_of = [&](int64_t l) { return (int)(l % (SUBS / 2)) * DQ + dq; };
+    auto row0_of = [&](int64_t l) { return ((l / SUBS) * 8 + xcd) * 64 + (int)((l % SUBS) / (SUBS / 2)) * 32 + d_of(l); };
+    auto load = [&](Fp6RowsRaw<TASKS>& raw, int64_t l) __attribute__((always_inline)) {
+        const int64_t row0 = row0_of(l);
+#pragma unroll
+        for (int i = 0; i < TASKS; ++i) {
+            // slices past the row repeat its last one (no effect on the maximum, never stored)
+            const int64_t e = el + ESTEP * i < E ? el + ESTEP * i : E - 1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const u32x4v_t* src = reinterpret_cast<const u32x4v_t*>(w + (row0 + 8 * j) * K + e * 16);
+                raw.v[i][j][0] = src[0];
+                raw.v[i][j][1] = src[1];
+            }
+        }
+    };
+    auto process = [&](const Fp6RowsRaw<TASKS>& raw, int64_t l, int parity) __attribute__((always_inline)) {
+        const int64_t a = (l / SUBS) * 8 + xcd, row0 = row0_of(l);
+        const int i1 = (int)((l % SUBS) / (SUBS / 2)), d = d_of(l);
+        // the rows' largest magnitude as a bit pattern (16-bit floats order like unsigned integers once the sign is
+        // masked; any NaN is above infinity)
+        uint32_t mx[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < TASKS; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+                        const uint32_t m = raw.v[i][j][h][c] & 0x7fff7fffu;
+                        const u16x2_t v = __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, m), __builtin_bit_cast(u16x2_t, mx[j]));
+                        mx[j] = __builtin_bit_cast(uint32_t, v);
+                    }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t m = mx[j] & 0xffffu;
+            const uint32_t hi = mx[j] >> 16;
+            m = m > hi ? m : hi;
+#pragma unroll
+            for (int o = 32; o >= DQ; o >>= 1) {   // over the lanes of the same row: lane % DQ
+                const uint32_t other = (uint32_t)__shfl_xor((int)m, o, 64);
+                m = m > other ? m : other;
+            }
+            if (lane < DQ) red[parity][wave][lane][j] = m;
+        }
+        // one barrier a group: the other half of `red` is not written again before every wave has passed this one.
+        // Not __syncthreads(): that also waits for the stores of the group before; the barrier only has to order
+        // the LDS writes above against the reads below.
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        float s[4], sq[4], rq[4];
+        bool fast[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t m = red[parity][0][dq][j];
+#pragma unroll
+            for (int v = 1; v < WAVES; ++v) m = m > red[parity][v][dq][j] ? m : red[parity][v][dq][j];
+            const float amax = BF16IN ? bf16_bits_to_f32((uint16_t)m) : f16_bits_to_f32((uint16_t)m);   // NaN if any was
+            s[j] = fp6_scale_of_amax(amax, max_normal);
+            fast[j] = s[j] >= 1e-20f && s[j] <= 1e20f;
+            sq[j] = s[j] * __uint_as_float((uint32_t)(127 + SHIFT) << 23);
+            rq[j] = __fdiv_rn(1.0f, sq[j]);
+            if (el == j) scale_out[row0 + 8 * j] = fp6_scale_bits(s[j]);
+        }
+#pragma unroll
+        for (int i = 0; i < TASKS; ++i) {
+            const int64_t e = el + ESTEP * i;
+            if (e >= E) break;
+            // D[j][c]: the bytes (sign << 7 | code & 31) of row j, columns 4 c .. 4 c + 3
+            uint32_t D[4][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t u0 = raw.v[i][j][c >> 1][(c & 1) * 2], u1 = raw.v[i][j][c >> 1][(c & 1) * 2 + 1];
+                    float x[4];
+                    if (BF16IN) {
+                        x[0] = __uint_as_float(u0 << 16); x[1] = __uint_as_float(u0 & 0xffff0000u);
+                        x[2] = __uint_as_float(u1 << 16); x[3] = __uint_as_float(u1 & 0xffff0000u);
+                    } else {
+                        x[0] = f16_bits_to_f32((uint16_t)(u0 & 0xffffu)); x[1] = f16_bits_to_f32((uint16_t)(u0 >> 16));
+                        x[2] = f16_bits_to_f32((uint16_t)(u1 & 0xffffu)); x[3] = f16_bits_to_f32((uint16_t)(u1 >> 16));
+                    }
+                    uint32_t dw;
+                    if (fast[j]) {   // the same for the whole workgroup
+                        float q[4];
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) q[v] = fp6_div_by_row(x[v], sq[j], rq[j]);
+                        dw = 0u;
+                        if (E3M2) {
+                            dw = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(q[0], q[1], (int)dw, false);
+                            dw = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(q[2], q[3], (int)dw, true);
+                        } else {
+                            dw = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], (int)dw, false);
+                            dw = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], (int)dw, true);
+                        }
+                        // signs from the inputs: the high bytes of the four 16-bit values
+                        const uint32_t sg = __builtin_amdgcn_perm(u1, u0, 0x07050301u);
+                        dw = (dw & 0x7f7f7f7fu) | (sg & 0x80808080u);
+                    } else {
+                        dw = fp6_bytes_by_division(x[0], x[1], x[2], x[3], s[j], ebits, mbits);
+                    }
+                    D[j][c] = dw;
+                }
+            }
+            // the 4-bit plane: byte (i2, g, p) = low 4 bits of row 16 i2 + 8 (1 - p) + d at columns g and 8 + g; g and
+            // p interleave, so rows j = 2 i2 + 1 (p = 0) and j = 2 i2 (p = 1) alternate bytewise
+            const int64_t tile = (a * E + e) * 2 + i1;
+#pragma unroll
+            for (int i2 = 0; i2 < 2; ++i2) {
+                uint32_t nib[2][2];   // [p][h]: 4 bytes, g = 4 h .. 4 h + 3
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int j = 2 * i2 + 1 - p;
+                        nib[p][h] = ((D[j][h] & 0x0f0f0f0fu) << 4) | (D[j][2 + h] & 0x0f0f0f0fu);
+                    }
+                u32x4v_t o;
+                o[0] = __builtin_amdgcn_perm(nib[1][0], nib[0][0], 0x05010400u);
+                o[1] = __builtin_amdgcn_perm(nib[1][0], nib[0][0], 0x07030602u);
+                o[2] = __builtin_amdgcn_perm(nib[1][1], nib[0][1], 0x05010400u);
+                o[3] = __builtin_amdgcn_perm(nib[1][1], nib[0][1], 0x07030602u);
+                *reinterpret_cast<u32x4v_t*>(p4 + ((tile * 2 + i2) * 8 + d) * 16) = o;
+            }
+            // the 2-bit plane: byte (g, p) = the two high code bits of rows 8 (1 - p) + d (i2 = 0) and + 16 (i2 = 1)
+            // at columns g and 8 + g, most significant first in the order (i2, f)
+            {
+                uint32_t top[4][4];   // code bits 5, 4 in place (from byte bits 7, 4)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) top[j][c] = ((D[j][c] & 0x80808080u) >> 2) | (D[j][c] & 0x10101010u);
+                uint32_t two[2][2];
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int ja = 1 - p, jb = 3 - p;
+                        two[p][h] = (top[ja][h] << 2) | top[ja][2 + h] | (top[jb][h] >> 2) | (top[jb][2 + h] >> 4);
+                    }
+                u32x4v_t o;
+                o[0] = __builtin_amdgcn_perm(two[1][0], two[0][0], 0x05010400u);
+                o[1] = __builtin_amdgcn_perm(two[1][0], two[0][0], 0x07030602u);
+                o[2] = __builtin_amdgcn_perm(two[1][1], two[0][1], 0x05010400u);
+                o[3] = __builtin_amdgcn_perm(two[1][1], two[0][1], 0x07030602u);
+                *reinterpret_cast<u32x4v_t*>(p2 + (tile * 8 + d) * 16) = o;
+            }
+        }
+    };
+
+    // One register set holds a group.  (A second set, loaded ahead while the first is worked on, measured slower: the
+    // registers it takes halve the waves on a CU, and the waves of other workgroups fill the load latency as well.)
+    int parity = 0;
+    for (int64_t l = first; l < total; l += stride, parity ^= 1) {
+        Fp6RowsRaw<TASKS> raw;
+        load(raw, l);
+        process(raw, l, parity);
     }
 }
 
@@ -883,6 +1126,44 @@ extern "C" int ao_amd_fp6_quantize_pack(const void* w, int w_dtype, int64_t N, i
                (long long)K);
     hipStream_t st = (hipStream_t)stream;
     const int64_t E = K / 16;
+    if ((w_dtype == AO_BF16 || w_dtype == AO_F16) && ebits + mbits == 5 && E <= 1024 && ((uintptr_t)w & 15) == 0 &&
+        N / 64 <= (1 << 20)) {
+        // FP6 from a 16-bit weight with rows of up to 16384 values: one pass, the rows held in registers; as many
+        // workgroups as run at once, each walking its share of the row groups
+        static const int cus = [] {
+            int dev = 0, n = 0;
+            if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+            return n;
+        }();
+        // rows of up to 4096 values: 8-row groups (32-byte pieces), 256 threads with two slices each, 3 workgroups a
+        // CU; up to 8192: the same with 512 threads, 2 a CU; up to 16384: 4-row groups, 512 threads, 2 a CU (the
+        // measured best of the shapes that fit the registers)
+        const int variant = E <= 256 ? 0 : (E <= 512 ? 1 : 2);
+        const int64_t groups = N / (variant == 2 ? 4 : 8);
+        int64_t wgs = (int64_t)cus * (variant == 0 ? 3 : 2);
+        if (wgs > groups) wgs = groups;
+        const dim3 grid((unsigned)((wgs + 7) / 8 * 8));
+#define AO_FP6_ROWS(BF, E3, T, TH, DQV)                                                                             \
+    hipLaunchKernelGGL((fp6_quantize_pack_rows_kernel<BF, E3, T, TH, DQV>), grid, dim3(TH), 0, st,                   \
+                       (const uint16_t*)w, N, K, (uint8_t*)out_tc, (uint16_t*)out_scale_f16)
+#define AO_FP6_ROWS_T(BF, E3)                                                                                       \
+    do {                                                                                                            \
+        if (variant == 0) AO_FP6_ROWS(BF, E3, 2, 256, 2);                                                           \
+        else if (variant == 1) AO_FP6_ROWS(BF, E3, 2, 512, 2);                                                      \
+        else AO_FP6_ROWS(BF, E3, 2, 512, 1);                                                                        \
+    } while (0)
+        if (w_dtype == AO_BF16) {
+            if (ebits == 3) AO_FP6_ROWS_T(true, true);
+            else AO_FP6_ROWS_T(true, false);
+        } else {
+            if (ebits == 3) AO_FP6_ROWS_T(false, true);
+            else AO_FP6_ROWS_T(false, false);
+        }
+#undef AO_FP6_ROWS_T
+#undef AO_FP6_ROWS
+        AO_LAUNCH_CHECK();
+        return 0;
+    }
     if (w_dtype == AO_BF16 || w_dtype == AO_F16) {
         // enough workgroups for the chip: about 2048, each with a run of 16-column slices of one 64-row block
         int64_t splits = (2048 + N / 64 - 1) / (N / 64);

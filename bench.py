@@ -524,6 +524,8 @@ def sweep(kind, iters=100):
             packed = torch.empty(pb // 4, dtype=torch.int32, device=dev)
             qp = torch.empty(qb // 4, dtype=torch.int32, device=dev)
             BF16, I32, ASYM, ZP_FLOAT = 1, 3, 1, 1
+            tc = torch.empty(N * K * 3 // 4, dtype=torch.uint8, device=dev)
+            sc16 = torch.empty(N, dtype=torch.float16, device=dev)
             qparam_bytes = 4 * N * K // g
             steps = [
                 ("choose_qparams_affine", N * K * 2 + qparam_bytes, lambda i: _lib.check(L.ao_amd_choose_qparams_affine(
@@ -538,6 +540,9 @@ def sweep(kind, iters=100):
                 ("int4wo_quantize_pack", N * K * 2 + N * K // 2 + qparam_bytes, lambda i: _lib.check(
                     L.ao_amd_int4wo_quantize_pack(w[i % copies].data_ptr(), N, K, K, g, packed.data_ptr(), qp.data_ptr(),
                                                   st))),
+                ("fp6_quantize_pack_e3m2", N * K * 2 + N * K * 3 // 4 + 2 * N, lambda i: _lib.check(
+                    L.ao_amd_fp6_quantize_pack(w[i % copies].data_ptr(), BF16, N, K, 3, 2, tc.data_ptr(), sc16.data_ptr(),
+                                               st))),
             ]
             for name, nbytes, launch in steps:
                 us = _time_linear(L, launch, iters, armed=False)

@@ -35,6 +35,54 @@ def test_quantize_pack_bit_exact(oracle, shape, dtype):
     assert np.array_equal(data.cpu().numpy(), packed_ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("fmt", [(3, 2), (2, 3)])
+@pytest.mark.parametrize("shape", [(64, 64), (128, 4096), (64, 8192), (128, 14336), (64, 16384), (64, 16448)])
+def test_quantize_pack_16_bit_rows_bit_exact_on_edge_cases(oracle, shape, fmt, dtype):
+    """The one-pass kernel for 16-bit weights (rows of up to 16384 values; the last shape is past it and takes the
+    three-launch path): the division by the row scale is a reciprocal with two corrections and the cast is the hardware's
+    8-bit float conversion, so the cases are the ones where either could differ from the reference's division and
+    bitwise cast: ties of the FP6 grid (scale a power of two), values a hair off the ties, signed zeros, a row that is
+    all zero, rows so small or large that the scale leaves the range the shortcut is used in, NaN and inf."""
+    from ao_amd import ops
+
+    N, K = shape
+    ebits, mbits = fmt
+    print(f"case fp6 quantize_pack edge rows N={N} K={K} e{ebits}m{mbits} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(N * 7 + K + ebits)
+    w = (torch.randn(N, K, generator=g) * torch.logspace(-3, 1, N).unsqueeze(1)).float()
+    max_normal = {(3, 2): 28.0, (2, 3): 7.5}[fmt]
+    # row 0: amax = max_normal * 2^-6, so the scale is 2^-6 and every multiple of the half step is a tie
+    steps = torch.arange(K) % 449
+    w[0] = (steps.float() - 224.0) * (max_normal / 224.0) * 2.0 ** -6 * (0.25 if fmt == (3, 2) else 1.0)
+    w[0, 0] = max_normal * 2.0 ** -6
+    # row 1: the same grid, nudged by the input dtype's own rounding
+    w[1] = w[0] * (1.0 + 2.0 ** -9)
+    w[2] = 0.0
+    w[2, 1::2] = -0.0
+    w[3] = w[3] * 0.0 + 1e-30 if dtype is torch.bfloat16 else w[3] * 1e-7     # far below the 1e-12 clamp / fp16 subnormals
+    w[4, ::3] = -0.0
+    w[5] = w[5].abs() * -1.0
+    if dtype is torch.bfloat16:
+        w[6] = w[6] * 1e30          # scale beyond the shortcut's range
+        w[7] = w[7] * 1e-25
+    w[8, 3] = float("inf")
+    w[9, 5] = float("nan")
+    w[10, 7] = float("-inf")
+    w[11] = 65504.0 if dtype is torch.float16 else 3.0e38
+    w[11, ::2] = -w[11, ::2] * 0.5
+    wd = w.to(dtype)
+    data, scale = ops.fp6_quantize_pack(wd.to(_dev()), ebits, mbits)
+    code = {torch.bfloat16: oracle.BF16, torch.float16: oracle.F16}[dtype]
+    codes_ref, scale_ref = oracle.fpx_quantize(bits16(wd), code, ebits, mbits)
+    packed_ref = oracle.pack_tc_fp6(codes_ref)
+    bad_scales = np.nonzero(bits16(scale) != scale_ref)[0].tolist()
+    got = oracle.unpack_tc_fp6(data.cpu().numpy(), N, K)
+    bad_rows = np.nonzero((got != codes_ref).any(axis=1))[0].tolist()
+    assert bad_scales == [] and bad_rows == []
+    assert np.array_equal(data.cpu().numpy(), packed_ref)
+
+
 def test_dequantize_and_repack_round_trip(oracle):
     from ao_amd import ops
 
