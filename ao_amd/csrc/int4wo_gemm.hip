@@ -372,6 +372,218 @@ __global__ __launch_bounds__(256) void int4wo_gemm_lds_kernel(const LinearArgs a
     }
 }
 
+// ---------------------------------------------------------------- 128-row tiles, K split over the waves
+// For activation counts whose 256-row tiles cannot fill the chip (128 to about 1000 rows on the narrower weights):
+// workgroup tile 128 x 64, and the four waves split K instead of N: wave w takes the 64-wide K steps w, w + 4, ... of
+// the whole tile (4 x 2 blocks of 32 x 32, 128 accumulator registers), and the four partial tiles are summed through
+// LDS at the end.  Nothing is shared between the waves inside the loop, so it has no barrier: every wave brings in its
+// own activation slices (128 x 64 bf16 = 16 KB, double buffered in the wave's own 32 KB of LDS, 16 LDS-DMA requests a
+// step) and waits for them with its own counters.  The weights are dequantized once per workgroup, as in the 256-row
+// kernel, but a 128-row tile has only 4 matrix instructions per weight dword, so the 39 VALU instructions of the
+// dequantization bound the loop (10 per matrix instruction): about 70 cycles per matrix instruction instead of 32.
+// Slot schedule of a step: as in the 256-row kernel with 8 slots per sub-step; the DMA requests of step t + 2 go one
+// per slot into sub-step 3 (after a wait for the LDS reads of the buffer they overwrite) and sub-step 0 of step t + 1.
+template <int G>
+__global__ __launch_bounds__(256) void int4wo_gemm_kwave_kernel(const LinearArgs a, int tiles_n, int tiles_total,
+                                                                 int tiles_per_xcd) {
+    constexpr int BM = 128, BN = 64, MT = 4, NT = 2, XCH = 16, SLOTS = MT * NT, OPS = (NT * DQ8_OPS + SLOTS - 1) / SLOTS;
+    __shared__ __align__(16) uint8_t lds[4][2][BM * 128];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tile = (int)(blockIdx.x & 7) * tiles_per_xcd + (int)(blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= tiles_per_xcd || tile >= tiles_total) return;
+    const int tile_m = tile / tiles_n, tile_n = tile - tile_m * tiles_n;
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int KS = (int)(a.Kp / 64);
+    const int KB = (int)(a.Kp / 128);
+    const int nst = (KS - wave + 3) / 4;   // this wave's steps: s = wave + 4 t
+    const int64_t nblocks = (a.N + 15) / 16;
+    const uint32_t magic = 0x64006400u;
+
+    // activations: request j fills rows 8 j .. 8 j + 7 of the wave's slice, 8 lanes a row; lane L holds, at row L / 8
+    // and 16-byte column L % 8, k chunk (L % 8) ^ (row % 8) (row % 8 = L / 8)
+    const int xr = lane >> 3, xp = lane & 7;
+    uint32_t xoff[XCH];
+#pragma unroll
+    for (int j = 0; j < XCH; ++j) {
+        const int row = xr + 8 * j;
+        const int64_t rel = (m0 + row < a.M ? m0 + row : a.M - 1) - m0;
+        xoff[j] = (uint32_t)(rel * a.ldx * 2) + ((xp ^ xr) << 4);
+    }
+    const uint16_t* const xbase = uniform_ptr(a.x + m0 * a.ldx);
+    uint8_t* const Lw = &lds[wave][0][0];
+    const uint32_t ldsw = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)Lw;
+    auto dma_x1 = [&](int j, int t) __attribute__((always_inline)) {
+        const int tc = t < nst ? t : nst - 1;   // steps past the end repeat the last one and are never used
+        const int s = wave + 4 * tc;
+        const uint32_t m0v = ldsw + (t & 1) * (BM * 128) + j * 1024;
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(xoff[j]), "s"(xbase + (int64_t)s * 64), "s"(m0v) : "memory");
+    };
+    const int frow = lane & 31, kq = lane >> 5;
+    const int64_t nb0 = n0 >> 4;
+    uint32_t woff[NT], qoff[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        int64_t nb = nb0 + ((j * 32 + frow) >> 4);
+        if (nb >= nblocks) nb = nblocks - 1;
+        woff[j] = (uint32_t)((nb - nb0) * KB * 1024) + kq * 256 + (frow & 15) * 16;
+        qoff[j] = (uint32_t)((nb - nb0) * (a.Kp / G) * 64) + (G == 32 ? kq * 64 : 0) + (frow & 15) * 4;
+    }
+    const uint4* const wbase = uniform_ptr(a.packed + nb0 * KB * 64);
+    const uint32_t* const qbase = uniform_ptr(a.qparams + nb0 * (a.Kp / G) * 16);
+    u32x4_t wr[2][NT];
+    uint32_t qr[2][NT];
+    auto load_w = [&](int set, int t) __attribute__((always_inline)) {
+        const int tc = t < nst ? t : nst - 1;
+        const int s = wave + 4 * tc;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            wr[set][j] = asm_load_b128(wbase + (int64_t)(s >> 1) * 64 + (s & 1) * 32, woff[j]);
+            qr[set][j] = asm_load_b32(qbase + (int64_t)((s * 64) / G) * 16, qoff[j]);
+        }
+    };
+
+    f32x16_t acc[MT][NT];
+    {
+        const u32x4_t zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+                asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %1, 0" : "=a"(acc[i][j]) : "v"(zero));
+    }
+    const uint32_t afrag0 = frow * 128 + (((kq * 4) ^ (frow & 7)) << 4);
+
+    Frag fa[2][MT], fb[2][NT];
+#pragma unroll
+    for (int j = 0; j < XCH; ++j) dma_x1(j, 0);
+    load_w(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    load_w(1, 1);
+#pragma unroll
+    for (int j = 0; j < XCH / 2; ++j) dma_x1(j, 1);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) fb[0][j].q = dq8_all(wr[0][j].x, make_group_f32(qr[0][j]), magic);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) fa[0][i].q = *reinterpret_cast<const u32x4_t*>(Lw + afrag0 + i * 4096);
+
+    auto step = [&](int t, const int set) __attribute__((always_inline)) {
+        const uint8_t* As = Lw + (t & 1) * (BM * 128);
+        const uint8_t* An = Lw + ((t + 1) & 1) * (BM * 128);
+        GroupF32 gc[NT];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) gc[j] = make_group_f32(qr[set][j]);
+        uint32_t w[NT][4];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            w[j][0] = wr[set][j].x; w[j][1] = wr[set][j].y; w[j][2] = wr[set][j].z; w[j][3] = wr[set][j].w;
+        }
+        static_for<0, 4>([&](auto ks_c) __attribute__((always_inline)) {
+            constexpr int ks = decltype(ks_c)::value, cur = ks & 1, nxt = cur ^ 1;
+            Dq8 d[NT];
+            uint32_t wn[NT];
+            if constexpr (ks < 3) {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) wn[j] = w[j][ks + 1];
+            } else {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    wn[j] = wr[set ^ 1][j].x;
+                    gc[j] = make_group_f32(qr[set ^ 1][j]);
+                }
+                // the LDS reads of this step's buffer have returned before the requests below overwrite it
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<0, SLOTS>([&](auto q_c) __attribute__((always_inline)) {
+                constexpr int q = decltype(q_c)::value, i = q / NT, j = q % NT;
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[cur][i].v), "v"(fb[cur][j].v));
+                static_for<0, OPS>([&](auto u_c) __attribute__((always_inline)) {
+                    constexpr int op = q * OPS + decltype(u_c)::value, pj = op / DQ8_OPS, o = op % DQ8_OPS;
+                    if constexpr (pj < NT) {
+                        dq8_op<o>(d[pj], wn[pj], gc[pj], magic);
+                        if constexpr (o == DQ8_OPS - 1) fb[nxt][pj].q = u32x4_t{d[pj].p0, d[pj].p1, d[pj].p2, d[pj].p3};
+                    }
+                });
+                if constexpr (q < MT) {
+                    if constexpr (ks < 3) fa[nxt][q].q = *reinterpret_cast<const u32x4_t*>(As + (afrag0 ^ ((ks + 1) << 4)) + q * 4096);
+                    else fa[nxt][q].q = *reinterpret_cast<const u32x4_t*>(An + afrag0 + q * 4096);
+                }
+                if constexpr (ks == 3 && q == 0) load_w(set, t + 2);
+                if constexpr (ks == 3) dma_x1(q, t + 2);
+                if constexpr (ks == 0) dma_x1(8 + q, t + 1);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            if constexpr (ks == 2) {
+                // the wave's activation slice of step t + 1 has landed, and the weights requested before its second half
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+        });
+    };
+    for (int t = 0; t < nst; t += 2) {
+        step(t, 0);
+        if (t + 1 < nst) step(t + 1, 1);
+    }
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+
+    // Sum of the four waves' partial tiles: every wave leaves its own in its 32 KB of LDS as fp32 [128][64] (the column
+    // index flipped by 32 in rows whose bit 2 is set: the two half-waves write rows 4 apart, 1024 bytes, the same
+    // banks otherwise), then wave w adds up rows 32 w .. 32 w + 31 of the four and stores them, 4 columns a lane.
+    // acc[i][j][e] = C[m = m0 + 32 i + 8 (e / 4) + 4 kq + e % 4][n = n0 + 32 j + frow]
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row = 32 * i + 8 * (e >> 2) + 4 * kq + (e & 3);
+                const int col = (32 * j + frow) ^ (kq << 5);
+                *reinterpret_cast<float*>(Lw + (row * 64 + col) * 4) = acc[i][j][e];
+            }
+    __syncthreads();
+    const int r = lane >> 4, c4 = lane & 15;
+    const int64_t n = n0 + c4 * 4;
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (a.bias) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            if (n + v < a.N) bv[v] = bf16_bits_to_f32(a.bias[n + v]);
+    }
+    const bool wide = n + 3 < a.N && (a.ldy & 3) == 0 && ((uintptr_t)a.y & 15) == 0;
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+        const int row = 32 * wave + 4 * pass + r;
+        const int pc = (c4 * 4) ^ (((row >> 2) & 1) << 5);
+        f32x4_t sum = *reinterpret_cast<const f32x4_t*>(&lds[0][0][0] + (row * 64 + pc) * 4);
+#pragma unroll
+        for (int p = 1; p < 4; ++p) {
+            const f32x4_t v = *reinterpret_cast<const f32x4_t*>(&lds[p][0][0] + (row * 64 + pc) * 4);
+            sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
+        }
+        const int64_t m = m0 + row;
+        if (m >= a.M) continue;
+        if (wide) {
+            if (a.y_is_f32) {
+                *reinterpret_cast<f32x4_t*>((float*)a.y + m * a.ldy + n) = f32x4_t{sum[0] + bv[0], sum[1] + bv[1], sum[2] + bv[2], sum[3] + bv[3]};
+            } else {
+                u32x2_t o;
+                o.x = (uint32_t)f32_to_bf16_bits(sum[0] + bv[0]) | ((uint32_t)f32_to_bf16_bits(sum[1] + bv[1]) << 16);
+                o.y = (uint32_t)f32_to_bf16_bits(sum[2] + bv[2]) | ((uint32_t)f32_to_bf16_bits(sum[3] + bv[3]) << 16);
+                *reinterpret_cast<u32x2_t*>((uint16_t*)a.y + m * a.ldy + n) = o;
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (n + v < a.N) {
+                    if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n + v] = sum[v] + bv[v];
+                    else ((uint16_t*)a.y)[m * a.ldy + n + v] = f32_to_bf16_bits(sum[v] + bv[v]);
+                }
+        }
+    }
+}
+
 struct GemmLdsPlan {
     int nt, tiles_m, tiles_n;
 };
@@ -397,11 +609,52 @@ static bool gemm_lds_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
     return (int64_t)p->tiles_m * p->tiles_n < (1 << 24);
 }
 
+// 128 x 64 tiles with K split over the waves: where the 256-row tiles do not apply, from about 100 rows, when the tiles
+// cover at least three quarters of the CUs (measured: with 128 tiles the older kernels are as fast)
+static bool gemm_kwave_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
+    static const bool disabled = [] { const char* e = getenv("AO_AMD_GEMM_KWAVE"); return e && e[0] == '0'; }();
+    if (disabled) return false;
+    static const int64_t min_rows = [] { const char* e = getenv("AO_AMD_GEMM_KWAVE_MIN_M"); return e ? atoll(e) : 100ll; }();
+    if (a.M < min_rows || a.K != a.Kp || a.Kp < 1024 || a.packed2 || a.residual || a.norm_w || a.pair8 || a.ksplit != 1) return false;
+    if (g != 32 && g != 64 && g != 128 && g != 256) return false;
+    if (128 * a.ldx * 2 >= ((int64_t)1 << 32) || 4 * (a.Kp / 128) * 1024 + 1024 >= ((int64_t)1 << 32)) return false;
+    p->nt = 0;
+    p->tiles_m = (int)((a.M + 127) / 128);
+    p->tiles_n = (int)((a.N + 63) / 64);
+    const int64_t tiles = (int64_t)p->tiles_m * p->tiles_n;
+    return tiles >= 192 && tiles < (1 << 24);
+}
+
 bool int4wo_gemm_lds_plan(const LinearArgs& a, int64_t g, char* out, size_t cap) {
     GemmLdsPlan p;
-    if (!gemm_lds_plan(a, g, &p)) return false;
-    snprintf(out, cap, "int4wo_gemm_lds_kernel<%lld,%d>", (long long)g, p.nt);
-    return true;
+    if (gemm_lds_plan(a, g, &p)) {
+        snprintf(out, cap, "int4wo_gemm_lds_kernel<%lld,%d>", (long long)g, p.nt);
+        return true;
+    }
+    if (gemm_kwave_plan(a, g, &p)) {
+        snprintf(out, cap, "int4wo_gemm_kwave_kernel<%lld>", (long long)g);
+        return true;
+    }
+    return false;
+}
+
+static void launch_gemm_kwave(const LinearArgs& a, int64_t g, const GemmLdsPlan& p, hipStream_t st) {
+    const int total = p.tiles_m * p.tiles_n, per_xcd = (total + 7) / 8;
+    const dim3 grid((unsigned)(per_xcd * 8)), block(256);
+    auto go = [&](auto kernel) {
+        if (g_prof_start && g_prof_stop) {
+            hipExtLaunchKernelGGL(kernel, grid, block, 0, st, g_prof_start, g_prof_stop, 0, a, p.tiles_n, total, per_xcd);
+            g_prof_start = g_prof_stop = nullptr;
+        } else {
+            hipLaunchKernelGGL(kernel, grid, block, 0, st, a, p.tiles_n, total, per_xcd);
+        }
+    };
+    switch (g) {
+        case 32: go(int4wo_gemm_kwave_kernel<32>); break;
+        case 64: go(int4wo_gemm_kwave_kernel<64>); break;
+        case 128: go(int4wo_gemm_kwave_kernel<128>); break;
+        default: go(int4wo_gemm_kwave_kernel<256>); break;
+    }
 }
 
 template <int NT>
@@ -426,10 +679,16 @@ static void launch_gemm_lds_nt(const LinearArgs& a, int64_t g, const GemmLdsPlan
 
 bool launch_int4wo_gemm_lds(const LinearArgs& a, int64_t g, hipStream_t st) {
     GemmLdsPlan p;
-    if (!gemm_lds_plan(a, g, &p)) return false;
-    if (p.nt == 1) launch_gemm_lds_nt<1>(a, g, p, st);
-    else launch_gemm_lds_nt<2>(a, g, p, st);
-    return true;
+    if (gemm_lds_plan(a, g, &p)) {
+        if (p.nt == 1) launch_gemm_lds_nt<1>(a, g, p, st);
+        else launch_gemm_lds_nt<2>(a, g, p, st);
+        return true;
+    }
+    if (gemm_kwave_plan(a, g, &p)) {
+        launch_gemm_kwave(a, g, p, st);
+        return true;
+    }
+    return false;
 }
 
 }  // namespace ao

@@ -46,12 +46,12 @@ def test_dispatch_walk_finds_every_kernel_family():
     plans = _walk()
     families = {n.split("<")[0] for n in plans}
     assert families == {"int4wo_gemv1_kernel", "int4wo_gemv_kernel", "int4wo_linear_kernel", "int4wo_gemm_kernel",
-                        "int4wo_gemm_ksplit_kernel", "int4wo_gemm_lds_kernel"}
+                        "int4wo_gemm_ksplit_kernel", "int4wo_gemm_lds_kernel", "int4wo_gemm_kwave_kernel"}
     # the tile variants of the matrix-core kernels and both K-split forms
     for g in GROUPS:
         for tile in ("int4wo_gemm_kernel<%d,2,8>", "int4wo_gemm_kernel<%d,1,4>", "int4wo_gemm_kernel<%d,1,2>",
                      "int4wo_gemm_ksplit_kernel<%d,4,4>", "int4wo_gemm_ksplit_kernel<%d,2,4>",
-                     "int4wo_gemm_lds_kernel<%d,1>", "int4wo_gemm_lds_kernel<%d,2>"):
+                     "int4wo_gemm_lds_kernel<%d,1>", "int4wo_gemm_lds_kernel<%d,2>", "int4wo_gemm_kwave_kernel<%d>"):
             assert tile % g in plans, tile % g
     # the single-row kernel: exactly the instantiations that int4wo_gemv1.hip compiles (waves, chunks per lane, norm)
     gemv1 = {n.split(" ")[0] for n in plans if n.startswith("int4wo_gemv1_kernel<")}
@@ -66,7 +66,13 @@ def test_dispatch_walk_finds_every_kernel_family():
     assert _lib.int4wo_linear_plan(2048, 14336, 4096, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
     assert not _lib.int4wo_linear_plan(512, 14336, 4096, 64).startswith("int4wo_gemm_lds_kernel")   # 64 tiles
     assert not _lib.int4wo_linear_plan(300, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel")   # 212 of 512 tile rows empty
-    assert len(plans) >= 68
+    # ... and the 128-row tiles with K split over the waves where those do not, from about 100 rows, when at least 192
+    # of them exist
+    assert _lib.int4wo_linear_plan(128, 4096, 14336, 64) == "int4wo_gemm_kwave_kernel<64>"
+    assert _lib.int4wo_linear_plan(512, 14336, 4096, 64) == "int4wo_gemm_kwave_kernel<64>"
+    assert not _lib.int4wo_linear_plan(128, 4096, 4096, 64).startswith("int4wo_gemm_kwave_kernel")   # 64 tiles
+    assert not _lib.int4wo_linear_plan(99, 1024, 14336, 64).startswith("int4wo_gemm_kwave_kernel")
+    assert len(plans) >= 72
 
 
 def _cases():

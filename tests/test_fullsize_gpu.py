@@ -211,19 +211,24 @@ def test_config1_output_tolerance(oracle):
     assert rel_l2(y16.float().cpu().numpy(), y_ref16) <= 1e-3
 
 
-@pytest.mark.parametrize("M,N,K,g,bias,fp32", [(2048, 14336, 4096, 64, False, False), (1000, 14336, 4096, 128, True, False),
-                                               (2048, 6100, 1024, 64, True, False), (1792, 4096, 2048, 32, False, True),
-                                               (2048, 4096, 14336, 256, True, False)])
-def test_prefill_gemm_tiles_edges_and_repeated_launches(cabi, M, N, K, g, bias, fp32):
-    """The 256-row prefill kernel (activations through LDS-direct loads, weights dequantized between the matrix
-    instructions): every output element is written (the output starts as NaN), ragged M and N, bias, both output
+@pytest.mark.parametrize("M,N,K,g,bias,fp32,kernel", [
+    (2048, 14336, 4096, 64, False, False, "lds"), (1000, 14336, 4096, 128, True, False, "lds"),
+    (2048, 6100, 1024, 64, True, False, "lds"), (1792, 4096, 2048, 32, False, True, "lds"),
+    (2048, 4096, 14336, 256, True, False, "lds"),
+    (128, 14336, 4096, 64, False, False, "kwave"), (200, 12352, 1024, 128, True, False, "kwave"),
+    (512, 4096, 14336, 256, False, True, "kwave"), (333, 6100, 2048, 32, True, False, "kwave"),
+    (1000, 4098, 4096, 64, True, True, "kwave"), (130, 14336, 1152, 64, False, False, "kwave")])
+def test_prefill_gemm_tiles_edges_and_repeated_launches(cabi, M, N, K, g, bias, fp32, kernel):
+    """The prefill kernels (activations through LDS-direct loads, weights dequantized between the matrix instructions;
+    256-row tiles, and 128-row tiles whose waves split K, with step counts per wave that differ when K / 64 is not a
+    multiple of 4): every output element is written (the output starts as NaN), ragged M and N, bias, both output
     types, and the same launch three times in a row with LDS of every CU overwritten in between by another kernel, so
     that a read that runs ahead of its data cannot find the previous launch's identical bytes there."""
-    print(f"case prefill gemm M={M} N={N} K={K} g={g} bias={bias} fp32={fp32}", flush=True)
+    print(f"case prefill gemm M={M} N={N} K={K} g={g} bias={bias} fp32={fp32} {kernel}", flush=True)
     dev = torch.device("cuda:0")
     L = cabi.lib()
     st = torch.cuda.current_stream().cuda_stream
-    assert cabi.int4wo_linear_plan(M, K, N, g).startswith("int4wo_gemm_lds_kernel")
+    assert cabi.int4wo_linear_plan(M, K, N, g).startswith(f"int4wo_gemm_{kernel}_kernel")
     gen = torch.Generator(device=dev).manual_seed(M + N + K)
     w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).bfloat16()
     _, _, pb, qb = cabi.packed_shape(N, K, g)

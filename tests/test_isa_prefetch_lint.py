@@ -167,8 +167,9 @@ def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched
       * between a weight load and the next vmcnt(0) wait (following the loop's back edge once) no instruction reads or
         writes the load's target registers, so a copy of stale contents or a reuse of a register under a load in flight
         (the epilogue's, after the last, unused requests of the loop) cannot happen;
-      * the K loop carries the 16 LDS-direct activation requests and the weight requests (a chunk and its scale / zero per
-        32-row block) of its two steps;
+      * the K loop carries the LDS-direct activation requests (16 per two steps and wave of the 256-row kernel, 32 of the
+        128-row kernel, whose waves each bring in their own slices) and the weight requests (a chunk and its scale / zero
+        per 32-row block) of its two steps;
       * no scratch access inside the K loop, every matrix instruction accumulates in accumulation registers."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
@@ -180,8 +181,12 @@ def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched
     kernels = list(re.finditer(r"^(_ZN2ao22int4wo_gemm_lds_kernelILi(\d+)ELi([12])EEEvNS_10LinearArgsEiii): ; @.*?\n(.*?)s_endpgm(.*?)\.end_amdhsa_kernel",
                                text, re.S | re.M))
     assert len(kernels) == 8
-    for m in kernels:
-        name, nt, body, meta = m.group(1), int(m.group(3)), m.group(4), m.group(5)
+    # the 128-row kernel whose waves split K: the same discipline, 16 activation requests per step and wave
+    kwave = list(re.finditer(r"^(_ZN2ao24int4wo_gemm_kwave_kernelILi(\d+)EEEvNS_10LinearArgsEiii): ; @.*?\n(.*?)s_endpgm(.*?)\.end_amdhsa_kernel",
+                             text, re.S | re.M))
+    assert len(kwave) == 4
+    cases = [(m.group(1), int(m.group(3)), 16, m.group(4)) for m in kernels] + [(m.group(1), 2, 32, m.group(3)) for m in kwave]
+    for name, nt, dma, body in cases:
         lines = [l.strip() for l in body.splitlines()]
         lines = [l for l in lines if l and not l.startswith(";") and not (l.startswith(".") and not l.startswith(".LBB"))]
         labels = {re.match(r"(\.LBB\d+_\d+):", l).group(1): i for i, l in enumerate(lines) if re.match(r"\.LBB\d+_\d+:", l)}
@@ -190,15 +195,15 @@ def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched
             b = re.match(r"s_c?branch\w* (\.LBB\d+_\d+)", l)
             if b and labels.get(b.group(1), i) < i:
                 back[i] = labels[b.group(1)]
-        assert len(back) == 1, (name, back)           # the K loop is the only loop
-        (loop_end, loop_head), = back.items()
+        assert len(set(back.values())) == 1, (name, back)   # the K loop is the only loop (its second step may be skipped
+        loop_end, loop_head = max(back), min(back.values())  # at the end of K: two branches back to the one head)
         loads = [i for i, l in enumerate(lines) if re.match(r"global_load_dword(x4)? v", l)]
         assert sum(1 for i in loads if loop_head < i < loop_end) == 2 * nt * 2, name   # chunk + qparams per block, two steps
-        assert sum(1 for l in lines[loop_head:loop_end] if l.startswith("global_load_lds_dwordx4")) == 16, name
+        assert sum(1 for l in lines[loop_head:loop_end] if l.startswith("global_load_lds_dwordx4")) == dma, name
         for i in loads:
             dest = _regs(lines[i].split(",")[0])
             j, jumped = i + 1, False
-            while j < len(lines) and lines[j] != "s_waitcnt vmcnt(0)":
+            while j < len(lines) and not lines[j].startswith("s_waitcnt vmcnt(0)"):
                 touched = not lines[j].startswith((".LBB", "s_", "global_load")) and _regs(lines[j]) & dest
                 assert not touched, (name, lines[i], lines[j])
                 if j == loop_end and not jumped:
@@ -208,4 +213,4 @@ def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched
             assert j < len(lines), (name, lines[i])
         # values the epilogue needs may be parked in scratch around the loop, never inside it
         assert not [l for l in lines[loop_head:loop_end] if l.startswith("scratch_")], name
-        assert len(re.findall(r"v_mfma_f32_32x32x16_bf16 a\[", body)) >= 64 * nt, name
+        assert len(re.findall(r"v_mfma_f32_32x32x16_bf16 a\[", body)) >= (64 * nt if dma == 16 else 64), name
