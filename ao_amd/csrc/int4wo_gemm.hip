@@ -622,7 +622,9 @@ static bool gemm_kwave_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
     p->tiles_m = (int)((a.M + 127) / 128);
     p->tiles_n = (int)((a.N + 63) / 64);
     const int64_t tiles = (int64_t)p->tiles_m * p->tiles_n;
-    return tiles >= 192 && tiles < (1 << 24);
+    // ... and at most four rounds of them: with more, the older 64-row kernels fill the chip as well and run the
+    // vocabulary head at 128 rows in 180 us against 208 us
+    return tiles >= 192 && tiles <= 1024;
 }
 
 bool int4wo_gemm_lds_plan(const LinearArgs& a, int64_t g, char* out, size_t cap) {
