@@ -8,10 +8,13 @@
 // What bounds the kernel (measured on MI355X, one wave per SIMD): a 32x32x16 matrix instruction holds the matrix pipe
 // for 32 cycles and the wave's issue port for about 8; an ordinary VALU instruction takes about 6 issue cycles, an LDS
 // read about the same, a global request about 35.  Four VALU instructions per matrix instruction are therefore free and
-// every further one costs its issue time.  The exact two-rounding dequantization is 39 VALU instructions per 8 codes,
-// and a 256-row tile spends 8 matrix instructions per 8 codes: 4.9 VALU instructions per matrix instruction, which is
-// what the loop runs at (about 40 cycles per matrix instruction instead of 32).  v_dot2 and the 4x4x4 matrix
-// instruction, which the single-row kernels dequantize with, run on the matrix pipe itself and are not used here.
+// every further one costs its issue time.  The exact two-rounding dequantization is 33 VALU instructions per 8 codes,
+// and a 256-row tile spends 8 matrix instructions per 8 codes: 4.1 VALU instructions per matrix instruction, which is
+// close to free.  What is left between the loop's 40 cycles per matrix instruction and the pipe's 32 are the memory
+// requests (12 per wave and 64-wide K step, each holding the wave's issue port for about 35 cycles), the LDS reads and
+// the barrier: with all but 9 of the 33 dequantization instructions removed (wrong results, measured once) a 2048-row
+// launch on 14336 x 4096 takes 212 instead of 236 us.  v_dot2 and the 4x4x4 matrix instruction, which the single-row
+// kernels dequantize with, run on the matrix pipe itself and are not used here.
 //
 // Workgroup -> tile mapping: consecutive workgroup ids go to different XCDs (8 of them, each with its own L2), so
 // XCD j takes the j-th eighth of the tiles in row-major order; the workgroups that run together on one XCD then
@@ -31,74 +34,73 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 // matrix pipe for 32 cycles and about four ordinary VALU instructions issued in its shadow are free, each further one
 // delays the next matrix instruction by its own 4 cycles.  v_dot2 and the small matrix instructions are not ordinary:
 // they run on the matrix pipe themselves (8 cycles each and a switch penalty, measured), which is why the widening of
-// t below is spelled out as shifts and masks instead of the v_dot2 the single-row kernels use.
+// t below is not the v_dot2 the single-row kernels use.  33 instructions:
 //
-//   (dword >> 4 j) & 0x000F000F | 0x64006400 is the fp16 pair (1024 + q_2j, 1024 + q_2j+1);
-//   v_fma_mix_f32 reads one half as fp16 and computes (1024 + q) * scale - 1032 * scale, exact in fp32;
-//   v_cvt_pk_bf16_f32 rounds two of them to the pair (t_2j, t_2j+1); shift / mask widen them again; add; round.
+//   5  unpack: the code pairs sit at bits (0, 16), (4, 20), (8, 24), (12, 28) of the dword.  dword & 0x000F000F |
+//      0x64006400 is the fp16 pair (1024 + q, 1024 + q') of the first; the second needs no shift: dword & 0x00F000F0 |
+//      0x64006400 is (1024 + 16 q, 1024 + 16 q'), whose factor 16 goes into the scale; one shift by 8 serves the other two;
+//   8  v_fma_mix_f32 reads one half as fp16 and computes (1024 + q) * scale - 1032 * scale, respectively
+//      (1024 + 16 q) * (scale / 16) - 72 * scale: (q - 8) * scale, exact in fp32;
+//   8  v_cvt_pk_bf16_f32 with a zero low operand rounds one value to bf16 and leaves it in the high half: t as fp32;
+//   8  add the zero point;
+//   4  v_cvt_pk_bf16_f32 rounds two of them to the pair (w, w') of the fragment.
 // Every instruction is an asm volatile statement: volatile statements keep their program order.
 struct Dq8 {
-    uint32_t p0, p1, p2, p3;
+    uint32_t p0, p1, p2, p3, ws;
     float a0, a1, a2, a3, a4, a5, a6, a7;
 };
 struct GroupF32 {
-    float s, c, z;   // scale, -1032 * scale, zero
+    float s, c, s16, c16, z;   // scale, -1032 * scale, scale / 16, -72 * scale, zero
 };
 __device__ __forceinline__ GroupF32 make_group_f32(uint32_t qp) {
     const float s = __uint_as_float(qp << 16);
-    return GroupF32{s, -1032.0f * s, __uint_as_float(qp & 0xffff0000u)};
+    return GroupF32{s, -1032.0f * s, 0.0625f * s, -72.0f * s, __uint_as_float(qp & 0xffff0000u)};
 }
-constexpr int DQ8_OPS = 39;
-#define AO_DQ_ANDOR(dst, src, magic) asm volatile("v_and_or_b32 %0, %1, %2, %3" : "=v"(dst) : "v"(src), "s"(0x000F000Fu), "v"(magic))
+constexpr int DQ8_OPS = 33;
+#define AO_DQ_ANDOR_EVEN(dst, src, magic) asm volatile("v_and_or_b32 %0, %1, %2, %3" : "=v"(dst) : "v"(src), "s"(0x000F000Fu), "v"(magic))
+#define AO_DQ_ANDOR_ODD(dst, src, magic) asm volatile("v_and_or_b32 %0, %1, %2, %3" : "=v"(dst) : "v"(src), "s"(0x00F000F0u), "v"(magic))
 #define AO_DQ_SHR(dst, n, src) asm volatile("v_lshrrev_b32 %0, " #n ", %1" : "=v"(dst) : "v"(src))
 #define AO_DQ_FMA_LO(dst, src, s, c) asm volatile("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(dst) : "v"(src), "v"(s), "v"(c))
 #define AO_DQ_FMA_HI(dst, src, s, c) asm volatile("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(dst) : "v"(src), "v"(s), "v"(c))
+#define AO_DQ_ROUND(dst) asm volatile("v_cvt_pk_bf16_f32 %0, 0, %0" : "+v"(dst))
 #define AO_DQ_CVT(dst, lo, hi) asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(dst) : "v"(lo), "v"(hi))
-#define AO_DQ_WIDEN_LO(dst, src) asm volatile("v_lshlrev_b32 %0, 16, %1" : "=v"(dst) : "v"(src))
-#define AO_DQ_WIDEN_HI(dst, src) asm volatile("v_and_b32 %0, 0xffff0000, %1" : "=v"(dst) : "v"(src))
 #define AO_DQ_ADD(dst, z) asm volatile("v_add_f32 %0, %0, %1" : "+v"(dst) : "v"(z))
 template <int op>
 __device__ __forceinline__ void dq8_op(Dq8& d, uint32_t w, const GroupF32& g, uint32_t magic) {
     switch (op) {
-        case 0: AO_DQ_ANDOR(d.p0, w, magic); break;
-        case 1: AO_DQ_SHR(d.p1, 4, w); break;
-        case 2: AO_DQ_SHR(d.p2, 8, w); break;
-        case 3: AO_DQ_SHR(d.p3, 12, w); break;
-        case 4: AO_DQ_ANDOR(d.p1, d.p1, magic); break;
-        case 5: AO_DQ_ANDOR(d.p2, d.p2, magic); break;
-        case 6: AO_DQ_ANDOR(d.p3, d.p3, magic); break;
-        case 7: AO_DQ_FMA_LO(d.a0, d.p0, g.s, g.c); break;
-        case 8: AO_DQ_FMA_HI(d.a1, d.p0, g.s, g.c); break;
-        case 9: AO_DQ_FMA_LO(d.a2, d.p1, g.s, g.c); break;
-        case 10: AO_DQ_FMA_HI(d.a3, d.p1, g.s, g.c); break;
-        case 11: AO_DQ_FMA_LO(d.a4, d.p2, g.s, g.c); break;
-        case 12: AO_DQ_FMA_HI(d.a5, d.p2, g.s, g.c); break;
-        case 13: AO_DQ_FMA_LO(d.a6, d.p3, g.s, g.c); break;
-        case 14: AO_DQ_FMA_HI(d.a7, d.p3, g.s, g.c); break;
-        case 15: AO_DQ_CVT(d.p0, d.a0, d.a1); break;
-        case 16: AO_DQ_CVT(d.p1, d.a2, d.a3); break;
-        case 17: AO_DQ_CVT(d.p2, d.a4, d.a5); break;
-        case 18: AO_DQ_CVT(d.p3, d.a6, d.a7); break;
-        case 19: AO_DQ_WIDEN_LO(d.a0, d.p0); break;
-        case 20: AO_DQ_WIDEN_HI(d.a1, d.p0); break;
-        case 21: AO_DQ_WIDEN_LO(d.a2, d.p1); break;
-        case 22: AO_DQ_WIDEN_HI(d.a3, d.p1); break;
-        case 23: AO_DQ_WIDEN_LO(d.a4, d.p2); break;
-        case 24: AO_DQ_WIDEN_HI(d.a5, d.p2); break;
-        case 25: AO_DQ_WIDEN_LO(d.a6, d.p3); break;
-        case 26: AO_DQ_WIDEN_HI(d.a7, d.p3); break;
-        case 27: AO_DQ_ADD(d.a0, g.z); break;
-        case 28: AO_DQ_ADD(d.a1, g.z); break;
-        case 29: AO_DQ_ADD(d.a2, g.z); break;
-        case 30: AO_DQ_ADD(d.a3, g.z); break;
-        case 31: AO_DQ_ADD(d.a4, g.z); break;
-        case 32: AO_DQ_ADD(d.a5, g.z); break;
-        case 33: AO_DQ_ADD(d.a6, g.z); break;
-        case 34: AO_DQ_ADD(d.a7, g.z); break;
-        case 35: AO_DQ_CVT(d.p0, d.a0, d.a1); break;
-        case 36: AO_DQ_CVT(d.p1, d.a2, d.a3); break;
-        case 37: AO_DQ_CVT(d.p2, d.a4, d.a5); break;
-        case 38: AO_DQ_CVT(d.p3, d.a6, d.a7); break;
+        case 0: AO_DQ_ANDOR_EVEN(d.p0, w, magic); break;
+        case 1: AO_DQ_ANDOR_ODD(d.p1, w, magic); break;
+        case 2: AO_DQ_SHR(d.ws, 8, w); break;
+        case 3: AO_DQ_ANDOR_EVEN(d.p2, d.ws, magic); break;
+        case 4: AO_DQ_ANDOR_ODD(d.p3, d.ws, magic); break;
+        case 5: AO_DQ_FMA_LO(d.a0, d.p0, g.s, g.c); break;
+        case 6: AO_DQ_FMA_HI(d.a1, d.p0, g.s, g.c); break;
+        case 7: AO_DQ_FMA_LO(d.a2, d.p1, g.s16, g.c16); break;
+        case 8: AO_DQ_FMA_HI(d.a3, d.p1, g.s16, g.c16); break;
+        case 9: AO_DQ_FMA_LO(d.a4, d.p2, g.s, g.c); break;
+        case 10: AO_DQ_FMA_HI(d.a5, d.p2, g.s, g.c); break;
+        case 11: AO_DQ_FMA_LO(d.a6, d.p3, g.s16, g.c16); break;
+        case 12: AO_DQ_FMA_HI(d.a7, d.p3, g.s16, g.c16); break;
+        case 13: AO_DQ_ROUND(d.a0); break;
+        case 14: AO_DQ_ROUND(d.a1); break;
+        case 15: AO_DQ_ROUND(d.a2); break;
+        case 16: AO_DQ_ROUND(d.a3); break;
+        case 17: AO_DQ_ROUND(d.a4); break;
+        case 18: AO_DQ_ROUND(d.a5); break;
+        case 19: AO_DQ_ROUND(d.a6); break;
+        case 20: AO_DQ_ROUND(d.a7); break;
+        case 21: AO_DQ_ADD(d.a0, g.z); break;
+        case 22: AO_DQ_ADD(d.a1, g.z); break;
+        case 23: AO_DQ_ADD(d.a2, g.z); break;
+        case 24: AO_DQ_ADD(d.a3, g.z); break;
+        case 25: AO_DQ_ADD(d.a4, g.z); break;
+        case 26: AO_DQ_ADD(d.a5, g.z); break;
+        case 27: AO_DQ_ADD(d.a6, g.z); break;
+        case 28: AO_DQ_ADD(d.a7, g.z); break;
+        case 29: AO_DQ_CVT(d.p0, d.a0, d.a1); break;
+        case 30: AO_DQ_CVT(d.p1, d.a2, d.a3); break;
+        case 31: AO_DQ_CVT(d.p2, d.a4, d.a5); break;
+        case 32: AO_DQ_CVT(d.p3, d.a6, d.a7); break;
         default: break;
     }
 }
@@ -142,7 +144,7 @@ __device__ __forceinline__ const T* uniform_ptr(const T* p) {
 // One K step = 4 sub-steps ks of 16 slots; a slot is one matrix instruction followed by the work that runs in its
 // shadow.  Entering step s, fragment set 0 holds sub-step 0 of both operands.
 //   every ks:  slots 0-7 read the activation fragments of the next sub-step (ks 3: sub-step 0 of step s + 1, from the
-//              other LDS buffer); all slots carry 5 of the 78 instructions that dequantize the next two weight dwords
+//              other LDS buffer); all slots carry 4 or 5 of the 66 instructions that dequantize the next two weight dwords
 //              (ks 3: the first dwords of step s + 1);
 //   ks 2:      ends with the barrier of the step, once the activation slice of step s + 1 has landed in the other LDS
 //              buffer: everything read after it (ks 3) is from that buffer, and this step's buffer is free again;
@@ -280,12 +282,11 @@ __global__ __launch_bounds__(256) void int4wo_gemm_lds_kernel(const LinearArgs a
             static_for<0, SLOTS>([&](auto q_c) __attribute__((always_inline)) {
                 constexpr int q = decltype(q_c)::value, i = q / NT, j = q % NT;
                 asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[cur][i].v), "v"(fb[cur][j].v));
-                static_for<0, 5>([&](auto u_c) __attribute__((always_inline)) {
-                    constexpr int op = q * 5 + decltype(u_c)::value, pj = op / DQ8_OPS, o = op % DQ8_OPS;
-                    if constexpr (pj < NT) {
-                        dq8_op<o>(d[pj], wn[pj], gc[pj], magic);
-                        if constexpr (o == DQ8_OPS - 1) fb[nxt][pj].q = u32x4_t{d[pj].p0, d[pj].p1, d[pj].p2, d[pj].p3};
-                    }
+                // this slot's share of the NT * 33 dequantization instructions of the sub-step, dealt out evenly
+                static_for<q * NT * DQ8_OPS / SLOTS, (q + 1) * NT * DQ8_OPS / SLOTS>([&](auto op_c) __attribute__((always_inline)) {
+                    constexpr int op = decltype(op_c)::value, pj = op / DQ8_OPS, o = op % DQ8_OPS;
+                    dq8_op<o>(d[pj], wn[pj], gc[pj], magic);
+                    if constexpr (o == DQ8_OPS - 1) fb[nxt][pj].q = u32x4_t{d[pj].p0, d[pj].p1, d[pj].p2, d[pj].p3};
                 });
                 if constexpr (q < 8) {
                     if constexpr (ks < 3) fa[nxt][q].q = *reinterpret_cast<const u32x4_t*>(As + (afrag0 ^ ((ks + 1) << 4)) + q * 4096);
@@ -379,14 +380,14 @@ __global__ __launch_bounds__(256) void int4wo_gemm_lds_kernel(const LinearArgs a
 // LDS at the end.  Nothing is shared between the waves inside the loop, so it has no barrier: every wave brings in its
 // own activation slices (128 x 64 bf16 = 16 KB, double buffered in the wave's own 32 KB of LDS, 16 LDS-DMA requests a
 // step) and waits for them with its own counters.  The weights are dequantized once per workgroup, as in the 256-row
-// kernel, but a 128-row tile has only 4 matrix instructions per weight dword, so the 39 VALU instructions of the
-// dequantization bound the loop (10 per matrix instruction): about 70 cycles per matrix instruction instead of 32.
+// kernel, but a 128-row tile has only 4 matrix instructions per weight dword, so the 33 VALU instructions of the
+// dequantization bound the loop (8 per matrix instruction): about 60 cycles per matrix instruction instead of 32.
 // Slot schedule of a step: as in the 256-row kernel with 8 slots per sub-step; the DMA requests of step t + 2 go one
 // per slot into sub-step 3 (after a wait for the LDS reads of the buffer they overwrite) and sub-step 0 of step t + 1.
 template <int G>
 __global__ __launch_bounds__(256) void int4wo_gemm_kwave_kernel(const LinearArgs a, int tiles_n, int tiles_total,
                                                                  int tiles_per_xcd) {
-    constexpr int BM = 128, BN = 64, MT = 4, NT = 2, XCH = 16, SLOTS = MT * NT, OPS = (NT * DQ8_OPS + SLOTS - 1) / SLOTS;
+    constexpr int BM = 128, BN = 64, MT = 4, NT = 2, XCH = 16, SLOTS = MT * NT;
     __shared__ __align__(16) uint8_t lds[4][2][BM * 128];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -500,12 +501,11 @@ __global__ __launch_bounds__(256) void int4wo_gemm_kwave_kernel(const LinearArgs
             static_for<0, SLOTS>([&](auto q_c) __attribute__((always_inline)) {
                 constexpr int q = decltype(q_c)::value, i = q / NT, j = q % NT;
                 asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[cur][i].v), "v"(fb[cur][j].v));
-                static_for<0, OPS>([&](auto u_c) __attribute__((always_inline)) {
-                    constexpr int op = q * OPS + decltype(u_c)::value, pj = op / DQ8_OPS, o = op % DQ8_OPS;
-                    if constexpr (pj < NT) {
-                        dq8_op<o>(d[pj], wn[pj], gc[pj], magic);
-                        if constexpr (o == DQ8_OPS - 1) fb[nxt][pj].q = u32x4_t{d[pj].p0, d[pj].p1, d[pj].p2, d[pj].p3};
-                    }
+                // this slot's share of the NT * 33 dequantization instructions of the sub-step, dealt out evenly
+                static_for<q * NT * DQ8_OPS / SLOTS, (q + 1) * NT * DQ8_OPS / SLOTS>([&](auto op_c) __attribute__((always_inline)) {
+                    constexpr int op = decltype(op_c)::value, pj = op / DQ8_OPS, o = op % DQ8_OPS;
+                    dq8_op<o>(d[pj], wn[pj], gc[pj], magic);
+                    if constexpr (o == DQ8_OPS - 1) fb[nxt][pj].q = u32x4_t{d[pj].p0, d[pj].p1, d[pj].p2, d[pj].p3};
                 });
                 if constexpr (q < MT) {
                     if constexpr (ks < 3) fa[nxt][q].q = *reinterpret_cast<const u32x4_t*>(As + (afrag0 ^ ((ks + 1) << 4)) + q * 4096);
