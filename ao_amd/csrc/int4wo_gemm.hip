@@ -124,6 +124,17 @@ union Frag {
     bf16x8_t v;
 };
 
+// One accumulator register into an ordinary register.  An asm statement, because the matrix instructions are asm
+// statements too: the compiler does not know that their results arrive 16 passes later, and would place its own copies
+// of the accumulators right behind the loop, in front of the wait that follows it (a read that early returns what the
+// register held before; seen as one wrong output element in a few launches of a thousand).  Volatile statements keep
+// their order, so these reads stay behind that wait.
+__device__ __forceinline__ float acc_read(const float& a) {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+}
+
 // a workgroup-uniform pointer, moved to scalar registers (64-bit multiplies run on the VALU: without this the
 // address of a tile would live in vector registers, which the scalar-base form of the loads cannot take)
 template <class T>
@@ -315,6 +326,7 @@ __global__ __launch_bounds__(256) void int4wo_gemm_lds_kernel(const LinearArgs a
     // asm statements' latency
     // ... and the requests of the last step are still in flight: their target registers and LDS rows are not free
     // (the compiler, which sees the loaded values unused, would hand the registers to the epilogue) before they landed
+    // (the epilogue reads the accumulators through acc_read, volatile asm statements that stay behind this one)
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // the LDS buffers are free: the epilogue turns the accumulators through them
 
@@ -337,7 +349,7 @@ __global__ __launch_bounds__(256) void int4wo_gemm_lds_kernel(const LinearArgs a
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int row = 8 * (e >> 2) + 4 * kq + (e & 3);
-                    *reinterpret_cast<uint16_t*>(T + row * TS + (j * 32 + frow) * 2) = f32_to_bf16_bits(acc[i][j][e] + bv[j]);
+                    *reinterpret_cast<uint16_t*>(T + row * TS + (j * 32 + frow) * 2) = f32_to_bf16_bits(acc_read(acc[i][j][e]) + bv[j]);
                 }
             // the wave's own writes: ordered by the LDS queue, a wait is all that is needed
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -365,7 +377,7 @@ __global__ __launch_bounds__(256) void int4wo_gemm_lds_kernel(const LinearArgs a
             for (int e = 0; e < 16; ++e) {
                 const int64_t m = m0 + i * 32 + 8 * (e >> 2) + 4 * kq + (e & 3);
                 if (m < a.M) {
-                    const float v = acc[i][j][e] + bv;
+                    const float v = acc_read(acc[i][j][e]) + bv;
                     if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = v;
                     else ((uint16_t*)a.y)[m * a.ldy + n] = f32_to_bf16_bits(v);
                 }
@@ -526,6 +538,8 @@ __global__ __launch_bounds__(256) void int4wo_gemm_kwave_kernel(const LinearArgs
         step(t, 0);
         if (t + 1 < nst) step(t + 1, 1);
     }
+    // a matrix instruction's result may be read 18 issue slots after it at the earliest; the epilogue reads the
+    // accumulators through acc_read, volatile asm statements that stay behind this one
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
     // Sum of the four waves' partial tiles: every wave leaves its own in its 32 KB of LDS as fp32 [128][64] (the column
@@ -540,7 +554,7 @@ __global__ __launch_bounds__(256) void int4wo_gemm_kwave_kernel(const LinearArgs
             for (int e = 0; e < 16; ++e) {
                 const int row = 32 * i + 8 * (e >> 2) + 4 * kq + (e & 3);
                 const int col = (32 * j + frow) ^ (kq << 5);
-                *reinterpret_cast<float*>(Lw + (row * 64 + col) * 4) = acc[i][j][e];
+                *reinterpret_cast<float*>(Lw + (row * 64 + col) * 4) = acc_read(acc[i][j][e]);
             }
     __syncthreads();
     const int r = lane >> 4, c4 = lane & 15;

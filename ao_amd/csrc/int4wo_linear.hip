@@ -1025,7 +1025,11 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // N = 4096: 64 workgroups on 256 CUs, each walking all of K); the streaming kernel over chunks of 16 rows
     // keeps every CU busy there and re-reads the weight from the last-level cache.
     const int64_t gemm_small_wgs = ((RB + 3) / 4) * ((M + 63) / 64);
-    const bool gemm_starved = (M <= 32 && gemm_small_wgs < 128) || (M <= 64 && gemm_small_wgs <= 64);
+    // (measured, us, streaming / 32 x 64 tiles with K split in the workgroup: 4096 x 14336 at 32, 40, 64 rows 34 / 40,
+    // 42.5 / 40.6, 62 / 40; 4096 x 4096 at 40, 48, 64 rows 13.4 / 13.8, 14.8 / 13.7, 18.7 / 14; 1024 x 4096 8.7 / 13.8 at
+    // every count up to 64)
+    const bool gemm_starved = (M <= 32 && gemm_small_wgs < 128) || (M <= 40 && gemm_small_wgs <= 64) ||
+                              (M <= 64 && gemm_small_wgs <= 16);
     AO_REQUIRE(ksplit == 1 || (xmode == X_LDS && M <= 16 && !dual && !pair8 && !bias_bf16 && !residual_bf16 && y_dtype == AO_F32),
                "partial sums over a split K need M <= 16, fp32 output, no bias / residual epilogue and activations that "
                "fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);

@@ -170,7 +170,8 @@ def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched
       * the K loop carries the LDS-direct activation requests (16 per two steps and wave of the 256-row kernel, 32 of the
         128-row kernel, whose waves each bring in their own slices) and the weight requests (a chunk and its scale / zero
         per 32-row block) of its two steps;
-      * no scratch access inside the K loop, every matrix instruction accumulates in accumulation registers."""
+      * no scratch access inside the K loop, every matrix instruction accumulates in accumulation registers;
+      * no accumulator is read before the wait that follows the loop."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         pytest.skip("hipcc not available")
@@ -211,6 +212,13 @@ def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched
                     continue
                 j += 1
             assert j < len(lines), (name, lines[i])
+        # the accumulators are first read behind the wait that follows the loop: the matrix instructions are asm
+        # statements, whose result latency the compiler does not know, so a copy placed right behind the loop would
+        # read a register the last matrix instructions have not written yet
+        last_mfma = max(i for i, l in enumerate(lines) if l.startswith("v_mfma"))
+        nops = [i for i, l in enumerate(lines) if l == "s_nop 15" and i > last_mfma]
+        assert nops, name
+        assert not [l for l in lines[:nops[0]] if l.startswith(("v_accvgpr_read", "v_accvgpr_mov"))], name
         # values the epilogue needs may be parked in scratch around the loop, never inside it
         assert not [l for l in lines[loop_head:loop_end] if l.startswith("scratch_")], name
         assert len(re.findall(r"v_mfma_f32_32x32x16_bf16 a\[", body)) >= (64 * nt if dma == 16 else 64), name
