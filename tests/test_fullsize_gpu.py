@@ -267,3 +267,38 @@ def test_prefill_gemm_tiles_edges_and_repeated_launches(cabi, M, N, K, g, bias, 
     torch.cuda.synchronize()
     exact = bool(torch.equal(yh, dq.float().t()[ks]))
     assert exact
+
+
+@pytest.mark.parametrize("M,N,K,g", [(2048, 14336, 4096, 64), (512, 14336, 4096, 128), (512, 4096, 14336, 256),
+                                     (128, 14336, 4096, 64)])
+def test_prefill_gemm_launches_repeat_bit_for_bit(cabi, M, N, K, g):
+    """The prefill kernels sum in a fixed order, so 40 launches on the same operands must give the same fp32 bits; a
+    result read before its matrix instruction has finished (their latency is the kernels' own business: the
+    instructions are asm statements) shows up as a launch that differs in a few elements."""
+    plan = cabi.int4wo_linear_plan(M, K, N, g)
+    print(f"case prefill gemm repeat M={M} N={N} K={K} g={g}: {plan}", flush=True)
+    assert plan.startswith(("int4wo_gemm_lds_kernel", "int4wo_gemm_kwave_kernel"))
+    dev = torch.device("cuda:0")
+    L = cabi.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device=dev).manual_seed(M + N + K + g)
+    w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).bfloat16()
+    _, _, pb, qb = cabi.packed_shape(N, K, g)
+    packed = torch.empty(pb // 4, dtype=torch.int32, device=dev)
+    qp = torch.empty(qb // 4, dtype=torch.int32, device=dev)
+    cabi.check(L.ao_amd_int4wo_quantize_pack(w.data_ptr(), N, K, K, g, packed.data_ptr(), qp.data_ptr(), st))
+    del w
+    x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
+    first = torch.empty(M, N, dtype=torch.float32, device=dev)
+    y = torch.empty_like(first)
+    differing = []
+    for rep in range(40):
+        out = first if rep == 0 else y
+        out.fill_(float("nan"))
+        cabi.check(L.ao_amd_int4wo_linear(x.data_ptr(), M, K, K, packed.data_ptr(), qp.data_ptr(), N, g, None, out.data_ptr(),
+                                          cabi.F32, N, st))
+        torch.cuda.synchronize()
+        if rep and not torch.equal(y, first):
+            differing.append((rep, int((y != first).sum())))
+    finite = bool(torch.isfinite(first).all())
+    assert finite and differing == []
