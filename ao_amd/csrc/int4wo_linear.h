@@ -56,16 +56,21 @@ typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
 struct GroupConst {
-    uint32_t s_lo, s_hi;  // packed bf16 (s, 0) and (0, s)
+    uint32_t s_lo, s_hi;  // packed bf16 (s, 0) and (0, s); s_hi is also the scale as fp32
     float c136;           // -136 * s (exact in fp32)
     float z;
+    float c1032, s16, c72;  // -1032 * s, s / 16, -72 * s: the constants of first_half (exact in fp32)
 };
 __device__ __forceinline__ GroupConst make_group(uint32_t qp) {
     GroupConst g;
     g.s_lo = qp & 0xffffu;
     g.s_hi = qp << 16;
-    g.c136 = -136.0f * __uint_as_float(qp << 16);
+    const float s = __uint_as_float(qp << 16);
+    g.c136 = -136.0f * s;
     g.z = __uint_as_float(qp & 0xffff0000u);
+    g.c1032 = -1032.0f * s;
+    g.s16 = 0.0625f * s;
+    g.c72 = -72.0f * s;
     return g;
 }
 

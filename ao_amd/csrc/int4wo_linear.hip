@@ -9,8 +9,9 @@
 // Dequantization is the reference's dequantize_affine (torchao/quantization/quant_primitives.py:265-274)
 // with both bf16 roundings kept: w = bf16( bf16((q-8)*s) + z ).  Dropping them costs 1.8e-3 relative
 // L2 error on the output, above the 1e-3 tolerance of the path.  Per pair of elements:
-//   P  = (dword >> 4v) & 0x000F000F | 0x43004300      two bf16 values 128+q          (1 v_and_or)
-//   t  = P.lo*s + P.hi*0 - 136*s  /  P.lo*0 + P.hi*s - 136*s   exact (q-8)*s in fp32  (2 v_dot2_f32_bf16)
+//   P  = dword & 0x000F000F | 0x64006400               two fp16 values 1024+q         (1 v_and_or; the pair at
+//        bits 4 / 20 is masked in place, 1024+16q, with the factor 16 in the scale; one shift serves the other two)
+//   t  = P.half * s - 1032*s                            exact (q-8)*s in fp32          (2 v_fma_mix_f32)
 //   T  = cvt_pk_bf16(t0, t1)                           first rounding                 (1 v_cvt_pk_bf16_f32)
 //   u  = T.lo*1 + T.hi*0 + z  /  T.lo*0 + T.hi*1 + z   fp32 add of the bf16 operands  (2 v_dot2_f32_bf16)
 //   W  = cvt_pk_bf16(u0, u1)                           second rounding                (1 v_cvt_pk_bf16_f32)
@@ -27,7 +28,7 @@ namespace ao {
 // matrix core overlap; each stage is one asm volatile block (volatile blocks keep their program order, which
 // is what carries the dependency distances the hardware needs):
 //
-//   stage 1  first_half   VALU: 8 codes -> T = bf16((q-8)*s) as 4 packed pairs       (19 instructions)
+//   stage 1  first_half   VALU: 8 codes -> T = bf16((q-8)*s) as 4 packed pairs       (17 instructions)
 //   stage 2  add_zero     MFMA x2: u = T + z for the lane's own 8 values, in fp32.  With B = T (lane (row, qd)
 //                         holds kk = 8*qd + e) and the 0/1 selection matrices sel_a[i][kk] = (kk == 8*(i/4) + i%4),
 //                         sel_b = the same + 4, the 16x16 results C[i][row] = T[row][8*(i/4) + i%4 (+4)] + z land
@@ -37,34 +38,38 @@ namespace ao {
 //
 // A 4-pass MFMA result may be read by the VALU 7 issue slots later at the earliest; the caller puts stage 1
 // of the NEXT dword between stage 2 and stage 3 of the current one, which fills those slots with useful work.
-__device__ __forceinline__ u32x4_t first_half(uint32_t w, const GroupConst& g, uint32_t magic) {
-    uint32_t p0, p1, p2, p3;
+__device__ __forceinline__ u32x4_t first_half(uint32_t w, const GroupConst& g, uint32_t) {
+    // t = bf16((q - 8) * s) for the 8 codes of a dword, on the ordinary VALU (v_dot2 shares the matrix pipe with the
+    // three matrix instructions a dword already costs there): the code pairs sit at bits (0, 16), (4, 20), (8, 24),
+    // (12, 28); dword & 0x000F000F | 0x64006400 is the fp16 pair (1024 + q, 1024 + q'), dword & 0x00F000F0 | 0x64006400
+    // is (1024 + 16 q, 1024 + 16 q') with the factor 16 moved into the scale, one shift by 8 serves the other two pairs;
+    // v_fma_mix_f32 reads one fp16 half and computes (1024 + q) * s - 1032 * s, exact in fp32.
+    uint32_t p0, p1, p2, p3, ws;
     float a0, a1, a2, a3, a4, a5, a6, a7;
+    const uint32_t magic16 = 0x64006400u;
     asm volatile(
-        "v_and_or_b32 %[p0], %[w], %[mask], %[magic]\n\t"
-        "v_lshrrev_b32 %[p1], 4, %[w]\n\t"
-        "v_lshrrev_b32 %[p2], 8, %[w]\n\t"
-        "v_lshrrev_b32 %[p3], 12, %[w]\n\t"
-        "v_and_or_b32 %[p1], %[p1], %[mask], %[magic]\n\t"
-        "v_and_or_b32 %[p2], %[p2], %[mask], %[magic]\n\t"
-        "v_and_or_b32 %[p3], %[p3], %[mask], %[magic]\n\t"
-        "v_dot2_f32_bf16 %[a0], %[p0], %[slo], %[c]\n\t"
-        "v_dot2_f32_bf16 %[a1], %[p0], %[shi], %[c]\n\t"
-        "v_dot2_f32_bf16 %[a2], %[p1], %[slo], %[c]\n\t"
-        "v_dot2_f32_bf16 %[a3], %[p1], %[shi], %[c]\n\t"
-        "v_dot2_f32_bf16 %[a4], %[p2], %[slo], %[c]\n\t"
-        "v_dot2_f32_bf16 %[a5], %[p2], %[shi], %[c]\n\t"
-        "v_dot2_f32_bf16 %[a6], %[p3], %[slo], %[c]\n\t"
-        "v_dot2_f32_bf16 %[a7], %[p3], %[shi], %[c]\n\t"
+        "v_and_or_b32 %[p0], %[w], %[me], %[magic]\n\t"
+        "v_and_or_b32 %[p1], %[w], %[mo], %[magic]\n\t"
+        "v_lshrrev_b32 %[ws], 8, %[w]\n\t"
+        "v_and_or_b32 %[p2], %[ws], %[me], %[magic]\n\t"
+        "v_and_or_b32 %[p3], %[ws], %[mo], %[magic]\n\t"
+        "v_fma_mix_f32 %[a0], %[p0], %[s], %[c] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %[a1], %[p0], %[s], %[c] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %[a2], %[p1], %[s16], %[c16] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %[a3], %[p1], %[s16], %[c16] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %[a4], %[p2], %[s], %[c] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %[a5], %[p2], %[s], %[c] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %[a6], %[p3], %[s16], %[c16] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %[a7], %[p3], %[s16], %[c16] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
         "v_cvt_pk_bf16_f32 %[p0], %[a0], %[a1]\n\t"
         "v_cvt_pk_bf16_f32 %[p1], %[a2], %[a3]\n\t"
         "v_cvt_pk_bf16_f32 %[p2], %[a4], %[a5]\n\t"
         "v_cvt_pk_bf16_f32 %[p3], %[a6], %[a7]\n\t"
         "s_nop 1"
-        : [p0] "=&v"(p0), [p1] "=&v"(p1), [p2] "=&v"(p2), [p3] "=&v"(p3), [a0] "=&v"(a0), [a1] "=&v"(a1),
+        : [p0] "=&v"(p0), [p1] "=&v"(p1), [p2] "=&v"(p2), [p3] "=&v"(p3), [ws] "=&v"(ws), [a0] "=&v"(a0), [a1] "=&v"(a1),
           [a2] "=&v"(a2), [a3] "=&v"(a3), [a4] "=&v"(a4), [a5] "=&v"(a5), [a6] "=&v"(a6), [a7] "=&v"(a7)
-        : [w] "v"(w), [mask] "s"(0x000F000Fu), [magic] "v"(magic), [slo] "v"(g.s_lo), [shi] "v"(g.s_hi),
-          [c] "v"(g.c136));
+        : [w] "v"(w), [me] "s"(0x000F000Fu), [mo] "s"(0x00F000F0u), [magic] "v"(magic16), [s] "v"(g.s_hi), [c] "v"(g.c1032),
+          [s16] "v"(g.s16), [c16] "v"(g.c72));
     const u32x4_t t = {p0, p1, p2, p3};
     return t;
 }
@@ -154,11 +159,14 @@ __device__ __forceinline__ GroupRegs make_group_asm(uint32_t qp) {
         "v_lshlrev_b32 %[shi], 16, %[q]\n\t"
         "v_and_b32 %[z0], 0xffff0000, %[q]\n\t"
         "v_mul_f32 %[c], 0xc3080000, %[shi]\n\t"
+        "v_mul_f32 %[c1032], 0xc4810000, %[shi]\n\t"
+        "v_mul_f32 %[s16], 0x3d800000, %[shi]\n\t"
+        "v_mul_f32 %[c72], 0xc2900000, %[shi]\n\t"
         "v_mov_b32 %[z1], %[z0]\n\t"
         "v_mov_b32 %[z2], %[z0]\n\t"
         "v_mov_b32 %[z3], %[z0]"
-        : [slo] "=&v"(r.g.s_lo), [shi] "=&v"(r.g.s_hi), [c] "=&v"(r.g.c136), [z0] "=&v"(z0), [z1] "=&v"(z1),
-          [z2] "=&v"(z2), [z3] "=&v"(z3)
+        : [slo] "=&v"(r.g.s_lo), [shi] "=&v"(r.g.s_hi), [c] "=&v"(r.g.c136), [c1032] "=&v"(r.g.c1032), [s16] "=&v"(r.g.s16),
+          [c72] "=&v"(r.g.c72), [z0] "=&v"(z0), [z1] "=&v"(z1), [z2] "=&v"(z2), [z3] "=&v"(z3)
         : [q] "v"(qp));
     r.g.z = z0;
     r.zz = f32x4_t{z0, z1, z2, z3};
@@ -394,7 +402,7 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
     constexpr int LPT = DUAL ? 4 : 2;  // loads per tile
     u32x4_t tcur = {0, 0, 0, 0};  // stage-1 result of the dword that enters stage 2 next
     GroupRegs gnext;              // group constants of the tile whose dword 0 is in tcur
-    gnext.g.s_lo = gnext.g.s_hi = 0; gnext.g.c136 = 0.f; gnext.g.z = 0.f;
+    gnext.g.s_lo = gnext.g.s_hi = 0; gnext.g.c136 = 0.f; gnext.g.z = 0.f; gnext.g.c1032 = gnext.g.s16 = gnext.g.c72 = 0.f;
     gnext.zz = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     auto compute_tile = [&](const GemvTile& b, int kb, const GemvTile& nb, bool has_next, int younger_of_next) {
