@@ -337,6 +337,134 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(const LinearA
     }
 }
 
+// The same kernel with four 16-row blocks of W per workgroup, for 5 to 16 activation rows that do not fit the LDS
+// staging of the skinny path (K = 4096 at 8 or 16 rows).  There every 16-row block re-reads all activation rows from L2,
+// four times the bytes of its weights at 16 rows (896 workgroups x 128 KB on 14336 x 4096), and the fill rate of a
+// CU's L1 (about 20 bytes per cycle), not memory, sets the time.  Here a wave loads the activation fragments of a K
+// tile once and runs them against the tiles of four row blocks: a quarter of the activation traffic, four accumulators.
+template <int G, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const LinearArgs a) {
+    constexpr int D = 2, RBW = 4;
+    static_assert(WAVES <= 8, "the reduction buffer is 4 KB per row block and wave");
+    __shared__ float red[RBW][WAVES][4][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, qd = lane >> 4;
+    const int64_t rb0 = (int64_t)blockIdx.x * RBW;
+    const int64_t m0 = (int64_t)blockIdx.y * 16;
+    const int KB = (int)(a.Kp / 128);
+    const uint32_t magic = 0x43004300u;
+    const bool sel_lane = qd == (r >> 2);
+    const uint32_t one_bits = (r & 1) ? 0x3F800000u : 0x00003F80u;
+    const uint32_t s_even = (sel_lane && ((r & 3) >> 1) == 0) ? one_bits : 0u;
+    const uint32_t s_odd = (sel_lane && ((r & 3) >> 1) == 1) ? one_bits : 0u;
+    const u32x4_t sel_a = {s_even, s_odd, 0u, 0u};
+    const u32x4_t sel_b = {0u, 0u, s_even, s_odd};
+
+    const bool xact = (m0 + r) < a.M;
+    const uint16_t* xp = a.x + (xact ? (m0 + r) : 0) * a.ldx + qd * 32;
+    f32x4_t acc[RBW];
+#pragma unroll
+    for (int j = 0; j < RBW; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    struct Buf {
+        u32x4_t w[RBW];
+        uint32_t q[RBW];
+        uint4 x[4];
+    };
+    auto load_tile = [&](Buf& b, int kb) {
+        const int gidx = ((kb * 128 + qd * 32) / G) * 16;
+#pragma unroll
+        for (int j = 0; j < RBW; ++j) {
+            b.w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(a.packed + ((rb0 + j) * KB + kb) * 64 + lane));
+            b.q[j] = a.qparams[(rb0 + j) * (a.Kp / G) * 16 + r + gidx];
+        }
+        if (xact) {
+            const uint4* xv = reinterpret_cast<const uint4*>(xp + (int64_t)kb * 128);
+#pragma unroll
+            for (int sl = 0; sl < 4; ++sl) b.x[sl] = xv[sl];
+        }
+    };
+    u32x4_t tcur = {0, 0, 0, 0};
+    // one tile = 16 dwords per lane (4 row blocks x 4); the three dequantization stages run as in int4wo_linear_kernel
+    auto compute_tile = [&](const Buf& b, const Buf& nb, bool has_next) {
+        GroupConst gc[RBW];
+#pragma unroll
+        for (int j = 0; j < RBW; ++j) gc[j] = make_group(b.q[j]);
+#pragma unroll
+        for (int e = 0; e < 4 * RBW; ++e) {
+            const int j = e >> 2;
+            union { uint4 q; bf16x8_t v; } xa;
+            xa.q = b.x[e & 3];
+            f32x4_t ua, ub;
+            const f32x4_t zz = {gc[j].z, gc[j].z, gc[j].z, gc[j].z};
+            add_zero(tcur, zz, sel_a, sel_b, ua, ub);
+            bf16x8_t bw;
+            if (e + 1 < 4 * RBW) {
+                tcur = first_half(b.w[(e + 1) >> 2][(e + 1) & 3], gc[(e + 1) >> 2], magic);
+                bw = round_pack<false>(ua, ub);
+            } else if (has_next) {
+                tcur = first_half(nb.w[0].x, make_group(nb.q[0]), magic);
+                bw = round_pack<false>(ua, ub);
+            } else {
+                bw = round_pack<true>(ua, ub);
+            }
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw, acc[j], 0, 0, 0);
+        }
+    };
+
+    Buf buf[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+#pragma unroll
+        for (int j = 0; j < RBW; ++j) {
+            buf[d].w[j] = u32x4_t{0, 0, 0, 0};
+            buf[d].q[j] = 0;
+        }
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) buf[d].x[sl] = make_uint4(0, 0, 0, 0);   // rows >= M keep these zeros
+    }
+    if (wave < KB) load_tile(buf[0], wave);
+    const int nt = wave < KB ? (KB - wave + WAVES - 1) / WAVES : 0;
+    if (nt > 0) tcur = first_half(buf[0].w[0].x, make_group(buf[0].q[0]), magic);
+    for (int i0 = 0; i0 < nt; i0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int i = i0 + d;
+            if (i < nt) {
+                if (i + 1 < nt) load_tile(buf[(d + 1) % D], wave + (i + 1) * WAVES);
+                compute_tile(buf[d], buf[(d + 1) % D], i + 1 < nt);
+            }
+        }
+    }
+
+    // acc[j][i] = C[m = 4*qd + i][n = 16 (rb0 + j) + r]
+#pragma unroll
+    for (int j = 0; j < RBW; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[j][wave][i][lane] = acc[j][i];
+    __syncthreads();
+    if (wave < RBW) {   // wave j finishes row block j
+        const int j = wave;
+        const int64_t n = (rb0 + j) * 16 + r;
+        float bv = 0.f;
+        if (a.bias && n < a.N) bv = bf16_bits_to_f32(a.bias[n]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) sum += red[j][w][i][lane];
+            const int64_t m = m0 + 4 * qd + i;
+            if (m < a.M && n < a.N) {
+                sum += bv;
+                if (a.residual) sum = rne_bf16(sum) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
+                if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = sum;
+                else ((uint16_t*)a.y)[m * a.ldy + n] = f32_to_bf16_bits(sum);
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- skinny path (M <= 16 rows staged in LDS)
 // The decode kernel.  Same tiling as int4wo_linear_kernel, tuned for instruction count: the wave index is
 // made scalar so that every tile-loop branch is a scalar branch, the weight / qparam streams are addressed as
@@ -1088,6 +1216,41 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
         if (int4wo_gemv1_plan(a, g, RB, name, sizeof(name))) {
             AO_PLAN("%s", name);
             launch_int4wo_gemv1(a, g, RB, st);
+            AO_LAUNCH_CHECK();
+            return 0;
+        }
+    }
+    // 4 to 16 rows (and the 16-row chunks of a few more): four row blocks per workgroup while that leaves at least 192
+    // workgroups (see int4wo_linear_rb4_kernel).  Measured on 14336 x 4096, us at 2 / 3 / 4 / 5 / 8 / 12 / 16 rows: 13.1 /
+    // 13.9 / 13.5 / 13.6 / 13.7 / 13.7 / 14.1 against 12.8 / 14.0 / 14.2 / 16.4 / 14.8 / 18.2 / 20.6 of the kernels below
+    // (LDS-staged up to 5 rows there); the vocabulary head at 16 rows 85 against 129.
+    if ((xmode == X_GLOBAL || (xmode == X_LDS && !norm_weight_bf16 && !pair8)) && !dual && ksplit == 1 && M >= 4 &&
+        RB % 4 == 0 && (RB / 4) * mchunks >= 192 && a.K == a.Kp) {
+        static const bool rb4_disabled = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
+        if (!rb4_disabled) {
+            const int64_t wgs = (RB / 4) * mchunks;
+            int w4 = 4;   // at least four waves: wave j finishes row block j
+            while (w4 < 8 && wgs * w4 * 2 <= 4096 + wgs && w4 * 2 <= a.Kp / 128) w4 *= 2;
+            AO_PLAN("int4wo_linear_rb4_kernel<%lld,%d>", (long long)g, w4);
+            const dim3 grid4((unsigned)(RB / 4), (unsigned)mchunks);
+            auto go = [&](auto kernel, int nw) {
+                if (g_prof_start && g_prof_stop) {
+                    hipExtLaunchKernelGGL(kernel, grid4, dim3(nw * 64), 0, st, g_prof_start, g_prof_stop, 0, a);
+                    g_prof_start = g_prof_stop = nullptr;
+                } else {
+                    hipLaunchKernelGGL(kernel, grid4, dim3(nw * 64), 0, st, a);
+                }
+            };
+#define AO_RB4(GG)                                                  \
+    if (w4 == 4) go(int4wo_linear_rb4_kernel<GG, 4>, 4);            \
+    else go(int4wo_linear_rb4_kernel<GG, 8>, 8)
+            switch (g) {
+                case 32: AO_RB4(32); break;
+                case 64: AO_RB4(64); break;
+                case 128: AO_RB4(128); break;
+                default: AO_RB4(256); break;
+            }
+#undef AO_RB4
             AO_LAUNCH_CHECK();
             return 0;
         }

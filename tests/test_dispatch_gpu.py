@@ -46,12 +46,14 @@ def test_dispatch_walk_finds_every_kernel_family():
     plans = _walk()
     families = {n.split("<")[0] for n in plans}
     assert families == {"int4wo_gemv1_kernel", "int4wo_gemv_kernel", "int4wo_linear_kernel", "int4wo_gemm_kernel",
-                        "int4wo_gemm_ksplit_kernel", "int4wo_gemm_lds_kernel", "int4wo_gemm_kwave_kernel"}
+                        "int4wo_gemm_ksplit_kernel", "int4wo_gemm_lds_kernel", "int4wo_gemm_kwave_kernel",
+                        "int4wo_linear_rb4_kernel"}
     # the tile variants of the matrix-core kernels and both K-split forms
     for g in GROUPS:
         for tile in ("int4wo_gemm_kernel<%d,2,8>", "int4wo_gemm_kernel<%d,1,4>", "int4wo_gemm_kernel<%d,1,2>",
                      "int4wo_gemm_ksplit_kernel<%d,4,4>", "int4wo_gemm_ksplit_kernel<%d,2,4>",
-                     "int4wo_gemm_lds_kernel<%d,1>", "int4wo_gemm_lds_kernel<%d,2>", "int4wo_gemm_kwave_kernel<%d>"):
+                     "int4wo_gemm_lds_kernel<%d,1>", "int4wo_gemm_lds_kernel<%d,2>", "int4wo_gemm_kwave_kernel<%d>",
+                     "int4wo_linear_rb4_kernel<%d,4>", "int4wo_linear_rb4_kernel<%d,8>"):
             assert tile % g in plans, tile % g
     # the single-row kernel: exactly the instantiations that int4wo_gemv1.hip compiles (waves, chunks per lane, norm)
     gemv1 = {n.split(" ")[0] for n in plans if n.startswith("int4wo_gemv1_kernel<")}
@@ -72,7 +74,12 @@ def test_dispatch_walk_finds_every_kernel_family():
     assert _lib.int4wo_linear_plan(512, 14336, 4096, 64) == "int4wo_gemm_kwave_kernel<64>"
     assert not _lib.int4wo_linear_plan(128, 4096, 4096, 64).startswith("int4wo_gemm_kwave_kernel")   # 64 tiles
     assert not _lib.int4wo_linear_plan(99, 1024, 14336, 64).startswith("int4wo_gemm_kwave_kernel")
-    assert len(plans) >= 72
+    # 4 to 16 rows on weights with 768 or more 16-row blocks: four row blocks per workgroup share the activation loads
+    assert _lib.int4wo_linear_plan(16, 4096, 14336, 64) == "int4wo_linear_rb4_kernel<64,8>"
+    assert _lib.int4wo_linear_plan(4, 4096, 128256, 64) == "int4wo_linear_rb4_kernel<64,4>"
+    assert not _lib.int4wo_linear_plan(16, 14336, 4096, 64).startswith("int4wo_linear_rb4_kernel")   # 64 workgroups
+    assert not _lib.int4wo_linear_plan(3, 4096, 14336, 64).startswith("int4wo_linear_rb4_kernel")
+    assert len(plans) >= 80
 
 
 def _cases():

@@ -302,3 +302,44 @@ def test_prefill_gemm_launches_repeat_bit_for_bit(cabi, M, N, K, g):
             differing.append((rep, int((y != first).sum())))
     finite = bool(torch.isfinite(first).all())
     assert finite and differing == []
+
+
+@pytest.mark.parametrize("M,N,K,g,bias,residual,fp32", [(13, 14400, 1024, 128, True, False, False), (16, 14336, 4096, 64, False, True, False),
+                                                        (4, 16384, 2048, 32, True, True, False), (9, 14336, 4096, 256, True, False, True)])
+def test_four_row_blocks_per_workgroup_kernel_epilogues(cabi, M, N, K, g, bias, residual, fp32):
+    """int4wo_linear_rb4_kernel (4 to 16 activation rows, four 16-row weight blocks per workgroup sharing the activation
+    loads): bias, residual (y = bf16(bf16(acc + bias) + residual), the order of the unfused modules), fp32 output and
+    ragged M, against an fp32 matmul on the bit-exact dequantized weight."""
+    plan = cabi.int4wo_linear_plan(M, K, N, g, residual=residual)
+    print(f"case rb4 M={M} N={N} K={K} g={g} bias={bias} residual={residual} fp32={fp32}: {plan}", flush=True)
+    assert plan.startswith("int4wo_linear_rb4_kernel")
+    dev = torch.device("cuda:0")
+    L = cabi.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device=dev).manual_seed(M + N + K)
+    w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).bfloat16()
+    _, _, pb, qb = cabi.packed_shape(N, K, g)
+    packed = torch.empty(pb // 4, dtype=torch.int32, device=dev)
+    qp = torch.empty(qb // 4, dtype=torch.int32, device=dev)
+    cabi.check(L.ao_amd_int4wo_quantize_pack(w.data_ptr(), N, K, K, g, packed.data_ptr(), qp.data_ptr(), st))
+    dq = torch.empty(N, K, dtype=torch.bfloat16, device=dev)
+    cabi.check(L.ao_amd_int4wo_dequantize(packed.data_ptr(), qp.data_ptr(), N, K, g, dq.data_ptr(), st))
+    b = (torch.randn(N, device=dev, generator=gen) * 0.1).bfloat16() if bias else None
+    res = torch.randn(M, N, device=dev, generator=gen).bfloat16() if residual else None
+    x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
+    ref = x.float() @ dq.float().t()
+    if bias:
+        ref = ref + b.float()
+    y = torch.full((M, N), float("nan"), dtype=torch.float32 if fp32 else torch.bfloat16, device=dev)
+    if residual:
+        ref = ref.bfloat16().float() + res.float()
+        cabi.check(L.ao_amd_int4wo_linear_residual(x.data_ptr(), M, K, K, packed.data_ptr(), qp.data_ptr(), N, g,
+                                                   None if b is None else b.data_ptr(), res.data_ptr(), N, y.data_ptr(), N, st))
+    else:
+        cabi.check(L.ao_amd_int4wo_linear(x.data_ptr(), M, K, K, packed.data_ptr(), qp.data_ptr(), N, g,
+                                          None if b is None else b.data_ptr(), y.data_ptr(), cabi.F32 if fp32 else cabi.BF16, N, st))
+    torch.cuda.synchronize()
+    finite = bool(torch.isfinite(y.float()).all())
+    want = ref if fp32 else ref.bfloat16().float()
+    err = float((y.float() - want).norm() / ref.norm())
+    assert finite and err <= (2e-5 if fp32 else 1.5e-3)
