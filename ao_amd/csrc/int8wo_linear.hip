@@ -314,6 +314,109 @@ __global__ __launch_bounds__(WAVES * 64) void int8wo_linear_kernel(const Int8Arg
     }
 }
 
+// The unstaged kernel with four 16-row blocks of W per workgroup, for activation rows that do not fit the LDS staging
+// (9 and more rows at K = 4096): every row block re-reads all activation rows from L2 there, twice the bytes of its int8
+// weights at 16 rows, and a CU's L1 fill rate (about 20 bytes per cycle), not memory, sets the time.  A wave loads the
+// activation fragments of a K tile once and runs them against the tiles of four row blocks; wave j finishes block j.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void int8wo_linear_rb4_kernel(const Int8Args a) {
+    constexpr int RBW = 4;
+    static_assert(WAVES >= RBW && WAVES <= 8, "wave j finishes row block j; 4 KB of reduction buffer per block and wave");
+    __shared__ float red[RBW][WAVES][4][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, qd = lane >> 4;
+    const int64_t rb0 = (int64_t)blockIdx.x * RBW, m0 = (int64_t)blockIdx.y * 16;
+    const int KB = (int)(a.K / 128);
+    const int64_t mrow = m0 + r < a.M ? m0 + r : a.M - 1;   // rows past M alias the last one, never stored
+    const int8_t* wp[RBW];
+#pragma unroll
+    for (int j = 0; j < RBW; ++j) {
+        const int64_t n = (rb0 + j) * 16 + r;
+        wp[j] = a.w + (n < a.N ? n : a.N - 1) * a.ldw + qd * 32;
+    }
+    const uint16_t* xp = a.x + mrow * a.ldx + qd * 32;
+    f32x4_t acc[RBW];
+#pragma unroll
+    for (int j = 0; j < RBW; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    struct Buf { u32x4_t w0[RBW], w1[RBW]; u32x4_t x[4]; };
+    auto load_tile = [&](Buf& b, int kb) {
+#pragma unroll
+        for (int j = 0; j < RBW; ++j) {
+            const u32x4_t* wv = reinterpret_cast<const u32x4_t*>(wp[j] + (int64_t)kb * 128);
+            b.w0[j] = __builtin_nontemporal_load(wv);
+            b.w1[j] = __builtin_nontemporal_load(wv + 1);
+        }
+        const u32x4_t* xv = reinterpret_cast<const u32x4_t*>(xp + (int64_t)kb * 128);
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) b.x[sl] = xv[sl];
+    };
+    auto compute_tile = [&](const Buf& b) {
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            union { u32x4_t q; bf16x8_t v; } xa;
+            xa.q = b.x[sl];
+#pragma unroll
+            for (int j = 0; j < RBW; ++j) {
+                const uint32_t ww[8] = {b.w0[j].x, b.w0[j].y, b.w0[j].z, b.w0[j].w, b.w1[j].x, b.w1[j].y, b.w1[j].z, b.w1[j].w};
+                union { uint32_t u[4]; bf16x8_t v; } bw;
+                int8x4_to_bf16(ww[2 * sl], bw.u[0], bw.u[1]);
+                int8x4_to_bf16(ww[2 * sl + 1], bw.u[2], bw.u[3]);
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw.v, acc[j], 0, 0, 0);
+            }
+        }
+    };
+    {
+        Buf b0, b1;
+        int kb = wave;
+        if (kb < KB) load_tile(b0, kb);
+        while (kb < KB) {
+            const int kb1 = kb + WAVES, kb2 = kb + 2 * WAVES;
+            if (kb1 < KB) load_tile(b1, kb1);
+            compute_tile(b0);
+            if (kb1 < KB) {
+                if (kb2 < KB) load_tile(b0, kb2);
+                compute_tile(b1);
+            }
+            kb = kb2;
+        }
+    }
+    // acc[j][i] = C[m = 4*qd + i][n = 16 (rb0 + j) + r]
+#pragma unroll
+    for (int j = 0; j < RBW; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[j][wave][i][lane] = acc[j][i];
+    __syncthreads();
+    if (wave < RBW) {
+        const int64_t n = (rb0 + wave) * 16 + r;
+        if (n < a.N) {
+            const float sc = bf16_bits_to_f32(a.scale[n]);
+            const float bv = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) s += red[wave][w][i][lane];
+                const int64_t m = m0 + 4 * qd + i;
+                if (m < a.M) {
+                    // the epilogue of int8wo_linear_kernel: mm result rounded to bf16, times scale, plus bias, then the
+                    // fused residual or gate
+                    float v = hw_rne_bf16(s) * sc;
+                    if (a.bias) v = hw_rne_bf16(v) + bv;
+                    if (a.residual) v = hw_rne_bf16(v) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
+                    if (a.gate) {
+                        const float gt = bf16_bits_to_f32(a.gate[m * a.ldgate + n]);
+                        v = hw_rne_bf16(gt / (1.0f + expf(-gt))) * hw_rne_bf16(v);
+                    }
+                    if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = v;
+                    else ((uint16_t*)a.y)[m * a.ldy + n] = hw_bf16_bits(v);
+                }
+            }
+        }
+    }
+}
+
 // int8 [N,K] (row stride ldw) -> bf16 [N,K]: the `w_int8.to(x.dtype)` of the reference's formula as its own pass, for
 // batches large enough that a plain bf16 GEMM on the converted weight beats re-streaming the int8 weight per 16 rows.
 // 16 codes in, 32 bytes out per thread; every int8 value is exact in bf16.
@@ -392,8 +495,23 @@ static int int8wo_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
                (const uint16_t*)bias_bf16, N, y, y_dtype == AO_F32, ldy, (const uint16_t*)residual_bf16, ldres,
                (const uint16_t*)gate_bf16, ldgate, (const uint16_t*)norm_weight_bf16, norm_eps, (const int8_t*)w_up_int8,
                (const uint16_t*)scale_up_bf16};
-    dim3 grid((unsigned)RB, (unsigned)mchunks);
     hipStream_t st = (hipStream_t)stream;
+    // unstaged rows on a weight with 768 or more row blocks: four row blocks per workgroup share the activation loads
+    // (14336 x 4096 at 16 rows: measured against the one-block kernel below)
+    static const bool rb4_disabled = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
+    if (!staged && !rb4_disabled && RB % 4 == 0 && (RB / 4) * mchunks >= 192 && KB >= 8) {
+        const int64_t wgs = (RB / 4) * mchunks;
+        int w4 = 4;
+        while (w4 < 8 && wgs * w4 * 2 <= 4096 + wgs && w4 * 2 <= KB) w4 *= 2;
+        const dim3 grid4((unsigned)(RB / 4), (unsigned)mchunks);
+        hipEvent_t ev0 = g_prof_start, ev1 = g_prof_stop;
+        g_prof_start = g_prof_stop = nullptr;
+        if (w4 == 4) hipExtLaunchKernelGGL((int8wo_linear_rb4_kernel<4>), grid4, dim3(256), 0, st, ev0, ev1, 0, a);
+        else hipExtLaunchKernelGGL((int8wo_linear_rb4_kernel<8>), grid4, dim3(512), 0, st, ev0, ev1, 0, a);
+        AO_LAUNCH_CHECK();
+        return 0;
+    }
+    dim3 grid((unsigned)RB, (unsigned)mchunks);
     const size_t smem = staged ? (size_t)xbytes : 0;
     switch (waves) {
         case 1: launch_int8<1>(grid, smem, st, a); break;

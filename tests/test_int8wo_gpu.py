@@ -238,3 +238,42 @@ def test_legacy_entry_points_map_to_quantize():
         with torch.no_grad():
             same_output = torch.equal(a(x), b(x))
         assert same_class and same_output
+
+
+@pytest.mark.parametrize("M,N,K,bias", [(16, 14336, 4096, False), (13, 12352, 1024, True), (40, 16384, 2048, True)])
+def test_four_row_blocks_per_workgroup_kernel(M, N, K, bias):
+    """int8wo_linear_rb4_kernel (activation rows that do not fit the LDS staging, weights with 768 or more 16-row
+    blocks: four row blocks per workgroup share the activation loads): the linear against an fp32 matmul on the int8
+    codes with the module's roundings, one-hot rows bit for bit, and the fused residual / gate epilogues against the
+    separate bf16 ops."""
+    from ao_amd import ops
+
+    print(f"case int8 rb4 M={M} N={N} K={K} bias={bias}", flush=True)
+    dev = _dev()
+    gen = torch.Generator().manual_seed(M + N + K)
+    q = torch.randint(-127, 128, (N, K), generator=gen, dtype=torch.int8).to(dev)
+    s = (torch.rand(N, generator=gen) * 1e-3 + 1e-4).bfloat16().to(dev)
+    b = (torch.randn(N, generator=gen) * 0.1).bfloat16().to(dev) if bias else None
+    x = make_act(M, K, seed=M + 1).to(dev)
+    acc = x.float() @ q.float().t()
+    pre = acc.bfloat16().float() * s.float()
+    if bias:
+        pre = pre.bfloat16().float() + b.float()
+    y32 = ops.int8wo_linear(x, q, s, b, True)
+    y16 = ops.int8wo_linear(x, q, s, b, False)
+    err32 = float((y32 - pre).norm() / pre.norm())
+    err16 = float((y16.float() - pre.bfloat16().float()).norm() / pre.norm())
+    assert err32 <= 1e-3 and err16 <= 1.5e-3
+    # one-hot rows: the codes times the scale, exactly
+    ks = torch.randint(0, K, (M,), generator=gen).to(dev)
+    xh = torch.zeros(M, K, dtype=torch.bfloat16, device=dev)
+    xh[torch.arange(M, device=dev), ks] = 1.0
+    yh = ops.int8wo_linear(xh, q, s, None, True)
+    exact = bool(torch.equal(yh, q.float().t()[ks] * s.float()))
+    assert exact
+    other = make_act(M, N, seed=M + 2).to(dev)
+    y = ops.int8wo_linear(x, q, s)
+    same_residual = bool(torch.equal(ops.int8wo_linear_residual(x, q, s, other), other + y))
+    got = ops.int8wo_linear_gated(x, q, s, other).float().cpu().numpy()
+    want = (torch.nn.functional.silu(other) * y).float().cpu().numpy()
+    assert same_residual and np.count_nonzero(got != want) <= 0.002 * got.size + 1 and rel_l2(got, want) <= 1e-3
