@@ -342,16 +342,18 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_kernel(const LinearA
 // four times the bytes of its weights at 16 rows (896 workgroups x 128 KB on 14336 x 4096), and the fill rate of a
 // CU's L1 (about 20 bytes per cycle), not memory, sets the time.  Here a wave loads the activation fragments of a K
 // tile once and runs them against the tiles of four row blocks: a quarter of the activation traffic, four accumulators.
-template <int G, int WAVES>
+template <int G, int WAVES, int MB>
 __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const LinearArgs a) {
+    // MB 16-row blocks of activations per workgroup (17 to 32 rows with MB = 2): every dequantized dword then feeds MB
+    // matrix instructions, and the dequantization, which bounds the kernel, is done once for all of them
     constexpr int D = 2, RBW = 4;
-    static_assert(WAVES <= 8, "the reduction buffer is 4 KB per row block and wave");
+    static_assert(WAVES <= 8, "the reduction buffer is 4 KB per row block, activation block and wave");
     __shared__ float red[RBW][WAVES][4][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, qd = lane >> 4;
     const int64_t rb0 = (int64_t)blockIdx.x * RBW;
-    const int64_t m0 = (int64_t)blockIdx.y * 16;
+    const int64_t m0 = (int64_t)blockIdx.y * (16 * MB);
     const int KB = (int)(a.Kp / 128);
     const uint32_t magic = 0x43004300u;
     const bool sel_lane = qd == (r >> 2);
@@ -361,16 +363,23 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const Lin
     const u32x4_t sel_a = {s_even, s_odd, 0u, 0u};
     const u32x4_t sel_b = {0u, 0u, s_even, s_odd};
 
-    const bool xact = (m0 + r) < a.M;
-    const uint16_t* xp = a.x + (xact ? (m0 + r) : 0) * a.ldx + qd * 32;
-    f32x4_t acc[RBW];
+    bool xact[MB];
+    const uint16_t* xp[MB];
 #pragma unroll
-    for (int j = 0; j < RBW; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int mb = 0; mb < MB; ++mb) {
+        xact[mb] = (m0 + 16 * mb + r) < a.M;
+        xp[mb] = a.x + (xact[mb] ? (m0 + 16 * mb + r) : 0) * a.ldx + qd * 32;
+    }
+    f32x4_t acc[RBW][MB];
+#pragma unroll
+    for (int j = 0; j < RBW; ++j)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[j][mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     struct Buf {
         u32x4_t w[RBW];
         uint32_t q[RBW];
-        uint4 x[4];
+        uint4 x[MB][4];
     };
     auto load_tile = [&](Buf& b, int kb) {
         const int gidx = ((kb * 128 + qd * 32) / G) * 16;
@@ -379,11 +388,13 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const Lin
             b.w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(a.packed + ((rb0 + j) * KB + kb) * 64 + lane));
             b.q[j] = a.qparams[(rb0 + j) * (a.Kp / G) * 16 + r + gidx];
         }
-        if (xact) {
-            const uint4* xv = reinterpret_cast<const uint4*>(xp + (int64_t)kb * 128);
 #pragma unroll
-            for (int sl = 0; sl < 4; ++sl) b.x[sl] = xv[sl];
-        }
+        for (int mb = 0; mb < MB; ++mb)
+            if (xact[mb]) {
+                const uint4* xv = reinterpret_cast<const uint4*>(xp[mb] + (int64_t)kb * 128);
+#pragma unroll
+                for (int sl = 0; sl < 4; ++sl) b.x[mb][sl] = xv[sl];
+            }
     };
     u32x4_t tcur = {0, 0, 0, 0};
     // one tile = 16 dwords per lane (4 row blocks x 4); the three dequantization stages run as in int4wo_linear_kernel
@@ -394,8 +405,6 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const Lin
 #pragma unroll
         for (int e = 0; e < 4 * RBW; ++e) {
             const int j = e >> 2;
-            union { uint4 q; bf16x8_t v; } xa;
-            xa.q = b.x[e & 3];
             f32x4_t ua, ub;
             const f32x4_t zz = {gc[j].z, gc[j].z, gc[j].z, gc[j].z};
             add_zero(tcur, zz, sel_a, sel_b, ua, ub);
@@ -409,7 +418,12 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const Lin
             } else {
                 bw = round_pack<true>(ua, ub);
             }
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw, acc[j], 0, 0, 0);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                union { uint4 q; bf16x8_t v; } xa;
+                xa.q = b.x[mb][e & 3];
+                acc[j][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw, acc[j][mb], 0, 0, 0);
+            }
         }
     };
 
@@ -422,7 +436,9 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const Lin
             buf[d].q[j] = 0;
         }
 #pragma unroll
-        for (int sl = 0; sl < 4; ++sl) buf[d].x[sl] = make_uint4(0, 0, 0, 0);   // rows >= M keep these zeros
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int sl = 0; sl < 4; ++sl) buf[d].x[mb][sl] = make_uint4(0, 0, 0, 0);   // rows >= M keep these zeros
     }
     if (wave < KB) load_tile(buf[0], wave);
     const int nt = wave < KB ? (KB - wave + WAVES - 1) / WAVES : 0;
@@ -438,28 +454,33 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const Lin
         }
     }
 
-    // acc[j][i] = C[m = 4*qd + i][n = 16 (rb0 + j) + r]
+    // acc[j][mb][i] = C[m = m0 + 16 mb + 4*qd + i][n = 16 (rb0 + j) + r]; one pass of the reduction buffer per
+    // activation block, wave j finishes row block j
 #pragma unroll
-    for (int j = 0; j < RBW; ++j)
+    for (int mb = 0; mb < MB; ++mb) {
+        if (mb) __syncthreads();
 #pragma unroll
-        for (int i = 0; i < 4; ++i) red[j][wave][i][lane] = acc[j][i];
-    __syncthreads();
-    if (wave < RBW) {   // wave j finishes row block j
-        const int j = wave;
-        const int64_t n = (rb0 + j) * 16 + r;
-        float bv = 0.f;
-        if (a.bias && n < a.N) bv = bf16_bits_to_f32(a.bias[n]);
+        for (int j = 0; j < RBW; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float sum = 0.f;
+            for (int i = 0; i < 4; ++i) red[j][wave][i][lane] = acc[j][mb][i];
+        __syncthreads();
+        if (wave < RBW) {
+            const int j = wave;
+            const int64_t n = (rb0 + j) * 16 + r;
+            float bv = 0.f;
+            if (a.bias && n < a.N) bv = bf16_bits_to_f32(a.bias[n]);
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) sum += red[j][w][i][lane];
-            const int64_t m = m0 + 4 * qd + i;
-            if (m < a.M && n < a.N) {
-                sum += bv;
-                if (a.residual) sum = rne_bf16(sum) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
-                if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = sum;
-                else ((uint16_t*)a.y)[m * a.ldy + n] = f32_to_bf16_bits(sum);
+            for (int i = 0; i < 4; ++i) {
+                float sum = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) sum += red[j][w][i][lane];
+                const int64_t m = m0 + 16 * mb + 4 * qd + i;
+                if (m < a.M && n < a.N) {
+                    sum += bv;
+                    if (a.residual) sum = rne_bf16(sum) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
+                    if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = sum;
+                    else ((uint16_t*)a.y)[m * a.ldy + n] = f32_to_bf16_bits(sum);
+                }
             }
         }
     }
@@ -1166,10 +1187,15 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // every count up to 64)
     const bool gemm_starved = (M <= 32 && gemm_small_wgs < 128) || (M <= 40 && gemm_small_wgs <= 64) ||
                               (M <= 64 && gemm_small_wgs <= 16);
+    // 17 to 32 rows on a weight with 768 or more row blocks: the streaming kernel with four row blocks and two
+    // activation blocks per workgroup (14336 x 4096: 16-18 us against 24.5 us of the 64-row tiles, the head 92-101
+    // against 160; from 33 rows, two passes of it, the tiles win again)
+    static const bool rb4_off = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
+    const bool rb4_two_blocks = !rb4_off && M > 16 && M <= 32 && RB % 4 == 0 && RB / 4 >= 192 && a.K == a.Kp;
     AO_REQUIRE(ksplit == 1 || (xmode == X_LDS && M <= 16 && !dual && !pair8 && !bias_bf16 && !residual_bf16 && y_dtype == AO_F32),
                "partial sums over a split K need M <= 16, fp32 output, no bias / residual epilogue and activations that "
                "fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);
-    if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16 && !gemm_starved) {
+    if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16 && !gemm_starved && !rb4_two_blocks) {
         {
             char name[96];
             if (int4wo_gemm_lds_plan(a, g, name, sizeof(name))) {
@@ -1225,14 +1251,19 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // 13.9 / 13.5 / 13.6 / 13.7 / 13.7 / 14.1 against 12.8 / 14.0 / 14.2 / 16.4 / 14.8 / 18.2 / 20.6 of the kernels below
     // (LDS-staged up to 5 rows there); the vocabulary head at 16 rows 85 against 129.
     if ((xmode == X_GLOBAL || (xmode == X_LDS && !norm_weight_bf16 && !pair8)) && !dual && ksplit == 1 && M >= 4 &&
-        RB % 4 == 0 && (RB / 4) * mchunks >= 192 && a.K == a.Kp) {
+        RB % 4 == 0 && a.K == a.Kp) {
         static const bool rb4_disabled = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
-        if (!rb4_disabled) {
-            const int64_t wgs = (RB / 4) * mchunks;
+        // two 16-row activation blocks per workgroup from 17 rows on: the dequantized dword feeds both (four of them
+        // do not fit the registers)
+        const int mb = M > 16 ? 2 : 1;
+        const int64_t mch = (M + 16 * mb - 1) / (16 * mb);
+        const int64_t wgs = (RB / 4) * mch;
+        if (!rb4_disabled && wgs >= 192) {
             int w4 = 4;   // at least four waves: wave j finishes row block j
             while (w4 < 8 && wgs * w4 * 2 <= 4096 + wgs && w4 * 2 <= a.Kp / 128) w4 *= 2;
-            AO_PLAN("int4wo_linear_rb4_kernel<%lld,%d>", (long long)g, w4);
-            const dim3 grid4((unsigned)(RB / 4), (unsigned)mchunks);
+            if (mb == 1) AO_PLAN("int4wo_linear_rb4_kernel<%lld,%d>", (long long)g, w4);
+            AO_PLAN("int4wo_linear_rb4_kernel<%lld,%d,%d>", (long long)g, w4, mb);
+            const dim3 grid4((unsigned)(RB / 4), (unsigned)mch);
             auto go = [&](auto kernel, int nw) {
                 if (g_prof_start && g_prof_stop) {
                     hipExtLaunchKernelGGL(kernel, grid4, dim3(nw * 64), 0, st, g_prof_start, g_prof_stop, 0, a);
@@ -1241,9 +1272,12 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
                     hipLaunchKernelGGL(kernel, grid4, dim3(nw * 64), 0, st, a);
                 }
             };
-#define AO_RB4(GG)                                                  \
-    if (w4 == 4) go(int4wo_linear_rb4_kernel<GG, 4>, 4);            \
-    else go(int4wo_linear_rb4_kernel<GG, 8>, 8)
+#define AO_RB4_MB(GG, MBV)                                                 \
+    if (w4 == 4) go(int4wo_linear_rb4_kernel<GG, 4, MBV>, 4);              \
+    else go(int4wo_linear_rb4_kernel<GG, 8, MBV>, 8)
+#define AO_RB4(GG)                                                         \
+    if (mb == 1) { AO_RB4_MB(GG, 1); }                                     \
+    else { AO_RB4_MB(GG, 2); }
             switch (g) {
                 case 32: AO_RB4(32); break;
                 case 64: AO_RB4(64); break;
@@ -1251,6 +1285,7 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
                 default: AO_RB4(256); break;
             }
 #undef AO_RB4
+#undef AO_RB4_MB
             AO_LAUNCH_CHECK();
             return 0;
         }

@@ -53,7 +53,8 @@ def test_dispatch_walk_finds_every_kernel_family():
         for tile in ("int4wo_gemm_kernel<%d,2,8>", "int4wo_gemm_kernel<%d,1,4>", "int4wo_gemm_kernel<%d,1,2>",
                      "int4wo_gemm_ksplit_kernel<%d,4,4>", "int4wo_gemm_ksplit_kernel<%d,2,4>",
                      "int4wo_gemm_lds_kernel<%d,1>", "int4wo_gemm_lds_kernel<%d,2>", "int4wo_gemm_kwave_kernel<%d>",
-                     "int4wo_linear_rb4_kernel<%d,4>", "int4wo_linear_rb4_kernel<%d,8>"):
+                     "int4wo_linear_rb4_kernel<%d,4>", "int4wo_linear_rb4_kernel<%d,8>", "int4wo_linear_rb4_kernel<%d,4,2>",
+                     "int4wo_linear_rb4_kernel<%d,8,2>"):
             assert tile % g in plans, tile % g
     # the single-row kernel: exactly the instantiations that int4wo_gemv1.hip compiles (waves, chunks per lane, norm)
     gemv1 = {n.split(" ")[0] for n in plans if n.startswith("int4wo_gemv1_kernel<")}
@@ -79,7 +80,10 @@ def test_dispatch_walk_finds_every_kernel_family():
     assert _lib.int4wo_linear_plan(4, 4096, 128256, 64) == "int4wo_linear_rb4_kernel<64,4>"
     assert not _lib.int4wo_linear_plan(16, 14336, 4096, 64).startswith("int4wo_linear_rb4_kernel")   # 64 workgroups
     assert not _lib.int4wo_linear_plan(3, 4096, 14336, 64).startswith("int4wo_linear_rb4_kernel")
-    assert len(plans) >= 80
+    # ... and 17 to 32 rows there take it with two activation blocks per workgroup instead of the 64-row tiles
+    assert _lib.int4wo_linear_plan(24, 4096, 14336, 64) == "int4wo_linear_rb4_kernel<64,8,2>"
+    assert not _lib.int4wo_linear_plan(33, 4096, 14336, 64).startswith("int4wo_linear_rb4_kernel")
+    assert len(plans) >= 88
 
 
 def _cases():
