@@ -693,6 +693,129 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_linear_kernel(const uint16_t* 
 // W[N,K] fp16 = fp16(fpx value * scale), the dequantization of the linear kernels as a pass of its own, for batches
 // large enough that the library fp16 GEMM on the converted weight beats the fused kernel.  One wave per 16-row x 128-k
 // tile: 24 bytes in, 64 bytes out per lane (the four quarter-lanes of a row write 256 contiguous bytes).
+// The streaming kernel for 17 to 32 activation rows (MB = 2): four row blocks of W and MB 16-row blocks of activations
+// per workgroup, so that a converted and scaled weight fragment feeds MB matrix instructions and the activation rows are
+// fetched once per four row blocks (the tiled kernel takes 18 us on 14336 x 4096 at any of these row counts, this
+// kernel's 16-row form 9.5 us at 16 rows).
+template <int WAVES, bool E3M2, int MB>
+__global__ __launch_bounds__(WAVES * 64) void fp6_linear_mb_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
+                                                                    const uint32_t* __restrict__ native,
+                                                                    const uint16_t* __restrict__ scale, int64_t N,
+                                                                    uint16_t* __restrict__ out) {
+    constexpr int RBW = 4;
+    static_assert(WAVES >= RBW && WAVES <= 8, "wave j finishes row block j; 4 KB of reduction buffer per block and wave");
+    __shared__ float red[RBW][WAVES][4][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, qd = lane >> 4;
+    const int64_t rb0 = (int64_t)blockIdx.x * RBW, m0 = (int64_t)blockIdx.y * (16 * MB);
+    const int KB = (int)(K / 128);
+    const uint32_t* tiles = native + rb0 * KB * 384;
+    bool xact[MB];
+    const uint16_t* xp[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        xact[mb] = (m0 + 16 * mb + r) < M;
+        xp[mb] = x + (xact[mb] ? (m0 + 16 * mb + r) : 0) * K + qd * 32;
+    }
+    f16x2_t sc2[RBW];
+#pragma unroll
+    for (int j = 0; j < RBW; ++j) {
+        union { uint16_t h; _Float16 f; } sc;
+        sc.h = scale[(rb0 + j) * 16 + r];
+        sc2[j] = f16x2_t{sc.f, sc.f};
+    }
+    f32x4_t acc[RBW][MB];
+#pragma unroll
+    for (int j = 0; j < RBW; ++j)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[j][mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    struct Buf { u32x6_t w[RBW]; u32x4v_t x[MB][4]; };
+    auto load_tile = [&](Buf& b, int kb) __attribute__((always_inline)) {
+        const uint32_t* t = tiles + (int64_t)kb * 384;
+#pragma unroll
+        for (int j = 0; j < RBW; ++j) {
+            const uint32_t* tj = t + (int64_t)j * KB * 384;
+            const u32x4v_t lo = reinterpret_cast<const u32x4v_t*>(tj)[lane];
+            const u32x2v_t hi = reinterpret_cast<const u32x2v_t*>(tj + 256)[lane];
+            b.w[j] = __builtin_shufflevector(lo, __builtin_shufflevector(hi, hi, 0, 1, -1, -1), 0, 1, 2, 3, 4, 5);
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            if (xact[mb]) {
+                const u32x4v_t* xv = reinterpret_cast<const u32x4v_t*>(xp[mb] + (int64_t)kb * 128);
+#pragma unroll
+                for (int sl = 0; sl < 4; ++sl) b.x[mb][sl] = xv[sl];
+            }
+    };
+    auto compute_tile = [&](const Buf& b) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < RBW; ++j) {
+            f16x32_t v;
+            if (E3M2) v = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(b.w[j], 1.0f);
+            else v = __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(b.w[j], 1.0f);
+#pragma unroll
+            for (int sl = 0; sl < 4; ++sl) {
+                union { f16x2_t p[4]; f16x8_t v; } w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const f16x2_t pr = {v[sl * 8 + 2 * e], v[sl * 8 + 2 * e + 1]};
+                    w.p[e] = pr * sc2[j];  // v_pk_mul_f16: fp16(fp6 * scale), the one rounding of the reference kernel
+                }
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    union { u32x4v_t q; f16x8_t v; } xa;
+                    xa.q = b.x[mb][sl];
+                    acc[j][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa.v, w.v, acc[j][mb], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    Buf b0, b1;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            b0.x[mb][sl] = u32x4v_t{0, 0, 0, 0};   // rows >= M keep these zeros
+            b1.x[mb][sl] = u32x4v_t{0, 0, 0, 0};
+        }
+    int kb = wave;
+    if (kb < KB) load_tile(b0, kb);
+    while (kb < KB) {
+        const int kb1 = kb + WAVES, kb2 = kb + 2 * WAVES;
+        if (kb1 < KB) load_tile(b1, kb1);
+        compute_tile(b0);
+        if (kb1 < KB) {
+            if (kb2 < KB) load_tile(b0, kb2);
+            compute_tile(b1);
+        }
+        kb = kb2;
+    }
+    // one pass of the reduction buffer per activation block; wave j sums and stores row block j
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        if (mb) __syncthreads();
+#pragma unroll
+        for (int j = 0; j < RBW; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[j][wave][i][lane] = acc[j][mb][i];
+        __syncthreads();
+        if (wave < RBW) {
+            const int64_t n = (rb0 + wave) * 16 + r;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) s += red[wave][w][i][lane];
+                const int64_t m = m0 + 16 * mb + 4 * qd + i;
+                if (m < M && n < N) out[m * N + n] = f32_to_f16_bits(s);
+            }
+        }
+    }
+}
+
 template <bool E3M2>
 __global__ __launch_bounds__(256) void fp6_native_to_f16_kernel(const uint32_t* __restrict__ native,
                                                                  const uint16_t* __restrict__ scale, int64_t N, int64_t K,
@@ -1315,6 +1438,24 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
         }
         AO_LAUNCH_CHECK();
         return 0;
+    }
+    if (M > 16 && M <= 32 && K % 128 == 0 && !res && !gt && RB % 4 == 0 && RB / 4 >= 192) {
+        // 17 to 32 rows on a weight with 768 or more row blocks: the streaming kernel with four row blocks and two
+        // activation blocks per workgroup (14336 x 4096: 11.3-13.4 us against 18 us of the tiled kernel, the head 82-97
+        // against 145; four activation blocks for 33 to 64 rows spill and measured slower than the tiles)
+        static const bool mb_disabled = [] { const char* e = getenv("AO_AMD_FP6_MB"); return e && e[0] == '0'; }();
+        if (!mb_disabled) {
+            const int64_t wgs = RB / 4;
+            int w4 = 4;
+            while (w4 < 8 && wgs * w4 * 2 <= 4096 + wgs && w4 * 2 <= KB) w4 *= 2;
+            const dim3 mgrid((unsigned)(RB / 4), 1u);
+#define AO_FP6_MB(W, E3) hipExtLaunchKernelGGL((fp6_linear_mb_kernel<W, E3, 2>), mgrid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o)
+            if (ebits == 3) { if (w4 == 4) AO_FP6_MB(4, true); else AO_FP6_MB(8, true); }
+            else { if (w4 == 4) AO_FP6_MB(4, false); else AO_FP6_MB(8, false); }
+#undef AO_FP6_MB
+            AO_LAUNCH_CHECK();
+            return 0;
+        }
     }
     if (M > 16 && K % 128 == 0 && !res && !gt) {
         // ... and 32 x 64 tiles when even those leave CUs idle

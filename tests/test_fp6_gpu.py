@@ -133,10 +133,12 @@ def test_linear_matches_oracle(oracle, shape, M):
     assert rel.mean() < 1e-3
 
 
-@pytest.mark.parametrize("N,K,M", [(14336, 1024, 16), (14336, 512, 8), (6144, 576, 5), (3072, 320, 40), (2048, 192, 100), (4096, 4096, 16)])
+@pytest.mark.parametrize("N,K,M", [(14336, 1024, 16), (14336, 512, 8), (6144, 576, 5), (3072, 320, 40), (2048, 192, 100), (4096, 4096, 16),
+                                   (14336, 1024, 17), (12288, 512, 32), (14336, 4096, 29)])
 def test_linear_with_shared_activation_tiles_matches_oracle(oracle, N, K, M):
     """Sizes at which a wave of the few-row kernel multiplies one activation tile against 4 or 2 row blocks (4 or more
-    activation rows, 192 or more workgroups left), with whole and half last K tiles and more than one 16-row chunk."""
+    activation rows, 192 or more workgroups left), with whole and half last K tiles and more than one 16-row chunk;
+    and 17 to 32 rows on weights with 768 or more row blocks, where two activation blocks share each weight fragment."""
     from ao_amd import ops
 
     print(f"case fp6 linear shared activation tiles N={N} K={K} M={M}", flush=True)
