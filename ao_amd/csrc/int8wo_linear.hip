@@ -318,29 +318,37 @@ __global__ __launch_bounds__(WAVES * 64) void int8wo_linear_kernel(const Int8Arg
 // (9 and more rows at K = 4096): every row block re-reads all activation rows from L2 there, twice the bytes of its int8
 // weights at 16 rows, and a CU's L1 fill rate (about 20 bytes per cycle), not memory, sets the time.  A wave loads the
 // activation fragments of a K tile once and runs them against the tiles of four row blocks; wave j finishes block j.
-template <int WAVES>
+template <int WAVES, int MB>
 __global__ __launch_bounds__(WAVES * 64) void int8wo_linear_rb4_kernel(const Int8Args a) {
+    // MB 16-row blocks of activations per workgroup (MB = 2 from 17 rows on): a converted weight fragment feeds MB
+    // matrix instructions and the weight is streamed once per 16 MB rows
     constexpr int RBW = 4;
     static_assert(WAVES >= RBW && WAVES <= 8, "wave j finishes row block j; 4 KB of reduction buffer per block and wave");
     __shared__ float red[RBW][WAVES][4][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, qd = lane >> 4;
-    const int64_t rb0 = (int64_t)blockIdx.x * RBW, m0 = (int64_t)blockIdx.y * 16;
+    const int64_t rb0 = (int64_t)blockIdx.x * RBW, m0 = (int64_t)blockIdx.y * (16 * MB);
     const int KB = (int)(a.K / 128);
-    const int64_t mrow = m0 + r < a.M ? m0 + r : a.M - 1;   // rows past M alias the last one, never stored
     const int8_t* wp[RBW];
 #pragma unroll
     for (int j = 0; j < RBW; ++j) {
         const int64_t n = (rb0 + j) * 16 + r;
         wp[j] = a.w + (n < a.N ? n : a.N - 1) * a.ldw + qd * 32;
     }
-    const uint16_t* xp = a.x + mrow * a.ldx + qd * 32;
-    f32x4_t acc[RBW];
+    const uint16_t* xp[MB];
 #pragma unroll
-    for (int j = 0; j < RBW; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int mb = 0; mb < MB; ++mb) {
+        const int64_t m = m0 + 16 * mb + r;
+        xp[mb] = a.x + (m < a.M ? m : a.M - 1) * a.ldx + qd * 32;   // rows past M alias the last one, never stored
+    }
+    f32x4_t acc[RBW][MB];
+#pragma unroll
+    for (int j = 0; j < RBW; ++j)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[j][mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    struct Buf { u32x4_t w0[RBW], w1[RBW]; u32x4_t x[4]; };
+    struct Buf { u32x4_t w0[RBW], w1[RBW]; u32x4_t x[MB][4]; };
     auto load_tile = [&](Buf& b, int kb) {
 #pragma unroll
         for (int j = 0; j < RBW; ++j) {
@@ -348,22 +356,28 @@ __global__ __launch_bounds__(WAVES * 64) void int8wo_linear_rb4_kernel(const Int
             b.w0[j] = __builtin_nontemporal_load(wv);
             b.w1[j] = __builtin_nontemporal_load(wv + 1);
         }
-        const u32x4_t* xv = reinterpret_cast<const u32x4_t*>(xp + (int64_t)kb * 128);
 #pragma unroll
-        for (int sl = 0; sl < 4; ++sl) b.x[sl] = xv[sl];
+        for (int mb = 0; mb < MB; ++mb) {
+            const u32x4_t* xv = reinterpret_cast<const u32x4_t*>(xp[mb] + (int64_t)kb * 128);
+#pragma unroll
+            for (int sl = 0; sl < 4; ++sl) b.x[mb][sl] = xv[sl];
+        }
     };
     auto compute_tile = [&](const Buf& b) {
 #pragma unroll
         for (int sl = 0; sl < 4; ++sl) {
-            union { u32x4_t q; bf16x8_t v; } xa;
-            xa.q = b.x[sl];
 #pragma unroll
             for (int j = 0; j < RBW; ++j) {
                 const uint32_t ww[8] = {b.w0[j].x, b.w0[j].y, b.w0[j].z, b.w0[j].w, b.w1[j].x, b.w1[j].y, b.w1[j].z, b.w1[j].w};
                 union { uint32_t u[4]; bf16x8_t v; } bw;
                 int8x4_to_bf16(ww[2 * sl], bw.u[0], bw.u[1]);
                 int8x4_to_bf16(ww[2 * sl + 1], bw.u[2], bw.u[3]);
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw.v, acc[j], 0, 0, 0);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    union { u32x4_t q; bf16x8_t v; } xa;
+                    xa.q = b.x[mb][sl];
+                    acc[j][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa.v, bw.v, acc[j][mb], 0, 0, 0);
+                }
             }
         }
     };
@@ -382,35 +396,40 @@ __global__ __launch_bounds__(WAVES * 64) void int8wo_linear_rb4_kernel(const Int
             kb = kb2;
         }
     }
-    // acc[j][i] = C[m = 4*qd + i][n = 16 (rb0 + j) + r]
+    // acc[j][mb][i] = C[m = m0 + 16 mb + 4*qd + i][n = 16 (rb0 + j) + r]; one pass of the reduction buffer per
+    // activation block
 #pragma unroll
-    for (int j = 0; j < RBW; ++j)
+    for (int mb = 0; mb < MB; ++mb) {
+        if (mb) __syncthreads();
 #pragma unroll
-        for (int i = 0; i < 4; ++i) red[j][wave][i][lane] = acc[j][i];
-    __syncthreads();
-    if (wave < RBW) {
-        const int64_t n = (rb0 + wave) * 16 + r;
-        if (n < a.N) {
-            const float sc = bf16_bits_to_f32(a.scale[n]);
-            const float bv = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.f;
+        for (int j = 0; j < RBW; ++j)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float s = 0.f;
+            for (int i = 0; i < 4; ++i) red[j][wave][i][lane] = acc[j][mb][i];
+        __syncthreads();
+        if (wave < RBW) {
+            const int64_t n = (rb0 + wave) * 16 + r;
+            if (n < a.N) {
+                const float sc = bf16_bits_to_f32(a.scale[n]);
+                const float bv = a.bias ? bf16_bits_to_f32(a.bias[n]) : 0.f;
 #pragma unroll
-                for (int w = 0; w < WAVES; ++w) s += red[wave][w][i][lane];
-                const int64_t m = m0 + 4 * qd + i;
-                if (m < a.M) {
-                    // the epilogue of int8wo_linear_kernel: mm result rounded to bf16, times scale, plus bias, then the
-                    // fused residual or gate
-                    float v = hw_rne_bf16(s) * sc;
-                    if (a.bias) v = hw_rne_bf16(v) + bv;
-                    if (a.residual) v = hw_rne_bf16(v) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
-                    if (a.gate) {
-                        const float gt = bf16_bits_to_f32(a.gate[m * a.ldgate + n]);
-                        v = hw_rne_bf16(gt / (1.0f + expf(-gt))) * hw_rne_bf16(v);
+                for (int i = 0; i < 4; ++i) {
+                    float s = 0.f;
+#pragma unroll
+                    for (int w = 0; w < WAVES; ++w) s += red[wave][w][i][lane];
+                    const int64_t m = m0 + 16 * mb + 4 * qd + i;
+                    if (m < a.M) {
+                        // the epilogue of int8wo_linear_kernel: mm result rounded to bf16, times scale, plus bias, then
+                        // the fused residual or gate
+                        float v = hw_rne_bf16(s) * sc;
+                        if (a.bias) v = hw_rne_bf16(v) + bv;
+                        if (a.residual) v = hw_rne_bf16(v) + bf16_bits_to_f32(a.residual[m * a.ldres + n]);
+                        if (a.gate) {
+                            const float gt = bf16_bits_to_f32(a.gate[m * a.ldgate + n]);
+                            v = hw_rne_bf16(gt / (1.0f + expf(-gt))) * hw_rne_bf16(v);
+                        }
+                        if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = v;
+                        else ((uint16_t*)a.y)[m * a.ldy + n] = hw_bf16_bits(v);
                     }
-                    if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = v;
-                    else ((uint16_t*)a.y)[m * a.ldy + n] = hw_bf16_bits(v);
                 }
             }
         }
@@ -499,15 +518,23 @@ static int int8wo_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // unstaged rows on a weight with 768 or more row blocks: four row blocks per workgroup share the activation loads
     // (14336 x 4096 at 16 rows: measured against the one-block kernel below)
     static const bool rb4_disabled = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
-    if (!staged && !rb4_disabled && RB % 4 == 0 && (RB / 4) * mchunks >= 192 && KB >= 8) {
-        const int64_t wgs = (RB / 4) * mchunks;
+    // two activation blocks per workgroup from 17 rows on (four do not fit the registers): 14336 x 4096 at 17 / 32 / 64 /
+    // 100 rows 31 / 34 / 59 / 97 -> 20.5 / 23 / 43 / 67 us, the head at 32 rows 243 -> 144
+    const int mbv = M > 16 ? 2 : 1;
+    const int64_t mch = (M + 16 * mbv - 1) / (16 * mbv);
+    if (!staged && !rb4_disabled && RB % 4 == 0 && (RB / 4) * mch >= 192 && KB >= 8) {
+        const int64_t wgs = (RB / 4) * mch;
         int w4 = 4;
         while (w4 < 8 && wgs * w4 * 2 <= 4096 + wgs && w4 * 2 <= KB) w4 *= 2;
-        const dim3 grid4((unsigned)(RB / 4), (unsigned)mchunks);
+        const dim3 grid4((unsigned)(RB / 4), (unsigned)mch);
         hipEvent_t ev0 = g_prof_start, ev1 = g_prof_stop;
         g_prof_start = g_prof_stop = nullptr;
-        if (w4 == 4) hipExtLaunchKernelGGL((int8wo_linear_rb4_kernel<4>), grid4, dim3(256), 0, st, ev0, ev1, 0, a);
-        else hipExtLaunchKernelGGL((int8wo_linear_rb4_kernel<8>), grid4, dim3(512), 0, st, ev0, ev1, 0, a);
+#define AO_I8_RB4(MBV)                                                                                                   \
+    if (w4 == 4) hipExtLaunchKernelGGL((int8wo_linear_rb4_kernel<4, MBV>), grid4, dim3(256), 0, st, ev0, ev1, 0, a);        \
+    else hipExtLaunchKernelGGL((int8wo_linear_rb4_kernel<8, MBV>), grid4, dim3(512), 0, st, ev0, ev1, 0, a)
+        if (mbv == 1) { AO_I8_RB4(1); }
+        else { AO_I8_RB4(2); }
+#undef AO_I8_RB4
         AO_LAUNCH_CHECK();
         return 0;
     }

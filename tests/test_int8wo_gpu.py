@@ -240,10 +240,11 @@ def test_legacy_entry_points_map_to_quantize():
         assert same_class and same_output
 
 
-@pytest.mark.parametrize("M,N,K,bias", [(16, 14336, 4096, False), (13, 12352, 1024, True), (40, 16384, 2048, True)])
+@pytest.mark.parametrize("M,N,K,bias", [(16, 14336, 4096, False), (13, 12352, 1024, True), (40, 16384, 2048, True),
+                                        (29, 14336, 1024, False)])
 def test_four_row_blocks_per_workgroup_kernel(M, N, K, bias):
     """int8wo_linear_rb4_kernel (activation rows that do not fit the LDS staging, weights with 768 or more 16-row
-    blocks: four row blocks per workgroup share the activation loads): the linear against an fp32 matmul on the int8
+    blocks: four row blocks per workgroup share the activation loads, two activation blocks from 17 rows on): the linear against an fp32 matmul on the int8
     codes with the module's roundings, one-hot rows bit for bit, and the fused residual / gate epilogues against the
     separate bf16 ops."""
     from ao_amd import ops
