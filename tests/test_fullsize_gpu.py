@@ -307,7 +307,8 @@ def test_prefill_gemm_launches_repeat_bit_for_bit(cabi, M, N, K, g):
 @pytest.mark.parametrize("M,N,K,g,bias,residual,fp32", [(13, 14400, 1024, 128, True, False, False), (16, 14336, 4096, 64, False, True, False),
                                                         (4, 16384, 2048, 32, True, True, False), (9, 14336, 4096, 256, True, False, True),
                                                         (17, 14336, 4096, 64, True, False, False), (29, 14400, 1024, 128, True, True, False),
-                                                        (32, 16384, 2048, 256, False, False, True)])
+                                                        (32, 16384, 2048, 256, False, False, True), (11, 14330, 1024, 64, True, False, False),
+                                                        (23, 12346, 1024, 64, False, True, False)])
 def test_four_row_blocks_per_workgroup_kernel_epilogues(cabi, M, N, K, g, bias, residual, fp32):
     """int4wo_linear_rb4_kernel (4 to 32 activation rows, four 16-row weight blocks per workgroup sharing the activation
     loads, two activation blocks from 17 rows): bias, residual (y = bf16(bf16(acc + bias) + residual), the order of the unfused modules), fp32 output and
