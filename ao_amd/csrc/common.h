@@ -87,7 +87,13 @@ __device__ __forceinline__ uint16_t hw_bf16_bits(float f) {
     __builtin_memcpy(&u, &b, 2);
     return u;
 }
-__device__ __forceinline__ float hw_rne_bf16(float v) { return bf16_bits_to_f32(hw_bf16_bits(v)); }
+// ... as an fp32 value, in one instruction: with a zero low operand the converter leaves bf16(v) in the high half of the
+// result, which is that value widened back to fp32 (converting to a 16-bit value and shifting it up takes two)
+__device__ __forceinline__ float hw_rne_bf16(float v) {
+    float r;
+    asm("v_cvt_pk_bf16_f32 %0, 0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
 __device__ __forceinline__ uint32_t hw_bf16_pack(float lo, float hi) {
     typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
     const bf16x2 p = {(__bf16)lo, (__bf16)hi};

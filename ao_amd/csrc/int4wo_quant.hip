@@ -383,8 +383,41 @@ __global__ __launch_bounds__(256) void int4wo_quantize_pack_kernel(const uint16_
     const bool vec_ok = ((ldw & 7) == 0) && ((((uintptr_t)w) & 15) == 0);
 
     float v[NSS][4][8];
+    // Whole tiles inside the weight (the common case) are fetched with loads whose 16 neighbouring lanes cover 256
+    // contiguous bytes of one row, four rows per instruction, and turned through LDS into the order the packing wants
+    // (lane (r, qd) owns the 64 bytes k = 32 qd .. 32 qd + 31 of row r).  Loading in that order directly makes every
+    // lane of an instruction its own 16-byte request, 7 million of them for a 14336 x 4096 weight, and the requests,
+    // not the bytes, set the time.
+    __shared__ __align__(16) uint8_t turn[4][16 * 272];   // per wave: 16 rows of 256 bytes, 16 bytes of padding each
+    const bool whole = vec_ok && rb * 16 + 16 <= N && kbase + SPAN <= K;
 #pragma unroll
-    for (int ss = 0; ss < NSS; ++ss)
+    for (int ss = 0; ss < NSS; ++ss) {
+        if (whole) {   // uniform over the wave
+            uint4 raw[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = 64 * j + lane;   // chunk c of the tile: row c / 16, 16-byte column c % 16
+                raw[j] = *reinterpret_cast<const uint4*>(w + (rb * 16 + (c >> 4)) * ldw + kbase + ss * 128 + (c & 15) * 8);
+            }
+            if (ss) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads of the slice before (own wave only)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = 64 * j + lane;
+                *reinterpret_cast<uint4*>(&turn[wave][(c >> 4) * 272 + (c & 15) * 16]) = raw[j];
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // written and read by the same wave: no barrier
+#pragma unroll
+            for (int sl = 0; sl < 4; ++sl) {
+                const uint4 q = *reinterpret_cast<const uint4*>(&turn[wave][r * 272 + (qd * 4 + sl) * 16]);
+                const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    v[ss][sl][2 * j] = __uint_as_float(u[j] << 16);
+                    v[ss][sl][2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u);
+                }
+            }
+            continue;
+        }
 #pragma unroll
         for (int sl = 0; sl < 4; ++sl) {
             const int64_t k0 = kbase + ss * 128 + qd * 32 + sl * 8;
@@ -402,6 +435,7 @@ __global__ __launch_bounds__(256) void int4wo_quantize_pack_kernel(const uint16_
                     v[ss][sl][e] = (row < N && k0 + e < K) ? bf16_bits_to_f32(w[row * ldw + k0 + e]) : 0.f;
             }
         }
+    }
 
     // per-lane partial min/max of each super-slice
     float mn[NSS], mx[NSS];
@@ -471,9 +505,9 @@ __global__ __launch_bounds__(256) void int4wo_quantize_pack_kernel(const uint16_
             uint32_t word = 0;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                float q = __builtin_rintf(hw_rne_bf16(tq[e]));
-                q = q < 0.f ? 0.f : (q > 15.f ? 15.f : q);
-                if (q != q) q = 0.f;
+                // clamp to 0..15; v_med3_f32 returns the smallest of its operands when one is a NaN, i.e. the 0 that the
+                // reference's cast of a NaN code gives
+                const float q = __builtin_amdgcn_fmed3f(__builtin_rintf(hw_rne_bf16(tq[e])), 0.f, 15.f);
                 word |= (uint32_t)(int)q << (4 * nib_pos(e));
             }
             words[sl] = word;
