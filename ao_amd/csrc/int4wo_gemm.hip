@@ -326,8 +326,20 @@ __global__ __launch_bounds__(256) void int4wo_gemm_lds_kernel(const LinearArgs a
     // asm statements' latency
     // ... and the requests of the last step are still in flight: their target registers and LDS rows are not free
     // (the compiler, which sees the loaded values unused, would hand the registers to the epilogue) before they landed
-    // (the epilogue reads the accumulators through acc_read, volatile asm statements that stay behind this one)
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)" ::: "memory");
+    // (the epilogue reads the accumulators through acc_read, volatile asm statements that stay behind this one).
+    // The wait takes the load targets as operands: that keeps them allocated up to here.  A plain asm statement does
+    // not: the scheduler puts the epilogue's first address computations in front of it, into registers it considers
+    // free, and a request that lands after them overwrites them.
+    if constexpr (NT == 2) {
+        asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)"
+                     : "+v"(wr[0][0]), "+v"(wr[0][1]), "+v"(wr[1][0]), "+v"(wr[1][1]), "+v"(qr[0][0]), "+v"(qr[0][1]),
+                       "+v"(qr[1][0]), "+v"(qr[1][1])
+                     :: "memory");
+    } else {
+        asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)"
+                     : "+v"(wr[0][0]), "+v"(wr[1][0]), "+v"(qr[0][0]), "+v"(qr[1][0])
+                     :: "memory");
+    }
     __syncthreads();  // the LDS buffers are free: the epilogue turns the accumulators through them
 
     // acc[i][j][e] = C[m = m0 + 32 i + 8 (e / 4) + 4 kq + e % 4][n = n0 + 64 wave + 32 j + frow]
@@ -536,11 +548,20 @@ __global__ __launch_bounds__(256) void int4wo_gemm_kwave_kernel(const LinearArgs
     };
     for (int t = 0; t < nst; t += 2) {
         step(t, 0);
-        if (t + 1 < nst) step(t + 1, 1);
+        if (t + 1 >= nst) break;
+        step(t + 1, 1);
     }
     // a matrix instruction's result may be read 18 issue slots after it at the earliest; the epilogue reads the
     // accumulators through acc_read, volatile asm statements that stay behind this one
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    // The wait takes the targets of the loop's weight requests as operands, which keeps them allocated up to here: the
+    // requests of the last step (issued for a step past the end) are still in flight, and without the operands the
+    // scheduler puts the epilogue's first address computations in front of the wait, into those registers; a request
+    // that lands after them overwrites the addresses (seen as one wave's partial tile written to the wrong place, a
+    // few launches in a hundred, on waves that leave the loop after an even-numbered step).
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0) lgkmcnt(0)"
+                 : "+v"(wr[0][0]), "+v"(wr[0][1]), "+v"(wr[1][0]), "+v"(wr[1][1]), "+v"(qr[0][0]), "+v"(qr[0][1]),
+                   "+v"(qr[1][0]), "+v"(qr[1][1])
+                 :: "memory");
 
     // Sum of the four waves' partial tiles: every wave leaves its own in its 32 KB of LDS as fp32 [128][64] (the column
     // index flipped by 32 in rows whose bit 2 is set: the two half-waves write rows 4 apart, 1024 bytes, the same

@@ -730,6 +730,7 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
             }
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the requests of a wave without tiles
 
     // acc[i] = C[m = 4*qd + i][n = r]
 #pragma unroll

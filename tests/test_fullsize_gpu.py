@@ -217,7 +217,8 @@ def test_config1_output_tolerance(oracle):
     (2048, 4096, 14336, 256, True, False, "lds"),
     (128, 14336, 4096, 64, False, False, "kwave"), (200, 12352, 1024, 128, True, False, "kwave"),
     (512, 4096, 14336, 256, False, True, "kwave"), (333, 6100, 2048, 32, True, False, "kwave"),
-    (1000, 4098, 4096, 64, True, True, "kwave"), (130, 14336, 1152, 64, False, False, "kwave")])
+    (1000, 4098, 4096, 64, True, True, "kwave"), (130, 14336, 1152, 64, False, False, "kwave"),
+    (213, 6144, 1920, 128, True, False, "kwave")])
 def test_prefill_gemm_tiles_edges_and_repeated_launches(cabi, M, N, K, g, bias, fp32, kernel):
     """The prefill kernels (activations through LDS-direct loads, weights dequantized between the matrix instructions;
     256-row tiles, and 128-row tiles whose waves split K, with step counts per wave that differ when K / 64 is not a
@@ -270,11 +271,14 @@ def test_prefill_gemm_tiles_edges_and_repeated_launches(cabi, M, N, K, g, bias, 
 
 
 @pytest.mark.parametrize("M,N,K,g", [(2048, 14336, 4096, 64), (512, 14336, 4096, 128), (512, 4096, 14336, 256),
-                                     (128, 14336, 4096, 64)])
+                                     (128, 14336, 4096, 64), (213, 6144, 1920, 128), (150, 12288, 1152, 64)])
 def test_prefill_gemm_launches_repeat_bit_for_bit(cabi, M, N, K, g):
     """The prefill kernels sum in a fixed order, so 40 launches on the same operands must give the same fp32 bits; a
     result read before its matrix instruction has finished (their latency is the kernels' own business: the
-    instructions are asm statements) shows up as a launch that differs in a few elements."""
+    instructions are asm statements) shows up as a launch that differs in a few elements.  K = 1920 and 1152 give the
+    four waves of the 128-row kernel different step counts: the waves that leave the loop after an even-numbered step
+    still have that step's look-ahead requests in flight, into registers the epilogue must not use before they landed
+    (it did, for its store addresses: one wave's partial tile went to the wrong place in a few launches of a hundred)."""
     plan = cabi.int4wo_linear_plan(M, K, N, g)
     print(f"case prefill gemm repeat M={M} N={N} K={K} g={g}: {plan}", flush=True)
     assert plan.startswith(("int4wo_gemm_lds_kernel", "int4wo_gemm_kwave_kernel"))

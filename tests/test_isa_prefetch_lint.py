@@ -164,9 +164,9 @@ def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched
     """int4wo_gemm_lds_kernel issues every load of its K loop as an asm statement and waits for them with explicit
     s_waitcnt vmcnt(0) statements; the compiler neither counts those loads nor knows that their target registers are
     being filled.  Checked on the generated ISA of every instantiation:
-      * between a weight load and the next vmcnt(0) wait (following the loop's back edge once) no instruction reads or
-        writes the load's target registers, so a copy of stale contents or a reuse of a register under a load in flight
-        (the epilogue's, after the last, unused requests of the loop) cannot happen;
+      * between a weight load and the next vmcnt(0) wait, on every path (around the loop's back edge and out of the loop by
+        either exit), no instruction reads or writes the load's target registers, so a copy of stale contents or a reuse
+        of a register under a load in flight (the epilogue's, after the last, unused requests of the loop) cannot happen;
       * the K loop carries the LDS-direct activation requests (16 per two steps and wave of the 256-row kernel, 32 of the
         128-row kernel, whose waves each bring in their own slices) and the weight requests (a chunk and its scale / zero
         per 32-row block) of its two steps;
@@ -201,17 +201,30 @@ def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched
         loads = [i for i, l in enumerate(lines) if re.match(r"global_load_dword(x4)? v", l)]
         assert sum(1 for i in loads if loop_head < i < loop_end) == 2 * nt * 2, name   # chunk + qparams per block, two steps
         assert sum(1 for l in lines[loop_head:loop_end] if l.startswith("global_load_lds_dwordx4")) == dma, name
+        # every path from a load to its first vmcnt(0) wait: around the back edge, and out of the loop by either exit
+        # (the requests of the last step are issued for a step past the end and are still in flight when the loop is
+        # left; the wait behind the loop names their targets as operands, which is what keeps the epilogue's first
+        # instructions, scheduled in front of that wait, out of those registers)
         for i in loads:
             dest = _regs(lines[i].split(",")[0])
-            j, jumped = i + 1, False
-            while j < len(lines) and not lines[j].startswith("s_waitcnt vmcnt(0)"):
+            todo, seen = [i + 1], set()
+            while todo:
+                j = todo.pop()
+                if j in seen:
+                    continue
+                seen.add(j)
+                assert j < len(lines), (name, lines[i], "no wait before the end of the kernel")
+                if lines[j].startswith("s_waitcnt vmcnt(0)"):
+                    continue
                 touched = not lines[j].startswith((".LBB", "s_", "global_load")) and _regs(lines[j]) & dest
                 assert not touched, (name, lines[i], lines[j])
-                if j == loop_end and not jumped:
-                    j, jumped = loop_head, True
-                    continue
-                j += 1
-            assert j < len(lines), (name, lines[i])
+                b = re.match(r"s_(c?)branch\w* (\.LBB\d+_\d+)", lines[j])
+                if b:
+                    todo.append(labels[b.group(2)])
+                    if b.group(1):
+                        todo.append(j + 1)
+                else:
+                    todo.append(j + 1)
         # the accumulators are first read behind the wait that follows the loop: the matrix instructions are asm
         # statements, whose result latency the compiler does not know, so a copy placed right behind the loop would
         # read a register the last matrix instructions have not written yet
