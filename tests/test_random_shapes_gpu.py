@@ -1,85 +1,148 @@
-"""GPU consistency sweep over random shapes: every linear kernel (decode kernel, tiled kernels with both tile sizes,
-general fallback; int4, FP6 / FP5, int8) against an fp32 matmul on the weight that the library's own dequantize kernels
-return.  Those dequantize kernels are compared bit for bit with the CPU oracle in the parity tests, so this
-sweep extends that parity to many shapes at the price of a GPU matmul: ragged N, K not a multiple of 128, M on
-both sides of every dispatch boundary.  fp32 outputs, tolerance 2e-5 relative L2 (accumulation order only)."""
-import numpy as np
+"""Seeded random shapes through the linear entry points, each compared with the matrix product of the library's own
+dequantized weight, and the fused quantize + pack kernels compared bit for bit with the step-by-step primitives.
+
+The kernel a call runs is chosen from (M, N, K, group) by a dispatch with a dozen branches per format; the hand-picked
+shapes of the other tests reach every branch, these reach the combinations nobody thought of (a 128-row tile kernel
+whose waves take different numbers of K steps was found wrong this way, at 213 x 6144 x 1920).  Every case prints its
+shape first.
+"""
+import random
+
 import pytest
 import torch
 
 pytestmark = pytest.mark.gpu
 
 
-def _dev():
-    assert torch.cuda.is_available()
-    return torch.device("cuda:0")
+def _rel_l2(y, ref):
+    return float((y.float() - ref.float()).norm() / ref.float().norm().clamp_min(1e-30))
 
 
-def _rel(a, b):
-    return float((a.double() - b.double()).norm() / b.double().norm().clamp(min=1e-30))
+def _rows(rng):
+    r = rng.random()
+    if r < 0.3:
+        return rng.randint(1, 16)
+    if r < 0.6:
+        return rng.randint(17, 64)
+    if r < 0.85:
+        return rng.randint(65, 300)
+    return rng.choice([384, 512, 777, 1024])
 
 
-def test_int4_linear_random_shapes():
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_linear_entry_points_on_random_shapes(seed):
     from ao_amd import ops
 
-    dev = _dev()
-    rng = np.random.default_rng(2024)
-    gen = torch.Generator(device=dev).manual_seed(7)
-    for case in range(40):
-        g = int(rng.choice([32, 64, 128, 256]))
-        N = int(rng.integers(1, 700))
-        K = int(rng.integers(1, 12)) * 128 if case % 3 else int(rng.integers(1, 1500))
-        M = int(rng.choice([1, 2, 3, 15, 16, 17, 33, 64, 65, 130, 300]))
-        print(f"case int4 random N={N} K={K} M={M} g={g}", flush=True)
-        Kq = -(-K // g) * g
-        w = (torch.randn(N, Kq, device=dev, generator=gen) * 0.05).bfloat16()
-        w[:, K:] = 0                              # the reference zero-pads K to a group multiple before quantizing
-        x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
-        packed, qp = ops.int4wo_quantize_pack(w[:, :K].contiguous() if K % g == 0 else w, g)
-        Kw = K if K % g == 0 else Kq
-        dq = ops.int4wo_dequantize(packed, qp, N, Kw, g).float()[:, :K]
-        xin = x if Kw == K else torch.nn.functional.pad(x, (0, Kw - K))
-        y = ops.int4wo_linear(xin, packed, qp, g, N, None, True)
-        assert _rel(y, x.float() @ dq.t()) <= 2e-5, (N, K, M, g)
+    dev = torch.device("cuda:0")
+    rng = random.Random(seed)
+    torch.manual_seed(seed)
+    for i in range(60):
+        kind = rng.choice(["int4", "int4", "int4", "int8", "fp6"])
+        M = _rows(rng)
+        if kind == "int4":
+            g = rng.choice([32, 64, 128, 256])
+            N = rng.choice([rng.randint(1, 600), 16 * rng.randint(1, 400), 64 * rng.randint(1, 230),
+                            rng.choice([4096, 6144, 14336, 12288, 1024])])
+            K = g * rng.randint(1, max(1, 4096 // g)) if rng.random() < 0.7 else rng.choice([4096, 8192, 14336, 1024, 2048])
+            if N * K > 14336 * 8192:
+                N = 4096
+            bias, resid = rng.random() < 0.4, rng.random() < 0.25
+            f32 = rng.random() < 0.3 and not resid
+            print(f"case random {seed}/{i} int4 M={M} N={N} K={K} g={g} bias={bias} residual={resid} fp32={f32}", flush=True)
+            w = (torch.randn(N, K, device=dev) * 0.02).bfloat16()
+            x = torch.randn(M, K, device=dev).bfloat16()
+            packed, qparams = ops.int4wo_quantize_pack(w, g)
+            dq = ops.int4wo_dequantize(packed, qparams, N, K, g)
+            b = torch.randn(N, device=dev).bfloat16() if bias else None
+            ref = x.float() @ dq.float().t()
+            if bias:
+                ref = ref + b.float()
+            if resid:
+                r = torch.randn(M, N, device=dev).bfloat16()
+                y = ops.int4wo_linear_residual(x, packed, qparams, g, N, r, b)
+                ref = ref.bfloat16().float() + r.float()
+            else:
+                y = ops.int4wo_linear(x, packed, qparams, g, N, b, f32)
+            tol = 2e-5 if f32 else 4e-3   # fp32 output: summation order only; bf16 output: its rounding (2^-9)
+        elif kind == "int8":
+            N = rng.choice([rng.randint(1, 600), 16 * rng.randint(1, 400), rng.choice([4096, 6144, 14336, 1024])])
+            K = rng.choice([128 * rng.randint(1, 32), 128 * rng.randint(1, 112), 4096, 14336])
+            if N * K > 14336 * 8192:
+                N = 4096
+            bias = rng.random() < 0.4
+            print(f"case random {seed}/{i} int8 M={M} N={N} K={K} bias={bias}", flush=True)
+            wq = torch.randint(-128, 128, (N, K), device=dev, dtype=torch.int8)
+            s = (torch.rand(N, device=dev) * 0.01 + 0.001).bfloat16()
+            x = torch.randn(M, K, device=dev).bfloat16()
+            b = torch.randn(N, device=dev).bfloat16() if bias else None
+            y = ops.int8wo_linear(x, wq, s, b)
+            ref = (x.float() @ wq.float().t()).bfloat16().float() * s.float()
+            if bias:
+                ref = ref.bfloat16().float() + b.float()
+            tol = 6e-3   # three bf16 roundings
+        else:
+            eb, mb = rng.choice([(3, 2), (2, 3), (2, 2)])
+            N = 64 * rng.randint(1, 230) if rng.random() < 0.7 else rng.choice([4096, 14336, 6144, 1024])
+            K = 64 * rng.randint(1, 128) if rng.random() < 0.7 else rng.choice([4096, 14336, 8192])
+            if N * K > 14336 * 8192:
+                N = 4096
+            print(f"case random {seed}/{i} fp e{eb}m{mb} M={M} N={N} K={K}", flush=True)
+            w = (torch.randn(N, K, device=dev) * 0.02).half()
+            x = torch.randn(M, K, device=dev).half()
+            data, s = ops.fp6_quantize_pack(w, eb, mb)
+            dq = ops.fp6_dequantize(data, s, eb, mb)
+            y = ops.quant_llm_linear(eb, mb, x, data, s, 1)
+            ref = x.float() @ dq.float().t()
+            tol = 2e-3   # fp16 output rounding (2^-12) and the fp16 rounding of weight * scale
+        err = _rel_l2(y, ref)
+        assert bool(torch.isfinite(y.float()).all()) and err <= tol, (seed, i, kind, M, N, K, err)
 
 
-def test_fp6_linear_random_shapes():
+@pytest.mark.parametrize("seed", [1, 2])
+def test_fused_quantize_pack_kernels_on_random_shapes_bit_exact(seed):
     from ao_amd import ops
+    from ao_amd.quantization.utils import get_groupwise_affine_qparams, groupwise_affine_quantize_tensor_from_qparams
 
-    dev = _dev()
-    rng = np.random.default_rng(99)
-    gen = torch.Generator(device=dev).manual_seed(8)
-    for case in range(24):
-        ebits, mbits = [(3, 2), (2, 3), (2, 2), (3, 1)][case % 4]
-        N = int(rng.integers(1, 12)) * 64
-        K = int(rng.integers(1, 24)) * 64
-        M = int(rng.choice([1, 3, 16, 17, 64, 65, 129, 300]))
-        print(f"case fpx random e{ebits}m{mbits} N={N} K={K} M={M}", flush=True)
-        w = (torch.randn(N, K, device=dev, generator=gen) * 0.05).half()
-        x = (torch.rand(M, K, device=dev, generator=gen) - 0.5).half()
-        data, scale = ops.fp6_quantize_pack(w, ebits, mbits)
-        dq = ops.fp6_dequantize(data, scale, ebits, mbits).half().float()   # the kernel rounds code * scale to fp16
-        y = ops.quant_llm_linear(ebits, mbits, x, data, scale)
-        ref = (x.float() @ dq.t())
-        assert _rel(y.float(), ref.half().float()) <= 1e-3, (N, K, M, ebits, mbits)
+    dev = torch.device("cuda:0")
+    rng = random.Random(100 + seed)
+    torch.manual_seed(100 + seed)
 
+    def special_values(w):
+        for v in (0.0, float("inf"), -float("inf"), float("nan"), 1e-30, -1e-30, 3e38, 65504.0, 6e-8):
+            if rng.random() < 0.25:
+                idx = torch.randint(0, w.numel(), (max(1, w.numel() // 5000),), device=dev)
+                w.view(-1)[idx] = v
+        return w
 
-def test_int8_linear_random_shapes():
-    from ao_amd import ops
-
-    dev = _dev()
-    rng = np.random.default_rng(5)
-    gen = torch.Generator(device=dev).manual_seed(9)
-    for case in range(24):
-        N = int(rng.integers(1, 900))
-        K = int(rng.integers(1, 20)) * 128
-        M = int(rng.choice([1, 2, 16, 17, 40]))
-        print(f"case int8 random N={N} K={K} M={M}", flush=True)
-        q = torch.randint(-128, 128, (N, K), device=dev, dtype=torch.int8, generator=gen)
-        s = (torch.rand(N, device=dev, generator=gen) * 1e-2 + 1e-3).bfloat16()
-        x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
-        y = ops.int8wo_linear(x, q, s, None, True)                        # bf16(x @ q^T) * s, before the last rounding
-        acc = x.float() @ q.float().t()
-        ref = acc.bfloat16().float() * s.float()
-        # an accumulator on a bf16 rounding boundary may land on the other side: allow a few one-ulp elements
-        assert _rel(y, ref) <= 1e-3 and float(((y - ref).abs() > 1e-6 * ref.abs() + 1e-12).float().mean()) <= 0.02
+    for i in range(60):
+        scale = rng.choice([0.02, 1.0, 100.0, 1e-3])
+        if rng.random() < 0.5:
+            g = rng.choice([32, 64, 128, 256])
+            N = rng.choice([rng.randint(1, 700), 16 * rng.randint(1, 300), rng.choice([4096, 1024])])
+            K = g * rng.randint(1, max(1, 6144 // g))
+            print(f"case random pack {seed}/{i} int4 N={N} K={K} g={g} scale={scale}", flush=True)
+            w = (torch.randn(N, K, device=dev) * scale).bfloat16()
+            if rng.random() < 0.3:
+                w[:, :g] = 0   # constant groups
+            if rng.random() < 0.3:
+                w = special_values(w)
+            packed, qparams = ops.int4wo_quantize_pack(w, g)
+            s, z = get_groupwise_affine_qparams(w, 4, g, torch.bfloat16)
+            codes = groupwise_affine_quantize_tensor_from_qparams(w, s, z, 4, g)
+            packed2, qparams2 = ops.int4wo_pack(codes, s, z, g)
+            assert torch.equal(packed, packed2) and torch.equal(qparams, qparams2), (seed, i, N, K, g)
+        else:
+            eb, mb = rng.choice([(3, 2), (2, 3), (2, 2)])
+            N = 64 * rng.randint(1, 40)
+            K = 64 * rng.randint(1, 40) if rng.random() < 0.8 else rng.choice([4096, 1024, 2048])
+            dt = rng.choice([torch.bfloat16, torch.float16])
+            print(f"case random pack {seed}/{i} fp e{eb}m{mb} N={N} K={K} {dt} scale={scale}", flush=True)
+            w = (torch.randn(N, K, device=dev) * scale).to(dt)
+            if rng.random() < 0.3:
+                w[rng.randrange(N)] = 0
+            if rng.random() < 0.3:
+                w = special_values(w)
+            # 16-bit rows take the one-launch kernel with the hardware conversions, fp32 rows the three-launch path
+            data, s = ops.fp6_quantize_pack(w, eb, mb)
+            data2, s2 = ops.fp6_quantize_pack(w.float(), eb, mb)
+            assert torch.equal(data, data2) and torch.equal(s.view(torch.int16), s2.view(torch.int16)), (seed, i, N, K)
