@@ -235,3 +235,87 @@ def test_prefill_gemm_requests_are_waited_for_before_their_registers_are_touched
         # values the epilogue needs may be parked in scratch around the loop, never inside it
         assert not [l for l in lines[loop_head:loop_end] if l.startswith("scratch_")], name
         assert len(re.findall(r"v_mfma_f32_32x32x16_bf16 a\[", body)) >= (64 * nt if dma == 16 else 64), name
+
+
+def _vmcnt(line):
+    m = re.search(r"vmcnt\((\d+)\)", line)
+    return int(m.group(1)) if m else None
+
+
+def _asm_load_violations(body):
+    """Walks every path from every asm-issued global load of a kernel to the wait that covers it and returns the
+    instructions on the way that read or write the load's target registers.
+
+    The count wait `s_waitcnt vmcnt(n)` covers a load when at least n vector memory loads were issued after it (they
+    return in order).  Loads the compiler issues count too; stores are ignored, which only makes the check stricter."""
+    raw = [l.strip() for l in body.splitlines()]
+    lines, in_asm, is_asm = [], False, []
+    for l in raw:
+        if l.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if l.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if not l or l.startswith(";") or (l.startswith(".") and not l.startswith(".LBB")):
+            continue
+        lines.append(l.split(";")[0].strip())
+        is_asm.append(in_asm)
+    labels = {re.match(r"(\.LBB\d+_\d+):", l).group(1): i for i, l in enumerate(lines) if re.match(r"\.LBB\d+_\d+:", l)}
+    is_load = [bool(re.match(r"(global|buffer|scratch|flat)_load", l)) for l in lines]
+    out = []
+    for i, l in enumerate(lines):
+        if not (is_asm[i] and re.match(r"global_load_dword(x[234])? v", l)):
+            continue
+        dest = _regs(l.split(",")[0])
+        todo, seen = [(i + 1, 0)], set()
+        while todo:
+            j, younger = todo.pop()
+            if (j, younger) in seen or j >= len(lines):
+                continue
+            seen.add((j, younger))
+            cur = lines[j]
+            if cur.startswith("s_endpgm"):
+                continue
+            if cur.startswith("s_waitcnt"):
+                n = _vmcnt(cur)
+                if n is not None and younger >= n:
+                    continue
+            elif is_load[j]:
+                younger = min(younger + 1, 63)
+            elif not cur.startswith((".LBB", "s_")) and _regs(cur) & dest:
+                out.append((l, cur))
+                continue
+            b = re.match(r"s_(c?)branch\w* (\.LBB\d+_\d+)", cur)
+            if b:
+                todo.append((labels[b.group(2)], younger))
+                if b.group(1):
+                    todo.append((j + 1, younger))
+            else:
+                todo.append((j + 1, younger))
+    return out
+
+
+@pytest.mark.parametrize("source", ["int4wo_gemm.hip", "int4wo_gemv1.hip"])
+def test_asm_loads_are_waited_for_on_every_path_before_their_registers_are_touched(tmp_path, source):
+    """Every kernel that issues global loads from asm statements (the weight streams of the GEMV rings and of the
+    prefill kernels): between such a load and the wait that covers it, on every path through loops and out of them,
+    nothing reads or writes the registers being filled.  The compiler knows neither that the load is outstanding nor,
+    once the loaded value is dead, that the register is not free yet."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not available")
+    asm = tmp_path / (source + ".s")
+    subprocess.run([hipcc, *_FLAGS, "-o", str(asm), os.path.join(_ROOT, "ao_amd", "csrc", source)], check=True,
+                   capture_output=True, timeout=900)
+    text = asm.read_text()
+    kernels = list(re.finditer(r"^(_ZN2ao\w+): ; @.*?\n(.*?)\.end_amdhsa_kernel", text, re.S | re.M))
+    checked = 0
+    for m in kernels:
+        name, body = m.group(1), m.group(2)
+        if ";;#ASMSTART\n\tglobal_load_dword" not in body:
+            continue
+        checked += 1
+        bad = _asm_load_violations(body)
+        assert not bad, (name, bad[:4])
+    assert checked >= 4, (source, checked)
