@@ -631,16 +631,22 @@ static bool gemm_lds_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
     // lane offsets are 32 bits wide: one tile's rows of the activations, the packed codes and the qparams within reach
     if (256 * a.ldx * 2 >= ((int64_t)1 << 32) || 16 * (a.Kp / 128) * 1024 + 1024 >= ((int64_t)1 << 32)) return false;
     p->tiles_m = (int)((a.M + 255) / 256);
-    // 256 x 256 tiles unless they leave more than a fifth of the 256 CUs without one and 256 x 128 tiles fill more
+    // One workgroup per CU, each walking all of K: worth it from 3/4 of the CUs busy
+    // (measured: N = 4096, K = 14336 at 512 rows gives 64 tiles and 175 us against 116 us of the 128-row kernel).
+    // 256 x 256 or 256 x 128 tiles, whichever needs less time for its rounds over the 256 CUs: a 256 x 128 tile takes
+    // 0.51 of a 256 x 256 tile's time (14336 x 4096 at 2048 rows: 217 us in four rounds against 212 us in two), so
+    // e.g. 14336 x 4096 at 640 rows runs 336 narrow tiles (95 us) where 168 wide ones would not fill the chip, and
+    // 28672 x 4096 at 2048 rows seven rounds of narrow tiles (405 us) instead of four rounds of wide ones (422 us).
     const int64_t t256 = (int64_t)p->tiles_m * ((a.N + 255) / 256), t128 = (int64_t)p->tiles_m * ((a.N + 127) / 128);
-    auto fill = [](int64_t t) { return (double)t / (double)((t + 255) / 256 * 256); };
-    p->nt = (fill(t256) < 0.8 && fill(t128) > fill(t256)) ? 1 : 2;
+    auto cost = [](int64_t t, double per_tile) { return t >= 192 ? (double)((t + 255) / 256) * per_tile : 1e30; };
+    const double c256 = cost(t256, 1.0), c128 = cost(t128, 0.51);
+    p->nt = c128 < c256 ? 1 : 2;
     if (const char* e = getenv("AO_AMD_GEMM_LDS_NT")) p->nt = e[0] == '1' ? 1 : 2;   // measurement aid
     p->tiles_n = (int)((a.N + 128 * p->nt - 1) / (128 * p->nt));
-    // One workgroup per CU, each walking all of K: worth it from 3/4 of the CUs busy and 3/4 of the tile rows real
-    // (measured: N = 4096, K = 14336 at 512 rows gives 64 tiles and 175 us against 116 us of the 128-row kernel)
     const int64_t tiles = (int64_t)p->tiles_m * p->tiles_n;
-    if (tiles < 192 || a.M * 4 < (int64_t)p->tiles_m * 256 * 3) return false;
+    // ... and more than half of the tile rows real: at exactly 128 rows the 128-row kernel is faster (28672 x 4096: 50
+    // against 61 us), from there on this one (288 rows on 28672 x 4096: 104 us against 127 us of the 64-row tiles)
+    if (tiles < 192 || a.M * 2 <= (int64_t)p->tiles_m * 256) return false;
     return (int64_t)p->tiles_m * p->tiles_n < (1 << 24);
 }
 

@@ -68,7 +68,11 @@ def test_dispatch_walk_finds_every_kernel_family():
     assert _lib.int4wo_linear_plan(512, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
     assert _lib.int4wo_linear_plan(2048, 14336, 4096, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
     assert not _lib.int4wo_linear_plan(512, 14336, 4096, 64).startswith("int4wo_gemm_lds_kernel")   # 64 tiles
-    assert not _lib.int4wo_linear_plan(300, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel")   # 212 of 512 tile rows empty
+    assert _lib.int4wo_linear_plan(300, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
+    assert not _lib.int4wo_linear_plan(128, 4096, 28672, 64).startswith("int4wo_gemm_lds_kernel")   # half of the tile rows empty
+    # 256 x 128 tiles where 256 x 256 ones would not fill the chip (168) or would need more time for their rounds
+    assert _lib.int4wo_linear_plan(768, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
+    assert _lib.int4wo_linear_plan(2048, 4096, 28672, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
     # ... and the 128-row tiles with K split over the waves where those do not, from about 100 rows, when at least 192
     # of them exist
     assert _lib.int4wo_linear_plan(128, 4096, 14336, 64) == "int4wo_gemm_kwave_kernel<64>"
