@@ -1426,7 +1426,12 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
     // (with four row blocks per activation tile in registers the rows need no staging: 12.7 / 12.9 us against 13.1 /
     // 17.4 us staged at 4 / 8 rows on 14336 x 4096; 16 rows, which never fit, 13.9 against 21.8 us)
     const bool shared_tiles = !need_lds && M >= 4 && fp6_row_blocks_per_wave(M, RB, mchunks) == 4;
-    if (fits && !shared_tiles && (need_lds || KB >= 4 * waves)) {
+    // ... and for one or two rows only (three on weights with 768 or more row blocks): from there on the streaming
+    // kernel whose lanes load their activation fragments themselves is faster without the staging pass and its barrier
+    // (us staged / not: 4096 x 4096 at 4 / 6 / 8 rows 5.9 / 5.4, 6.1 / 5.4, 6.5 / 5.7; 6144 x 4096 7.5 / 6.5, 7.9 / 6.8,
+    // 8.2 / 7.2; 4096 x 14336 at 4 rows 12.1 / 11.4; at 2 rows staged wins everywhere: 14336 x 4096 9.6 / 11.7)
+    const bool stage_pays = M <= 2 || (M == 3 && RB >= 768);
+    if (fits && !shared_tiles && (need_lds || (KB >= 4 * waves && stage_pays))) {
         Fp6GemvArgs a{xx, M, K, Kp, nat, sc, N, o, res, gt, (const uint16_t*)norm_weight_f16, norm_eps,
                       (const uint32_t*)native_up, (const uint16_t*)scale_up_f16};
         if (ebits == 3) {

@@ -1163,7 +1163,13 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // static arrays (cross-wave reduction: 1 KB per wave and weight, RMSNorm partials), fits one workgroup's limit
     const size_t static_lds = (size_t)(dual ? 2 : 1) * waves * 1024 + 256;
     const bool lds_ok = xbytes <= (size_t)waves * 10 * 1024 && xbytes + static_lds <= 160 * 1024;
-    int xmode = aligned ? (lds_ok ? X_LDS : X_GLOBAL) : X_CHECKED;
+    // ... and only where it pays: for one row, for the fused forms that exist on the staged kernel only, and for two
+    // rows on the widest weights.  From two rows on the kernel whose lanes load their activation fragments themselves
+    // (served by the CU's L1) is faster without the staging pass and its barrier (us, staged / not, 4096 x 4096 at 2 / 4 /
+    // 8 / 16 rows: 7.0 / 5.8, 7.7 / 6.3, 8.2 / 6.5, 9.9 / 7.9; 6144 x 4096 at 2 / 4 / 10 rows: 9.1 / 7.8, 9.6 / 8.2, 14.8 / 9.5;
+    // 4096 x 14336 at 2 / 4 rows: 13.2 / 12.5, 14.0 / 12.6; 14336 x 4096 at 2 rows 13.6 / 13.6; 28672 x 4096 at 2 rows 21.2 / 23.1).
+    const bool want_lds = M == 1 || norm_weight_bf16 || pair8 || packed2 != nullptr || ksplit > 1 || (M == 2 && RB >= 1536);
+    int xmode = aligned ? (lds_ok && want_lds ? X_LDS : X_GLOBAL) : X_CHECKED;
     LinearArgs a{(const uint16_t*)x_bf16, M, K, ldx, (const uint4*)packed, (const uint32_t*)qparams,
                  (const uint4*)packed2, (const uint32_t*)qparams2, n_out, Kp, (const uint16_t*)bias_bf16,
                  (const uint16_t*)residual_bf16, ldres, y, y_dtype == AO_F32, ldy,

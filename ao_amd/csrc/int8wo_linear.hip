@@ -506,7 +506,11 @@ static int int8wo_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // staging costs a pass over the rows and a barrier: it pays once a wave has 4 or more K tiles to stream
     // (the staged path addresses the weight with 32-bit per-lane offsets)
     const bool fits = xbytes <= 64 * 1024 && xbytes <= (int64_t)waves * 16 * 1024 && N * ldw < ((int64_t)1 << 32);
-    const bool staged = fits && (need_lds || KB >= 4 * waves);
+    // ... and, from three rows on, only where the kernel with four row blocks per workgroup below does not apply: it
+    // needs no staging pass (14336 x 4096 at 3 / 4 / 5 / 8 rows: 17.2 / 17.7 / 21.9 / 23.3 us staged, 16.6 / 16.9 / 17.2 /
+    // 17.4 us not; at 2 rows the staged kernel is as fast or faster everywhere: 28672 x 4096 25.9 against 30.6 us)
+    const bool four_blocks_ok = RB % 4 == 0 && (RB / 4) * ((M + 15) / 16) >= 192 && KB >= 8;
+    const bool staged = fits && (need_lds || (KB >= 4 * waves && (M <= 2 || !four_blocks_ok)));
     AO_REQUIRE(!need_lds || (staged && (((uintptr_t)norm_weight_bf16) & 15) == 0),
                "the fused RMSNorm and the two-weight SwiGLU need the activation rows to fit in LDS (M=%lld K=%lld) and a "
                "16-byte aligned norm weight", (long long)M, (long long)K);
