@@ -81,8 +81,21 @@ _LIB.define("fp6_linear_native_fused(int ebits, int mbits, Tensor x, Tensor nati
 TWO_PASS_MIN_M = 4096
 
 
+# int8 and FPx: the same choice.  The conversion pass costs the same whatever the row count, so the narrower the weight
+# the later it pays (fused / two-pass in us, int8: 14336 x 4096 at 96 / 128 / 256 rows 57 / 58, 73 / 61, 128 / 76;
+# 4096 x 4096 at 128 / 256 / 384 rows 22 / 42, 40 / 42, 53 / 41; 4096 x 14336 at 128 / 192 / 256 rows 64 / 93, 125 / 113,
+# 125 / 80; 1024 x 4096 at 512 / 1536 rows 22 / 37, 51 / 38.  FP6: 14336 x 4096 at 768 / 1024 rows 115 / 126, 142 / 134;
+# 4096 x 4096 at 1024 / 1536 / 3072 rows 50 / 54, 71 / 66, 113 / 96; 1024 x 4096 at 2048 / 3072 rows 32 / 36, 46 / 41).
 INT8_TWO_PASS_MIN_M = 128
 FP6_TWO_PASS_MIN_M = 1024
+
+
+def int8wo_two_pass(M: int, N: int, K: int) -> bool:
+    return M >= INT8_TWO_PASS_MIN_M and (M * N >= 1500000 or (K >= 8192 and M * N >= 700000))
+
+
+def fp6_two_pass(M: int, N: int, K: int) -> bool:
+    return M >= (3 * FP6_TWO_PASS_MIN_M if N < 2048 else (3 * FP6_TWO_PASS_MIN_M // 2 if N <= 4096 else FP6_TWO_PASS_MIN_M))
 
 
 def int4wo_two_pass(M: int, N: int, K: int) -> bool:
@@ -241,7 +254,7 @@ def _int8wo_linear_cuda(x, w_int8, scale, bias, fp32_out):
     if bias is not None:
         torch._check(bias.dtype is torch.bfloat16 and bias.numel() == N, lambda: "bias must be bfloat16 of size N")
         bias = bias.contiguous()
-    if M >= INT8_TWO_PASS_MIN_M and not fp32_out and K % 16 == 0:
+    if int8wo_two_pass(M, N, K) and not fp32_out and K % 16 == 0:
         # prefill-sized batch: bf16 copy of the codes (HIP kernel), library bf16 GEMM, scale, bias: the reference's
         # `torch.mm(x, w_int8.t().to(x.dtype)) * scale` (+ bias) op by op.  The streaming kernel below re-reads the
         # weight for every 16 activation rows and falls behind from about 128 rows on.
@@ -646,7 +659,7 @@ def _fp6_linear_native_cuda(ebits, mbits, x, native, scale):
     M, K = x.shape
     N = scale.shape[0]
     torch._check(native.dtype is torch.int32 and native.numel() == _fp6_native_numel(N, K), lambda: "Dimensions mismatched")
-    if M >= FP6_TWO_PASS_MIN_M:
+    if fp6_two_pass(M, N, K):
         # prefill-sized batch: the weight as an fp16 matrix (HIP kernel, the same fp16(fpx * scale) values the fused
         # kernel multiplies) and the library fp16 GEMM; the fused kernel tops out near 0.95 PFLOP/s, the library GEMM
         # at 1.3-1.5, and the conversion costs about as much as 300 activation rows

@@ -234,7 +234,7 @@ def test_weight_subclass_and_api(oracle):
 
 @pytest.mark.parametrize("fmt,shape", [((3, 2), (256, 1024)), ((3, 2), (512, 192)), ((2, 3), (320, 256)), ((2, 2), (128, 320)),
                                        ((3, 1), (64, 128))])
-def test_native_to_fp16_is_the_scaled_weight_and_feeds_the_two_pass_linear(oracle, fmt, shape):
+def test_native_to_fp16_is_the_scaled_weight_and_feeds_the_two_pass_linear(oracle, fmt, shape, monkeypatch):
     """Prefill path: the native tiles converted to an fp16 matrix are bit for bit fp16(fpx value * scale) (oracle codes
     and scales, one fp16 multiply each, zero rows / ragged last K tile included), and the op's result from 1024 rows on
     (library GEMM on that matrix) stays within the op's tolerance of the oracle."""
@@ -256,10 +256,13 @@ def test_native_to_fp16_is_the_scaled_weight_and_feeds_the_two_pass_linear(oracl
     want = (values.half() * scale.view(-1, 1))                  # one fp16 multiply, as the kernels do
     assert np.array_equal(bits16(w16), bits16(want))
     M = ops.FP6_TWO_PASS_MIN_M
+    assert ops.fp6_two_pass(M, 14336, 4096) and not ops.fp6_two_pass(M, 1024, 4096) and ops.fp6_two_pass(3 * M, 1024, 4096)
     x = (torch.rand(M, K, generator=g) + 0.5).half().to(dev)
+    monkeypatch.setattr(ops, "fp6_two_pass", lambda M, N, K: True)   # these small weights would stay on the fused kernel
     y = ops.fp6_linear_native(e, m, x, native, scale).float().cpu().numpy()
     ref = (x.double() @ want.double().t()).cpu().numpy()
     ref16 = ref.astype(np.float16).astype(np.float32)
     assert rel_l2(y, ref16) <= 1e-3
+    monkeypatch.setattr(ops, "fp6_two_pass", lambda M, N, K: False)
     y_small = ops.fp6_linear_native(e, m, x[:64], native, scale).float().cpu().numpy()   # fused kernel, same rows
     assert rel_l2(y[:64], y_small) <= 1e-3

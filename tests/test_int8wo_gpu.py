@@ -47,9 +47,9 @@ def test_quantize_bit_exact(oracle, shape):
     assert np.array_equal(zero.cpu().numpy().reshape(-1), z.reshape(-1))
 
 
-@pytest.mark.parametrize("M", [1, 4, 16, 33, 130, 300])  # from 128 rows on the bf16 result comes from the two-pass path
+@pytest.mark.parametrize("M", [1, 4, 16, 33, 130, 300])  # from 128 rows on the two-pass path is checked as well
 @pytest.mark.parametrize("shape", [(256, 1024), (48, 256), (1000, 4096)])
-def test_linear_matches_oracle(oracle, shape, M):
+def test_linear_matches_oracle(oracle, shape, M, monkeypatch):
     from ao_amd import ops
 
     N, K = shape
@@ -75,6 +75,12 @@ def test_linear_matches_oracle(oracle, shape, M):
     assert rel_l2(y32, pre) <= 1e-3
     assert rel_l2(y16, expect) <= 1e-3
     assert np.count_nonzero(y16 != expect) <= 0.02 * y16.size + 1
+    if M >= ops.INT8_TWO_PASS_MIN_M:
+        # large weights take the bf16 copy of the codes + the library GEMM from here on (ops.int8wo_two_pass): same bar
+        monkeypatch.setattr(ops, "int8wo_two_pass", lambda M, N, K: True)
+        y2p = ops.int8wo_linear(x.to(dev), qd, sd, bd, False).float().cpu().numpy()
+        assert rel_l2(y2p, expect) <= 1e-3
+        assert np.count_nonzero(y2p != expect) <= 0.02 * y2p.size + 1
 
 
 def test_one_hot_rows_return_scaled_codes(oracle):
