@@ -650,12 +650,13 @@ static bool gemm_lds_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
     return (int64_t)p->tiles_m * p->tiles_n < (1 << 24);
 }
 
-// 128 x 64 tiles with K split over the waves: where the 256-row tiles do not apply, from about 100 rows, when the tiles
+// 128 x 64 tiles with K split over the waves: where the 256-row tiles do not apply, from 65 rows (14336 x 4096 at 65-99
+// rows: 39 us on the 64-row tiles, two passes, against 26 us; at 33-64 rows those are as fast or faster), when the tiles
 // cover at least three quarters of the CUs (measured: with 128 tiles the older kernels are as fast)
 static bool gemm_kwave_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
     static const bool disabled = [] { const char* e = getenv("AO_AMD_GEMM_KWAVE"); return e && e[0] == '0'; }();
     if (disabled) return false;
-    static const int64_t min_rows = [] { const char* e = getenv("AO_AMD_GEMM_KWAVE_MIN_M"); return e ? atoll(e) : 100ll; }();
+    static const int64_t min_rows = [] { const char* e = getenv("AO_AMD_GEMM_KWAVE_MIN_M"); return e ? atoll(e) : 65ll; }();
     if (a.M < min_rows || a.K != a.Kp || a.Kp < 1024 || a.packed2 || a.residual || a.norm_w || a.pair8 || a.ksplit != 1) return false;
     if (g != 32 && g != 64 && g != 128 && g != 256) return false;
     if (128 * a.ldx * 2 >= ((int64_t)1 << 32) || 4 * (a.Kp / 128) * 1024 + 1024 >= ((int64_t)1 << 32)) return false;

@@ -526,7 +526,9 @@ static int int8wo_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // 100 rows 31 / 34 / 59 / 97 -> 20.5 / 23 / 43 / 67 us, the head at 32 rows 243 -> 144
     const int mbv = M > 16 ? 2 : 1;
     const int64_t mch = (M + 16 * mbv - 1) / (16 * mbv);
-    if (!staged && !rb4_disabled && RB % 4 == 0 && (RB / 4) * mch >= 192 && KB >= 8) {
+    // (from 49 rows on 128 workgroups are enough: 4096 x 14336 at 56 / 64 rows 80 / 84 -> 63 us, 4096 x 4096 24 / 26 -> 21;
+    // below, the one-block kernel's two or three passes are as fast or faster: 57 against 64 us at 33 rows)
+    if (!staged && !rb4_disabled && RB % 4 == 0 && (RB / 4) * mch >= (M > 48 ? 128 : 192) && KB >= 8) {
         const int64_t wgs = (RB / 4) * mch;
         int w4 = 4;
         while (w4 < 8 && wgs * w4 * 2 <= 4096 + wgs && w4 * 2 <= KB) w4 *= 2;

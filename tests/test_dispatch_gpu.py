@@ -73,12 +73,13 @@ def test_dispatch_walk_finds_every_kernel_family():
     # 256 x 128 tiles where 256 x 256 ones would not fill the chip (168) or would need more time for their rounds
     assert _lib.int4wo_linear_plan(768, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
     assert _lib.int4wo_linear_plan(2048, 4096, 28672, 64).startswith("int4wo_gemm_lds_kernel<64,1>")
-    # ... and the 128-row tiles with K split over the waves where those do not, from about 100 rows, when at least 192
+    # ... and the 128-row tiles with K split over the waves where those do not, from 65 rows, when at least 192
     # of them exist
     assert _lib.int4wo_linear_plan(128, 4096, 14336, 64) == "int4wo_gemm_kwave_kernel<64>"
     assert _lib.int4wo_linear_plan(512, 14336, 4096, 64) == "int4wo_gemm_kwave_kernel<64>"
     assert not _lib.int4wo_linear_plan(128, 4096, 4096, 64).startswith("int4wo_gemm_kwave_kernel")   # 64 tiles
-    assert not _lib.int4wo_linear_plan(99, 1024, 14336, 64).startswith("int4wo_gemm_kwave_kernel")
+    assert _lib.int4wo_linear_plan(65, 1024, 14336, 64) == "int4wo_gemm_kwave_kernel<64>"
+    assert not _lib.int4wo_linear_plan(64, 1024, 14336, 64).startswith("int4wo_gemm_kwave_kernel")
     # 4 to 16 rows on weights with 768 or more 16-row blocks: four row blocks per workgroup share the activation loads
     assert _lib.int4wo_linear_plan(16, 4096, 14336, 64) == "int4wo_linear_rb4_kernel<64,8>"
     assert _lib.int4wo_linear_plan(4, 4096, 128256, 64) == "int4wo_linear_rb4_kernel<64,4>"
