@@ -346,7 +346,7 @@ template <int G, int WAVES, int MB>
 __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const LinearArgs a) {
     // MB 16-row blocks of activations per workgroup (17 to 32 rows with MB = 2): every dequantized dword then feeds MB
     // matrix instructions, and the dequantization, which bounds the kernel, is done once for all of them
-    constexpr int D = 2, RBW = 4;
+    constexpr int RBW = 4;
     static_assert(WAVES <= 8, "the reduction buffer is 4 KB per row block, activation block and wave");
     __shared__ float red[RBW][WAVES][4][64];
     const int lane = threadIdx.x & 63;
@@ -398,10 +398,11 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const Lin
     };
     u32x4_t tcur = {0, 0, 0, 0};
     // one tile = 16 dwords per lane (4 row blocks x 4); the three dequantization stages run as in int4wo_linear_kernel
-    auto compute_tile = [&](const Buf& b, const Buf& nb, bool has_next) {
+    auto compute_tile = [&](const Buf& b) {
         GroupConst gc[RBW];
 #pragma unroll
         for (int j = 0; j < RBW; ++j) gc[j] = make_group(b.q[j]);
+        tcur = first_half(b.w[0].x, gc[0], magic);
 #pragma unroll
         for (int e = 0; e < 4 * RBW; ++e) {
             const int j = e >> 2;
@@ -411,9 +412,6 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const Lin
             bf16x8_t bw;
             if (e + 1 < 4 * RBW) {
                 tcur = first_half(b.w[(e + 1) >> 2][(e + 1) & 3], gc[(e + 1) >> 2], magic);
-                bw = round_pack<false>(ua, ub);
-            } else if (has_next) {
-                tcur = first_half(nb.w[0].x, make_group(nb.q[0]), magic);
                 bw = round_pack<false>(ua, ub);
             } else {
                 bw = round_pack<true>(ua, ub);
@@ -427,31 +425,24 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_linear_rb4_kernel(const Lin
         }
     };
 
-    Buf buf[D];
+    // One tile buffer and no look-ahead: with a second buffer the kernel needs 160 to 200 registers, which leaves one
+    // 8-wave workgroup per CU; with one it needs 105 to 140, and the second workgroup on the CU hides the load latency
+    // better than the look-ahead did (14336 x 4096 at 4-16 rows 14.2 -> 13.9 us; 28672 x 4096, 448 workgroups, 24 -> 21;
+    // the vocabulary head 81 -> 71).
+    Buf buf;
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-#pragma unroll
-        for (int j = 0; j < RBW; ++j) {
-            buf[d].w[j] = u32x4_t{0, 0, 0, 0};
-            buf[d].q[j] = 0;
-        }
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int sl = 0; sl < 4; ++sl) buf[d].x[mb][sl] = make_uint4(0, 0, 0, 0);   // rows >= M keep these zeros
+    for (int j = 0; j < RBW; ++j) {
+        buf.w[j] = u32x4_t{0, 0, 0, 0};
+        buf.q[j] = 0;
     }
-    if (wave < KB) load_tile(buf[0], wave);
-    const int nt = wave < KB ? (KB - wave + WAVES - 1) / WAVES : 0;
-    if (nt > 0) tcur = first_half(buf[0].w[0].x, make_group(buf[0].q[0]), magic);
-    for (int i0 = 0; i0 < nt; i0 += D) {
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const int i = i0 + d;
-            if (i < nt) {
-                if (i + 1 < nt) load_tile(buf[(d + 1) % D], wave + (i + 1) * WAVES);
-                compute_tile(buf[d], buf[(d + 1) % D], i + 1 < nt);
-            }
-        }
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) buf.x[mb][sl] = make_uint4(0, 0, 0, 0);   // rows >= M keep these zeros
+    const int nt = wave < KB ? (KB - wave + WAVES - 1) / WAVES : 0;
+    for (int i = 0; i < nt; ++i) {
+        load_tile(buf, wave + i * WAVES);
+        compute_tile(buf);
     }
 
     // acc[j][mb][i] = C[m = m0 + 16 mb + 4*qd + i][n = 16 (rb0 + j) + r]; one pass of the reduction buffer per
@@ -1268,6 +1259,9 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
         if (!rb4_disabled && wgs >= 192) {
             int w4 = 4;   // at least four waves: wave j finishes row block j
             while (w4 < 8 && wgs * w4 * 2 <= 4096 + wgs && w4 * 2 <= a.Kp / 128) w4 *= 2;
+            // two activation blocks (140 registers): beyond one workgroup per CU, three 4-wave workgroups share a CU
+            // where 8-wave ones would queue (28672 x 4096 at 24-32 rows: 32 -> 25.5 us)
+            if (mb == 2 && wgs > 256) w4 = 4;
             if (mb == 1) AO_PLAN("int4wo_linear_rb4_kernel<%lld,%d>", (long long)g, w4);
             AO_PLAN("int4wo_linear_rb4_kernel<%lld,%d,%d>", (long long)g, w4, mb);
             const dim3 grid4((unsigned)(RB / 4), (unsigned)mch);
