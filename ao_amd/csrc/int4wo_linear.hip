@@ -1189,7 +1189,11 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // activation blocks per workgroup (14336 x 4096: 16-18 us against 24.5 us of the 64-row tiles, the head 92-101
     // against 160; from 33 rows, two passes of it, the tiles win again)
     static const bool rb4_off = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
-    const bool rb4_two_blocks = !rb4_off && M > 16 && M <= 32 && RB % 4 == 0 && RB / 4 >= 192 && a.K == a.Kp;
+    // ... and 33 to 48 rows (to 64 on weights with 4096 or more row blocks) with four activation blocks, which fit the
+    // registers since the kernel keeps one tile buffer: 14336 x 4096 at 33-48 rows 25.5 -> 20.4-21.0 us, 28672 x 4096 38 ->
+    // 32-33.5, the head at 33-64 rows 164-167 -> 115-145 (at 56-64 rows the tiles are as fast or faster on the others)
+    const int64_t rb4_max_m = RB / 4 >= 1024 ? 64 : 48;
+    const bool rb4_two_blocks = !rb4_off && M > 16 && M <= rb4_max_m && RB % 4 == 0 && RB / 4 >= 192 && a.K == a.Kp;
     AO_REQUIRE(ksplit == 1 || (xmode == X_LDS && M <= 16 && !dual && !pair8 && !bias_bf16 && !residual_bf16 && y_dtype == AO_F32),
                "partial sums over a split K need M <= 16, fp32 output, no bias / residual epilogue and activations that "
                "fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);
@@ -1253,7 +1257,7 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
         static const bool rb4_disabled = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
         // two 16-row activation blocks per workgroup from 17 rows on: the dequantized dword feeds both (four of them
         // do not fit the registers)
-        const int mb = M > 16 ? 2 : 1;
+        const int mb = M > 32 && M <= rb4_max_m ? 4 : (M > 16 ? 2 : 1);
         const int64_t mch = (M + 16 * mb - 1) / (16 * mb);
         const int64_t wgs = (RB / 4) * mch;
         if (!rb4_disabled && wgs >= 192) {
@@ -1261,7 +1265,7 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
             while (w4 < 8 && wgs * w4 * 2 <= 4096 + wgs && w4 * 2 <= a.Kp / 128) w4 *= 2;
             // two activation blocks (140 registers): beyond one workgroup per CU, three 4-wave workgroups share a CU
             // where 8-wave ones would queue (28672 x 4096 at 24-32 rows: 32 -> 25.5 us)
-            if (mb == 2 && wgs > 256) w4 = 4;
+            if (mb >= 2 && wgs > 256) w4 = 4;
             if (mb == 1) AO_PLAN("int4wo_linear_rb4_kernel<%lld,%d>", (long long)g, w4);
             AO_PLAN("int4wo_linear_rb4_kernel<%lld,%d,%d>", (long long)g, w4, mb);
             const dim3 grid4((unsigned)(RB / 4), (unsigned)mch);
@@ -1278,7 +1282,8 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     else go(int4wo_linear_rb4_kernel<GG, 8, MBV>, 8)
 #define AO_RB4(GG)                                                         \
     if (mb == 1) { AO_RB4_MB(GG, 1); }                                     \
-    else { AO_RB4_MB(GG, 2); }
+    else if (mb == 2) { AO_RB4_MB(GG, 2); }                                \
+    else { AO_RB4_MB(GG, 4); }
             switch (g) {
                 case 32: AO_RB4(32); break;
                 case 64: AO_RB4(64); break;

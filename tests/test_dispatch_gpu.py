@@ -54,7 +54,7 @@ def test_dispatch_walk_finds_every_kernel_family():
                      "int4wo_gemm_ksplit_kernel<%d,4,4>", "int4wo_gemm_ksplit_kernel<%d,2,4>",
                      "int4wo_gemm_lds_kernel<%d,1>", "int4wo_gemm_lds_kernel<%d,2>", "int4wo_gemm_kwave_kernel<%d>",
                      "int4wo_linear_rb4_kernel<%d,4>", "int4wo_linear_rb4_kernel<%d,8>", "int4wo_linear_rb4_kernel<%d,4,2>",
-                     "int4wo_linear_rb4_kernel<%d,8,2>"):
+                     "int4wo_linear_rb4_kernel<%d,8,2>", "int4wo_linear_rb4_kernel<%d,4,4>", "int4wo_linear_rb4_kernel<%d,8,4>"):
             assert tile % g in plans, tile % g
     # the single-row kernel: exactly the instantiations that int4wo_gemv1.hip compiles (waves, chunks per lane, norm)
     gemv1 = {n.split(" ")[0] for n in plans if n.startswith("int4wo_gemv1_kernel<")}
@@ -87,7 +87,10 @@ def test_dispatch_walk_finds_every_kernel_family():
     assert not _lib.int4wo_linear_plan(3, 4096, 14336, 64).startswith("int4wo_linear_rb4_kernel")
     # ... and 17 to 32 rows there take it with two activation blocks per workgroup instead of the 64-row tiles
     assert _lib.int4wo_linear_plan(24, 4096, 14336, 64) == "int4wo_linear_rb4_kernel<64,8,2>"
-    assert not _lib.int4wo_linear_plan(33, 4096, 14336, 64).startswith("int4wo_linear_rb4_kernel")
+    # ... 33 to 48 rows (64 on the widest weights) with four
+    assert _lib.int4wo_linear_plan(40, 4096, 14336, 64) == "int4wo_linear_rb4_kernel<64,8,4>"
+    assert _lib.int4wo_linear_plan(64, 4096, 128256, 64) == "int4wo_linear_rb4_kernel<64,4,4>"
+    assert not _lib.int4wo_linear_plan(49, 4096, 14336, 64).startswith("int4wo_linear_rb4_kernel")
     assert len(plans) >= 88
 
 

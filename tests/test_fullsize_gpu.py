@@ -312,10 +312,12 @@ def test_prefill_gemm_launches_repeat_bit_for_bit(cabi, M, N, K, g):
                                                         (4, 16384, 2048, 32, True, True, False), (9, 14336, 4096, 256, True, False, True),
                                                         (17, 14336, 4096, 64, True, False, False), (29, 14400, 1024, 128, True, True, False),
                                                         (32, 16384, 2048, 256, False, False, True), (11, 14330, 1024, 64, True, False, False),
-                                                        (23, 12346, 1024, 64, False, True, False)])
+                                                        (23, 12346, 1024, 64, False, True, False), (33, 14336, 4096, 64, True, False, False),
+                                                        (48, 14400, 1024, 128, False, True, False), (41, 16384, 2048, 32, True, False, True),
+                                                        (64, 65536, 512, 256, True, True, False)])
 def test_four_row_blocks_per_workgroup_kernel_epilogues(cabi, M, N, K, g, bias, residual, fp32):
-    """int4wo_linear_rb4_kernel (4 to 32 activation rows, four 16-row weight blocks per workgroup sharing the activation
-    loads, two activation blocks from 17 rows): bias, residual (y = bf16(bf16(acc + bias) + residual), the order of the unfused modules), fp32 output and
+    """int4wo_linear_rb4_kernel (4 to 48 or 64 activation rows, four 16-row weight blocks per workgroup sharing the
+    activation loads, two activation blocks from 17 rows, four from 33): bias, residual (y = bf16(bf16(acc + bias) + residual), the order of the unfused modules), fp32 output and
     ragged M, against an fp32 matmul on the bit-exact dequantized weight."""
     plan = cabi.int4wo_linear_plan(M, K, N, g, residual=residual)
     print(f"case rb4 M={M} N={N} K={K} g={g} bias={bias} residual={residual} fp32={fp32}: {plan}", flush=True)
