@@ -383,20 +383,30 @@ def _quantized_linear_op(input_tensor, weight_qtensor, bias):
         and weight_qtensor.block_size[0] == 1
         and weight_qtensor.block_size[1] == weight_qtensor.shape[1]
         and weight_qtensor.zero_point_domain == ZeroPointDomain.INT
-        and weight_qtensor.dtype is torch.bfloat16
-        and layout.int_data.is_cuda
-        and weight_qtensor.shape[1] % 128 == 0
-        and layout.int_data.stride(1) == 1 and layout.int_data.stride(0) % 16 == 0
     ):
         # per-channel int8 weight-only (reference :641-665): mm(x, w_int8.t().to(x.dtype)) * scale, the symmetric
         # recipe's zero point is zero and, as in the reference, does not enter
         orig_shape, orig_dtype = input_tensor.shape, input_tensor.dtype
-        act = input_tensor.reshape(-1, orig_shape[-1]).to(torch.bfloat16)
-        fused_bias = bias if (bias is not None and bias.dtype is torch.bfloat16) else None
-        y = ops.int8wo_linear(act, layout.int_data, layout.scale.reshape(-1).to(torch.bfloat16), fused_bias)
-        y = y.reshape(*orig_shape[:-1], weight_qtensor.shape[0])
-        if bias is not None and fused_bias is None:
-            y = y + bias
+        if (
+            orig_dtype is torch.bfloat16
+            and weight_qtensor.dtype is torch.bfloat16
+            and layout.int_data.is_cuda
+            and weight_qtensor.shape[1] % 128 == 0
+            and layout.int_data.stride(1) == 1 and layout.int_data.stride(0) % 16 == 0
+        ):
+            act = input_tensor.reshape(-1, orig_shape[-1])
+            fused_bias = bias if (bias is not None and bias.dtype is torch.bfloat16) else None
+            y = ops.int8wo_linear(act, layout.int_data, layout.scale.reshape(-1).to(torch.bfloat16), fused_bias)
+            y = y.reshape(*orig_shape[:-1], weight_qtensor.shape[0])
+            if bias is not None and fused_bias is None:
+                y = y + bias
+            return y.to(orig_dtype)
+        # other activation dtypes (the product is formed in the activation's dtype there) and in_features that are
+        # not a multiple of 128: the reference's own op sequence
+        y = torch.mm(input_tensor.reshape(-1, orig_shape[-1]), layout.int_data.t().to(orig_dtype)) * layout.scale
+        y = y.reshape(*orig_shape[:-1], y.shape[-1])
+        if bias is not None:
+            y += bias
         return y.to(orig_dtype)
     raise NotImplementedError("No specialized dispatch found for quantized linear op")
 

@@ -103,8 +103,10 @@ def test_one_hot_rows_return_scaled_codes(oracle):
 
 
 def test_module_api_and_fallback():
-    """quantize_(model, int8_weight_only()) swaps nn.Linear weights; F.linear runs the HIP kernel when
-    in_features is a multiple of 128 and the dequantize path (reference :683-690) otherwise."""
+    """quantize_(model, int8_weight_only()) swaps nn.Linear weights; F.linear runs the HIP kernel for bf16
+    activations when in_features is a multiple of 128, and the reference's own op sequence (:655-665: the product
+    formed in the activation's dtype, times scale, plus bias, cast back) for other activation dtypes and ragged
+    in_features."""
     from ao_amd import int8_weight_only, quantize_
     from ao_amd.dtypes import AffineQuantizedTensor
 
@@ -123,6 +125,16 @@ def test_module_api_and_fallback():
         assert y.shape == (5, 96) and y.dtype is torch.bfloat16
         assert rel_l2(y.float().cpu().numpy(), y_ref.float().cpu().numpy()) <= 1e-2   # two bf16 rounding chains
         assert rel_l2(y.float().cpu().numpy(), y_fp.float().cpu().numpy()) <= 3e-2    # 8-bit quantization error
+        # fp16 / fp32 activations on the bf16 module (the reference multiplies in the activation's dtype and returns it)
+        for dt in (torch.float16, torch.float32):
+            xd = torch.randn(2, 3, K, device=dev, dtype=dt)
+            with torch.no_grad():
+                yd = lin(xd)
+                w_t = lin.weight.layout_tensor.int_data.t().to(dt)
+                want = (torch.mm(xd.reshape(-1, K), w_t) * lin.weight.layout_tensor.scale).reshape(2, 3, 96)
+                want += lin.bias
+            assert yd.shape == (2, 3, 96) and yd.dtype is dt
+            assert torch.equal(yd, want.to(dt))
 
 
 def test_rejects_bad_arguments(cabi):
