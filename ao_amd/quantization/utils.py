@@ -26,30 +26,42 @@ __all__ = [
 
 def compute_error(x, y):
     """Signal to quantization noise ratio in dB (reference :50-53)."""
-    Ps = torch.linalg.norm(x)
-    Pn = torch.linalg.norm(x - y)
-    return 20 * torch.log10(Ps / Pn)
+    signal, noise = torch.linalg.norm(x), torch.linalg.norm(x - y)
+    return 20 * torch.log10(signal / noise)
 
 
 def guard_dtype_size(tensor_arg, arg_name, dtype=None, size=None):
-    if dtype is not None and tensor_arg.dtype != dtype:
-        raise ValueError(f"Expected Tensor argument {arg_name} to have dtype {dtype}, but got {tensor_arg.dtype} instead.")
-    if size is not None and tensor_arg.size() != size:
-        raise ValueError(f"Expected Tensor argument {arg_name} to have size {size}, but got {tensor_arg.size()} instead.")
+    """ValueError unless the tensor has the given dtype / size (reference :125-129, same messages)."""
+    for what, want, got in (("dtype", dtype, tensor_arg.dtype), ("size", size, tensor_arg.size())):
+        if want is not None and got != want:
+            raise ValueError(f"Expected Tensor argument {arg_name} to have {what} {want}, but got {got} instead.")
+
+
+def _row_groups(t, groupsize, qparams=None):
+    """Block size (1, g) of a groupwise operation on the 2-d tensor `t`, with the reference's argument checks.
+    A group larger than the row means one group per row: always when choosing qparams (`qparams` None), and for the
+    GPTQ loop's single-column slices when the qparams passed in have one column."""
+    if groupsize > t.shape[-1] and (qparams is None or qparams.shape[-1] == 1):
+        groupsize = t.shape[-1]
+    assert groupsize > 1
+    assert t.shape[-1] % groupsize == 0
+    assert t.dim() == 2
+    return (1, groupsize)
+
+
+def _uint_range(n_bit):
+    return 0, 2**n_bit - 1
 
 
 def get_groupwise_affine_qparams(w, n_bit=4, groupsize=128, dtype=torch.bfloat16):
     """Per-group (scale, zero) of an asymmetric uint`n_bit` quantization, float zero point (reference :274-308)."""
-    if groupsize > w.shape[-1]:
-        groupsize = w.shape[-1]
-    assert groupsize > 1
-    assert w.shape[-1] % groupsize == 0
-    assert w.dim() == 2
+    block = _row_groups(w, groupsize)
     assert n_bit <= 8, f"only n_bit smaller than 8 is supported, got: {n_bit}"
     scale, zero_point = choose_qparams_affine(
-        w, MappingType.ASYMMETRIC, (1, groupsize), torch.int32, 0, 2**n_bit - 1, 1e-6, scale_dtype=dtype,
+        w, MappingType.ASYMMETRIC, block, torch.int32, *_uint_range(n_bit), 1e-6, scale_dtype=dtype,
         zero_point_dtype=dtype, preserve_zero=False, zero_point_domain=ZeroPointDomain.FLOAT)
-    return scale.to(dtype=dtype).reshape(w.shape[0], -1), zero_point.to(dtype=dtype).reshape(w.shape[0], -1)
+    rows = w.shape[0]
+    return scale.to(dtype=dtype).reshape(rows, -1), zero_point.to(dtype=dtype).reshape(rows, -1)
 
 
 def pack_tinygemm_scales_and_zeros(scales, zeros):
@@ -60,39 +72,31 @@ def pack_tinygemm_scales_and_zeros(scales, zeros):
 
 
 def unpack_tinygemm_scales_and_zeros(scales_and_zeros):
-    assert len(scales_and_zeros.shape) == 3 and scales_and_zeros.shape[2] == 2
+    assert scales_and_zeros.dim() == 3 and scales_and_zeros.shape[2] == 2
     return torch.split(scales_and_zeros.transpose(0, 1), 1, 2)
 
 
 def groupwise_affine_quantize_tensor_from_qparams(w, scales, zeros, n_bit=4, groupsize=128):
     assert groupsize > 1
-    if groupsize > w.shape[-1] and scales.shape[-1] == 1:  # GPTQ single-column case
-        groupsize = w.shape[-1]
-    assert w.shape[-1] % groupsize == 0
-    assert w.dim() == 2
-    return quantize_affine(w, (1, groupsize), scales, zeros, torch.int32, 0, 2**n_bit - 1,
+    return quantize_affine(w, _row_groups(w, groupsize, scales), scales, zeros, torch.int32, *_uint_range(n_bit),
                            zero_point_domain=ZeroPointDomain.FLOAT)
 
 
 def groupwise_affine_dequantize_tensor_from_qparams(w_int4x8, scales, zeros, n_bit=4, groupsize=128):
     assert groupsize > 1
-    if groupsize > w_int4x8.shape[-1] and scales.shape[-1] == 1:
-        groupsize = w_int4x8.shape[-1]
-    assert w_int4x8.shape[-1] % groupsize == 0
-    assert w_int4x8.dim() == 2
-    return dequantize_affine(w_int4x8, (1, groupsize), scales, zeros, torch.int32, 0, 2**n_bit - 1,
-                             zero_point_domain=ZeroPointDomain.FLOAT, output_dtype=scales.dtype)
+    return dequantize_affine(w_int4x8, _row_groups(w_int4x8, groupsize, scales), scales, zeros, torch.int32,
+                             *_uint_range(n_bit), zero_point_domain=ZeroPointDomain.FLOAT, output_dtype=scales.dtype)
 
 
 def groupwise_affine_quantize_tensor(w, n_bit=4, groupsize=128, dtype=torch.bfloat16):
-    scales, zeros = get_groupwise_affine_qparams(w, n_bit, groupsize, dtype)
-    w_int4x8 = groupwise_affine_quantize_tensor_from_qparams(w, scales, zeros, n_bit, groupsize)
-    return w_int4x8, pack_tinygemm_scales_and_zeros(scales, zeros)
+    qparams = get_groupwise_affine_qparams(w, n_bit, groupsize, dtype)
+    codes = groupwise_affine_quantize_tensor_from_qparams(w, *qparams, n_bit, groupsize)
+    return codes, pack_tinygemm_scales_and_zeros(*qparams)
 
 
 def groupwise_affine_dequantize_tensor(w_int4x8, scales_and_zeros, n_bit=4, groupsize=128):
-    scales, zeros = unpack_tinygemm_scales_and_zeros(scales_and_zeros)
-    return groupwise_affine_dequantize_tensor_from_qparams(w_int4x8, scales, zeros, n_bit, groupsize)
+    return groupwise_affine_dequantize_tensor_from_qparams(
+        w_int4x8, *unpack_tinygemm_scales_and_zeros(scales_and_zeros), n_bit, groupsize)
 
 
 def recommended_inductor_config_setter():
