@@ -41,9 +41,12 @@ def _row_groups(t, groupsize, qparams=None):
     """Block size (1, g) of a groupwise operation on the 2-d tensor `t`, with the reference's argument checks.
     A group larger than the row means one group per row: always when choosing qparams (`qparams` None), and for the
     GPTQ loop's single-column slices when the qparams passed in have one column."""
+    if qparams is not None:
+        assert groupsize > 1   # as asked for; the single-column slice below then is its own group of one
     if groupsize > t.shape[-1] and (qparams is None or qparams.shape[-1] == 1):
         groupsize = t.shape[-1]
-    assert groupsize > 1
+    if qparams is None:
+        assert groupsize > 1
     assert t.shape[-1] % groupsize == 0
     assert t.dim() == 2
     return (1, groupsize)
@@ -77,13 +80,11 @@ def unpack_tinygemm_scales_and_zeros(scales_and_zeros):
 
 
 def groupwise_affine_quantize_tensor_from_qparams(w, scales, zeros, n_bit=4, groupsize=128):
-    assert groupsize > 1
     return quantize_affine(w, _row_groups(w, groupsize, scales), scales, zeros, torch.int32, *_uint_range(n_bit),
                            zero_point_domain=ZeroPointDomain.FLOAT)
 
 
 def groupwise_affine_dequantize_tensor_from_qparams(w_int4x8, scales, zeros, n_bit=4, groupsize=128):
-    assert groupsize > 1
     return dequantize_affine(w_int4x8, _row_groups(w_int4x8, groupsize, scales), scales, zeros, torch.int32,
                              *_uint_range(n_bit), zero_point_domain=ZeroPointDomain.FLOAT, output_dtype=scales.dtype)
 
