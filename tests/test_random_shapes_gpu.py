@@ -146,3 +146,49 @@ def test_fused_quantize_pack_kernels_on_random_shapes_bit_exact(seed):
             data, s = ops.fp6_quantize_pack(w, eb, mb)
             data2, s2 = ops.fp6_quantize_pack(w.float(), eb, mb)
             assert torch.equal(data, data2) and torch.equal(s.view(torch.int16), s2.view(torch.int16)), (seed, i, N, K)
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_module_api_on_random_layers(seed):
+    """quantize_(nn.Linear, ...) on random layer shapes, activation dtypes and leading dimensions: the forward returns
+    the activation's dtype and shape and agrees with F.linear on the layer's own dequantized weight.  in_features that
+    are not a multiple of the group (int4: zero-extended to a whole group) or of 128 (int8: the reference's op
+    sequence instead of the HIP kernel) and layers the FPx recipe leaves in floating point are part of the draw."""
+    import torch.nn as nn
+    import torch.nn.functional as F
+
+    from ao_amd.dtypes import AffineQuantizedTensor
+    from ao_amd.prototype.quant_llm import QuantLlmLinearWeight
+    from ao_amd.quantization import fp6_llm_weight_only, int4_weight_only, int8_weight_only, quantize_
+
+    dev = torch.device("cuda:0")
+    rng = random.Random(200 + seed)
+    torch.manual_seed(200 + seed)
+    for i in range(60):
+        kind = rng.choice(["int4", "int4", "int8", "fpx"])
+        N = rng.choice([rng.randint(1, 300), 8 * rng.randint(1, 200), 256 * rng.randint(1, 16), rng.choice([4096, 1024, 11008])])
+        K = rng.choice([rng.randint(8, 600), 32 * rng.randint(1, 64), 128 * rng.randint(1, 40), rng.choice([4096, 1024])])
+        lead = rng.choice([(1,), (3,), (2, 5), (17,), (40,), (130,), (1, 1, 7)])
+        g = rng.choice([32, 64, 128, 256])
+        bias = rng.random() < 0.5
+        if kind == "fpx":
+            K = max(64, K // 64 * 64)
+            wdt = torch.float16
+            dt = rng.choice([torch.float16, torch.float16, torch.bfloat16, torch.float32])
+        else:
+            wdt = torch.bfloat16
+            dt = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        print(f"case random api {seed}/{i} {kind} N={N} K={K} lead={lead} dtype={dt} bias={bias} g={g}", flush=True)
+        lin = nn.Linear(K, N, bias=bias, device=dev, dtype=wdt)
+        quantize_(lin, int4_weight_only(group_size=g) if kind == "int4" else int8_weight_only() if kind == "int8" else fp6_llm_weight_only())
+        if not isinstance(lin.weight, (AffineQuantizedTensor, QuantLlmLinearWeight)):
+            assert kind == "fpx" and (N % 256 or K % 64), (kind, N, K)   # the recipe's own shape rule
+            continue
+        x = torch.randn(*lead, K, device=dev, dtype=dt)
+        with torch.no_grad():
+            y = lin(x)
+            ref = F.linear(x.float(), lin.weight.dequantize().float(), None if lin.bias is None else lin.bias.float())
+        assert y.shape == ref.shape and y.dtype is dt, (kind, N, K, lead, dt)
+        err = _rel_l2(y, ref)
+        # the 16-bit roundings of the chains (product, scale, bias; fp16 products for FPx) against an fp32 reference
+        assert bool(torch.isfinite(y.float()).all()) and err <= 8e-3, (seed, i, kind, N, K, lead, dt, err)
