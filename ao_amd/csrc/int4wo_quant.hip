@@ -170,6 +170,57 @@ __global__ __launch_bounds__(256) void choose_qparams_vec8_kernel(QParamArgs a, 
     if (active && part == 0) finish_qparams(a, mn, mx, has_nan, blk);
 }
 
+// The same for 16-bit inputs without converting a single element: a bf16 / fp16 pattern b orders like the integer
+// key b ^ (b & 0x8000 ? 0xffff : 0x8000) (negative values mirrored below the positive ones), so the minimum and the
+// maximum of a pair of elements are one packed 16-bit integer instruction each, five instructions per two elements
+// with the key (the fp32 form spends a conversion, a NaN test, a canonicalisation and two min / max per element and is
+// bound by them: 3.3 TB/s).  NaN patterns have keys above +inf's (or below -inf's) and are recognised on the two
+// results; min(-0, +0) is -0 here, which no later step of the recipe distinguishes from +0 (it enters sums only).
+typedef unsigned short u16x2v_t __attribute__((ext_vector_type(2)));
+typedef short i16x2v_t __attribute__((ext_vector_type(2)));
+
+template <int CH>
+__global__ __launch_bounds__(256) void choose_qparams_vec8_b16_kernel(QParamArgs a, uint32_t units, uint32_t tpg, uint32_t GK) {
+    const uint32_t ui = blockIdx.x * 256u + threadIdx.x;
+    const bool active = ui < units;
+    const uint32_t uu = active ? ui : units - 1;
+    const uint32_t blk = uu / tpg, part = uu % tpg;
+    const uint32_t r = blk / GK, gk = blk % GK;
+    const int64_t off = (int64_t)r * a.ld + (int64_t)gk * a.bK + part * (8 * CH);
+    uint4 v[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) v[c] = *reinterpret_cast<const uint4*>((const uint16_t*)a.in + off + 8 * c);
+    u16x2v_t mn2 = {0xffffu, 0xffffu}, mx2 = {0u, 0u};
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            union { uint32_t u; i16x2v_t s; u16x2v_t k; } p, m;
+            p.u = w[j];
+            m.s = p.s >> 15;                       // 0xffff in the halves that hold negative values
+            p.u ^= m.u | 0x80008000u;
+            mn2 = __builtin_elementwise_min(mn2, p.k);
+            mx2 = __builtin_elementwise_max(mx2, p.k);
+        }
+    }
+    uint32_t mnk = mn2[0] < mn2[1] ? mn2[0] : mn2[1], mxk = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+    for (uint32_t o = tpg >> 1; o >= 1; o >>= 1) {
+        const uint32_t omn = (uint32_t)__shfl_xor((int)mnk, (int)o, 64), omx = (uint32_t)__shfl_xor((int)mxk, (int)o, 64);
+        mnk = omn < mnk ? omn : mnk;
+        mxk = omx > mxk ? omx : mxk;
+    }
+    if (active && part == 0) {
+        const uint32_t inf = a.in_dtype == AO_BF16 ? 0x7f80u : 0x7c00u;
+        const int has_nan = mxk > (inf | 0x8000u) || mnk < (0x7fffu ^ inf);
+        const uint16_t mnb = (uint16_t)(mnk ^ ((mnk & 0x8000u) ? 0x8000u : 0xffffu));
+        const uint16_t mxb = (uint16_t)(mxk ^ ((mxk & 0x8000u) ? 0x8000u : 0xffffu));
+        const float mn = a.in_dtype == AO_BF16 ? bf16_bits_to_f32(mnb) : f16_bits_to_f32(mnb);
+        const float mx = a.in_dtype == AO_BF16 ? bf16_bits_to_f32(mxb) : f16_bits_to_f32(mxb);
+        finish_qparams(a, mn, mx, has_nan, blk);
+    }
+}
+
 // ---------------------------------------------------------------- quantize_affine / dequantize_affine (elementwise)
 struct QuantArgs {
     const void* in;
@@ -714,7 +765,13 @@ extern "C" int ao_amd_choose_qparams_affine(const void* in, int in_dtype, int64_
                       (uintptr_t)in % 16 == 0 && N * (K / 8) < (int64_t)0xffffff00u;
     if (vec8) {
         const uint32_t units = (uint32_t)(N * (K / (8 * ch)));
-        if (ch == 4) {
+        if (in_dtype != AO_F32 && ch == 4) {
+            hipLaunchKernelGGL(choose_qparams_vec8_b16_kernel<4>, dim3((units + 255u) / 256u), dim3(256), 0, st, a, units,
+                               (uint32_t)tpg, (uint32_t)(K / bK));
+        } else if (in_dtype != AO_F32) {
+            hipLaunchKernelGGL(choose_qparams_vec8_b16_kernel<1>, dim3((units + 255u) / 256u), dim3(256), 0, st, a, units,
+                               (uint32_t)tpg, (uint32_t)(K / bK));
+        } else if (ch == 4) {
             hipLaunchKernelGGL(choose_qparams_vec8_kernel<4>, dim3((units + 255u) / 256u), dim3(256), 0, st, a, units,
                                (uint32_t)tpg, (uint32_t)(K / bK));
         } else {
