@@ -32,7 +32,7 @@ def _weight(N, K, dtype, seed, zero_row=True):
 _SHAPES = [
     (64, 256, (1, 64)), (16, 4096, (1, 128)), (33, 512, (1, 512)), (8, 64, (1, 8)), (40, 200, (1, 8)),
     (24, 192, (1, 192)), (17, 64, (1, 64)), (32, 96, (1, 4)), (32, 128, (32, 128)), (16, 64, (4, 16)), (7, 9, (1, 9)),
-    (12, 1024, (1, 1024)),
+    (12, 1024, (1, 1024)), (5, 136, (1, 8)), (3, 1032, (1, 24)),
 ]
 
 
