@@ -221,6 +221,56 @@ __global__ __launch_bounds__(256) void choose_qparams_vec8_b16_kernel(QParamArgs
     }
 }
 
+// Long row blocks of a 16-bit dtype (per-channel quantization: the block is the whole row): one wave per block, lane l
+// takes the 16-byte chunks l, l + 64, ... so that every load instruction of the wave covers a contiguous kilobyte, four
+// loads in flight per lane; keys, reduction and finish as in choose_qparams_vec8_b16_kernel.
+__global__ __launch_bounds__(256) void choose_qparams_row_b16_kernel(QParamArgs a, uint32_t nblocks, uint32_t nch, uint32_t GK) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t bi = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const bool active = bi < nblocks;
+    const uint32_t blk = active ? bi : nblocks - 1;
+    const uint32_t r = blk / GK, gk = blk % GK;
+    const uint4* src = reinterpret_cast<const uint4*>((const uint16_t*)a.in + ((int64_t)r * a.ld + (int64_t)gk * a.bK));
+    u16x2v_t mn2 = {0xffffu, 0xffffu}, mx2 = {0u, 0u};
+    for (uint32_t i0 = lane; i0 < nch; i0 += 256u) {
+        uint4 v[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t i = i0 + 64u * c;
+            v[c] = src[i < nch ? i : i0];  // past the end: the lane's first chunk again, which changes no minimum or maximum
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                union { uint32_t u; i16x2v_t s; u16x2v_t k; } p, m;
+                p.u = w[j];
+                m.s = p.s >> 15;
+                p.u ^= m.u | 0x80008000u;
+                mn2 = __builtin_elementwise_min(mn2, p.k);
+                mx2 = __builtin_elementwise_max(mx2, p.k);
+            }
+        }
+    }
+    uint32_t mnk = mn2[0] < mn2[1] ? mn2[0] : mn2[1], mxk = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const uint32_t omn = (uint32_t)__shfl_xor((int)mnk, o, 64), omx = (uint32_t)__shfl_xor((int)mxk, o, 64);
+        mnk = omn < mnk ? omn : mnk;
+        mxk = omx > mxk ? omx : mxk;
+    }
+    if (active && lane == 0) {
+        const uint32_t inf = a.in_dtype == AO_BF16 ? 0x7f80u : 0x7c00u;
+        const int has_nan = mxk > (inf | 0x8000u) || mnk < (0x7fffu ^ inf);
+        const uint16_t mnb = (uint16_t)(mnk ^ ((mnk & 0x8000u) ? 0x8000u : 0xffffu));
+        const uint16_t mxb = (uint16_t)(mxk ^ ((mxk & 0x8000u) ? 0x8000u : 0xffffu));
+        const float mn = a.in_dtype == AO_BF16 ? bf16_bits_to_f32(mnb) : f16_bits_to_f32(mnb);
+        const float mx = a.in_dtype == AO_BF16 ? bf16_bits_to_f32(mxb) : f16_bits_to_f32(mxb);
+        finish_qparams(a, mn, mx, has_nan, blk);
+    }
+}
+
 // ---------------------------------------------------------------- quantize_affine / dequantize_affine (elementwise)
 struct QuantArgs {
     const void* in;
@@ -292,7 +342,17 @@ __global__ __launch_bounds__(256) void quantize_affine_kernel(QuantArgs a) {
 // arithmetic and the scale / zero point loads happen once per eight elements, the input arrives as one 16-byte
 // (fp32: two) load and the codes leave as 16-byte (int8: 8-byte) stores.
 
-__global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a, uint32_t chunks, uint32_t K8) {
+// I8_RECIPE: the arguments of the int8 weight-only call (bf16 input and scale, int64 or no zero point in the integer
+// domain, int8 codes, a clamp range within +-2^24) as constants, which folds the per-element dtype switches away.
+template <bool I8_RECIPE>
+__global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a0, uint32_t chunks, uint32_t K8) {
+    QuantArgs a = a0;
+    if (I8_RECIPE) {
+        a.in_dtype = a.scale_dtype = AO_BF16;
+        a.zp_dtype = AO_I64;
+        a.zp_domain = AO_ZP_INT;
+        a.out_dtype = AO_I8;
+    }
     const uint32_t ci = blockIdx.x * 256u + threadIdx.x;
     if (ci >= chunks) return;
     const uint32_t r = ci / K8, c = (ci % K8) * 8u;
@@ -302,7 +362,7 @@ __global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a, 
     const float s = load_f(a.scale, a.scale_dtype, g);
     const float z = a.zp ? load_f(a.zp, a.zp_dtype, g) : 0.f;
     int64_t q[8];
-    if (a.qmin >= -(1 << 24) && a.qmax <= (1 << 24)) {
+    if (I8_RECIPE || (a.qmin >= -(1 << 24) && a.qmax <= (1 << 24))) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) q[j] = quantize_elem<true>(a, x[j], s, z);
     } else {
@@ -851,6 +911,10 @@ extern "C" int ao_amd_choose_qparams_affine(const void* in, int in_dtype, int64_
             hipLaunchKernelGGL(choose_qparams_vec8_kernel<1>, dim3((units + 255u) / 256u), dim3(256), 0, st, a, units,
                                (uint32_t)tpg, (uint32_t)(K / bK));
         }
+    } else if (in_dtype != AO_F32 && bN == 1 && bK % 8 == 0 && bK >= 512 && ld % 8 == 0 && (uintptr_t)in % 16 == 0 &&
+               nblocks < (int64_t)0xfffffff0u) {
+        hipLaunchKernelGGL(choose_qparams_row_b16_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, a,
+                           (uint32_t)nblocks, (uint32_t)(bK / 8), (uint32_t)(K / bK));
     } else if (bN * bK <= 2048) {
         hipLaunchKernelGGL(choose_qparams_kernel<64>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, a);
     } else {
@@ -895,8 +959,14 @@ extern "C" int ao_amd_quantize_affine(const void* in, int in_dtype, int64_t N, i
                            (hipStream_t)stream, a, total, (uint32_t)K, (uint32_t)bK, (uint32_t)(K / bK));
     } else if (vec8) {
         const uint32_t chunks = (uint32_t)(N * (K / 8));
-        hipLaunchKernelGGL(quantize_affine_vec8_kernel, dim3((chunks + 255u) / 256u), dim3(256), 0, (hipStream_t)stream, a,
-                           chunks, (uint32_t)(K / 8));
+        const bool i8_recipe = in_dtype == AO_BF16 && scale_dtype == AO_BF16 && (!zero_point || zp_dtype == AO_I64) &&
+                               zp_domain == AO_ZP_INT && out_dtype == AO_I8 && qmin >= -(1 << 24) && qmax <= (1 << 24);
+        if (i8_recipe)
+            hipLaunchKernelGGL(quantize_affine_vec8_kernel<true>, dim3((chunks + 255u) / 256u), dim3(256), 0,
+                               (hipStream_t)stream, a, chunks, (uint32_t)(K / 8));
+        else
+            hipLaunchKernelGGL(quantize_affine_vec8_kernel<false>, dim3((chunks + 255u) / 256u), dim3(256), 0,
+                               (hipStream_t)stream, a, chunks, (uint32_t)(K / 8));
     } else {
         hipLaunchKernelGGL(quantize_affine_kernel, dim3(elementwise_grid(N * K)), dim3(256), 0, (hipStream_t)stream, a);
     }

@@ -544,6 +544,21 @@ def sweep(kind, iters=100):
                     L.ao_amd_fp6_quantize_pack(w[i % copies].data_ptr(), BF16, N, K, 3, 2, tc.data_ptr(), sc16.data_ptr(),
                                                st))),
             ]
+            if g == 64:
+                # the int8 weight-only call (quant_api.py:390-405): symmetric, one block per row, int8 codes, int64 zeros
+                I64, I8, SYM, ZP_INT = 4, 5, 0, 0
+                srow = torch.empty(N, dtype=torch.bfloat16, device=dev)
+                zrow = torch.zeros(N, dtype=torch.int64, device=dev)
+                codes8 = codes.view(torch.int8).view(copies, -1)[:, : N * K].view(copies, N, K)
+                steps += [
+                    ("choose_qparams_affine int8 per row", N * K * 2 + 10 * N, lambda i: _lib.check(
+                        L.ao_amd_choose_qparams_affine(w[i % copies].data_ptr(), BF16, N, K, K, 1, K, SYM, -128, 127,
+                                                       float(torch.finfo(torch.float32).eps), 1, ZP_INT, BF16, I64,
+                                                       srow.data_ptr(), zrow.data_ptr(), st))),
+                    ("quantize_affine int8 per row", N * K * 3 + 10 * N, lambda i: _lib.check(L.ao_amd_quantize_affine(
+                        w[i % copies].data_ptr(), BF16, N, K, K, 1, K, srow.data_ptr(), BF16, zrow.data_ptr(), I64, -128,
+                        127, ZP_INT, codes8[i % copies].data_ptr(), I8, st))),
+                ]
             for name, nbytes, launch in steps:
                 us = _time_linear(L, launch, iters, armed=False)
                 print(json.dumps({"kernel": name, "N": N, "K": K, "group": g, "us": round(us, 2),

@@ -28,11 +28,13 @@ def _weight(N, K, dtype, seed, zero_row=True):
     return w
 
 
-# (N, K, block): 8-per-thread paths for both kernels, groups of 8..512, rows of any length, 2-D and per-tensor blocks
+# (N, K, block): 8-per-thread paths for both kernels, groups of 8..512, rows of any length, 2-D and per-tensor blocks,
+# long row blocks (one wave per block: whole and partial rounds of 64 and 256 chunks, several blocks per row)
 _SHAPES = [
     (64, 256, (1, 64)), (16, 4096, (1, 128)), (33, 512, (1, 512)), (8, 64, (1, 8)), (40, 200, (1, 8)),
     (24, 192, (1, 192)), (17, 64, (1, 64)), (32, 96, (1, 4)), (32, 128, (32, 128)), (16, 64, (4, 16)), (7, 9, (1, 9)),
     (12, 1024, (1, 1024)), (5, 136, (1, 8)), (3, 1032, (1, 24)),
+    (6, 4096, (1, 4096)), (5, 2560, (1, 2560)), (4, 1544, (1, 1544)), (2, 12288, (1, 3072)), (9, 14336, (1, 14336)),
 ]
 
 
