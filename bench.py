@@ -551,11 +551,11 @@ def sweep(kind, iters=100):
                 zrow = torch.zeros(N, dtype=torch.int64, device=dev)
                 codes8 = codes.view(torch.int8).view(copies, -1)[:, : N * K].view(copies, N, K)
                 steps += [
-                    ("choose_qparams_affine int8 per row", N * K * 2 + 10 * N, lambda i: _lib.check(
+                    ("choose_qparams_i8_row", N * K * 2 + 10 * N, lambda i: _lib.check(
                         L.ao_amd_choose_qparams_affine(w[i % copies].data_ptr(), BF16, N, K, K, 1, K, SYM, -128, 127,
                                                        float(torch.finfo(torch.float32).eps), 1, ZP_INT, BF16, I64,
                                                        srow.data_ptr(), zrow.data_ptr(), st))),
-                    ("quantize_affine int8 per row", N * K * 3 + 10 * N, lambda i: _lib.check(L.ao_amd_quantize_affine(
+                    ("quantize_affine_i8_row", N * K * 3 + 10 * N, lambda i: _lib.check(L.ao_amd_quantize_affine(
                         w[i % copies].data_ptr(), BF16, N, K, K, 1, K, srow.data_ptr(), BF16, zrow.data_ptr(), I64, -128,
                         127, ZP_INT, codes8[i % copies].data_ptr(), I8, st))),
                 ]
