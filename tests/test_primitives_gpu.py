@@ -120,3 +120,39 @@ def test_nan_and_offset_views(oracle):
     dq2 = dequantize_affine(q2, block, s2, None, torch.int8, -128, 127, ZeroPointDomain.INT, output_dtype=torch.bfloat16)
     dq2o = oracle.dequantize_affine(q2o, oracle.I8, block, s2o, 1, None, 0, -128, 127, zp_domain=0, out_dtype=1)
     assert np.array_equal(_to_np(dq2), dq2o)
+
+
+@pytest.mark.parametrize("N,K,bK", [(24, 256, 64), (7, 4096, 4096), (5, 2560, 2560), (9, 1024, 128), (6, 200, 8)])
+def test_row_stride_larger_than_k_through_the_c_abi(N, K, bK):
+    """ao_amd_choose_qparams_affine / ao_amd_quantize_affine on rows that lie `ld` > K elements apart (the columns of a
+    wider matrix) give the bits they give on a contiguous copy, for the int4 and the int8 weight-only argument sets."""
+    from ao_amd import _lib
+
+    print(f"case row stride N={N} K={K} bK={bK}", flush=True)
+    L = _lib.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    dev = torch.device("cuda:0")
+    BF16, I32, I64, I8 = 1, 3, 4, 5
+    ld = K + 24
+    wide = (torch.randn(N, ld, device=dev) * 0.05).bfloat16()
+    view = wide[:, 16:16 + K]
+    dense = view.contiguous()
+    assert view.data_ptr() % 16 == 0 and view.stride(0) == ld
+    eps32 = float(torch.finfo(torch.float32).eps)
+    for name, args in (("int4", (1, 0, 15, 1e-6, 0, 1, BF16, BF16)), ("int8", (0, -128, 127, eps32, 1, 0, BF16, I64))):
+        mapping, qmin, qmax, eps, preserve_zero, domain, sdt, zdt = args
+        zt = torch.bfloat16 if zdt == BF16 else torch.int64
+        ct, cdt = (torch.int32, I32) if name == "int4" else (torch.int8, I8)
+        got = []
+        for src, stride in ((view, ld), (dense, K)):
+            s = torch.empty(N, K // bK, dtype=torch.bfloat16, device=dev)
+            z = torch.empty(N, K // bK, dtype=zt, device=dev)
+            q = torch.empty(N, K, dtype=ct, device=dev)
+            _lib.check(L.ao_amd_choose_qparams_affine(src.data_ptr(), BF16, N, K, stride, 1, bK, mapping, qmin, qmax, eps,
+                                                      preserve_zero, domain, sdt, zdt, s.data_ptr(), z.data_ptr(), st))
+            _lib.check(L.ao_amd_quantize_affine(src.data_ptr(), BF16, N, K, stride, 1, bK, s.data_ptr(), sdt, z.data_ptr(),
+                                                zdt, qmin, qmax, domain, q.data_ptr(), cdt, st))
+            torch.cuda.synchronize()
+            got.append((s.view(torch.int16), z.view(torch.int16) if zdt == BF16 else z, q))
+        for a, b in zip(*got):
+            assert torch.equal(a, b), (name, N, K, bK)
