@@ -911,8 +911,8 @@ extern "C" int ao_amd_choose_qparams_affine(const void* in, int in_dtype, int64_
             hipLaunchKernelGGL(choose_qparams_vec8_kernel<1>, dim3((units + 255u) / 256u), dim3(256), 0, st, a, units,
                                (uint32_t)tpg, (uint32_t)(K / bK));
         }
-    } else if (in_dtype != AO_F32 && bN == 1 && bK % 8 == 0 && bK >= 512 && ld % 8 == 0 && (uintptr_t)in % 16 == 0 &&
-               nblocks < (int64_t)0xfffffff0u) {
+    } else if (in_dtype != AO_F32 && bN == 1 && bK % 8 == 0 && bK >= 512 && bK < ((int64_t)1 << 34) && ld % 8 == 0 &&
+               (uintptr_t)in % 16 == 0 && nblocks < (int64_t)0xfffffff0u) {
         hipLaunchKernelGGL(choose_qparams_row_b16_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, st, a,
                            (uint32_t)nblocks, (uint32_t)(bK / 8), (uint32_t)(K / bK));
     } else if (bN * bK <= 2048) {
