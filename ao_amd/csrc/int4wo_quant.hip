@@ -342,17 +342,7 @@ __global__ __launch_bounds__(256) void quantize_affine_kernel(QuantArgs a) {
 // arithmetic and the scale / zero point loads happen once per eight elements, the input arrives as one 16-byte
 // (fp32: two) load and the codes leave as 16-byte (int8: 8-byte) stores.
 
-// I8_RECIPE: the arguments of the int8 weight-only call (bf16 input and scale, int64 or no zero point in the integer
-// domain, int8 codes, a clamp range within +-2^24) as constants, which folds the per-element dtype switches away.
-template <bool I8_RECIPE>
-__global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a0, uint32_t chunks, uint32_t K8) {
-    QuantArgs a = a0;
-    if (I8_RECIPE) {
-        a.in_dtype = a.scale_dtype = AO_BF16;
-        a.zp_dtype = AO_I64;
-        a.zp_domain = AO_ZP_INT;
-        a.out_dtype = AO_I8;
-    }
+__global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a, uint32_t chunks, uint32_t K8) {
     const uint32_t ci = blockIdx.x * 256u + threadIdx.x;
     if (ci >= chunks) return;
     const uint32_t r = ci / K8, c = (ci % K8) * 8u;
@@ -362,7 +352,7 @@ __global__ __launch_bounds__(256) void quantize_affine_vec8_kernel(QuantArgs a0,
     const float s = load_f(a.scale, a.scale_dtype, g);
     const float z = a.zp ? load_f(a.zp, a.zp_dtype, g) : 0.f;
     int64_t q[8];
-    if (I8_RECIPE || (a.qmin >= -(1 << 24) && a.qmax <= (1 << 24))) {
+    if (a.qmin >= -(1 << 24) && a.qmax <= (1 << 24)) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) q[j] = quantize_elem<true>(a, x[j], s, z);
     } else {
@@ -424,6 +414,47 @@ __global__ __launch_bounds__(256) void quantize_affine_bf16_fzp_i32_kernel(Quant
 #pragma unroll
         for (int j = 0; j < 4; ++j) q[j] = (int)quantize_elem<true>(a, x[j], s[h], z[h]);
         *reinterpret_cast<int4*>((int32_t*)a.out + f) = make_int4(q[0], q[1], q[2], q[3]);
+    }
+}
+
+// The int8 weight-only call (bf16 input and scale, int64 or no zero point in the integer domain, int8 codes, clamp range
+// within +-2^24) laid out like the kernel above: a lane owns RUNS runs of eight elements 512 apart (16-byte loads and
+// 8-byte stores, contiguous over the wave), every run's load before the first store.
+template <int RUNS>
+__global__ __launch_bounds__(256) void quantize_affine_bf16_izp_i8_kernel(QuantArgs a0, uint32_t chunks, uint32_t K8,
+                                                                          uint32_t bK, uint32_t GK) {
+    QuantArgs a = a0;
+    a.in_dtype = a.scale_dtype = AO_BF16;
+    a.zp_dtype = AO_I64;
+    a.zp_domain = AO_ZP_INT;
+    const uint32_t ci = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t base = (ci >> 6) * (64u * RUNS) + (ci & 63u);
+    uint4 v[RUNS];
+    float s[RUNS], z[RUNS];
+#pragma unroll
+    for (int h = 0; h < RUNS; ++h) {
+        const uint32_t c = base + 64u * h;
+        if (c >= chunks) continue;
+        const uint32_t r = c / K8, col = (c - r * K8) * 8u;
+        const uint32_t g = (a.bN == 1 ? r : r / (uint32_t)a.bN) * GK + col / bK;
+        v[h] = *reinterpret_cast<const uint4*>((const uint16_t*)a.in + ((int64_t)r * a.ld + col));
+        s[h] = bf16_bits_to_f32(((const uint16_t*)a.scale)[g]);
+        z[h] = a.zp ? load_f(a.zp, AO_I64, g) : 0.f;
+    }
+#pragma unroll
+    for (int h = 0; h < RUNS; ++h) {
+        const uint32_t c = base + 64u * h;
+        if (c >= chunks) continue;
+        const uint32_t w[4] = {v[h].x, v[h].y, v[h].z, v[h].w};
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t q0 = (uint32_t)quantize_elem<true>(a, bf16_bits_to_f32((uint16_t)(w[j] & 0xffffu)), s[h], z[h]) & 0xffu;
+            const uint32_t q1 = (uint32_t)quantize_elem<true>(a, bf16_bits_to_f32((uint16_t)(w[j] >> 16)), s[h], z[h]) & 0xffu;
+            if (j < 2) lo |= (q0 | (q1 << 8)) << (16 * j);
+            else hi |= (q0 | (q1 << 8)) << (16 * (j - 2));
+        }
+        *reinterpret_cast<uint2*>((uint8_t*)a.out + (int64_t)c * 8) = make_uint2(lo, hi);
     }
 }
 
@@ -542,6 +573,49 @@ __global__ __launch_bounds__(256) void dequantize_affine_i32_fzp_bf16_kernel(Qua
 #pragma unroll
         for (int j = 0; j < 4; ++j) b[j] = f32_to_bf16_bits(dequantize_elem<int32_t>(a, qs[j], s[h], 0, z[h])) & 0xffffu;
         *reinterpret_cast<uint2*>((uint16_t*)a.out + f) = make_uint2(b[0] | (b[1] << 16), b[2] | (b[3] << 16));
+    }
+}
+
+// dequantize_affine for the int8 weight-only call (int8 codes, bf16 scale and output, int64 or no zero point in the
+// integer domain), laid out as quantize_affine_bf16_izp_i8_kernel: 8-byte loads, 16-byte stores.
+template <int RUNS>
+__global__ __launch_bounds__(256) void dequantize_affine_i8_izp_bf16_kernel(QuantArgs a0, uint32_t chunks, uint32_t K8,
+                                                                            uint32_t bK, uint32_t GK) {
+    QuantArgs a = a0;
+    a.in_dtype = AO_I8;
+    a.scale_dtype = a.out_dtype = AO_BF16;
+    a.zp_dtype = AO_I64;
+    a.zp_domain = AO_ZP_INT;
+    const uint32_t ci = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t base = (ci >> 6) * (64u * RUNS) + (ci & 63u);
+    uint2 v[RUNS];
+    float s[RUNS];
+    int64_t zi[RUNS];
+#pragma unroll
+    for (int h = 0; h < RUNS; ++h) {
+        const uint32_t c = base + 64u * h;
+        if (c >= chunks) continue;
+        const uint32_t r = c / K8, col = (c - r * K8) * 8u;
+        const uint32_t g = (a.bN == 1 ? r : r / (uint32_t)a.bN) * GK + col / bK;
+        v[h] = *reinterpret_cast<const uint2*>((const uint8_t*)a.in + (int64_t)c * 8);
+        s[h] = bf16_bits_to_f32(((const uint16_t*)a.scale)[g]);
+        zi[h] = a.zp ? ((const int64_t*)a.zp)[g] : 0;
+    }
+#pragma unroll
+    for (int h = 0; h < RUNS; ++h) {
+        const uint32_t c = base + 64u * h;
+        if (c >= chunks) continue;
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t word = j < 2 ? v[h].x : v[h].y;
+            const int32_t q0 = (int32_t)(int8_t)((word >> (16 * (j & 1))) & 0xffu);
+            const int32_t q1 = (int32_t)(int8_t)((word >> (16 * (j & 1) + 8)) & 0xffu);
+            const uint32_t b0 = f32_to_bf16_bits(dequantize_elem<int32_t>(a, q0, s[h], zi[h], 0.f));
+            const uint32_t b1 = f32_to_bf16_bits(dequantize_elem<int32_t>(a, q1, s[h], zi[h], 0.f));
+            o[j] = (b0 & 0xffffu) | (b1 << 16);
+        }
+        *reinterpret_cast<uint4*>((uint16_t*)a.out + (int64_t)c * 8) = make_uint4(o[0], o[1], o[2], o[3]);
     }
 }
 
@@ -960,12 +1034,13 @@ extern "C" int ao_amd_quantize_affine(const void* in, int in_dtype, int64_t N, i
     } else if (vec8) {
         const uint32_t chunks = (uint32_t)(N * (K / 8));
         const bool i8_recipe = in_dtype == AO_BF16 && scale_dtype == AO_BF16 && (!zero_point || zp_dtype == AO_I64) &&
-                               zp_domain == AO_ZP_INT && out_dtype == AO_I8 && qmin >= -(1 << 24) && qmax <= (1 << 24);
+                               zp_domain == AO_ZP_INT && out_dtype == AO_I8 && qmin >= -(1 << 24) && qmax <= (1 << 24) &&
+                               chunks < 0xfffff000u;
         if (i8_recipe)
-            hipLaunchKernelGGL(quantize_affine_vec8_kernel<true>, dim3((chunks + 255u) / 256u), dim3(256), 0,
-                               (hipStream_t)stream, a, chunks, (uint32_t)(K / 8));
+            hipLaunchKernelGGL(quantize_affine_bf16_izp_i8_kernel<2>, dim3(((chunks + 1u) / 2u + 255u) / 256u), dim3(256), 0,
+                               (hipStream_t)stream, a, chunks, (uint32_t)(K / 8), (uint32_t)bK, (uint32_t)(K / bK));
         else
-            hipLaunchKernelGGL(quantize_affine_vec8_kernel<false>, dim3((chunks + 255u) / 256u), dim3(256), 0,
+            hipLaunchKernelGGL(quantize_affine_vec8_kernel, dim3((chunks + 255u) / 256u), dim3(256), 0,
                                (hipStream_t)stream, a, chunks, (uint32_t)(K / 8));
     } else {
         hipLaunchKernelGGL(quantize_affine_kernel, dim3(elementwise_grid(N * K)), dim3(256), 0, (hipStream_t)stream, a);
@@ -992,8 +1067,13 @@ extern "C" int ao_amd_dequantize_affine(const void* in, int in_dtype, int64_t N,
                            (hipStream_t)stream, a, total, (uint32_t)K, (uint32_t)bK, (uint32_t)(K / bK));
     } else if (vec8) {
         const uint32_t chunks = (uint32_t)(N * (K / 8));
-        hipLaunchKernelGGL(dequantize_affine_vec8_kernel, dim3((chunks + 255u) / 256u), dim3(256), 0, (hipStream_t)stream,
-                           a, chunks, (uint32_t)(K / 8));
+        if (in_dtype == AO_I8 && scale_dtype == AO_BF16 && (!zero_point || zp_dtype == AO_I64) && zp_domain == AO_ZP_INT &&
+            out_dtype == AO_BF16 && chunks < 0xfffff000u)
+            hipLaunchKernelGGL(dequantize_affine_i8_izp_bf16_kernel<2>, dim3(((chunks + 1u) / 2u + 255u) / 256u), dim3(256), 0,
+                               (hipStream_t)stream, a, chunks, (uint32_t)(K / 8), (uint32_t)bK, (uint32_t)(K / bK));
+        else
+            hipLaunchKernelGGL(dequantize_affine_vec8_kernel, dim3((chunks + 255u) / 256u), dim3(256), 0,
+                               (hipStream_t)stream, a, chunks, (uint32_t)(K / 8));
     } else {
         hipLaunchKernelGGL(dequantize_affine_kernel, dim3(elementwise_grid(N * K)), dim3(256), 0, (hipStream_t)stream, a);
     }
