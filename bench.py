@@ -558,7 +558,7 @@ def sweep(kind, iters=100):
                     ("quantize_affine_i8_row", N * K * 3 + 10 * N, lambda i: _lib.check(L.ao_amd_quantize_affine(
                         w[i % copies].data_ptr(), BF16, N, K, K, 1, K, srow.data_ptr(), BF16, zrow.data_ptr(), I64, -128,
                         127, ZP_INT, codes8[i % copies].data_ptr(), I8, st))),
-                    ("dequantize_affine_i8_row", N * K * 3 + 10 * N, lambda i: _lib.check(L.ao_amd_dequantize_affine(
+                    ("dequant_affine_i8_row", N * K * 3 + 10 * N, lambda i: _lib.check(L.ao_amd_dequantize_affine(
                         codes8[i % copies].data_ptr(), I8, N, K, 1, K, srow.data_ptr(), BF16, zrow.data_ptr(), I64, -128,
                         127, ZP_INT, deq.data_ptr(), BF16, st))),
                 ]
