@@ -101,6 +101,26 @@ def build_torch_binding(verbose: bool = False) -> str:
     return TORCH_BINDING_PATH
 
 
+CEILINGS_PATH = os.path.join(LIB_DIR, "ao_amd_ceilings")
+
+
+def build_ubench(verbose: bool = False) -> str:
+    """Compiles csrc/ubench/ceilings.hip, the standalone program that measures the fixed costs the kernels are bounded
+    by (empty kernel, load-only stream, the GEMV's tile loop on cached weights, LDS reads, grid barriers).  Nothing in
+    the package loads it."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    os.makedirs(LIB_DIR, exist_ok=True)
+    tmp = CEILINGS_PATH + ".tmp"
+    cmd = [hipcc, *[f for f in HIPCC_FLAGS if f != "-fPIC"], "-I", os.path.join(_HERE, "..", "include"), "-o", tmp,
+           os.path.join(CSRC, "ubench", "ceilings.hip")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    os.replace(tmp, CEILINGS_PATH)
+    return CEILINGS_PATH
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
     print(build_torch_binding(verbose=True))
+    print(build_ubench(verbose=True))

@@ -37,8 +37,21 @@ requested whole before its first tile is touched.  A tile's body waits for the N
 the exact count of younger requests; once the run's last tile has been requested the loop stops requesting (a
 repeated request would be served by memory again).  The (scale, zero) words come from LDS too, 128 bytes per tile in the order
 [k half][row], staged by the caller.
+
+`python gen_int4wo_gemv1.py --v2 > int4wo_gemv2_loop.inc` prints the variant for int4wo_gemv2_kernel (one 16-wave
+workgroup per CU): a wave's run is a contiguous piece of the workgroup's tile stream and may cross unit boundaries
+(a unit = the K range of one row block, or one of its equal parts when K is split).  Differences:
+  * the activation row sits ONCE in the workgroup's LDS, 256 bytes per K tile; the loop keeps the address of the current
+    and of the next tile (xa, xn) and wraps the tile index at the end of a row block (scalars ktn, kbx);
+  * at a unit boundary, and after the last tile, the accumulator is reduced over the four lanes of a row exactly as the
+    kernel's epilogue does (own element, times 1 / f, two quad-permute adds) and stored to the wave's next 256-byte
+    slot of partial sums in LDS (every lane stores; the four lanes of a row hold the same sum); the block has no
+    register output.  The flush of a finished unit runs in step 3 of the next tile, after that unit's last product.
 """
 import sys
+
+V2 = "--v2" in sys.argv
+PFX = "GEMV2" if V2 else "GEMV1"
 
 D = 4            # ring depth: up to D - 1 tiles requested ahead of the one being consumed
 VBASE_TOP = 128  # registers are allocated downwards from v127
@@ -83,6 +96,10 @@ def build_regs():
     r.alloc("ee")
     r.alloc("xa")
     r.alloc("qx")
+    if V2:
+        r.alloc("xn")   # LDS address of the next tile's activations
+        r.alloc("rd")   # LDS address of the wave's next slot of partial sums
+        r.alloc("fl")
     total = r.next
     total += total % 2
     base = VBASE_TOP - total
@@ -94,10 +111,13 @@ def build_regs():
 
 REG, VBASE = build_regs()
 SREG = {n: SBASE + i for i, n in enumerate(
-    ["wp_lo", "wp_hi", "ldi", "ntm1", "rem", "c3c00", "cur", "t0"])}
+    ["wp_lo", "wp_hi", "ldi", "ntm1", "rem", "c3c00", "cur", "t0"] +
+    (["ktn", "kbx", "urem", "ut", "m1_lo", "m1_hi", "m2_lo", "m2_hi", "m3_lo", "m3_hi", "fflag"] if V2 else []))}
 
 
-SCALAR_INPUTS = ("wp_lo", "wp_hi", "ldi", "ntm1")
+# v2: ktn = K tile index of the run's first tile (on entry), kbx = K tiles per row block, urem = tiles of the first
+# unit that belong to this run or lie behind it (tiles until the first unit boundary), ut = tiles per unit
+SCALAR_INPUTS = ("wp_lo", "wp_hi", "ldi", "ntm1") + (("ktn", "kbx", "urem", "ut") if V2 else ())
 
 
 def v(name, off=0):
@@ -162,6 +182,56 @@ def wait_next_tile():
     return L
 
 
+QP_SWAP1 = "quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf"
+QP_SWAP2 = "quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf"
+
+
+def flush(final):
+    """v2: the accumulator's row sums -> the wave's next slot of partial sums.  Element l % 4 of the accumulator is the
+    lane's own dot product (times f); the sum over the four lanes of a row uses the same operations in the same order
+    as the kernel's own reduction, so a run that crosses no boundary gives the same bits either way."""
+    L = [
+        "v_cndmask_b32 %s, %s, %s, s[%d:%d]" % (v("fl"), v("acc", 0), v("acc", 1), SREG["m1_lo"], SREG["m1_hi"]),
+        "v_cndmask_b32 %s, %s, %s, s[%d:%d]" % (v("fl"), v("fl"), v("acc", 2), SREG["m2_lo"], SREG["m2_hi"]),
+        "v_cndmask_b32 %s, %s, %s, s[%d:%d]" % (v("fl"), v("fl"), v("acc", 3), SREG["m3_lo"], SREG["m3_hi"]),
+        "v_mul_f32 %s, %s, %%[finv]" % (v("fl"), v("fl")),
+        "s_nop 1",
+        "v_add_f32_dpp %s, %s, %s %s" % (v("fl"), v("fl"), v("fl"), QP_SWAP1),
+        "s_nop 1",
+        "v_add_f32_dpp %s, %s, %s %s" % (v("fl"), v("fl"), v("fl"), QP_SWAP2),
+        "ds_write_b32 %s, %s" % (v("rd"), v("fl")),
+    ]
+    if not final:
+        L.append("v_add_u32 %s, 256, %s" % (v("rd"), v("rd")))
+        for i in range(4):
+            L.append("v_mov_b32 %s, 0" % v("acc", i))
+    return L
+
+
+def next_x_address():
+    """v2, end of a tile: the next tile becomes the current one; K tile index of the one after it, wrapped at the end of
+    the row block"""
+    return [
+        "v_mov_b32 %s, %s" % (v("xa"), v("xn")),
+        "s_add_u32 %s, %s, 1" % (s("ktn"), s("ktn")),
+        "s_cmp_eq_u32 %s, %s" % (s("ktn"), s("kbx")),
+        "s_cselect_b32 %s, 0, %s" % (s("ktn"), s("ktn")),
+        "v_lshl_add_u32 %s, %s, 8, %%[xlane]" % (v("xn"), s("ktn")),
+    ]
+
+
+def unit_bookkeeping():
+    """v2, after a tile: one tile less in the current unit; at its end arm the flush that the next tile runs"""
+    return [
+        "s_sub_u32 %s, %s, 1" % (s("urem"), s("urem")),
+        "s_cmp_eq_u32 %s, 0" % s("urem"),
+        "s_cbranch_scc0 42f",
+        "s_mov_b32 %s, 1" % s("fflag"),
+        "s_mov_b32 %s, %s" % (s("urem"), s("ut")),
+        "42:",
+    ]
+
+
 def tile_body(pos, first):
     """the 8 steps of the tile in ring slot `pos`; `first`: the pipeline is empty (stages of earlier quads are idle)"""
     cur = "AB"[pos % 2]
@@ -173,10 +243,13 @@ def tile_body(pos, first):
     for u in range(8):
         if u == 3:
             L.append("s_waitcnt lgkmcnt(0)")
-            L.append("ds_read_b128 %s, %s offset:%d" % (vv("x", 4, 8), v("xa"), pos * 256 + 128))
-            L.append("ds_read_b128 %s, %s offset:%d" % (vv("x", 4, 12), v("xa"), pos * 256 + 192))
+            L.append("ds_read_b128 %s, %s offset:%d" % (vv("x", 4, 8), v("xa"), 128 if V2 else pos * 256 + 128))
+            L.append("ds_read_b128 %s, %s offset:%d" % (vv("x", 4, 12), v("xa"), 192 if V2 else pos * 256 + 192))
             # (scale, zero) of the tile after the next one (its register's previous content was last read a tile ago)
             L.append("ds_read_b32 %s, %s offset:%d" % (v("Q%d" % (pos % 2)), v("qx"), (pos + 2) * 128))
+            if V2 and not first:
+                # the previous tile closed a unit: its last product ran in step 2, park its sums before P(0)
+                L += ["s_cmp_eq_u32 %s, 0" % s("fflag"), "s_cbranch_scc1 41f"] + flush(False) + ["s_mov_b32 %s, 0" % s("fflag"), "41:"]
         if u == 7:
             L.append("s_waitcnt lgkmcnt(0)")
             L += wait_next_tile()   # X(8) below reads the next tile's first dword
@@ -219,8 +292,13 @@ def tile_body(pos, first):
         if u == 7:
             L.append(setup[8])
             # first half of the next tile's activations (its registers were last read by P(3) in step 6)
-            L.append("ds_read_b128 %s, %s offset:%d" % (vv("x", 4, 0), v("xa"), (pos + 1) * 256))
-            L.append("ds_read_b128 %s, %s offset:%d" % (vv("x", 4, 4), v("xa"), (pos + 1) * 256 + 64))
+            if V2:
+                L.append("ds_read_b128 %s, %s offset:0" % (vv("x", 4, 0), v("xn")))
+                L.append("ds_read_b128 %s, %s offset:64" % (vv("x", 4, 4), v("xn")))
+                L += next_x_address()
+            else:
+                L.append("ds_read_b128 %s, %s offset:%d" % (vv("x", 4, 0), v("xa"), (pos + 1) * 256))
+                L.append("ds_read_b128 %s, %s offset:%d" % (vv("x", 4, 4), v("xa"), (pos + 1) * 256 + 64))
     return L
 
 
@@ -254,7 +332,19 @@ def program():
     L.append("s_mov_b32 %s, 0x3c00" % s("c3c00"))
     L.append("s_add_u32 %s, %s, 1" % (s("rem"), s("ntm1")))
     L.append("s_mov_b32 %s, 0" % s("cur"))
-    L.append("v_mov_b32 %s, %%[xaddr]" % v("xa"))
+    if V2:
+        # lane masks of the lanes 1, 2, 3 of every 4-lane block, the flush flag, the first two activation addresses
+        for k, pat in (("m1", 0x22222222), ("m2", 0x44444444), ("m3", 0x88888888)):
+            L.append("s_mov_b32 %s, 0x%x" % (s(k + "_lo"), pat))
+            L.append("s_mov_b32 %s, 0x%x" % (s(k + "_hi"), pat))
+        L.append("s_mov_b32 %s, 0" % s("fflag"))
+        L.append("v_mov_b32 %s, %%[redaddr]" % v("rd"))
+        L.append("v_lshl_add_u32 %s, %s, 8, %%[xlane]" % (v("xa"), s("ktn")))
+        L += ["s_add_u32 %s, %s, 1" % (s("ktn"), s("ktn")), "s_cmp_eq_u32 %s, %s" % (s("ktn"), s("kbx")),
+              "s_cselect_b32 %s, 0, %s" % (s("ktn"), s("ktn")),
+              "v_lshl_add_u32 %s, %s, 8, %%[xlane]" % (v("xn"), s("ktn"))]
+    else:
+        L.append("v_mov_b32 %s, %%[xaddr]" % v("xa"))
     L.append("v_mov_b32 %s, %%[qaddr]" % v("qx"))
     L.append("v_mov_b32 %s, 0" % v("m16", 1))
     for sl in range(2):
@@ -274,14 +364,19 @@ def program():
     L.append("s_nop 7")
     # ---- first tile, then the ring
     L += tile_body(0, True)
+    if V2:
+        L += unit_bookkeeping()
     L += ["s_add_u32 %s, %s, 1" % (s("cur"), s("cur")), "s_sub_u32 %s, %s, 1" % (s("rem"), s("rem")), "s_cmp_eq_u32 %s, 0" % s("rem"), "s_cbranch_scc1 70f", "s_branch 11f"]
     L.append("10:")
     for pos in range(D):
         if pos == 1:
             L.append("11:")
         L += tile_body(pos, False)
+        if V2:
+            L += unit_bookkeeping()
         L += ["s_add_u32 %s, %s, 1" % (s("cur"), s("cur")), "s_sub_u32 %s, %s, 1" % (s("rem"), s("rem")), "s_cmp_eq_u32 %s, 0" % s("rem"), "s_cbranch_scc1 %df" % (70 + pos % 2)]
-    L.append("v_add_u32 %s, %d, %s" % (v("xa"), D * 256, v("xa")))
+    if not V2:
+        L.append("v_add_u32 %s, %d, %s" % (v("xa"), D * 256, v("xa")))
     L.append("v_add_u32 %s, %d, %s" % (v("qx"), D * 128, v("qx")))
     L.append("s_branch 10b")
     L.append("70:")
@@ -289,6 +384,8 @@ def program():
     L.append("71:")
     L += drain(1)
     L.append("9:")
+    if V2:
+        L += flush(True)
     L.append("s_waitcnt vmcnt(0) lgkmcnt(0)")  # repeated requests of the last tile and the next tile's activations
     return L
 
@@ -298,7 +395,7 @@ def clobbers():
     ring = set()
     for sl in range(D - 1):
         ring |= set(range(REG["W%d" % sl], REG["W%d" % sl] + 4))
-    acc = set(range(REG["acc"], REG["acc"] + 4))
+    acc = set() if V2 else set(range(REG["acc"], REG["acc"] + 4))
     for i in range(VBASE, VBASE_TOP):
         if i not in ring and i not in acc:
             regs.append('"v%d"' % i)
@@ -312,17 +409,17 @@ def clobbers():
 def main():
     out = []
     out.append("// Generated by gen_int4wo_gemv1.py -- do not edit; see that script for the schedule.")
-    out.append("#ifndef GEMV1_RING_DEPTH")
-    out.append("#define GEMV1_RING_DEPTH %d" % D)
-    out.append("#define GEMV1_VBASE %d" % VBASE)
-    out.append("#define GEMV1_S_WP \"{s[%d:%d]}\"" % (SREG["wp_lo"], SREG["wp_hi"]))
-    for n in ("ldi", "ntm1"):
-        out.append("#define GEMV1_S_%s \"{s%d}\"" % (n.upper(), SREG[n]))
+    out.append("#ifndef %s_RING_DEPTH" % PFX)
+    out.append("#define %s_RING_DEPTH %d" % (PFX, D))
+    out.append("#define %s_VBASE %d" % (PFX, VBASE))
+    out.append("#define %s_S_WP \"{s[%d:%d]}\"" % (PFX, SREG["wp_lo"], SREG["wp_hi"]))
+    for n in SCALAR_INPUTS[2:]:
+        out.append("#define %s_S_%s \"{s%d}\"" % (PFX, n.upper(), SREG[n]))
     for sl in range(D):
-        out.append("#define GEMV1_W%d \"{v[%d:%d]}\"" % (sl, REG["W%d" % sl], REG["W%d" % sl] + 3))
-    out.append("#define GEMV1_ACC \"{v[%d:%d]}\"" % (REG["acc"], REG["acc"] + 3))
-    out.append("#define GEMV1_CLOBBERS " + ", ".join(clobbers()))
-    out.append("#define GEMV1_LOOP_ASM \\")
+        out.append("#define %s_W%d \"{v[%d:%d]}\"" % (PFX, sl, REG["W%d" % sl], REG["W%d" % sl] + 3))
+    out.append("#define %s_ACC \"{v[%d:%d]}\"" % (PFX, REG["acc"], REG["acc"] + 3))
+    out.append("#define %s_CLOBBERS " % PFX + ", ".join(clobbers()))
+    out.append("#define %s_LOOP_ASM \\" % PFX)
     for l in program():
         out.append('    "%s\\n\\t" \\' % l)
     out.append('    ""')

@@ -142,6 +142,11 @@ bool launch_int4wo_gemv1(const LinearArgs& a, int64_t g, int64_t RB, hipStream_t
 bool int4wo_gemv1_plan(const LinearArgs& a, int64_t g, int64_t RB, char* out, size_t cap);
 
 
+// The same product with one 16-wave workgroup per CU and runs of tiles that cross row blocks (int4wo_gemv2.hip); it takes
+// the launches whose unit count spreads evenly over the CUs, int4wo_gemv1_kernel keeps the others.
+bool launch_int4wo_gemv2(const LinearArgs& a, int64_t g, int64_t RB, hipStream_t st);
+bool int4wo_gemv2_plan(const LinearArgs& a, int64_t g, int64_t RB, char* out, size_t cap);
+
 // Prefill GEMM with the weight tile dequantized once per workgroup into LDS (int4wo_gemm.hip); same contract as above.
 bool launch_int4wo_gemm_lds(const LinearArgs& a, int64_t g, hipStream_t st);
 bool int4wo_gemm_lds_plan(const LinearArgs& a, int64_t g, char* out, size_t cap);

@@ -1241,6 +1241,12 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // one activation row: the kernel built on the 4x4x4 matrix instructions (group size 64 and up, K up to 16384)
     if (M == 1 && aligned && !dual) {
         char name[96];
+        if (int4wo_gemv2_plan(a, g, RB, name, sizeof(name))) {
+            AO_PLAN("%s", name);
+            if (!launch_int4wo_gemv2(a, g, RB, st)) return -2;
+            AO_LAUNCH_CHECK();
+            return 0;
+        }
         if (int4wo_gemv1_plan(a, g, RB, name, sizeof(name))) {
             AO_PLAN("%s", name);
             launch_int4wo_gemv1(a, g, RB, st);

@@ -54,8 +54,8 @@ class Int4WeightOnlyQuantizedLinearWeight(torch.Tensor):
     # ------------------------------------------------------------------ construction
     @classmethod
     def to_qtensor_components(cls, input_float, groupsize=128, inner_k_tiles=8):
-        """(packed codes, scales_and_zeros, transposed, logical shape, groupsize, inner_k_tiles) of a float weight
-        [out_features, in_features]; in_features is zero-extended to a whole number of groups (the reference pads to
+        """(packed codes, scales_and_zeros, transposed, groupsize, inner_k_tiles) of a float weight
+        [out_features, in_features], the reference's 5-tuple (:583-601); in_features is zero-extended to a whole number of groups (the reference pads to
         1024: its kernel needs it, these do not)."""
         assert groupsize in (256, 128, 64, 32), f"groupsize {groupsize} not supported"
         assert inner_k_tiles in (8, 4, 2), f"inner_k_tiles {inner_k_tiles} not supported"
@@ -68,14 +68,16 @@ class Int4WeightOnlyQuantizedLinearWeight(torch.Tensor):
         codes, scales_and_zeros = groupwise_affine_quantize_tensor(w, 4, groupsize, dtype=torch.bfloat16)
         scales, zeros = unpack_tinygemm_scales_and_zeros(scales_and_zeros)
         packed, _ = torch.ops.torchao.int4wo_pack(codes, scales.reshape(N, -1).contiguous(), zeros.reshape(N, -1).contiguous(), groupsize)
-        return packed, scales_and_zeros, False, input_float.shape, groupsize, inner_k_tiles
+        return packed, scales_and_zeros, False, groupsize, inner_k_tiles
 
     @classmethod
     def from_float(cls, input_float, groupsize=128, inner_k_tiles=8, dtype=None):
         """Legacy conversion entry point (reference :551-571)."""
         if dtype is None:
             dtype = input_float.dtype
-        return cls(*cls.to_qtensor_components(input_float, groupsize, inner_k_tiles), dtype=dtype)
+        int_data, scales_and_zeros, transposed, groupsize, inner_k_tiles = cls.to_qtensor_components(
+            input_float, groupsize, inner_k_tiles)
+        return cls(int_data, scales_and_zeros, transposed, input_float.shape, groupsize, inner_k_tiles, dtype=dtype)
 
     # ------------------------------------------------------------------ accessors
     def _interleaved_qparams(self):

@@ -166,6 +166,15 @@ class Wave:
             self._gload(op, args)
         elif op.startswith("ds_read"):
             self._dsread(op, args)
+        elif op == "ds_write_b32":
+            addr = self._src(args[0]).astype(np.int64)
+            data = self._src(args[1])
+            for lane in range(NLANES):
+                ad = int(addr[lane])
+                if ad < 0 or ad + 4 > self.lds.size:
+                    raise HazardError("ds_write outside the LDS image: %d" % ad)
+                self.lds[ad: ad + 4] = np.frombuffer(np.uint32(data[lane]).tobytes(), dtype=np.uint8)
+            self.lgkm_pending.append(([], []))
         elif op.startswith("v_"):
             self._valu(op, args, rest)
         else:
@@ -254,6 +263,23 @@ class Wave:
             r = (self._src(a[1]) << (self._src(a[2]) & 31)) | self._src(a[3])
         elif op == "v_add_u32":
             r = self._src(a[1]) + self._src(a[2])
+        elif op == "v_lshl_add_u32":
+            r = (self._src(a[1]) << (self._src(a[2]) & 31)) + self._src(a[3])
+        elif op == "v_cndmask_b32":
+            sr = self._sregs(a[3])
+            m = int(self.s[sr[0]]) | (int(self.s[sr[1]]) << 32)
+            bits = np.array([(m >> i) & 1 for i in range(NLANES)], dtype=bool)
+            r = np.where(bits, self._src(a[2]), self._src(a[1]))
+        elif op == "v_mul_f32":
+            r = (self._src(a[1]).view(np.float32) * self._src(a[2]).view(np.float32)).astype(np.float32).view(np.uint32)
+        elif op == "v_add_f32_dpp":
+            last = a[2].split()
+            m = re.search(r"quad_perm:\[(\d),(\d),(\d),(\d)\]", rest)
+            perm = [int(m.group(i)) for i in range(1, 5)]
+            src0 = self._src(a[1], "dpp")
+            lanes = np.arange(NLANES)
+            sel = (lanes & ~3) + np.array(perm)[lanes & 3]
+            r = (src0[sel].view(np.float32) + self._src(last[0]).view(np.float32)).astype(np.float32).view(np.uint32)
         elif op == "v_perm_b32":
             s0, s1, sel = self._src(a[1]), self._src(a[2]), self._src(a[3])
             pool = (s0.astype(np.uint64) << 32) | s1.astype(np.uint64)

@@ -16,7 +16,8 @@ import pytest
 import torch
 
 SHAPES = [(48, 192), (64, 512), (256, 1024), (512, 2048), (1024, 4096), (4096, 4096), (3072, 8192), (14336, 4096),
-          (4096, 14336), (1024, 16384), (128256, 4096), (28672, 4096), (8192, 16384), (16384, 16384)]   # (N, K)
+          (4096, 14336), (1024, 16384), (128256, 4096), (28672, 4096), (8192, 16384), (16384, 16384), (4096, 16384),
+          (16384, 4096), (36864, 4096)]   # (N, K)
 MS = [1, 2, 4, 16, 17, 32, 33, 64, 65, 128, 256, 512, 1024]
 GROUPS = [32, 64, 128, 256]
 
@@ -45,7 +46,7 @@ def _walk():
 def test_dispatch_walk_finds_every_kernel_family():
     plans = _walk()
     families = {n.split("<")[0] for n in plans}
-    assert families == {"int4wo_gemv1_kernel", "int4wo_gemv_kernel", "int4wo_linear_kernel", "int4wo_gemm_kernel",
+    assert families == {"int4wo_gemv1_kernel", "int4wo_gemv2_kernel", "int4wo_gemv_kernel", "int4wo_linear_kernel", "int4wo_gemm_kernel",
                         "int4wo_gemm_ksplit_kernel", "int4wo_gemm_lds_kernel", "int4wo_gemm_kwave_kernel",
                         "int4wo_linear_rb4_kernel"}
     # the tile variants of the matrix-core kernels and both K-split forms
@@ -61,8 +62,17 @@ def test_dispatch_walk_finds_every_kernel_family():
     want = {"int4wo_gemv1_kernel<%d,2,%d>" % (w, nm) for w in (4, 8, 16) for nm in (0, 1)}
     want |= {"int4wo_gemv1_kernel<4,4,0>", "int4wo_gemv1_kernel<4,4,1>", "int4wo_gemv1_kernel<8,4,0>", "int4wo_gemv1_kernel<4,8,0>"}
     assert gemv1 == want, sorted(gemv1 ^ want)
-    # the prefill kernel takes a problem only when its 256-row tiles fill most of the chip
+    # the single-row kernel with one workgroup per CU: exactly the instantiations that int4wo_gemv2.hip compiles (activation
+    # chunks per thread, qparam chunks per lane); it takes fused-norm launches whose row blocks spread evenly over the CUs
+    gemv2 = {n.split(" ")[0] for n in plans if n.startswith("int4wo_gemv2_kernel<")}
+    assert gemv2 == {"int4wo_gemv2_kernel<%d,%d>" % (xc, ql) for xc in (1, 2) for ql in (1, 2, 4)}, sorted(gemv2)
     from ao_amd import _lib
+
+    assert _lib.int4wo_linear_plan(1, 4096, 28672, 64, norm=True) == "int4wo_gemv2_kernel<1,2> upw=7 run=14"
+    assert _lib.int4wo_linear_plan(1, 4096, 28672, 64).startswith("int4wo_gemv1_kernel")          # no norm
+    assert _lib.int4wo_linear_plan(1, 4096, 14336, 64, norm=True).startswith("int4wo_gemv1_kernel")   # 224 workgroups
+    assert _lib.int4wo_linear_plan(1, 4096, 128256, 64, norm=True).startswith("int4wo_gemv1_kernel")  # 32 units per workgroup
+    # the prefill kernel takes a problem only when its 256-row tiles fill most of the chip
 
     assert _lib.int4wo_linear_plan(2048, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel<64,2>")
     assert _lib.int4wo_linear_plan(512, 4096, 14336, 64).startswith("int4wo_gemm_lds_kernel<64,1>")

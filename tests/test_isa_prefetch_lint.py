@@ -296,7 +296,65 @@ def _asm_load_violations(body):
     return out
 
 
-@pytest.mark.parametrize("source", ["int4wo_gemm.hip", "int4wo_gemv1.hip"])
+def test_gemv2_loop_operands_and_ring(tmp_path):
+    """int4wo_gemv2_kernel: in every instantiation the three requests of the prologue land in the ring registers the
+    generated loop reads them from, every operand the compiler hands the loop lives below the loop's own register range
+    (the loop overwrites its registers while it still reads its operands) and is a register of its own, the loop text is
+    the generated one, and no scratch memory is used."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not available")
+    asm = tmp_path / "gemv2.s"
+    subprocess.run([hipcc, *_FLAGS, "-o", str(asm), os.path.join(_ROOT, "ao_amd", "csrc", "int4wo_gemv2.hip")], check=True,
+                   capture_output=True, timeout=600)
+    text = asm.read_text()
+    inc = open(os.path.join(_ROOT, "ao_amd", "csrc", "int4wo_gemv2_loop.inc")).read()
+    vbase = int(re.search(r"#define GEMV2_VBASE (\d+)", inc).group(1))
+    template = [t.replace("\\n", "").replace("\\t", "").strip()
+                for t in re.findall(r'"((?:[^"\\]|\\.)*)"', inc.split("#define GEMV2_LOOP_ASM", 1)[1])]
+    template = [t for t in template if t]
+    ring = set()
+    for j in range(3):
+        w = re.search(r'#define GEMV2_W%d "\{v\[(\d+):(\d+)\]\}"' % j, inc)
+        ring.update(range(int(w.group(1)), int(w.group(2)) + 1))
+    kernels = list(re.finditer(r"^(_ZN2ao19int4wo_gemv2_kernelILi\d+ELi\d+EEE\w*): ; @.*?\n(.*?)s_endpgm(.*?)\.end_amdhsa_kernel", text, re.S | re.M))
+    assert len(kernels) == 6
+    for m in kernels:
+        name, body, meta = m.group(1), m.group(2), m.group(3)
+        lines = [l.strip() for l in body.splitlines() if l.strip() and not l.strip().startswith(";") and
+                 (not l.strip().startswith(".") or l.strip().startswith(".LBB"))]
+        loop = next(i for i, l in enumerate(lines) if l == template[0])
+        requests = [l for l in lines[:loop] if re.match(r"global_load_dwordx4 v\[\d+:\d+\], v\d+, s\[.* nt", l)]
+        assert len(requests) == 3, (name, len(requests))
+        got = set()
+        for l in requests:
+            got |= _regs(l.split(",")[0])
+        assert got == ring, (name, sorted(got ^ ring))
+        actual = lines[loop:loop + len(template)]
+        operands = {}
+        for t, a in zip(template, actual):
+            if "%[" not in t:
+                assert t == a, (name, t, a)
+                continue
+            keys = re.findall(r"%\[(\w+)\]", t)
+            pat = re.sub(r"%\\\[\w+\\\]", lambda mm: r"(v\[\d+:\d+\]|v\d+)", re.escape(t))
+            mm = re.fullmatch(pat, a)
+            assert mm, (name, t, a)
+            for key, val in zip(keys, mm.groups()):
+                operands.setdefault(key, set()).add(val)
+        assert set(operands) == {"woff", "qaddr", "xlane", "redaddr", "finv", "mask", "sello", "selhi", "bc1", "bc2"}, (name, sorted(operands))
+        used = set()
+        for key, vals in operands.items():
+            assert len(vals) == 1, (name, key, vals)
+            regs = _regs(next(iter(vals)))
+            assert max(regs) < vbase, (name, key, vals)
+            assert not (regs & used), (name, key, vals)
+            used |= regs
+        scratch = re.search(r"\.amdhsa_private_segment_fixed_size (\d+)", meta)
+        assert scratch is None or int(scratch.group(1)) == 0, (name, scratch.group(0))
+
+
+@pytest.mark.parametrize("source", ["int4wo_gemm.hip", "int4wo_gemv1.hip", "int4wo_gemv2.hip"])
 def test_asm_loads_are_waited_for_on_every_path_before_their_registers_are_touched(tmp_path, source):
     """Every kernel that issues global loads from asm statements (the weight streams of the GEMV rings and of the
     prefill kernels): between such a load and the wait that covers it, on every path through loops and out of them,

@@ -63,7 +63,9 @@ def test_linear_entry_points_on_random_shapes(seed):
                 ref = ref.bfloat16().float() + r.float()
             else:
                 y = ops.int4wo_linear(x, packed, qparams, g, N, b, f32)
-            tol = 2e-5 if f32 else 4e-3   # fp32 output: summation order only; bf16 output: its rounding (2^-9)
+            if not f32:
+                ref = ref.bfloat16().float()   # the output's own rounding, as the kernel applies it to its fp32 sum
+            tol = 2e-5 if f32 else 1e-3   # summation order only; with a bf16 output an element at a rounding boundary may flip
         elif kind == "int8":
             N = rng.choice([rng.randint(1, 600), 16 * rng.randint(1, 400), rng.choice([4096, 6144, 14336, 1024])])
             K = rng.choice([128 * rng.randint(1, 32), 128 * rng.randint(1, 112), 4096, 14336])

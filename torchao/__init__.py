@@ -14,13 +14,21 @@ import ao_amd
 
 __version__ = ao_amd.__version__
 
-_SUBMODULES = [
-    "quantization", "quantization.quant_api", "quantization.quant_primitives", "quantization.GPTQ", "quantization.unified",
-    "quantization.utils", "dtypes", "dtypes.affine_quantized_tensor", "dtypes.utils", "ops", "utils", "prototype",
-    "prototype.quant_llm", "prototype.quant_llm.quant_llm", "prototype.hqq", "prototype.hqq.hqq_tinygemm_linear",
-    "prototype.hqq.mixed_mm", "_models", "_models.llama", "_models.llama.model", "_models.llama.generate",
-]
-for _name in _SUBMODULES:
+import pkgutil
+
+
+def _submodules():
+    """every module of the ao_amd package tree (packages before their members), private helpers excluded"""
+    names = []
+    for info in pkgutil.walk_packages(ao_amd.__path__, "ao_amd."):
+        rel = info.name[len("ao_amd."):]
+        if any(part.startswith("_") and part != "_models" for part in rel.split(".")) or rel.startswith(("csrc", "lib")):
+            continue
+        names.append(rel)
+    return names
+
+
+for _name in _submodules():
     _mod = importlib.import_module("ao_amd." + _name)
     sys.modules[__name__ + "." + _name] = _mod
     if "." not in _name:
