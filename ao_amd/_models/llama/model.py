@@ -291,37 +291,43 @@ class Transformer(nn.Module):
             ff._gate_up_pair_cache = cached
         return cached[1:]
 
-    def _fused_decode(self, idx: Tensor, input_pos: Tensor) -> Tensor:
-        """One token, batch 1: five launches per layer (norm + qkv, attention, wo + residual, norm + gate/up +
-        SwiGLU over the interleaved pair, down + residual).  Same roundings as the module-by-module path."""
+    def _fused_layer(self, b, x: Tensor, pos: Tensor) -> Tensor:
+        """One transformer block of the int4 decode step on the hidden state x [1, dim]: five launches (norm + qkv,
+        attention, wo + residual, norm + gate/up + SwiGLU over the interleaved pair, down + residual)."""
         from ... import ops
 
         cfg = self.config
 
-        def lin(x, layer, residual=None):
+        def lin(x, layer, residual):
             lay = layer.weight.layout_tensor
-            if residual is None:
-                return ops.int4wo_linear(x, lay.packed_weight, lay.scale_and_zero, lay.group_size, lay.N)
             return ops.int4wo_linear_residual(x, lay.packed_weight, lay.scale_and_zero, lay.group_size, lay.N, residual)
 
+        att = b.attention
+        qw = att.wqkv.weight.layout_tensor
+        if self.qkv_ksplit(qw.N) > 1:
+            # fp32 partial rows over two halves of K; the attention kernel adds and rounds them
+            qkv = ops.int4wo_linear_partials(x, qw.packed_weight, qw.scale_and_zero, qw.group_size, qw.N,
+                                             self.qkv_ksplit(qw.N), b.attention_norm.weight, b.attention_norm.eps)
+        else:
+            qkv = ops.int4wo_rmsnorm_linear(x, b.attention_norm.weight, b.attention_norm.eps, qw.packed_weight,
+                                            qw.scale_and_zero, qw.group_size, qw.N)
+        y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
+                                       cfg.n_head, cfg.n_local_heads)
+        h = lin(y, att.wo, x)
+        pair, pair_q, group, n_ff = self._gate_up_pair(b.feed_forward)
+        ff = ops.int4wo_swiglu_interleaved(h, pair, pair_q, group, n_ff, b.ffn_norm.weight, b.ffn_norm.eps)
+        return lin(ff, b.feed_forward.w2, h)
+
+    def _fused_decode(self, idx: Tensor, input_pos: Tensor) -> Tensor:
+        """One token, batch 1: five launches per layer, then norm + head.  Same roundings as the module-by-module
+        path."""
+        from ... import ops
+
+        cfg = self.config
         x = self.tok_embeddings(idx).view(1, cfg.dim)
         pos = input_pos.to(torch.int32) if input_pos.dtype is not torch.int32 else input_pos
         for b in self.layers:
-            att = b.attention
-            qw = att.wqkv.weight.layout_tensor
-            if self.qkv_ksplit(qw.N) > 1:
-                # fp32 partial rows over two halves of K; the attention kernel adds and rounds them
-                qkv = ops.int4wo_linear_partials(x, qw.packed_weight, qw.scale_and_zero, qw.group_size, qw.N,
-                                                 self.qkv_ksplit(qw.N), b.attention_norm.weight, b.attention_norm.eps)
-            else:
-                qkv = ops.int4wo_rmsnorm_linear(x, b.attention_norm.weight, b.attention_norm.eps, qw.packed_weight,
-                                                qw.scale_and_zero, qw.group_size, qw.N)
-            y = ops.llama_decode_attention(qkv, self.freqs_cis, pos, att.kv_cache.k_cache, att.kv_cache.v_cache,
-                                           cfg.n_head, cfg.n_local_heads)
-            h = lin(y, att.wo, residual=x)
-            pair, pair_q, group, n_ff = self._gate_up_pair(b.feed_forward)
-            ff = ops.int4wo_swiglu_interleaved(h, pair, pair_q, group, n_ff, b.ffn_norm.weight, b.ffn_norm.eps)
-            x = lin(ff, b.feed_forward.w2, residual=h)
+            x = self._fused_layer(b, x, pos)
         ow = self.output.weight.layout_tensor
         logits = ops.int4wo_rmsnorm_linear(x, self.norm.weight, self.norm.eps, ow.packed_weight, ow.scale_and_zero,
                                            ow.group_size, ow.N)

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <stdio.h>
 #include <string.h>
 
@@ -35,6 +36,17 @@ char* last_error_buf();  // thread-local, 512 bytes
 // timestamps into it (hipExtLaunchKernelGGL) and disarms; hipEventElapsedTime(start, stop) is then the
 // kernel's execution time without launch gaps.
 extern thread_local hipEvent_t g_prof_start, g_prof_stop;
+
+// Measurement switches (kernel families turned off, shape rules overridden) exist only in builds made with
+// -DAO_AMD_KNOBS; the shipped library reads no environment variable.
+inline const char* knob(const char* name) {
+#ifdef AO_AMD_KNOBS
+    return getenv(name);
+#else
+    (void)name;
+    return nullptr;
+#endif
+}
 
 inline bool is_float_dtype(int d) { return d == AO_F32 || d == AO_BF16 || d == AO_F16; }
 inline int dtype_size(int d) {

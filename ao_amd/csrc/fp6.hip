@@ -1448,7 +1448,7 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
         // 17 to 32 rows on a weight with 768 or more row blocks: the streaming kernel with four row blocks and two
         // activation blocks per workgroup (14336 x 4096: 11.3-13.4 us against 18 us of the tiled kernel, the head 82-97
         // against 145; four activation blocks for 33 to 64 rows spill and measured slower than the tiles)
-        static const bool mb_disabled = [] { const char* e = getenv("AO_AMD_FP6_MB"); return e && e[0] == '0'; }();
+        static const bool mb_disabled = [] { const char* e = knob("AO_AMD_FP6_MB"); return e && e[0] == '0'; }();
         if (!mb_disabled) {
             const int64_t wgs = RB / 4;
             int w4 = 4;

@@ -624,7 +624,7 @@ struct GemmLdsPlan {
 };
 
 static bool gemm_lds_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
-    static const bool disabled = [] { const char* e = getenv("AO_AMD_GEMM_LDS"); return e && e[0] == '0'; }();
+    static const bool disabled = [] { const char* e = knob("AO_AMD_GEMM_LDS"); return e && e[0] == '0'; }();
     if (disabled) return false;
     if (a.M < 128 || a.K != a.Kp || a.packed2 || a.residual || a.norm_w || a.pair8 || a.ksplit != 1) return false;
     if (g != 32 && g != 64 && g != 128 && g != 256) return false;
@@ -641,7 +641,8 @@ static bool gemm_lds_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
     auto cost = [](int64_t t, double per_tile) { return t >= 192 ? (double)((t + 255) / 256) * per_tile : 1e30; };
     const double c256 = cost(t256, 1.0), c128 = cost(t128, 0.51);
     p->nt = c128 < c256 ? 1 : 2;
-    if (const char* e = getenv("AO_AMD_GEMM_LDS_NT")) p->nt = e[0] == '1' ? 1 : 2;   // measurement aid
+    static const int forced_nt = [] { const char* e = knob("AO_AMD_GEMM_LDS_NT"); return e ? (e[0] == '1' ? 1 : 2) : 0; }();   // measurement aid
+    if (forced_nt) p->nt = forced_nt;
     p->tiles_n = (int)((a.N + 128 * p->nt - 1) / (128 * p->nt));
     const int64_t tiles = (int64_t)p->tiles_m * p->tiles_n;
     // ... and more than half of the tile rows real: at exactly 128 rows the 128-row kernel is faster (28672 x 4096: 50
@@ -654,9 +655,9 @@ static bool gemm_lds_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
 // rows: 39 us on the 64-row tiles, two passes, against 26 us; at 33-64 rows those are as fast or faster), when the tiles
 // cover at least three quarters of the CUs (measured: with 128 tiles the older kernels are as fast)
 static bool gemm_kwave_plan(const LinearArgs& a, int64_t g, GemmLdsPlan* p) {
-    static const bool disabled = [] { const char* e = getenv("AO_AMD_GEMM_KWAVE"); return e && e[0] == '0'; }();
+    static const bool disabled = [] { const char* e = knob("AO_AMD_GEMM_KWAVE"); return e && e[0] == '0'; }();
     if (disabled) return false;
-    static const int64_t min_rows = [] { const char* e = getenv("AO_AMD_GEMM_KWAVE_MIN_M"); return e ? atoll(e) : 65ll; }();
+    static const int64_t min_rows = [] { const char* e = knob("AO_AMD_GEMM_KWAVE_MIN_M"); return e ? atoll(e) : 65ll; }();
     if (a.M < min_rows || a.K != a.Kp || a.Kp < 1024 || a.packed2 || a.residual || a.norm_w || a.pair8 || a.ksplit != 1) return false;
     if (g != 32 && g != 64 && g != 128 && g != 256) return false;
     if (128 * a.ldx * 2 >= ((int64_t)1 << 32) || 4 * (a.Kp / 128) * 1024 + 1024 >= ((int64_t)1 << 32)) return false;

@@ -1188,7 +1188,7 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // 17 to 32 rows on a weight with 768 or more row blocks: the streaming kernel with four row blocks and two
     // activation blocks per workgroup (14336 x 4096: 16-18 us against 24.5 us of the 64-row tiles, the head 92-101
     // against 160; from 33 rows, two passes of it, the tiles win again)
-    static const bool rb4_off = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
+    static const bool rb4_off = [] { const char* e = knob("AO_AMD_RB4"); return e && e[0] == '0'; }();
     // ... and 33 to 48 rows (to 64 on weights with 4096 or more row blocks) with four activation blocks, which fit the
     // registers since the kernel keeps one tile buffer: 14336 x 4096 at 33-48 rows 25.5 -> 20.4-21.0 us, 28672 x 4096 38 ->
     // 32-33.5, the head at 33-64 rows 164-167 -> 115-145 (at 56-64 rows the tiles are as fast or faster on the others)
@@ -1260,7 +1260,7 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // (LDS-staged up to 5 rows there); the vocabulary head at 16 rows 85 against 129.
     if ((xmode == X_GLOBAL || (xmode == X_LDS && !norm_weight_bf16 && !pair8)) && !dual && ksplit == 1 && M >= 4 &&
         RB % 4 == 0 && a.K == a.Kp) {
-        static const bool rb4_disabled = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
+        static const bool rb4_disabled = [] { const char* e = knob("AO_AMD_RB4"); return e && e[0] == '0'; }();
         // two 16-row activation blocks per workgroup from 17 rows on: the dequantized dword feeds both (four of them
         // do not fit the registers)
         const int mb = M > 32 && M <= rb4_max_m ? 4 : (M > 16 ? 2 : 1);

@@ -521,7 +521,7 @@ static int int8wo_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     hipStream_t st = (hipStream_t)stream;
     // unstaged rows on a weight with 768 or more row blocks: four row blocks per workgroup share the activation loads
     // (14336 x 4096 at 16 rows: measured against the one-block kernel below)
-    static const bool rb4_disabled = [] { const char* e = getenv("AO_AMD_RB4"); return e && e[0] == '0'; }();
+    static const bool rb4_disabled = [] { const char* e = knob("AO_AMD_RB4"); return e && e[0] == '0'; }();
     // two activation blocks per workgroup from 17 rows on (four do not fit the registers): 14336 x 4096 at 17 / 32 / 64 /
     // 100 rows 31 / 34 / 59 / 97 -> 20.5 / 23 / 43 / 67 us, the head at 32 rows 243 -> 144
     const int mbv = M > 16 ? 2 : 1;
