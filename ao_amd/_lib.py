@@ -41,6 +41,7 @@ _SIGNATURES = {
     "ao_amd_int4wo_unpack": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _p], _int),
     "ao_amd_int4wo_dequantize": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
     "ao_amd_int4wo_linear": ([_p, _i64, _i64, _i64, _p, _p, _i64, _i64, _p, _p, _int, _i64, _p], _int),
+    "ao_amd_fp6_linear_plan": ([_i64, _i64, _i64, _int, _int, _int, _int, _int, _int, ctypes.c_char_p, _i64], _int),
     "ao_amd_int4wo_linear_plan": ([_i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _int, _int, ctypes.c_char_p, _i64], _int),
     "ao_amd_profile_next_linear": ([_p, _p], _int),
     "ao_amd_fp6_quantize_pack": ([_p, _int, _i64, _i64, _int, _int, _p, _p, _p], _int),
@@ -145,4 +146,12 @@ def int4wo_linear_plan(M: int, K: int, N: int, g: int, *, aligned: bool = True, 
     buf = ctypes.create_string_buffer(128)
     check(lib().ao_amd_int4wo_linear_plan(M, K, N, g, int(aligned), int(residual), int(norm), int(dual), int(pair8), ksplit,
                                           y_dtype, buf, 128))
+    return buf.value.decode()
+
+
+def fp6_linear_plan(M: int, K: int, N: int, ebits: int = 3, mbits: int = 2, *, norm: bool = False, residual: bool = False,
+                    gate: bool = False, dual: bool = False) -> str:
+    """Name of the kernel instantiation the FPx linear entry points run for this problem (host-side decision only)."""
+    buf = ctypes.create_string_buffer(128)
+    check(lib().ao_amd_fp6_linear_plan(M, K, N, ebits, mbits, int(norm), int(residual), int(gate), int(dual), buf, 128))
     return buf.value.decode()

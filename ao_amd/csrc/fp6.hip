@@ -1382,7 +1382,14 @@ static int fp6_row_blocks_per_wave(int64_t M, int64_t RB, int64_t mchunks) {
 static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
                                int64_t N, int ebits, int mbits, const void* residual_f16, const void* gate_f16,
                                void* out_f16, void* stream, const void* norm_weight_f16 = nullptr, float norm_eps = 0.f,
-                               const void* native_up = nullptr, const void* scale_up_f16 = nullptr) {
+                               const void* native_up = nullptr, const void* scale_up_f16 = nullptr, char* plan_out = nullptr,
+                               size_t plan_cap = 0) {
+    // plan_out: do not launch; write the name of the kernel instantiation the arguments select (ao_amd_fp6_linear_plan)
+#define AO_PLAN(...)                                    \
+    if (plan_out) {                                     \
+        snprintf(plan_out, plan_cap, __VA_ARGS__);      \
+        return 0;                                       \
+    }
     AO_REQUIRE(x_f16 && weights_native && scale_f16 && out_f16, "null pointer argument");
     AO_REQUIRE(!(residual_f16 && gate_f16), "residual and gate epilogues are exclusive");
     AO_REQUIRE(!(residual_f16 || gate_f16) || M <= 16, "the fused epilogues exist for at most 16 activation rows, got %lld",
@@ -1432,6 +1439,7 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
     // 8.2 / 7.2; 4096 x 14336 at 4 rows 12.1 / 11.4; at 2 rows staged wins everywhere: 14336 x 4096 9.6 / 11.7)
     const bool stage_pays = M <= 2 || (M == 3 && RB >= 768);
     if (fits && !shared_tiles && (need_lds || (KB >= 4 * waves && stage_pays))) {
+        AO_PLAN("fp6_gemv_kernel<%d,%d,%d>", waves, ebits == 3 ? 1 : 0, native_up ? 1 : 0);
         Fp6GemvArgs a{xx, M, K, Kp, nat, sc, N, o, res, gt, (const uint16_t*)norm_weight_f16, norm_eps,
                       (const uint32_t*)native_up, (const uint16_t*)scale_up_f16};
         if (ebits == 3) {
@@ -1454,6 +1462,7 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
             int w4 = 4;
             while (w4 < 8 && wgs * w4 * 2 <= 4096 + wgs && w4 * 2 <= KB) w4 *= 2;
             const dim3 mgrid((unsigned)(RB / 4), 1u);
+            AO_PLAN("fp6_linear_mb_kernel<%d,%d,2>", w4, ebits == 3 ? 1 : 0);
 #define AO_FP6_MB(W, E3) hipExtLaunchKernelGGL((fp6_linear_mb_kernel<W, E3, 2>), mgrid, dim3(W * 64), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o)
             if (ebits == 3) { if (w4 == 4) AO_FP6_MB(4, true); else AO_FP6_MB(8, true); }
             else { if (w4 == 4) AO_FP6_MB(4, false); else AO_FP6_MB(8, false); }
@@ -1469,6 +1478,7 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
         dim3 ggrid(big ? (unsigned)((RB + 7) / 8) : (unsigned)((RB + 3) / 4),
                    big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64));
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
+        AO_PLAN("fp6_gemm_kernel<%d,%s>", ebits == 3 ? 1 : 0, big ? "2,8,2,1" : (tiny ? "1,2,8,8" : "1,4,4,4"));
         if (ebits == 3) {
             if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 2, 8, 2, 1>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
             else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 2, 8, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
@@ -1504,6 +1514,8 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
         while (waves < wmax && (RB / rbw) * mchunks * waves * 2 <= 4096 + (RB / rbw) * mchunks && waves * 2 <= KB) waves *= 2;
     }
     dim3 lgrid((unsigned)(RB / rbw), (unsigned)mchunks);
+    AO_PLAN("fp6_linear_kernel<%d,%d,%d>", waves > (rbw == 4 ? 8 : 16) ? (rbw == 4 ? 8 : 16) : waves, ebits == 3 ? 1 : 0, rbw);
+#undef AO_PLAN
     if (rbw == 4) { AO_FP6_LAUNCH_WAVES(4, 8) }
     else if (rbw == 2) { AO_FP6_LAUNCH_WAVES(2, 16) }
     else { AO_FP6_LAUNCH_WAVES(1, 16) }
@@ -1511,6 +1523,17 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
 #undef AO_FP6_LAUNCH
     AO_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" int ao_amd_fp6_linear_plan(int64_t M, int64_t K, int64_t N, int ebits, int mbits, int has_norm, int has_residual,
+                                      int has_gate, int dual, char* out, int64_t out_cap) {
+    AO_REQUIRE(out && out_cap > 0, "null pointer argument");
+    // dummy operands: 16-byte aligned addresses that are never dereferenced
+    const void* p = reinterpret_cast<const void*>((uintptr_t)4096);
+    out[0] = 0;
+    return fp6_linear_dispatch(p, M, K, p, p, N, ebits, mbits, has_residual ? p : nullptr, has_gate ? p : nullptr,
+                               const_cast<void*>(p), nullptr, has_norm ? p : nullptr, 1e-5f, dual ? p : nullptr, dual ? p : nullptr,
+                               out, (size_t)out_cap);
 }
 
 extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native,

@@ -336,6 +336,14 @@ int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, int nbits, void* nat
 int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
                       int64_t N, int ebits, int mbits, void* out_f16, void* stream);
 
+/* Which kernel instantiation the FPx linear entry points run for a problem, without launching anything: writes a name
+ * such as "fp6_gemm_kernel<1,1,4,4,4>" (e3m2 flag, then the tile variant) or "fp6_gemv_kernel<8,1,0>" to `out`.  The
+ * flags say which fused variant is meant (RMSNorm on the activations, residual / gate epilogue, two weights).  The test
+ * suite walks the dispatch with it.  No counterpart in the reference (its launcher picks a kernel by batch bucket,
+ * torchao/csrc/cuda/fp6_llm/fp6_linear.cu:72-93). */
+int ao_amd_fp6_linear_plan(int64_t M, int64_t K, int64_t N, int ebits, int mbits, int has_norm, int has_residual,
+                           int has_gate, int dual, char* out, int64_t out_cap);
+
 /* The same linear for at most 16 activation rows with the module's next elementwise op on its fp16 result fused into the
  * epilogue (exactly one of the two operands, fp16 [M, N], is non-null): out = fp16(linear) + residual (h + attention(...),
  * h + feed_forward(...), TransformerBlock.forward, torchao/_models/llama/model.py:160-163) or

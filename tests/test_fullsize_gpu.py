@@ -139,6 +139,35 @@ def test_fp6_properties(shape):
             assert rel_l2(y[m].float().cpu().numpy(), dq[:, ks[m]].cpu().numpy()) <= 1e-3, (M, m)
 
 
+@pytest.mark.parametrize("M", [16, 128])
+@pytest.mark.parametrize("shape", [(4096, 4096), (14336, 4096), (4096, 14336)])
+def test_fp6_linear_full_size(shape, M):
+    """The FP6 configuration's many-row cases at the real Llama-3-8B shapes (the tile variants these shapes select are
+    not the ones small shapes select): one-hot activation rows return columns of fp16(value * scale) bit for bit, random
+    rows agree with an fp32 matmul on that weight to 1e-3 relative L2 and to the reference test's mean relative error
+    (test/test_ops.py:47-62)."""
+    from ao_amd import _lib, ops
+
+    N, K = shape
+    print(f"case fp6 linear full-size N={N} K={K} M={M}: {_lib.fp6_linear_plan(M, K, N)}", flush=True)
+    dev = _dev()
+    gen = torch.Generator(device=dev).manual_seed(N + M)
+    w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).half()
+    tc, scale = ops.fp6_quantize_pack(w, 3, 2)
+    w16 = ops.fp6_dequantize(tc, scale, 3, 2).half()
+    ks = torch.randint(0, K, (M,), device=dev, generator=gen)
+    ks[0], ks[-1] = 0, K - 1
+    xh = torch.zeros(M, K, dtype=torch.float16, device=dev)
+    xh[torch.arange(M, device=dev), ks] = 1.0
+    yh = ops.quant_llm_linear(3, 2, xh, tc, scale)
+    assert torch.equal(yh, w16.t()[ks])
+    x = torch.randn(M, K, device=dev, generator=gen).half()
+    y = ops.quant_llm_linear(3, 2, x, tc, scale).float()
+    ref = x.float() @ w16.float().t()
+    assert rel_l2(y.cpu().numpy(), ref.cpu().numpy()) <= 1e-3
+    assert float((y - ref).abs().mean() / ref.abs().mean()) < 1e-3
+
+
 @pytest.mark.parametrize("M", [128, 512, 2048])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_int4_prefill_gemm_full_size(shape, M):
