@@ -15,6 +15,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "../int4wo_gemv1.hip"
@@ -45,6 +46,10 @@ static float median(std::vector<float>& t) {
 
 // ------------------------------------------------------------------------------------------------ empty kernel
 __global__ void empty_kernel(int* p) {
+    if (p && threadIdx.x == 12345) p[0] = 1;
+}
+// the same, as the node of a graph (a name of its own, so that a profiler's per-kernel statistics keep the two apart)
+__global__ void empty_graph_node_kernel(int* p) {
     if (p && threadIdx.x == 12345) p[0] = 1;
 }
 // reads and rewrites an 8 KB vector: the smallest kernel with the data dependency of a decode launch
@@ -84,8 +89,8 @@ static void section_graph() {
         hipGraphExec_t exec;
         CK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
         for (int i = 0; i < N; ++i) {
-            if (kind == 0) hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, st, (int*)nullptr);
-            else if (kind == 1) hipLaunchKernelGGL(empty_kernel, dim3(896), dim3(256), 0, st, (int*)nullptr);
+            if (kind == 0) hipLaunchKernelGGL(empty_graph_node_kernel, dim3(1), dim3(64), 0, st, (int*)nullptr);
+            else if (kind == 1) hipLaunchKernelGGL(empty_graph_node_kernel, dim3(896), dim3(256), 0, st, (int*)nullptr);
             else hipLaunchKernelGGL(touch_kernel, dim3(8), dim3(256), 0, st, (i & 1) ? b : a, (i & 1) ? a : b);
         }
         CK(hipStreamEndCapture(st, &graph));
@@ -220,7 +225,8 @@ static void section_anyorder() {
 // ------------------------------------------------------------------------------------------------ load-only stream
 // A wave reads `tiles` consecutive 1 KiB tiles (16 bytes per lane, non-temporal), D requests in flight, and keeps an
 // xor of what it read; the store never happens.
-template <int D>
+// (CASE only gives every measured case a kernel name of its own)
+template <int D, int CASE>
 __global__ __launch_bounds__(256) void stream_nt_kernel(const char* base, int tiles, uint32_t* sink) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -257,6 +263,7 @@ static void section_stream() {
     const Case cases[] = {{"29.4MB tiles/wave=8", 29360128, 8},   {"29.4MB tiles/wave=4", 29360128, 4},
                           {"29.4MB tiles/wave=16", 29360128, 16}, {"29.4MB tiles/wave=28", 29360128, 28},
                           {"262.7MB tiles/wave=16", 262668288, 16}, {"262.7MB tiles/wave=32", 262668288, 32}};
+    int case_id = 0;
     for (auto& c : cases) {
         const int waves = (int)(c.bytes / 1024 / c.tiles);
         const int wgs = waves / 4;
@@ -265,15 +272,23 @@ static void section_stream() {
         std::vector<float> t;
         for (int it = 0; it < 60; ++it) {
             const char* p = buf + (size_t)(it % copies) * used;
-            hipExtLaunchKernelGGL(stream_nt_kernel<4>, dim3(wgs), dim3(256), 0, 0, g_e0, g_e1, 0, p, c.tiles, sink);
+            switch (case_id) {
+                case 0: hipExtLaunchKernelGGL((stream_nt_kernel<4, 0>), dim3(wgs), dim3(256), 0, 0, g_e0, g_e1, 0, p, c.tiles, sink); break;
+                case 1: hipExtLaunchKernelGGL((stream_nt_kernel<4, 1>), dim3(wgs), dim3(256), 0, 0, g_e0, g_e1, 0, p, c.tiles, sink); break;
+                case 2: hipExtLaunchKernelGGL((stream_nt_kernel<4, 2>), dim3(wgs), dim3(256), 0, 0, g_e0, g_e1, 0, p, c.tiles, sink); break;
+                case 3: hipExtLaunchKernelGGL((stream_nt_kernel<4, 3>), dim3(wgs), dim3(256), 0, 0, g_e0, g_e1, 0, p, c.tiles, sink); break;
+                case 4: hipExtLaunchKernelGGL((stream_nt_kernel<4, 4>), dim3(wgs), dim3(256), 0, 0, g_e0, g_e1, 0, p, c.tiles, sink); break;
+                default: hipExtLaunchKernelGGL((stream_nt_kernel<4, 5>), dim3(wgs), dim3(256), 0, 0, g_e0, g_e1, 0, p, c.tiles, sink); break;
+            }
             CK(hipEventSynchronize(g_e1));
             float ms;
             CK(hipEventElapsedTime(&ms, g_e0, g_e1));
             if (it >= 10) t.push_back(ms * 1e3f);
         }
         const float med = median(t);
-        printf("stream_nt %s wgs=%d (cold, %d copies) kernel_us median %.2f min %.2f  = %.2f TB/s (%.3f of 8 TB/s)\n", c.name, wgs,
-               copies, med, t[0], used / med * 1e-6, used / med * 1e-6 / 8.0);
+        printf("stream_nt<4,%d> %s wgs=%d (cold, %d copies) kernel_us median %.2f min %.2f  = %.2f TB/s (%.3f of 8 TB/s)\n", case_id, c.name,
+               wgs, copies, med, t[0], used / med * 1e-6, used / med * 1e-6 / 8.0);
+        ++case_id;
     }
     CK(hipFree(buf));
     CK(hipFree(sink));
@@ -360,9 +375,7 @@ __global__ __launch_bounds__(256) void lds_read_kernel(uint32_t* out, int iters)
     __syncthreads();
     uint32_t addr;
     const int row = (wave * 32 + (lane & 31)), col = lane >> 5;
-    if (MODE == 0) addr = row * 128 + ((col ^ (row & 7)) << 4);  // XOR-swizzled 16-byte fragment read (the GEMM's)
-    else if (MODE == 1) addr = (wave * 64 + lane) * 16;          // linear
-    else addr = row * 128 + col * 16;                            // unswizzled rows of 128 bytes (bank conflicts)
+    addr = row * 128 + ((col ^ (row & 7)) << 4);  // XOR-swizzled 16-byte fragment read (the prefill GEMM's)
     ao::u32x4_t acc = {0, 0, 0, 0};
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
@@ -393,8 +406,6 @@ static void section_lds() {
     uint32_t* out;
     CK(hipMalloc(&out, 512 * 256 * 4));
     lds_case<0>("swizzled-fragments", out);
-    lds_case<1>("linear", out);
-    lds_case<2>("unswizzled-rows", out);
     CK(hipFree(out));
 }
 
@@ -402,6 +413,7 @@ static void section_lds() {
 constexpr int kSpinLimit = 1 << 16;   // polls; a barrier that has not opened by then sets err and every wave leaves
 
 // (a) one counter, agent-scope release / acquire with a fence (what __threadfence + atomics give by default)
+template <int NWG>
 __global__ void barrier_fenced_kernel(unsigned* st, int iters, unsigned nwg) {
     unsigned* cnt = st;
     unsigned* err = st + 64;
@@ -425,6 +437,7 @@ __global__ void barrier_fenced_kernel(unsigned* st, int iters, unsigned nwg) {
     }
 }
 // (b) the same counter with relaxed agent-scope atomics only (no cache write-back / invalidate)
+template <int NWG>
 __global__ void barrier_relaxed_kernel(unsigned* st, int iters, unsigned nwg) {
     unsigned* cnt = st;
     unsigned* err = st + 64;
@@ -451,7 +464,7 @@ __global__ void barrier_relaxed_kernel(unsigned* st, int iters, unsigned nwg) {
 // 32 bytes of a vector before its flag (agent-scope stores, waited for before the flag store), and after the barrier
 // every workgroup reads the whole vector back with agent-scope loads and counts the words that are not this
 // iteration's: the data handoff of one decode dependency, with a correctness check of the fence-free protocol.
-template <bool PAYLOAD>
+template <bool PAYLOAD, int NWG>
 __global__ void barrier_flags_kernel(unsigned* st, int iters, unsigned nwg, unsigned* vec, unsigned* bad) {
     unsigned* flags = st + 128;   // nwg words
     unsigned* err = st + 64;
@@ -533,18 +546,22 @@ static void section_barrier() {
     CK(hipMemset(bad, 0, 4));
     CK(hipMemset(vec, 0, 4096 * 4));
     const int iters = 400;
+    auto run_all = [&](auto tag, int threads) {
+        constexpr unsigned nwg = decltype(tag)::value;
+        char name[160];
+        snprintf(name, sizeof name, "grid_barrier fenced-counter nwg=%u threads=%d", nwg, threads);
+        time_barrier(name, st, iters, [&] { hipExtLaunchKernelGGL(barrier_fenced_kernel<(int)nwg>, dim3(nwg), dim3(threads), 0, 0, g_e0, g_e1, 0, st, iters, nwg); });
+        snprintf(name, sizeof name, "grid_barrier relaxed-counter nwg=%u threads=%d", nwg, threads);
+        time_barrier(name, st, iters, [&] { hipExtLaunchKernelGGL(barrier_relaxed_kernel<(int)nwg>, dim3(nwg), dim3(threads), 0, 0, g_e0, g_e1, 0, st, iters, nwg); });
+        snprintf(name, sizeof name, "grid_barrier flag-array nwg=%u threads=%d", nwg, threads);
+        time_barrier(name, st, iters, [&] { hipExtLaunchKernelGGL((barrier_flags_kernel<false, (int)nwg>), dim3(nwg), dim3(threads), 0, 0, g_e0, g_e1, 0, st, iters, nwg, vec, bad); });
+        snprintf(name, sizeof name, "grid_barrier flag-array + %u-byte vector handoff nwg=%u threads=%d", nwg * 32, nwg, threads);
+        time_barrier(name, st, iters, [&] { hipExtLaunchKernelGGL((barrier_flags_kernel<true, (int)nwg>), dim3(nwg), dim3(threads), 0, 0, g_e0, g_e1, 0, st, iters, nwg, vec, bad); });
+    };
     for (int threads : {64, 1024}) {
-        for (unsigned nwg : {8u, 64u, 256u}) {
-            char name[160];
-            snprintf(name, sizeof name, "grid_barrier fenced-counter nwg=%u threads=%d", nwg, threads);
-            time_barrier(name, st, iters, [&] { hipExtLaunchKernelGGL(barrier_fenced_kernel, dim3(nwg), dim3(threads), 0, 0, g_e0, g_e1, 0, st, iters, nwg); });
-            snprintf(name, sizeof name, "grid_barrier relaxed-counter nwg=%u threads=%d", nwg, threads);
-            time_barrier(name, st, iters, [&] { hipExtLaunchKernelGGL(barrier_relaxed_kernel, dim3(nwg), dim3(threads), 0, 0, g_e0, g_e1, 0, st, iters, nwg); });
-            snprintf(name, sizeof name, "grid_barrier flag-array nwg=%u threads=%d", nwg, threads);
-            time_barrier(name, st, iters, [&] { hipExtLaunchKernelGGL(barrier_flags_kernel<false>, dim3(nwg), dim3(threads), 0, 0, g_e0, g_e1, 0, st, iters, nwg, vec, bad); });
-            snprintf(name, sizeof name, "grid_barrier flag-array + %u-byte vector handoff nwg=%u threads=%d", nwg * 32, nwg, threads);
-            time_barrier(name, st, iters, [&] { hipExtLaunchKernelGGL(barrier_flags_kernel<true>, dim3(nwg), dim3(threads), 0, 0, g_e0, g_e1, 0, st, iters, nwg, vec, bad); });
-        }
+        run_all(std::integral_constant<unsigned, 8>{}, threads);
+        run_all(std::integral_constant<unsigned, 64>{}, threads);
+        run_all(std::integral_constant<unsigned, 256>{}, threads);
     }
     unsigned hb;
     CK(hipMemcpy(&hb, bad, 4, hipMemcpyDeviceToHost));
