@@ -1040,7 +1040,14 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_gemv_kernel(const Fp6GemvArgs 
             }
         }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // duplicate requests of a short wave
+    // duplicate requests of a short wave may still be in flight; the ring registers are inputs of this wait, which keeps
+    // them allocated up to it (dead loaded values would otherwise free their registers under a load)
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+        if (DUAL) asm volatile("" : : "v"(buf_up[j].lo), "v"(buf_up[j].hi));
+        if (j + 1 < D) asm volatile("" : : "v"(buf[j].lo), "v"(buf[j].hi));
+        else asm volatile("s_waitcnt vmcnt(0)" : : "v"(buf[j].lo), "v"(buf[j].hi) : "memory");
+    }
 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

@@ -721,7 +721,14 @@ __global__ __launch_bounds__(WAVES * 64) void int4wo_gemv_kernel(const LinearArg
             }
         }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the requests of a wave without tiles
+    // the requests of a wave without tiles may still be in flight; the ring registers are inputs of this wait, which
+    // keeps them allocated up to it
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+        if (DUAL) asm volatile("" : : "v"(buf[j].w2), "v"(buf[j].q2));
+        if (j + 1 < D) asm volatile("" : : "v"(buf[j].w), "v"(buf[j].q));
+        else asm volatile("s_waitcnt vmcnt(0)" : : "v"(buf[j].w), "v"(buf[j].q) : "memory");
+    }
 
     // acc[i] = C[m = 4*qd + i][n = r]
 #pragma unroll

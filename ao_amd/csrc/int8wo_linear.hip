@@ -266,7 +266,14 @@ __global__ __launch_bounds__(WAVES * 64) void int8wo_linear_kernel(const Int8Arg
                 }
             }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // duplicate requests of a short wave
+        // duplicate requests of a short wave may still be in flight; the ring registers are inputs of this wait, which
+        // keeps them allocated up to it (dead loaded values would otherwise free their registers under a load)
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            if (DUAL) asm volatile("" : : "v"(buf[j].u0), "v"(buf[j].u1));
+            if (j + 1 < D) asm volatile("" : : "v"(buf[j].w0), "v"(buf[j].w1));
+            else asm volatile("s_waitcnt vmcnt(0)" : : "v"(buf[j].w0), "v"(buf[j].w1) : "memory");
+        }
     }
     // acc[i] = C[m = 4*qd + i][n = r]
 #pragma unroll
