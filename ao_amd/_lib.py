@@ -74,6 +74,8 @@ _SIGNATURES = {
     "ao_amd_hqq_dequantize": ([_p, _int, _i64, _i64, _p, _p, _i64, _int, _p, _p], _int),
     "ao_amd_hqq_mixed_mm_workspace": ([_i64, _i64, _i64, ctypes.POINTER(ctypes.c_int64)], _int),
     "ao_amd_hqq_mixed_mm": ([_p, _i64, _i64, _i64, _p, _int, _i64, _p, _p, _i64, _int, _p, _i64, _p, _p], _int),
+    "ao_amd_hqq_mixed_mm_mfma_workspace": ([_i64, _i64, _i64, _int, ctypes.POINTER(ctypes.c_int64)], _int),
+    "ao_amd_hqq_mixed_mm_mfma": ([_p, _i64, _i64, _p, _int, _i64, _i64, _p, _p, _i64, _int, _int, _p, _i64, _p, _p], _int),
     "ao_amd_rmsnorm_bf16": ([_p, _p, _i64, _i64, ctypes.c_float, _p, _p], _int),
     "ao_amd_argmax_bf16": ([_p, _i64, _p, _p], _int),
     "ao_amd_argmax_f16": ([_p, _i64, _p, _p], _int),

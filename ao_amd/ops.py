@@ -58,6 +58,7 @@ _LIB.define("int8wo_swiglu(Tensor x, Tensor? norm_weight, float eps, Tensor w_ga
 _LIB.define("int8wo_rmsnorm_linear(Tensor x, Tensor norm_weight, float eps, Tensor w_int8, Tensor scale, Tensor? gate) -> Tensor")
 _LIB.define("hqq_dequantize(Tensor packed_2xint4, Tensor scales, Tensor zeros, int group_size) -> Tensor")
 _LIB.define("hqq_mixed_mm_small(Tensor a, Tensor packed_2xint4, Tensor scales, Tensor zeros, int group_size) -> Tensor")
+_LIB.define("hqq_mixed_mm_mfma(Tensor a, Tensor packed_2xint4, Tensor scales, Tensor zeros, int group_size, bool transposed) -> Tensor")
 _LIB.define("rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor")
 _LIB.define("argmax_bf16(Tensor x) -> Tensor")
 _LIB.define("llama_decode_attention(Tensor qkv, Tensor freqs_cis, Tensor input_pos, Tensor(a!) k_cache, Tensor(b!) v_cache, int n_head, int n_kv) -> Tensor")
@@ -481,6 +482,37 @@ def _hqq_mixed_mm_small_cuda(a, packed_2xint4, scales, zeros, group_size):
     return y
 
 
+def _hqq_mixed_mm_mfma_cuda(a, packed_2xint4, scales, zeros, group_size, transposed):
+    """a [M <= 64, K] @ W [K, N], or a [M <= 64, N] @ W^T when `transposed`, W the dequantized HQQ weight; fused."""
+    require_cuda(a, packed_2xint4, scales, zeros)
+    torch._check(packed_2xint4.dim() == 2 and packed_2xint4.dtype in (torch.uint8, torch.int8),
+                 lambda: "b must be a 2d int8 or uint8 tensor")
+    torch._check(a.dim() == 2 and a.dtype in (torch.float16, torch.bfloat16) and scales.dtype is a.dtype and zeros.dtype is a.dtype,
+                 lambda: f"a, scales and zeros must share float16 or bfloat16, got {a.dtype}, {scales.dtype}, {zeros.dtype}")
+    K2, N = packed_2xint4.shape
+    K = 2 * K2
+    M = a.shape[0]
+    if transposed:
+        torch._check(a.shape[1] == N, lambda: "transpose requires (M x N) x (K x N), where reduction dim is N")
+    else:
+        torch._check(a.shape[1] == K, lambda: "incompatible dimensions")
+    torch._check(1 <= M <= 64, lambda: f"the fused product takes 1 to 64 rows, got {M}")
+    torch._check(scales.dim() == 2 and scales.shape == zeros.shape and scales.shape == (K // group_size, N),
+                 lambda: f"scales / zeros must have shape ({K // group_size}, {N}), got {tuple(scales.shape)} and {tuple(zeros.shape)}")
+    if a.stride(1) != 1 or a.stride(0) % 8 or a.data_ptr() % 16:
+        a = a.contiguous()
+    packed_2xint4, scales, zeros = packed_2xint4.contiguous(), scales.contiguous(), zeros.contiguous()
+    need = ctypes.c_int64(0)
+    check(lib().ao_amd_hqq_mixed_mm_mfma_workspace(M, K, N, int(transposed), ctypes.byref(need)))
+    ws = torch.empty((need.value // 4,), dtype=torch.float32, device=a.device)
+    y = torch.empty((M, K if transposed else N), dtype=a.dtype, device=a.device)
+    check(lib().ao_amd_hqq_mixed_mm_mfma(a.data_ptr(), M, a.stride(0), packed_2xint4.data_ptr(),
+                                         int(packed_2xint4.dtype is torch.int8), K, N, scales.data_ptr(), zeros.data_ptr(),
+                                         group_size, BF16 if a.dtype is torch.bfloat16 else F16, int(transposed),
+                                         ws.data_ptr(), need.value, y.data_ptr(), current_stream(a.device)))
+    return y
+
+
 def _rmsnorm_cuda(x, weight, eps):
     require_cuda(x, weight)
     torch._check(x.dtype in (torch.bfloat16, torch.float16) and weight.dtype is x.dtype,
@@ -776,6 +808,7 @@ _LIB.impl("int8wo_rmsnorm_linear", _int8wo_rmsnorm_linear_cuda, "CUDA")
 _LIB.impl("int8wo_swiglu", _int8wo_swiglu_cuda, "CUDA")
 _LIB.impl("hqq_dequantize", _hqq_dequantize_cuda, "CUDA")
 _LIB.impl("hqq_mixed_mm_small", _hqq_mixed_mm_small_cuda, "CUDA")
+_LIB.impl("hqq_mixed_mm_mfma", _hqq_mixed_mm_mfma_cuda, "CUDA")
 _LIB.impl("rmsnorm", _rmsnorm_cuda, "CUDA")
 _LIB.impl("llama_decode_attention", _decode_attention_cuda, "CUDA")
 _LIB.impl("argmax_bf16", _argmax_bf16_cuda, "CUDA")
@@ -794,7 +827,7 @@ def _no_cpu(name):
 
 for _name in ("int4wo_quantize_pack", "int4wo_pack", "int4wo_unpack", "int4wo_dequantize", "int4wo_linear",
               "int4wo_linear_residual", "int4wo_swiglu", "int4wo_rmsnorm_linear", "int4wo_rmsnorm_swiglu", "int4wo_linear_partials", "int4wo_interleave_pair",
-              "int4wo_swiglu_interleaved", "int8wo_linear", "int8wo_linear_fused", "int8wo_rmsnorm_linear", "int8wo_swiglu", "hqq_dequantize", "hqq_mixed_mm_small", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
+              "int4wo_swiglu_interleaved", "int8wo_linear", "int8wo_linear_fused", "int8wo_rmsnorm_linear", "int8wo_swiglu", "hqq_dequantize", "hqq_mixed_mm_small", "hqq_mixed_mm_mfma", "rmsnorm", "llama_decode_attention", "argmax_bf16", "quant_llm_linear",
               "fp6_quantize_pack", "fp6_dequantize", "fp6_repack", "fp6_linear_native", "fp6_linear_native_fused", "fp6_rmsnorm_linear",
               "fp6_swiglu"):
     _LIB.impl(_name, _no_cpu(_name), "CPU")
@@ -905,6 +938,11 @@ def _(packed_2xint4, scales, zeros, group_size):
 @torch.library.register_fake("torchao::hqq_mixed_mm_small")
 def _(a, packed_2xint4, scales, zeros, group_size):
     return a.new_empty((a.shape[0], packed_2xint4.shape[1]))
+
+
+@torch.library.register_fake("torchao::hqq_mixed_mm_mfma")
+def _(a, packed_2xint4, scales, zeros, group_size, transposed):
+    return a.new_empty((a.shape[0], 2 * packed_2xint4.shape[0] if transposed else packed_2xint4.shape[1]))
 
 
 @torch.library.register_fake("torchao::rmsnorm")
@@ -1067,6 +1105,13 @@ def int8wo_linear(x: Tensor, w_int8: Tensor, scale: Tensor, bias=None, fp32_out:
 def hqq_mixed_mm_small(a: Tensor, packed_2xint4: Tensor, scales: Tensor, zeros: Tensor, group_size: int) -> Tensor:
     """a [M <= 16, K] @ ((q - zero) * scale) [K, N], dequantization fused into the product."""
     return torch.ops.torchao.hqq_mixed_mm_small.default(a, packed_2xint4, scales, zeros, group_size)
+
+
+def hqq_mixed_mm_mfma(a: Tensor, packed_2xint4: Tensor, scales: Tensor, zeros: Tensor, group_size: int,
+                      transposed: bool = False) -> Tensor:
+    """a [M <= 64, K] @ W, or a [M <= 64, N] @ W^T when `transposed`, with W = (q - zero) * scale [K, N] dequantized
+    inside the matrix-core kernel."""
+    return torch.ops.torchao.hqq_mixed_mm_mfma.default(a, packed_2xint4, scales, zeros, group_size, transposed)
 
 
 def hqq_dequantize(packed_2xint4: Tensor, scales: Tensor, zeros: Tensor, group_size: int) -> Tensor:

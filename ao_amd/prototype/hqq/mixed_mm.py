@@ -1,8 +1,8 @@
 """Mixed matmul over HQQ-format int4 weights (reference torchao/prototype/hqq/mixed_mm.py).
 
-The reference fuses the dequantization into a Triton GEMM.  Here the forward product of up to 8 activation rows (the
-decode case the kernel exists for; `ops.hqq_mixed_mm_small` takes up to 16) runs a fused HIP kernel that streams the packed codes once; more rows, and the
-transposed product, dequantize the weight with a HIP kernel into a matrix of the activation dtype, op by op as the
+The reference fuses the dequantization into a Triton GEMM.  Here both products (forward over K, transposed over N) of up
+to 64 activation rows run a fused matrix-core HIP kernel that streams the packed codes once and dequantizes them in
+registers; more rows dequantize the weight with a HIP kernel into a matrix of the activation dtype, op by op as the
 reference's kernel does ((q - zero) * scale, kernels.py:318-358), and call the vendor GEMM on it.
 """
 import torch
@@ -10,9 +10,11 @@ import torch
 from ... import ops
 
 
-# activation rows up to which the forward product runs the fused kernel (measured on MI355X, kernels only: 4096 x 4096 at
-# 1-4 rows 11 + 4 us against 12 + 16 us for dequantize + library GEMM, 8 rows 16 + 4 against 12 + 16; at 16 rows the
-# fused kernel's per-row FMAs make it the slower of the two on wide weights)
+# activation rows up to which the fused kernels run (measured on MI355X, kernels only, bf16, graph replays: 4096 x 4096
+# at 1-16 rows 10.5-10.8 us, 64 rows 16 us, either product, against 26-35 us for dequantize + library GEMM; 11008 x 4096
+# 19-34 us against 41-50 us).  Shapes the matrix-core kernel does not take (K or the group size not a multiple of 8
+# forward, N not a multiple of 16 transposed) fall back to the scalar fused kernel up to FUSED_MAX_ROWS rows, forward only.
+MFMA_MAX_ROWS = 64
 FUSED_MAX_ROWS = 8
 
 
@@ -43,7 +45,13 @@ def mixed_mm(a, b, scales, zeros, group_size, transposed=False, acc_dtype=None, 
         assert a.shape[1] == b.shape[0] * 2, "incompatible dimensions"
     else:
         assert a.shape[1] == b.shape[1], "transpose requires (M x N) x (K x N), where reduction dim is N"
-    if not transposed and 1 <= a.shape[0] <= FUSED_MAX_ROWS and b.shape[1] % 4 == 0:
+    M, (K2, N) = a.shape[0], b.shape
+    if 1 <= M <= MFMA_MAX_ROWS and scales.shape[0] * group_size == 2 * K2:
+        if transposed and N % 16 == 0 and group_size % 2 == 0:
+            return ops.hqq_mixed_mm_mfma(a, b, scales, zeros, group_size, True)
+        if not transposed and K2 % 4 == 0 and group_size % 8 == 0 and N % 4 == 0:
+            return ops.hqq_mixed_mm_mfma(a, b, scales, zeros, group_size, False)
+    if not transposed and 1 <= M <= FUSED_MAX_ROWS and N % 4 == 0:
         return ops.hqq_mixed_mm_small(a, b, scales, zeros, group_size)
     w = ops.hqq_dequantize(b, scales, zeros, group_size)  # [K, N]
     return torch.matmul(a, w.t() if transposed else w)

@@ -184,12 +184,25 @@ int ao_amd_hqq_dequantize(const void* packed_2xint4, int is_signed, int64_t K, i
  * above (every weight rounded twice to `dtype` exactly as ao_amd_hqq_dequantize rounds it), fp32 accumulation, y in
  * `dtype`, row stride N.  a: `dtype` [M, K] with row stride lda (even, rows 4-byte aligned); N a multiple of 4, packed
  * codes 4-byte and scales / zeros 8-byte aligned.  K is cut into slices whose fp32 partial sums go through `workspace`
- * (ao_amd_hqq_mixed_mm_workspace gives its size; caller-owned, device memory).  More rows, or the transposed product,
- * take ao_amd_hqq_dequantize and a library GEMM. */
+ * (ao_amd_hqq_mixed_mm_workspace gives its size; caller-owned, device memory). */
 int ao_amd_hqq_mixed_mm_workspace(int64_t M, int64_t K, int64_t N, int64_t* bytes);
 int ao_amd_hqq_mixed_mm(const void* a, int64_t M, int64_t K, int64_t lda, const void* packed_2xint4, int is_signed, int64_t N,
                         const void* scales, const void* zeros, int64_t group_size, int dtype, void* workspace,
                         int64_t workspace_bytes, void* y, void* stream);
+
+/* Both products of that kernel for 1 to 64 activation rows on the matrix cores, the weight dequantized in registers
+ * (torchao/prototype/hqq/kernels.py:162-388; `transposed` is the TRANSPOSED switch of the Triton kernel,
+ * triton_mixed_mm(..., transposed=True), mixed_mm.py:38-62).  transposed == 0: y[M,N] = a[M,K] @ W[K,N]; needs K and
+ * group_size multiples of 8, N a multiple of 4.  transposed != 0: y[M,K] = a[M,N] @ W^T, the product over N that a
+ * backward pass needs; needs N a multiple of 16, K and group_size even.  Every weight is rounded twice to `dtype`
+ * exactly as ao_amd_hqq_dequantize rounds it; fp32 accumulation; y in `dtype`, contiguous.  a: `dtype`, row stride lda
+ * a multiple of 8 elements, 16-byte aligned like the packed codes, scales and zeros.  The reduction is cut into slices
+ * whose fp32 partial sums go through `workspace` (ao_amd_hqq_mixed_mm_mfma_workspace gives its size; caller-owned,
+ * device memory, 16-byte aligned).  More than 64 rows take ao_amd_hqq_dequantize and a library GEMM. */
+int ao_amd_hqq_mixed_mm_mfma_workspace(int64_t M, int64_t K, int64_t N, int transposed, int64_t* bytes);
+int ao_amd_hqq_mixed_mm_mfma(const void* a, int64_t M, int64_t lda, const void* packed_2xint4, int is_signed, int64_t K,
+                             int64_t N, const void* scales, const void* zeros, int64_t group_size, int dtype,
+                             int transposed, void* workspace, int64_t workspace_bytes, void* y, void* stream);
 
 /* ---------------------------------------------------------------- int8 weight-only linear
  * y[M,N] = bf16( bf16(x[M,K] @ bf16(w)^T) * scale[N] ) (+ bias, rounded to bf16 again): the per-channel int8

@@ -167,16 +167,10 @@ def test_fused_small_m_product_matches_the_dequantized_matmul(oracle, M, N, K, g
     ref_r = torch.from_numpy(ref).to(dtype).float().numpy()
     err = rel_l2(y.float().cpu().numpy(), ref_r)
     assert err <= 1e-3, err
-    # the module-level entry point takes the fused kernel up to FUSED_MAX_ROWS rows, the two-pass route beyond
-    from ao_amd.prototype.hqq.mixed_mm import FUSED_MAX_ROWS
-    if N % 16 == 0 or M <= FUSED_MAX_ROWS:
-        y2 = mixed_mm(x, packed, s, z, g)
-        if M <= FUSED_MAX_ROWS:
-            same = bool(torch.equal(y, y2))
-            assert same
-        else:
-            err2 = rel_l2(y2.float().cpu().numpy(), ref_r)
-            assert err2 <= 2e-3, err2
+    # the module-level entry point takes the matrix-core kernel for these shapes
+    if N % 16 == 0 or K % 8 == 0:
+        err2 = rel_l2(mixed_mm(x, packed, s, z, g).float().cpu().numpy(), ref_r)
+        assert err2 <= 1e-3, err2
     # one-hot rows read single weights back, bit for bit
     ks = torch.randint(0, K, (M,), generator=torch.Generator().manual_seed(4))
     ks[0], ks[-1] = 0, K - 1
@@ -201,3 +195,79 @@ def test_fused_product_limits():
     # 17 rows go the two-pass way through the module-level entry point
     y = mixed_mm(torch.randn(17, 128, dtype=torch.float16, device=dev), b, s, z, 64)
     assert y.shape == (17, 64)
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("transposed", [False, True])
+@pytest.mark.parametrize("M,N,K,g", [(1, 4096, 4096, 64), (16, 128, 128, 128), (17, 1008, 520, 8), (33, 4096, 11008, 128),
+                                     (64, 11008, 4096, 64), (9, 48, 100, 2), (40, 64, 2048, 32)])
+def test_matrix_core_product_matches_the_dequantized_matmul(oracle, M, N, K, g, dtype, transposed, signed):
+    """The matrix-core kernel (1-64 rows, forward and transposed): within 1e-3 relative L2 of the float64 product with
+    the oracle's dequantized weight (rounded to the output dtype), and exactly the dequantized weight on one-hot rows:
+    the kernel rounds every weight as ao_amd_hqq_dequantize does.  N = 1008 and 48 leave lanes of the last tile without
+    columns, K = 520 and 100 leave the last reduction step / the last tile of byte rows partly empty; K = 100 and
+    group 2 are legal only for the transposed product: the forward one refuses them."""
+    from ao_amd import ops
+    from ao_amd.prototype.hqq import pack_2xint4
+
+    if not transposed and (K % 8 or g % 8):
+        with pytest.raises(RuntimeError, match="multiples of 8"):
+            W_q, scale, zero = _hqq_like(N, K, g, dtype, seed=1, signed=signed)
+            ops.hqq_mixed_mm_mfma(torch.zeros(M, K, dtype=dtype, device=_dev()), pack_2xint4(W_q.T.contiguous()).to(_dev()),
+                                  scale.T.contiguous().to(_dev()), zero.T.contiguous().to(_dev()), g, False)
+        return
+    print(f"case hqq mfma M={M} N={N} K={K} g={g} {dtype} transposed={transposed} signed={signed}", flush=True)
+    dev = _dev()
+    W_q, scale, zero = _hqq_like(N, K, g, dtype, seed=M + N + g, signed=signed)
+    packed = pack_2xint4(W_q.T.contiguous()).to(dev)
+    s, z = scale.T.contiguous().to(dev), zero.T.contiguous().to(dev)
+    code = oracle.BF16 if dtype is torch.bfloat16 else oracle.F16
+    w_ref = oracle.hqq_dequantize(packed.cpu().numpy(), bits16(s.cpu()), bits16(z.cpu()), g, code)   # [K, N] bits
+    w_f64 = (oracle.bf16_bits_to_f32(w_ref) if dtype is torch.bfloat16 else w_ref.view(np.float16)).astype(np.float64)
+    R = N if transposed else K          # reduction length
+    x = torch.randn(M, R, dtype=dtype, generator=torch.Generator().manual_seed(3)).to(dev)
+    y = ops.hqq_mixed_mm_mfma(x, packed, s, z, g, transposed)
+    assert y.shape == (M, K if transposed else N) and y.dtype is dtype
+    ref = x.float().cpu().numpy().astype(np.float64) @ (w_f64.T if transposed else w_f64)
+    ref_r = torch.from_numpy(ref).to(dtype).float().numpy()
+    err = rel_l2(y.float().cpu().numpy(), ref_r)
+    assert err <= 1e-3, err
+    # a second call with a padded, strided activation gives the same bits
+    xp = torch.zeros(M, R + 8, dtype=dtype, device=dev)
+    xp[:, :R] = x
+    same = bool(torch.equal(ops.hqq_mixed_mm_mfma(xp[:, :R], packed, s, z, g, transposed), y))
+    assert same
+    # one-hot rows read single rows (forward) or columns (transposed) of the weight back, bit for bit
+    idx = torch.randint(0, R, (M,), generator=torch.Generator().manual_seed(4))
+    idx[0], idx[-1] = 0, R - 1
+    xh = torch.zeros(M, R, dtype=dtype)
+    xh[torch.arange(M), idx] = 1.0
+    yh = ops.hqq_mixed_mm_mfma(xh.to(dev), packed, s, z, g, transposed)
+    picked = w_ref[:, idx.numpy()].T if transposed else w_ref[idx.numpy()]
+    want = torch.from_numpy(np.ascontiguousarray(picked).astype(np.int16)).view(dtype)
+    exact = bool(torch.equal(yh.cpu(), want))
+    assert exact
+
+
+def test_matrix_core_product_limits():
+    from ao_amd import ops
+    from ao_amd.prototype.hqq import pack_2xint4
+
+    dev = _dev()
+    W_q, scale, zero = _hqq_like(64, 128, 64, torch.float16, seed=1)
+    b = pack_2xint4(W_q.T.contiguous()).to(dev)
+    s, z = scale.T.contiguous().to(dev), zero.T.contiguous().to(dev)
+    with pytest.raises(RuntimeError, match="1 to 64 rows"):
+        ops.hqq_mixed_mm_mfma(torch.randn(65, 128, dtype=torch.float16, device=dev), b, s, z, 64, False)
+    with pytest.raises(RuntimeError, match="incompatible dimensions"):
+        ops.hqq_mixed_mm_mfma(torch.randn(4, 64, dtype=torch.float16, device=dev), b, s, z, 64, False)
+    with pytest.raises(RuntimeError, match="transpose requires"):
+        ops.hqq_mixed_mm_mfma(torch.randn(4, 128, dtype=torch.float16, device=dev), b, s, z, 64, True)
+    # N = 40: fine forward (multiple of 4), refused transposed (needs a multiple of 16)
+    W_q, scale, zero = _hqq_like(40, 128, 64, torch.float16, seed=2)
+    b = pack_2xint4(W_q.T.contiguous()).to(dev)
+    s, z = scale.T.contiguous().to(dev), zero.T.contiguous().to(dev)
+    assert ops.hqq_mixed_mm_mfma(torch.randn(4, 128, dtype=torch.float16, device=dev), b, s, z, 64, False).shape == (4, 40)
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        ops.hqq_mixed_mm_mfma(torch.randn(4, 40, dtype=torch.float16, device=dev), b, s, z, 64, True)

@@ -58,3 +58,24 @@ def test_opcheck_fp6_pack_operators():
     fpx, scale = torch.ops.torchao.fp6_quantize_pack(w, 3, 2)
     torch.library.opcheck(torch.ops.torchao.fp6_dequantize.default, (fpx, scale, 3, 2), test_utils=_UTILS)
     torch.library.opcheck(torch.ops.torchao.fp6_repack.default, (fpx, 6), test_utils=_UTILS)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_opcheck_hqq_operators(dtype):
+    from ao_amd import ops  # noqa: F401
+    from ao_amd.prototype.hqq import pack_2xint4
+
+    print(f"case opcheck hqq {dtype}", flush=True)
+    dev = torch.device("cuda:0")
+    torch.manual_seed(3)
+    N, K, g = 256, 512, 64
+    packed = pack_2xint4(torch.randint(0, 16, (K, N), dtype=torch.uint8)).to(dev)
+    s = (torch.rand(K // g, N, device=dev) * 0.02 + 1e-3).to(dtype)
+    z = (torch.rand(K // g, N, device=dev) * 6 + 5).to(dtype)
+    torch.library.opcheck(torch.ops.torchao.hqq_dequantize.default, (packed, s, z, g), test_utils=_UTILS)
+    x = torch.randn(5, K, device=dev).to(dtype)
+    torch.library.opcheck(torch.ops.torchao.hqq_mixed_mm_small.default, (x, packed, s, z, g), test_utils=_UTILS)
+    torch.library.opcheck(torch.ops.torchao.hqq_mixed_mm_mfma.default, (x, packed, s, z, g, False), test_utils=_UTILS)
+    xt = torch.randn(33, N, device=dev).to(dtype)
+    torch.library.opcheck(torch.ops.torchao.hqq_mixed_mm_mfma.default, (xt, packed, s, z, g, True), test_utils=_UTILS)
