@@ -59,6 +59,9 @@ _SIGNATURES = {
     "ao_amd_int4wo_swiglu": ([_p, _i64, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p], _int),
     "ao_amd_int4wo_rmsnorm_linear": ([_p, _i64, _i64, _i64, _p, ctypes.c_float, _p, _p, _i64, _i64, _p, _p, _int, _i64, _p], _int),
     "ao_amd_int4wo_rmsnorm_swiglu": ([_p, _i64, _i64, _i64, _p, ctypes.c_float, _p, _p, _p, _p, _i64, _i64, _p, _i64, _p], _int),
+    "ao_amd_int4wo_linear_ws_bytes": ([_i64, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_int64)], _int),
+    "ao_amd_int4wo_linear_ws_parts": ([_i64, _i64, _i64, _i64], _int),
+    "ao_amd_int4wo_linear_ws": ([_p, _i64, _i64, _i64, _p, _p, _i64, _i64, _p, _p, _int, _i64, _p, _i64, _p], _int),
     "ao_amd_int4wo_linear_partials": ([_p, _i64, _i64, _i64, _p, ctypes.c_float, _p, _p, _i64, _i64, _int, _p, _i64, _p], _int),
     "ao_amd_llama_decode_attention_split": ([_p, _p, _int, _p, _p, _p, _p, _int, _int, _int, _i64, _int, _p, _p, _p], _int),
     "ao_amd_llama_decode_attention_split_static": ([_p, _p, _int, _p, _p, _p, _p, _int, _int, _int, _i64, _int, _p, _p], _int),

@@ -927,15 +927,19 @@ __global__ __launch_bounds__(256 * KP) void int4wo_gemm_ksplit_kernel(const Line
     const int wave = __builtin_amdgcn_readfirstlane((threadIdx.x >> 6) & 3);
     const int r = lane & 15, qd = lane >> 4;
     const int KB = (int)(a.Kp / 128);
-    const int IT = (KB + KP - 1) / KP;  // iterations of every group
+    // K tiles of this workgroup: all of them, or the blockIdx.z-th run when K is also split across workgroups (fp32
+    // partial tiles at y + z * M * ldy, added by int4wo_ws_finish_kernel)
+    const int kb_lo = (int)blockIdx.z * a.kb_per_split;
+    const int kb_hi = kb_lo + a.kb_per_split < KB ? kb_lo + a.kb_per_split : KB;
+    const int IT = (kb_hi - kb_lo + KP - 1) / KP;  // iterations of every group
     const int64_t nblocks = (a.N + 15) / 16;
     const int64_t nb0 = (int64_t)blockIdx.x * 4 + wave;
     const bool has0 = nb0 < nblocks;
     const int64_t m0 = (int64_t)blockIdx.y * BM;
     const uint32_t magic = 0x43004300u, one_lo = 0x00003F80u, one_hi = 0x3F800000u;
     auto tile = [&](int i) __attribute__((always_inline)) {
-        const int kb = part + KP * i;
-        return kb < KB ? kb : KB - 1;
+        const int kb = kb_lo + part + KP * i;
+        return kb < kb_hi ? kb : kb_hi - 1;
     };
 
     const int xrow = tid >> 4, xchunk = tid & 15;
@@ -1001,16 +1005,16 @@ __global__ __launch_bounds__(256 * KP) void int4wo_gemm_ksplit_kernel(const Line
     for (int i = 0; i + 1 < IT; i += 2) {
         store_x(1);
         load_x(tile(i + 2));
-        if (part + KP * i < KB) compute(b0, 0);
+        if (kb_lo + part + KP * i < kb_hi) compute(b0, 0);
         load_w(b0, tile(i + 2));
         __syncthreads();
         store_x(0);
         load_x(tile(i + 3));
-        if (part + KP * (i + 1) < KB) compute(b1, 1);
+        if (kb_lo + part + KP * (i + 1) < kb_hi) compute(b1, 1);
         load_w(b1, tile(i + 3));
         __syncthreads();
     }
-    if ((IT & 1) && part + KP * (IT - 1) < KB) compute(b0, 0);
+    if ((IT & 1) && kb_lo + part + KP * (IT - 1) < kb_hi) compute(b0, 0);
 
     // partial sums of groups 1.. -> LDS -> group 0
     __syncthreads();
@@ -1040,10 +1044,37 @@ __global__ __launch_bounds__(256 * KP) void int4wo_gemm_ksplit_kernel(const Line
             const int64_t m = m0 + mb * 16 + 4 * qd + i;
             if (m < a.M) {
                 const float v = acc0[mb][i] + bv;
-                if (a.y_is_f32) ((float*)a.y)[m * a.ldy + n] = v;
+                if (a.y_is_f32) ((float*)a.y)[((int64_t)blockIdx.z * a.M + m) * a.ldy + n] = v;
                 else ((uint16_t*)a.y)[m * a.ldy + n] = f32_to_bf16_bits(v);
             }
         }
+}
+
+// sum of the fp32 partial outputs of a launch whose K range was split over workgroups, plus the bias, rounded once
+template <bool F32OUT>
+__global__ __launch_bounds__(256) void int4wo_ws_finish_kernel(const float* __restrict__ parts, int nparts, int64_t M, int64_t N,
+                                                               const uint16_t* __restrict__ bias, void* __restrict__ y,
+                                                               int64_t ldy) {
+    // N is a multiple of 4 here (the packed layout pads it to 16 and the partial rows are that wide)
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= M * N) return;
+    const int64_t m = i / N, n = i - m * N;
+    float4 v = *reinterpret_cast<const float4*>(parts + i);
+    for (int z = 1; z < nparts; ++z) {
+        const float4 p = *reinterpret_cast<const float4*>(parts + (int64_t)z * M * N + i);
+        v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+    }
+    if (bias) {
+        v.x += bf16_bits_to_f32(bias[n]); v.y += bf16_bits_to_f32(bias[n + 1]);
+        v.z += bf16_bits_to_f32(bias[n + 2]); v.w += bf16_bits_to_f32(bias[n + 3]);
+    }
+    if (F32OUT) {
+        float* o = (float*)y + m * ldy + n;
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    } else {
+        uint16_t* o = (uint16_t*)y + m * ldy + n;
+        o[0] = hw_bf16_bits(v.x); o[1] = hw_bf16_bits(v.y); o[2] = hw_bf16_bits(v.z); o[3] = hw_bf16_bits(v.w);
+    }
 }
 
 template <int G, int WAVES, int XMODE, bool DUAL>
@@ -1201,11 +1232,19 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
     // 32-33.5, the head at 33-64 rows 164-167 -> 115-145 (at 56-64 rows the tiles are as fast or faster on the others)
     const int64_t rb4_max_m = RB / 4 >= 1024 ? 64 : 48;
     const bool rb4_two_blocks = !rb4_off && M > 16 && M <= rb4_max_m && RB % 4 == 0 && RB / 4 >= 192 && a.K == a.Kp;
-    AO_REQUIRE(ksplit == 1 || (xmode == X_LDS && M <= 16 && !dual && !pair8 && !bias_bf16 && !residual_bf16 && y_dtype == AO_F32),
-               "partial sums over a split K need M <= 16, fp32 output, no bias / residual epilogue and activations that "
-               "fit the LDS staging (M=%lld K=%lld)", (long long)M, (long long)K);
-    if (M > 16 && aligned && !dual && !residual_bf16 && !norm_weight_bf16 && !gemm_starved && !rb4_two_blocks) {
-        {
+    // K split over workgroups from 17 rows on: the 32- and 64-row tiles whose K loop is already split over four groups of waves
+    // (and below that when the rows do not fit the LDS staging of the streaming kernel)
+    const bool ws_tiles = ksplit > 1 && (M > 16 || !(aligned && lds_ok));
+    AO_REQUIRE(ksplit == 1 || (!dual && !pair8 && !bias_bf16 && !residual_bf16 && y_dtype == AO_F32 &&
+                               (ws_tiles ? aligned && !norm_weight_bf16 : xmode == X_LDS)),
+               "partial sums over a split K need fp32 output, no bias / residual epilogue and, up to 16 rows, activations that "
+               "fit the LDS staging, beyond, K a multiple of max(128, group) and 16-byte aligned rows (M=%lld K=%lld)",
+               (long long)M, (long long)K);
+    AO_REQUIRE(ksplit == 1 || (int64_t)(ksplit - 1) * KB < KB_all, "K split %d leaves a part without K tiles (%lld tiles)", ksplit,
+               (long long)KB_all);
+    if ((M > 16 || ws_tiles) && aligned && !dual && !residual_bf16 && !norm_weight_bf16 &&
+        (ws_tiles || (!gemm_starved && !rb4_two_blocks))) {
+        if (!ws_tiles) {
             char name[96];
             if (int4wo_gemm_lds_plan(a, g, name, sizeof(name))) {
                 AO_PLAN("%s", name);
@@ -1217,15 +1256,16 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
         // 128 x 128 workgroup tiles when they fill a good part of the 256 CUs, else 64 x 64 tiles: four times
         // the workgroups, each dequantizing for 64 activation rows only
         // ... and 32 x 64 tiles when even those leave CUs idle
-        const bool big = ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
-        const bool tiny = !big && gemm_small_wgs < 192;
+        const bool big = !ws_tiles && ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
+        const bool tiny = ws_tiles ? M <= 32 : (!big && gemm_small_wgs < 192);
         dim3 ggrid(big ? (unsigned)((RB + 7) / 8) : (unsigned)((RB + 3) / 4),
-                   big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64));
+                   big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64),
+                   (unsigned)ksplit);
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
         // the small tiles split their K loop over 4 groups of waves: the 32-row tiles (at most one workgroup per CU) once
         // each group has 2 or more K tiles; the 64-row tiles (192 or more workgroups, which already overlap each other)
         // from 64 K tiles on (K = 14336, 512 rows: -4 %; K = 4096: +4 % and therefore not split)
-        const bool ksplit_tiles = !big && KB_all >= (tiny ? 8 : 64);
+        const bool ksplit_tiles = ws_tiles || (!big && KB_all >= (tiny ? 8 : 64));
         AO_PLAN("%s<%lld,%d,%d>", (!big && ksplit_tiles) ? "int4wo_gemm_ksplit_kernel" : "int4wo_gemm_kernel", (long long)g,
                 big ? 2 : (tiny && ksplit_tiles ? 2 : (tiny ? 1 : (ksplit_tiles ? 4 : 1))),
                 big ? 8 : (tiny && ksplit_tiles ? 4 : (tiny ? 2 : 4)));
@@ -1356,6 +1396,79 @@ extern "C" int ao_amd_int4wo_linear(const void* x_bf16, int64_t M, int64_t K, in
     return linear_dispatch(x_bf16, M, K, ldx, packed, qparams, nullptr, nullptr, N, g, bias_bf16, nullptr, 0, y, y_dtype,
                            ldy, stream);
 }
+
+// K split over workgroups through a caller's workspace: where it is used and how many parts.  The fp32 partial outputs
+// cost 8 bytes per output and part (written, then read by the finish kernel) and a second, small launch (about 3 us
+// with its gap), so the split is kept for grids of the 32- and 64-row tiles that leave most CUs idle.  Measured, group
+// size 64, us without / with the split (parts): 4096 x 14336 at 16 / 32 / 64 / 128 rows 19.6 / 17.0 (4), 34.7 / 17.9 (4),
+// 42.3 / 23.5 (4), 50.6 / 38.2 (2); 4096 x 4096 at 32 / 64 rows 12.3 / 10.2 (4), 14.7 / 13.4 (4), at 128 rows 16.6 / 17.8 (2:
+// not split); 6144 x 4096 at 16 / 32 rows 11.8 / 11.0 (2), 15.7 / 11.9 (2), at 64 rows 15.6 / 16.2 (not split); 1024 x 4096 at
+// 128 / 256 rows 14.1 / 11.6 (4), 14.8 / 13.5 (4), at 32 / 64 rows 7.1 / 8.5, 7.5 / 10.9 (not split: the streaming kernel serves
+// those); 14336 x 4096: slower at every row count (224 workgroups already).  Below 16 rows the streaming kernels win
+// everywhere (4096 x 14336 at 8 rows 14.3 / 16.6).
+static int ws_parts(int64_t M, int64_t K, int64_t N, int64_t g) {
+    int64_t Np, Kp;
+    if (ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return 1;
+    static const int forced = [] { const char* e = knob("AO_AMD_WS_PARTS"); return e ? atoi(e) : 0; }();
+    const int64_t KB = Kp / 128, RB = Np / 16;
+    int z = 1;
+    if (forced > 0) {
+        z = forced;
+    } else if (M >= 16 && M <= 256 && (RB >= 256 || M > 64)) {
+        const int64_t wgs = ((RB + 3) / 4) * (M <= 32 ? 1 : (M + 63) / 64);
+        // parts while the grid stays within the CUs, at least 8 K tiles (2 per group of waves) each
+        while (z < 4 && wgs * z * 2 <= 256 && KB / (z * 2) >= 8) z *= 2;
+        // short K: only the emptiest grids gain
+        if (KB < 64 && (M == 16 || wgs > (M <= 32 ? 96 : 64))) z = 1;
+    }
+    while (z > 1 && (int64_t)(z - 1) * ((KB + z - 1) / z) >= KB) --z;
+    if (z > KB) z = (int)KB;
+    return z < 1 ? 1 : z;
+}
+
+extern "C" int ao_amd_int4wo_linear_ws_bytes(int64_t M, int64_t K, int64_t N, int64_t g, int64_t* bytes) {
+    AO_REQUIRE(bytes, "null pointer argument");
+    int64_t Np, Kp;
+    if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
+    AO_REQUIRE(M >= 0, "negative batch");
+    const int z = ws_parts(M, K, N, g);
+    *bytes = z > 1 ? (int64_t)z * M * N * (int64_t)sizeof(float) : 0;
+    return 0;
+}
+
+extern "C" int ao_amd_int4wo_linear_ws(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed,
+                                       const void* qparams, int64_t N, int64_t g, const void* bias_bf16, void* y,
+                                       int y_dtype, int64_t ldy, void* workspace, int64_t workspace_bytes, void* stream) {
+    int64_t Np, Kp;
+    if (int rc = ao_amd_int4wo_packed_shape(N, K, g, &Np, &Kp, nullptr, nullptr)) return rc;
+    const bool aligned = (K == Kp) && ((ldx & 7) == 0) && ((((uintptr_t)x_bf16) & 15) == 0);
+    const int z = M > 0 && aligned && N % 4 == 0 ? ws_parts(M, K, N, g) : 1;
+    if (z <= 1)
+        return linear_dispatch(x_bf16, M, K, ldx, packed, qparams, nullptr, nullptr, N, g, bias_bf16, nullptr, 0, y, y_dtype,
+                               ldy, stream);
+    AO_REQUIRE(y && (y_dtype == AO_BF16 || y_dtype == AO_F32), "output must be bf16 or f32");
+    AO_REQUIRE(ldy >= N, "output row stride %lld smaller than N=%lld", (long long)ldy, (long long)N);
+    const int64_t need = (int64_t)z * M * N * (int64_t)sizeof(float);
+    AO_REQUIRE(workspace && workspace_bytes >= need && (((uintptr_t)workspace) & 15) == 0,
+               "16-byte aligned workspace of %lld bytes needed (ao_amd_int4wo_linear_ws_bytes), got %lld", (long long)need,
+               (long long)workspace_bytes);
+    if (int rc = linear_dispatch(x_bf16, M, K, ldx, packed, qparams, nullptr, nullptr, N, g, nullptr, nullptr, 0, workspace,
+                                 AO_F32, N, stream, nullptr, 0.f, false, z))
+        return rc;
+    const int64_t quads = M * N / 4;
+    const dim3 grid((unsigned)((quads + 255) / 256));
+    hipStream_t st = (hipStream_t)stream;
+    if (y_dtype == AO_F32)
+        hipLaunchKernelGGL(int4wo_ws_finish_kernel<true>, grid, dim3(256), 0, st, (const float*)workspace, z, M, N,
+                           (const uint16_t*)bias_bf16, y, ldy);
+    else
+        hipLaunchKernelGGL(int4wo_ws_finish_kernel<false>, grid, dim3(256), 0, st, (const float*)workspace, z, M, N,
+                           (const uint16_t*)bias_bf16, y, ldy);
+    AO_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ao_amd_int4wo_linear_ws_parts(int64_t M, int64_t K, int64_t N, int64_t g) { return ws_parts(M, K, N, g); }
 
 extern "C" int ao_amd_int4wo_linear_residual(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed,
                                              const void* qparams, int64_t N, int64_t g, const void* bias_bf16,

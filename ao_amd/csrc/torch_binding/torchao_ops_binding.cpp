@@ -175,9 +175,16 @@ at::Tensor int4wo_linear_hip(at::Tensor x, at::Tensor packed, at::Tensor qparams
     if (bias.has_value()) b = bias->contiguous();
     const int64_t M = x.size(0), K = x.size(1);
     auto y = at::empty({M, N}, x.options().dtype(fp32_out ? at::kFloat : at::kBFloat16));
-    TORCH_CHECK(ao_amd_int4wo_linear(x.data_ptr(), M, K, M > 0 ? x.stride(0) : K, packed.data_ptr(), qparams.data_ptr(), N, group_size,
-                                     b.defined() ? b.data_ptr() : nullptr, y.data_ptr(), fp32_out ? AO_F32 : AO_BF16, N,
-                                     at::hip::getCurrentHIPStream().stream()) == 0,
+    // shapes whose K range the library splits over workgroups bring a workspace from the caching allocator (0 bytes: the
+    // call is the plain linear)
+    int64_t ws_bytes = 0;
+    TORCH_CHECK(ao_amd_int4wo_linear_ws_bytes(M, K, N, group_size, &ws_bytes) == 0, ao_amd_last_error());
+    at::Tensor ws;
+    if (ws_bytes > 0) ws = at::empty({ws_bytes / 4}, x.options().dtype(at::kFloat));
+    TORCH_CHECK(ao_amd_int4wo_linear_ws(x.data_ptr(), M, K, M > 0 ? x.stride(0) : K, packed.data_ptr(), qparams.data_ptr(), N,
+                                        group_size, b.defined() ? b.data_ptr() : nullptr, y.data_ptr(),
+                                        fp32_out ? AO_F32 : AO_BF16, N, ws.defined() ? ws.data_ptr() : nullptr, ws_bytes,
+                                        at::hip::getCurrentHIPStream().stream()) == 0,
                 ao_amd_last_error());
     return y;
 }

@@ -199,6 +199,17 @@ def _linear_cuda(x: Tensor, packed: Tensor, qparams: Tensor, group_size: int, N:
         # definition of the result: dequantize, then F.linear.
         return torch.nn.functional.linear(x, _dequantize_cuda(packed, qparams, N, K, group_size), bias)
     y = torch.empty((M, N), dtype=torch.float32 if fp32_out else torch.bfloat16, device=x.device)
+    if 16 <= M <= 256:
+        # the row counts at which the library may split K over workgroups through a workspace (narrow weights, long K)
+        need = ctypes.c_int64(0)
+        check(lib().ao_amd_int4wo_linear_ws_bytes(M, K, N, group_size, ctypes.byref(need)))
+        if need.value:
+            ws = torch.empty((need.value // 4,), dtype=torch.float32, device=x.device)
+            check(lib().ao_amd_int4wo_linear_ws(x.data_ptr(), M, K, x.stride(0), packed.data_ptr(), qparams.data_ptr(), N,
+                                                group_size, None if bias is None else bias.data_ptr(), y.data_ptr(),
+                                                F32 if fp32_out else BF16, N, ws.data_ptr(), need.value,
+                                                current_stream(x.device)))
+            return y
     check(lib().ao_amd_int4wo_linear(x.data_ptr(), M, K, x.stride(0) if M > 0 else K, packed.data_ptr(),
                                      qparams.data_ptr(), N, group_size, None if bias is None else bias.data_ptr(),
                                      y.data_ptr(), F32 if fp32_out else BF16, N, current_stream(x.device)))

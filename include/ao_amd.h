@@ -144,6 +144,19 @@ int ao_amd_int4wo_rmsnorm_swiglu(const void* x_bf16, int64_t M, int64_t K, int64
 int ao_amd_int4wo_linear_plan(int64_t M, int64_t K, int64_t N, int64_t g, int aligned, int has_residual, int has_norm,
                               int dual, int pair8, int ksplit, int y_dtype, char* out, int64_t out_cap);
 
+/* ao_amd_int4wo_linear with a caller-owned workspace (device memory, 16-byte aligned): for batches of 2 to 256 rows on
+ * weights whose tiles leave most CUs idle (4096-row weights, long K), the K range is split over 2 to 8 groups of
+ * workgroups, fp32 partial outputs [parts][M][N] go to the workspace and a second small launch adds them, adds the bias
+ * and rounds once.  ao_amd_int4wo_linear_ws_bytes gives the size for a shape (0 where the split is not used: the call is
+ * then ao_amd_int4wo_linear itself and `workspace` may be NULL); ao_amd_int4wo_linear_ws_parts the number of parts.
+ * Same product as ao_amd_int4wo_linear (`aten::_weight_int4pack_mm`, torchao/dtypes/affine_quantized_tensor.py:600-640),
+ * summed in another order.  Calls that share a workspace must not overlap. */
+int ao_amd_int4wo_linear_ws_bytes(int64_t M, int64_t K, int64_t N, int64_t g, int64_t* bytes);
+int ao_amd_int4wo_linear_ws_parts(int64_t M, int64_t K, int64_t N, int64_t g);
+int ao_amd_int4wo_linear_ws(const void* x_bf16, int64_t M, int64_t K, int64_t ldx, const void* packed, const void* qparams,
+                            int64_t N, int64_t g, const void* bias_bf16, void* y, int y_dtype, int64_t ldy, void* workspace,
+                            int64_t workspace_bytes, void* stream);
+
 /* Linear with the K range split over `ksplit` (1..8) groups of workgroups, for weights whose row-block count does not fill
  * the CUs evenly (Llama-3-8B wqkv: 384 row blocks on 256 CUs): y_f32_parts[z][M][ldy] = sum over the z-th run of K tiles
  * of x' W^T in fp32, x' = x or its RMSNorm as in ao_amd_int4wo_rmsnorm_linear.  The consumer adds the parts and rounds
