@@ -2,7 +2,7 @@
 // step.  Standalone program (built by ao_amd/_build.py::build_ubench into ao_amd/lib/ao_amd_ceilings); not part of the
 // product library.  Every kernel here exits after a bounded number of iterations or polls.
 //
-//   ceilings [section ...]     sections: empty graph ifetch anyorder stream loop lds atomics barrier   (default: all)
+//   ceilings [section ...]     sections: empty graph ifetch anyorder stream l2read loop lds atomics barrier   (default: all)
 //
 // Each line printed is one measurement; "kernel_us" is the kernel's own begin-to-end time from the timestamps that
 // hipExtLaunchKernelGGL records (what rocprofv3 --kernel-trace reports as the kernel's duration).
@@ -290,6 +290,75 @@ static void section_stream() {
                wgs, copies, med, t[0], used / med * 1e-6, used / med * 1e-6 / 8.0);
         ++case_id;
     }
+    CK(hipFree(buf));
+    CK(hipFree(sink));
+}
+
+// ------------------------------------------------------------------------------------------------ L2 -> CU re-reads
+// What bounds a tile kernel whose workgroups all re-read the same activation slice (128 rows x 4096 x bf16 = 1 MiB)
+// from the L2: every workgroup (one per CU) reads the same 1 MiB buffer `passes` times, wave w taking the 1 KiB tiles
+// w, w + WAVES, ...; 4 requests in flight per wave; into registers (plain cached loads) or straight into LDS.
+template <int WAVES, bool TO_LDS>
+__global__ __launch_bounds__(WAVES * 64) void l2_reread_kernel(const char* base, int tiles, int passes, uint32_t* sink) {
+    __shared__ __align__(16) char lds[WAVES][4][1024];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    ao::u32x4_t acc = {0, 0, 0, 0};
+    const uint32_t off = lane * 16;
+    const int mine = (tiles - wave + WAVES - 1) / WAVES;   // tiles of this wave per pass
+    for (int ps = 0; ps < passes; ++ps) {
+        for (int t = 0; t + 4 <= mine; t += 4) {
+            if (TO_LDS) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t m0v = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)&lds[wave][j][0];
+                    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                                 :: "v"(off), "s"(base + (uint64_t)(wave + (t + j) * WAVES) * 1024), "s"(m0v) : "memory");
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            } else {
+                ao::u32x4_t r[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) r[j] = ao::asm_load_b128(base + (uint64_t)(wave + (t + j) * WAVES) * 1024, off);
+                asm volatile("s_waitcnt vmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) :: "memory");
+                acc ^= r[0] ^ r[1] ^ r[2] ^ r[3];
+            }
+        }
+    }
+    if (TO_LDS) acc.x = *reinterpret_cast<const uint32_t*>(&lds[wave][lane & 3][lane * 4]);
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u && tiles < 0) sink[0] = acc.x;
+}
+
+template <int WAVES, bool TO_LDS>
+static void l2_reread_case(const char* buf, uint32_t* sink) {
+    const int tiles = 1024, passes = 8;
+    std::vector<float> t;
+    for (int it = 0; it < 30; ++it) {
+        hipExtLaunchKernelGGL((l2_reread_kernel<WAVES, TO_LDS>), dim3(256), dim3(WAVES * 64), 0, 0, g_e0, g_e1, 0, buf, tiles, passes, sink);
+        CK(hipEventSynchronize(g_e1));
+        float ms;
+        CK(hipEventElapsedTime(&ms, g_e0, g_e1));
+        if (it >= 5) t.push_back(ms * 1e3f);
+    }
+    const float med = median(t);
+    const double per_cu = (double)tiles * 1024 * passes;   // bytes one workgroup reads
+    printf("l2_reread<%d,%s> 256 workgroups x %d waves, each re-reads 1 MiB x %d: kernel_us median %.2f  = %.1f B/ns per CU (%.1f B per "
+           "cycle at 2.4 GHz), %.1f TB/s over the chip\n", WAVES, TO_LDS ? "lds" : "regs", WAVES, passes, med, per_cu / med * 1e-3,
+           per_cu / med * 1e-3 / 2.4, per_cu * 256 / med * 1e-6);
+}
+
+static void section_l2read() {
+    char* buf;
+    uint32_t* sink;
+    CK(hipMalloc(&buf, 1 << 20));
+    CK(hipMalloc(&sink, 4));
+    CK(hipMemset(buf, 1, 1 << 20));
+    l2_reread_case<4, false>(buf, sink);
+    l2_reread_case<8, false>(buf, sink);
+    l2_reread_case<16, false>(buf, sink);
+    l2_reread_case<4, true>(buf, sink);
+    l2_reread_case<8, true>(buf, sink);
+    l2_reread_case<16, true>(buf, sink);
     CK(hipFree(buf));
     CK(hipFree(sink));
 }
@@ -623,6 +692,7 @@ int main(int argc, char** argv) {
     if (want("ifetch")) section_ifetch();
     if (want("anyorder")) section_anyorder();
     if (want("stream")) section_stream();
+    if (want("l2read")) section_l2read();
     if (want("loop")) section_loop();
     if (want("lds")) section_lds();
     if (want("atomics")) section_atomics();
