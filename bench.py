@@ -147,7 +147,7 @@ def roofline_leg(model, passes=3):
     achieved = total_bytes / total_us / 1e3  # GB/s
     return {
         "bound": "hbm",
-        "kernel": "ao::int4wo_gemv1_kernel (M=1, g=64)",
+        "kernel": "ao::int4wo_gemv1_kernel / int4wo_gemv2_kernel (M=1, g=64)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
