@@ -2,7 +2,7 @@
 // step.  Standalone program (built by ao_amd/_build.py::build_ubench into ao_amd/lib/ao_amd_ceilings); not part of the
 // product library.  Every kernel here exits after a bounded number of iterations or polls.
 //
-//   ceilings [section ...]     sections: empty graph ifetch anyorder stream l2read loop lds atomics barrier   (default: all)
+//   ceilings [section ...]     sections: empty graph ifetch anyorder stream l2read loop lds chain atomics barrier   (default: all)
 //
 // Each line printed is one measurement; "kernel_us" is the kernel's own begin-to-end time from the timestamps that
 // hipExtLaunchKernelGGL records (what rocprofv3 --kernel-trace reports as the kernel's duration).
@@ -645,6 +645,142 @@ static void section_barrier() {
     CK(hipFree(bad));
 }
 
+// ------------------------------------------------------------------------------------------------ dependent chain
+// What overlapping a kernel's own start-up with its predecessor's tail would buy: a chain of 64 dependent launches, each
+// a load-only pass over 29.4 MB (896 workgroups x 4 waves x 8 tiles) preceded by `pro` dependent VALU instructions per wave
+// (a stand-in for the 250-650 instructions a GEMV wave executes before its loop).  (a) one stream, stream order is the
+// dependency; (b) the launches alternate between two streams and every wave, after its first loads are requested and its
+// prologue is done, polls a counter that the predecessor's workgroups bump when they finish (agent-scope relaxed atomics,
+// bounded polling).  Both kernels of a pair fit the chip together (2 x 3584 waves of 8192), and a launch's successor on
+// the same stream cannot start before it ends, so at most two launches are resident and the predecessor always fits.
+constexpr int kChainSpin = 1 << 16;
+template <bool FLAGS>
+__global__ __launch_bounds__(256) void chain_kernel(const char* base, int tiles, int pro, const unsigned* done_prev, unsigned target,
+                                                    unsigned* done_mine, unsigned* err, uint32_t* sink) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const char* p = base + ((uint64_t)blockIdx.x * 4 + wave) * (uint64_t)tiles * 1024;
+    ao::u32x4_t acc = {0, 0, 0, 0};
+    ao::u32x4_t r[4];
+    const uint32_t off = lane * 16;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = ao::asm_load_b128_nt(p + (uint64_t)(j < tiles ? j : 0) * 1024, off);
+    uint32_t v = lane;
+    for (int i = 0; i < pro; ++i) asm volatile("v_mad_u32_u24 %0, %0, 3, 1" : "+v"(v));
+    if (FLAGS && done_prev) {
+        int spins = 0;
+        while (__builtin_amdgcn_readfirstlane(__hip_atomic_load(done_prev, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) < target) {
+            __builtin_amdgcn_s_sleep(1);
+            if (++spins > kChainSpin) {
+                __hip_atomic_store(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+        }
+    }
+    int t = 0;
+    for (; t + 4 <= tiles; t += 4) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            asm volatile("s_waitcnt vmcnt(3)" : "+v"(r[j]) : : "memory");
+            acc ^= r[j];
+            const int nx = t + 4 + j < tiles ? t + 4 + j : 0;
+            r[j] = ao::asm_load_b128_nt(p + (uint64_t)nx * 1024, off);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : : "memory");
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w ^ v) == 0x12345678u && tiles < 0) sink[0] = acc.x;
+    if (FLAGS) {
+        __syncthreads();
+        if (threadIdx.x == 0) __hip_atomic_fetch_add(done_mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+__global__ void chain_clear_kernel(unsigned* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+static void section_chain() {
+    const int NK = 64, NBUF = 8, tiles = 8, wgs = 896;
+    const size_t one = (size_t)wgs * 4 * tiles * 1024;
+    char* buf;
+    unsigned* flags;   // [NK] done counters, [NK] = error word
+    uint32_t* sink;
+    CK(hipMalloc(&buf, one * NBUF));
+    CK(hipMalloc(&flags, (NK + 1) * sizeof(unsigned)));
+    CK(hipMalloc(&sink, 4));
+    CK(hipMemset(buf, 1, one * NBUF));
+    hipStream_t s0, s1;
+    CK(hipStreamCreate(&s0));
+    CK(hipStreamCreate(&s1));
+    hipEvent_t e_begin, e_end, e_fork, e_join;
+    CK(hipEventCreate(&e_begin));
+    CK(hipEventCreate(&e_end));
+    CK(hipEventCreateWithFlags(&e_fork, hipEventDisableTiming));
+    CK(hipEventCreateWithFlags(&e_join, hipEventDisableTiming));
+    auto enqueue = [&](int mode, int pro) {
+        // mode 0: one stream, no flags; 1: one stream, flags; 2: two streams, flags
+        hipLaunchKernelGGL(chain_clear_kernel, dim3(1), dim3(128), 0, s0, flags, NK + 1);
+        if (mode == 2) {
+            CK(hipEventRecord(e_fork, s0));
+            CK(hipStreamWaitEvent(s1, e_fork, 0));
+        }
+        for (int k = 0; k < NK; ++k) {
+            hipStream_t st = mode == 2 && (k & 1) ? s1 : s0;
+            const char* b = buf + (size_t)(k % NBUF) * one;
+            const unsigned* prev = k > 0 ? flags + (k - 1) : nullptr;
+            if (mode == 0) hipLaunchKernelGGL(chain_kernel<false>, dim3(wgs), dim3(256), 0, st, b, tiles, pro, prev, (unsigned)wgs, flags + k, flags + NK, sink);
+            else hipLaunchKernelGGL(chain_kernel<true>, dim3(wgs), dim3(256), 0, st, b, tiles, pro, prev, (unsigned)wgs, flags + k, flags + NK, sink);
+        }
+        if (mode == 2) {
+            CK(hipEventRecord(e_join, s1));
+            CK(hipStreamWaitEvent(s0, e_join, 0));
+        }
+    };
+    const char* names[3] = {"one stream, stream order", "one stream, flags polled", "two streams, flags polled"};
+    for (int pro : {0, 300, 600}) {
+        for (int mode = 0; mode < 3; ++mode) {
+            for (int graph = 0; graph < 2; ++graph) {
+                hipGraph_t g = nullptr;
+                hipGraphExec_t ge = nullptr;
+                if (graph) {
+                    CK(hipStreamBeginCapture(s0, hipStreamCaptureModeGlobal));
+                    enqueue(mode, pro);
+                    CK(hipStreamEndCapture(s0, &g));
+                    CK(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
+                }
+                std::vector<float> t;
+                for (int it = 0; it < 12; ++it) {
+                    CK(hipEventRecord(e_begin, s0));
+                    if (graph) CK(hipGraphLaunch(ge, s0));
+                    else enqueue(mode, pro);
+                    CK(hipEventRecord(e_end, s0));
+                    CK(hipEventSynchronize(e_end));
+                    float ms;
+                    CK(hipEventElapsedTime(&ms, e_begin, e_end));
+                    if (it >= 2) t.push_back(ms * 1e3f / NK);
+                }
+                unsigned err = 0;
+                CK(hipMemcpy(&err, flags + NK, 4, hipMemcpyDeviceToHost));
+                const float med = median(t);
+                printf("chain of %d dependent 29.4 MB passes, %3d prologue instructions, %s%s: %.2f us per launch (min %.2f)%s\n", NK, pro,
+                       names[mode], graph ? ", as a graph" : "", med, t[0], err ? "  POLL LIMIT HIT" : "");
+                if (ge) CK(hipGraphExecDestroy(ge));
+                if (g) CK(hipGraphDestroy(g));
+            }
+        }
+    }
+    CK(hipStreamSynchronize(s1));
+    CK(hipEventDestroy(e_begin));
+    CK(hipEventDestroy(e_end));
+    CK(hipEventDestroy(e_fork));
+    CK(hipEventDestroy(e_join));
+    CK(hipStreamDestroy(s0));
+    CK(hipStreamDestroy(s1));
+    CK(hipFree(buf));
+    CK(hipFree(flags));
+    CK(hipFree(sink));
+}
+
 // ------------------------------------------------------------------------------------------------ atomics
 template <bool SAME>
 __global__ void atomics_kernel(unsigned* cnt, int iters) {
@@ -695,6 +831,7 @@ int main(int argc, char** argv) {
     if (want("l2read")) section_l2read();
     if (want("loop")) section_loop();
     if (want("lds")) section_lds();
+    if (want("chain")) section_chain();
     if (want("atomics")) section_atomics();
     if (want("barrier")) section_barrier();
     fflush(stdout);
