@@ -812,6 +812,7 @@ static void section_atomics() {
 }
 
 int main(int argc, char** argv) {
+    setvbuf(stdout, nullptr, _IOLBF, 0);   // every measurement line reaches a redirected log as it is printed
     CK(hipEventCreate(&g_e0));
     CK(hipEventCreate(&g_e1));
     auto want = [&](const char* s) {
