@@ -49,6 +49,9 @@ _SIGNATURES = {
     "ao_amd_fp6_native_bytes": ([_i64, _i64, _i64p], _int),
     "ao_amd_fp6_repack": ([_p, _i64, _i64, _int, _p, _p], _int),
     "ao_amd_fp6_linear": ([_p, _i64, _i64, _p, _p, _i64, _int, _int, _p, _p], _int),
+    "ao_amd_fp6_linear_ws_bytes": ([_i64, _i64, _i64, ctypes.POINTER(ctypes.c_int64)], _int),
+    "ao_amd_fp6_linear_ws_parts": ([_i64, _i64, _i64], _int),
+    "ao_amd_fp6_linear_ws": ([_p, _i64, _i64, _p, _p, _i64, _int, _int, _p, _p, _i64, _p], _int),
     "ao_amd_fp6_rmsnorm_linear": ([_p, _i64, _i64, _p, ctypes.c_float, _p, _p, _i64, _int, _int, _p, _p], _int),
     "ao_amd_fp6_swiglu": ([_p, _i64, _i64, _p, ctypes.c_float, _p, _p, _p, _p, _i64, _int, _int, _p, _p], _int),
     "ao_amd_fp6_native_to_f16": ([_p, _p, _i64, _i64, _int, _int, _p, _p], _int),

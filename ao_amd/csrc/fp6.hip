@@ -1096,7 +1096,10 @@ template <bool E3M2, int NBW, int MBLK, int PF, int XD>
 __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
                                                            const uint32_t* __restrict__ native,
                                                            const uint16_t* __restrict__ scale, int64_t N,
-                                                           uint16_t* __restrict__ out) {
+                                                           uint16_t* __restrict__ out, int kb_per_part,
+                                                           float* __restrict__ parts) {
+    // parts != null: blockIdx.z takes the z-th run of kb_per_part K tiles and stores its fp32 partial tile at
+    // parts + (z * M + m) * N + n (fp6_ws_finish_kernel adds the runs and rounds once)
     typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
     typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
     constexpr int BM = 16 * MBLK, XSTRIDE = 136;  // fp16 elements per LDS row
@@ -1105,7 +1108,9 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, qd = lane >> 4;
-    const int KB = (int)(K / 128);
+    const int KB_row = (int)(K / 128);   // K tiles of a row block (the stride between row blocks)
+    const int kb_lo = parts ? (int)blockIdx.z * kb_per_part : 0;
+    const int KB = parts ? (KB_row - kb_lo < kb_per_part ? KB_row - kb_lo : kb_per_part) : KB_row;   // tiles of this workgroup
     const int64_t nblocks = N / 16;
     const int64_t nb0 = (int64_t)blockIdx.x * (4 * NBW) + NBW * wave;
     const bool has0 = nb0 < nblocks, has1 = NBW > 1 && nb0 + 1 < nblocks;
@@ -1116,7 +1121,7 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
 #pragma unroll
     for (int j = 0; j < XCH; ++j) {
         const int64_t m = m0 + xrow + 16 * j;
-        xrow_ptr[j] = x + (m < M ? m : M - 1) * K + xchunk * 8;
+        xrow_ptr[j] = x + (m < M ? m : M - 1) * K + xchunk * 8 + (int64_t)kb_lo * 128;
     }
     static_assert(PF >= 2 && PF % 2 == 0, "the ring of prefetched tiles alternates between the two LDS buffers");
     static_assert(PF % XD == 0, "a round of the weight ring is a whole number of rounds of the activation ring");
@@ -1133,8 +1138,8 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
 
     // the 24 bytes of a lane per tile, joined into the conversion's operand right at the load
     struct WBuf { u32x6_t w0, w1; };
-    const uint32_t* t0 = native + (has0 ? nb0 : 0) * KB * 384;
-    const uint32_t* t1 = native + (has1 ? nb0 + 1 : 0) * KB * 384;
+    const uint32_t* t0 = native + ((has0 ? nb0 : 0) * KB_row + kb_lo) * 384;
+    const uint32_t* t1 = native + ((has1 ? nb0 + 1 : 0) * KB_row + kb_lo) * 384;
     auto load_w6 = [&](const uint32_t* t) __attribute__((always_inline)) {
         const u32x4_t lo = reinterpret_cast<const u32x4_t*>(t)[lane];
         const u32x2_t hi = reinterpret_cast<const u32x2_t*>(t + 256)[lane];
@@ -1230,9 +1235,29 @@ __global__ __launch_bounds__(256, 2) void fp6_gemm_kernel(const uint16_t* __rest
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int64_t m = m0 + mb * 16 + 4 * qd + i;
-                if (m < M) out[m * N + n] = f32_to_f16_bits(h == 0 ? acc0[mb][i] : acc1[mb][i]);
+                if (m < M) {
+                    const float v = h == 0 ? acc0[mb][i] : acc1[mb][i];
+                    if (parts) parts[((int64_t)blockIdx.z * M + m) * N + n] = v;
+                    else out[m * N + n] = f32_to_f16_bits(v);
+                }
             }
     }
+}
+
+// sum of the fp32 partial outputs of a launch whose K range was split over workgroups, rounded once to fp16
+__global__ __launch_bounds__(256) void fp6_ws_finish_kernel(const float* __restrict__ parts, int nparts, int64_t MN,
+                                                            uint16_t* __restrict__ out) {
+    // M * N is a multiple of 4 (N is a multiple of 16)
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= MN) return;
+    float4 v = *reinterpret_cast<const float4*>(parts + i);
+    for (int z = 1; z < nparts; ++z) {
+        const float4 p = *reinterpret_cast<const float4*>(parts + (int64_t)z * MN + i);
+        v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+    }
+    const uint32_t lo = (uint32_t)f32_to_f16_bits(v.x) | ((uint32_t)f32_to_f16_bits(v.y) << 16);
+    const uint32_t hi = (uint32_t)f32_to_f16_bits(v.z) | ((uint32_t)f32_to_f16_bits(v.w) << 16);
+    *reinterpret_cast<uint2*>(out + i) = uint2{lo, hi};
 }
 
 static int check_fp6_format(int ebits, int mbits) {
@@ -1390,7 +1415,7 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
                                int64_t N, int ebits, int mbits, const void* residual_f16, const void* gate_f16,
                                void* out_f16, void* stream, const void* norm_weight_f16 = nullptr, float norm_eps = 0.f,
                                const void* native_up = nullptr, const void* scale_up_f16 = nullptr, char* plan_out = nullptr,
-                               size_t plan_cap = 0) {
+                               size_t plan_cap = 0, int ws_parts = 1, float* ws = nullptr) {
     // plan_out: do not launch; write the name of the kernel instantiation the arguments select (ao_amd_fp6_linear_plan)
 #define AO_PLAN(...)                                    \
     if (plan_out) {                                     \
@@ -1425,6 +1450,8 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
     // few rows: staged in LDS (at most 64 KB, and no more per wave than keeps several workgroups on a CU); worth the
     // pass over the rows and the barrier once a wave has 4 or more K tiles to stream
     const bool need_lds = norm_weight_f16 || native_up;
+    // K split over workgroups through a caller's workspace (ao_amd_fp6_linear_ws): the 32- and 64-row tiles, any row count
+    const bool ws_tiles = ws_parts > 1;
     const int64_t xbytes = (M < 16 ? M : 16) * Kp * 2;
     if (need_lds)
         while (waves < 16 && xbytes > (int64_t)waves * 16 * 1024) waves *= 2;
@@ -1445,7 +1472,7 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
     // (us staged / not: 4096 x 4096 at 4 / 6 / 8 rows 5.9 / 5.4, 6.1 / 5.4, 6.5 / 5.7; 6144 x 4096 7.5 / 6.5, 7.9 / 6.8,
     // 8.2 / 7.2; 4096 x 14336 at 4 rows 12.1 / 11.4; at 2 rows staged wins everywhere: 14336 x 4096 9.6 / 11.7)
     const bool stage_pays = M <= 2 || (M == 3 && RB >= 768);
-    if (fits && !shared_tiles && (need_lds || (KB >= 4 * waves && stage_pays))) {
+    if (!ws_tiles && fits && !shared_tiles && (need_lds || (KB >= 4 * waves && stage_pays))) {
         AO_PLAN("fp6_gemv_kernel<%d,%d,%d>", waves, ebits == 3 ? 1 : 0, native_up ? 1 : 0);
         Fp6GemvArgs a{xx, M, K, Kp, nat, sc, N, o, res, gt, (const uint16_t*)norm_weight_f16, norm_eps,
                       (const uint32_t*)native_up, (const uint16_t*)scale_up_f16};
@@ -1459,7 +1486,7 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
         AO_LAUNCH_CHECK();
         return 0;
     }
-    if (M > 16 && M <= 32 && K % 128 == 0 && !res && !gt && RB % 4 == 0 && RB / 4 >= 192) {
+    if (!ws_tiles && M > 16 && M <= 32 && K % 128 == 0 && !res && !gt && RB % 4 == 0 && RB / 4 >= 192) {
         // 17 to 32 rows on a weight with 768 or more row blocks: the streaming kernel with four row blocks and two
         // activation blocks per workgroup (14336 x 4096: 11.3-13.4 us against 18 us of the tiled kernel, the head 82-97
         // against 145; four activation blocks for 33 to 64 rows spill and measured slower than the tiles)
@@ -1478,24 +1505,35 @@ static int fp6_linear_dispatch(const void* x_f16, int64_t M, int64_t K, const vo
             return 0;
         }
     }
-    if (M > 16 && K % 128 == 0 && !res && !gt) {
+    AO_REQUIRE(!ws_tiles || (ws && K % 128 == 0 && !res && !gt && !need_lds && (int64_t)(ws_parts - 1) * ((KB + ws_parts - 1) / ws_parts) < KB),
+               "a split K needs a workspace, K a multiple of 128, no fused epilogue and a part count that leaves no part empty "
+               "(K=%lld, parts=%d)", (long long)K, ws_parts);
+    if ((M > 16 || ws_tiles) && K % 128 == 0 && !res && !gt) {
         // ... and 32 x 64 tiles when even those leave CUs idle
-        const bool big = ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
-        const bool tiny = !big && ((RB + 3) / 4) * ((M + 63) / 64) < 192;
+        const bool big = !ws_tiles && ((RB + 7) / 8) * ((M + 127) / 128) >= 256;
+        const bool tiny = ws_tiles ? M <= 32 : (!big && ((RB + 3) / 4) * ((M + 63) / 64) < 192);
         dim3 ggrid(big ? (unsigned)((RB + 7) / 8) : (unsigned)((RB + 3) / 4),
-                   big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64));
+                   big ? (unsigned)((M + 127) / 128) : tiny ? (unsigned)((M + 31) / 32) : (unsigned)((M + 63) / 64),
+                   (unsigned)ws_parts);
         AO_REQUIRE(ggrid.y <= 65535, "batch too large for one launch: M=%lld", (long long)M);
         AO_PLAN("fp6_gemm_kernel<%d,%s>", ebits == 3 ? 1 : 0, big ? "2,8,2,1" : (tiny ? "1,2,8,8" : "1,4,4,4"));
+        const int kbp = (int)((KB + ws_parts - 1) / ws_parts);
+        float* parts = ws_tiles ? ws : nullptr;
         if (ebits == 3) {
-            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 2, 8, 2, 1>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
-            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 2, 8, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
-            else hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 4, 4, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 2, 8, 2, 1>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o, kbp, parts);
+            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 2, 8, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o, kbp, parts);
+            else hipExtLaunchKernelGGL((fp6_gemm_kernel<true, 1, 4, 4, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o, kbp, parts);
         } else {
-            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 2, 8, 2, 1>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
-            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 2, 8, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
-            else hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 4, 4, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o);
+            if (big) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 2, 8, 2, 1>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o, kbp, parts);
+            else if (tiny) hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 2, 8, 8>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o, kbp, parts);
+            else hipExtLaunchKernelGGL((fp6_gemm_kernel<false, 1, 4, 4, 4>), ggrid, dim3(256), 0, st, ev0, ev1, 0, xx, M, K, nat, sc, N, o, kbp, parts);
         }
         AO_LAUNCH_CHECK();
+        if (ws_tiles) {
+            const int64_t MN = M * N;
+            hipLaunchKernelGGL(fp6_ws_finish_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, st, ws, ws_parts, MN, o);
+            AO_LAUNCH_CHECK();
+        }
         return 0;
     }
 #define AO_FP6_LAUNCH(W, R)                                                                                              \
@@ -1546,6 +1584,55 @@ extern "C" int ao_amd_fp6_linear_plan(int64_t M, int64_t K, int64_t N, int ebits
 extern "C" int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native,
                                  const void* scale_f16, int64_t N, int ebits, int mbits, void* out_f16, void* stream) {
     return fp6_linear_dispatch(x_f16, M, K, weights_native, scale_f16, N, ebits, mbits, nullptr, nullptr, out_f16, stream);
+}
+
+// K split over workgroups through a caller's workspace: where it is used and how many parts.  The reference's operator
+// has the same device (`splitK`, a [splitK, M, N] fp32 workspace and SplitK_Reduction, torchao/csrc/cuda/fp6_llm/
+// fp6_linear.cu:104-111, 167-168) chosen by the caller; here the library chooses.  Measured, e3m2, us without / with the
+// split (parts): 4096 x 14336 at 16 / 32 / 64 / 128 rows 17.9 / 15.5 (4), 33.2 / 16.2 (4), 34.5 / 21.4 (4), 38.0 / 34.5 (2);
+// 4096 x 4096 at 32 / 64 rows 11.9 / 9.0 (4), 12.5 / 11.7 (4), at 128 rows 13.5 / 15.3 (not split); 6144 x 4096 at 32 rows
+// 12.4 / 10.6 (2), at 64 rows 13.0 / 14.3 (not split); 1024 x 4096 at 32 / 64 / 128 / 256 rows 11.5 / 7.8, 11.6 / 9.7, 12.1 / 10.3,
+// 12.5 / 11.8 (4); 14336 x 4096: slower at every row count; at 16 rows only the long K gains (4096 x 4096: 6.6 / 8.1).
+static int fp6_ws_parts(int64_t M, int64_t K, int64_t N) {
+    if (K % 128 != 0 || N % 16 != 0 || M < 1) return 1;
+    static const int forced = [] { const char* e = knob("AO_AMD_WS_PARTS"); return e ? atoi(e) : 0; }();
+    const int64_t KB = K / 128, RB = N / 16;
+    int z = 1;
+    if (forced > 0) {
+        z = forced;
+    } else if (M >= 16 && M <= 256) {
+        const int64_t wgs = ((RB + 3) / 4) * (M <= 32 ? 1 : (M + 63) / 64);
+        // parts while the grid stays within the CUs, at least 8 K tiles each
+        while (z < 4 && wgs * z * 2 <= 256 && KB / (z * 2) >= 8) z *= 2;
+        // short K: only the emptiest grids gain
+        if (KB < 64 && (M == 16 || wgs > (M <= 32 ? 96 : 64))) z = 1;
+    }
+    while (z > 1 && (int64_t)(z - 1) * ((KB + z - 1) / z) >= KB) --z;
+    return z < 1 ? 1 : z;
+}
+
+extern "C" int ao_amd_fp6_linear_ws_bytes(int64_t M, int64_t K, int64_t N, int64_t* bytes) {
+    AO_REQUIRE(bytes, "null pointer argument");
+    AO_REQUIRE(M >= 0 && K > 0 && N > 0, "need M >= 0 and positive K, N");
+    const int z = fp6_ws_parts(M, K, N);
+    *bytes = z > 1 ? (int64_t)z * M * N * (int64_t)sizeof(float) : 0;
+    return 0;
+}
+
+extern "C" int ao_amd_fp6_linear_ws_parts(int64_t M, int64_t K, int64_t N) { return fp6_ws_parts(M, K, N); }
+
+extern "C" int ao_amd_fp6_linear_ws(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
+                                    int64_t N, int ebits, int mbits, void* out_f16, void* workspace, int64_t workspace_bytes,
+                                    void* stream) {
+    const int z = fp6_ws_parts(M, K, N);
+    if (z <= 1)
+        return fp6_linear_dispatch(x_f16, M, K, weights_native, scale_f16, N, ebits, mbits, nullptr, nullptr, out_f16, stream);
+    const int64_t need = (int64_t)z * M * N * (int64_t)sizeof(float);
+    AO_REQUIRE(workspace && workspace_bytes >= need && (((uintptr_t)workspace) & 15) == 0,
+               "16-byte aligned workspace of %lld bytes needed (ao_amd_fp6_linear_ws_bytes), got %lld", (long long)need,
+               (long long)workspace_bytes);
+    return fp6_linear_dispatch(x_f16, M, K, weights_native, scale_f16, N, ebits, mbits, nullptr, nullptr, out_f16, stream, nullptr,
+                               0.f, nullptr, nullptr, nullptr, 0, z, (float*)workspace);
 }
 
 extern "C" int ao_amd_fp6_linear_fused(const void* x_f16, int64_t M, int64_t K, const void* weights_native,

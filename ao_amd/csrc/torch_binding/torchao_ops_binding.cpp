@@ -93,8 +93,14 @@ at::Tensor quant_llm_linear_hip(int64_t EXPONENT, int64_t MANTISSA, at::Tensor _
     auto stream = at::hip::getCurrentHIPStream().stream();
     auto native = native_weight(_weights, N, K, (int)(1 + EXPONENT + MANTISSA), stream);
     auto out = at::empty({M, N}, x.options());
-    TORCH_CHECK(ao_amd_fp6_linear(x.data_ptr(), M, K, native.data_ptr(), scales.data_ptr(), N, (int)EXPONENT, (int)MANTISSA,
-                                  out.data_ptr(), stream) == 0,
+    // where the reference's caller passes splitK and the operator allocates [splitK, M, N] floats (fp6_linear.cu:167), the
+    // library says whether it splits K for this shape and how much workspace that takes (0: plain call)
+    int64_t ws_bytes = 0;
+    TORCH_CHECK(ao_amd_fp6_linear_ws_bytes(M, K, N, &ws_bytes) == 0, ao_amd_last_error());
+    at::Tensor ws;
+    if (ws_bytes > 0) ws = at::empty({ws_bytes / 4}, x.options().dtype(at::kFloat));
+    TORCH_CHECK(ao_amd_fp6_linear_ws(x.data_ptr(), M, K, native.data_ptr(), scales.data_ptr(), N, (int)EXPONENT, (int)MANTISSA,
+                                     out.data_ptr(), ws.defined() ? ws.data_ptr() : nullptr, ws_bytes, stream) == 0,
                 ao_amd_last_error());
     return out;
 }

@@ -711,6 +711,17 @@ def _fp6_linear_native_cuda(ebits, mbits, x, native, scale):
                                              w16.data_ptr(), current_stream(x.device)))
         return torch.nn.functional.linear(x, w16)
     out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    if 16 <= M <= 256:
+        # the row counts at which the library may split K over workgroups through a workspace, as the reference's
+        # operator does with its `splitK` argument (here the library picks the part count)
+        need = ctypes.c_int64(0)
+        check(lib().ao_amd_fp6_linear_ws_bytes(M, K, N, ctypes.byref(need)))
+        if need.value:
+            ws = torch.empty((need.value // 4,), dtype=torch.float32, device=x.device)
+            check(lib().ao_amd_fp6_linear_ws(x.contiguous().data_ptr(), M, K, native.data_ptr(), scale.contiguous().data_ptr(),
+                                             N, ebits, mbits, out.data_ptr(), ws.data_ptr(), need.value,
+                                             current_stream(x.device)))
+            return out
     check(lib().ao_amd_fp6_linear(x.contiguous().data_ptr(), M, K, native.data_ptr(), scale.contiguous().data_ptr(), N,
                                   ebits, mbits, out.data_ptr(), current_stream(x.device)))
     return out

@@ -362,6 +362,20 @@ int ao_amd_fp6_repack(const void* tc, int64_t N, int64_t K, int nbits, void* nat
 int ao_amd_fp6_linear(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16,
                       int64_t N, int ebits, int mbits, void* out_f16, void* stream);
 
+/* ao_amd_fp6_linear with a caller-owned workspace (device memory, 16-byte aligned): for batches of 16 to 256 rows on
+ * weights whose 32- / 64-row tiles leave most CUs idle (4096-row weights), the K range is split over 2 or 4 groups of
+ * workgroups, fp32 partial outputs [parts][M][N] go to the workspace and a second small launch adds them and rounds once
+ * to fp16.  ao_amd_fp6_linear_ws_bytes gives the size for a shape (0 where the split is not used: the call is then
+ * ao_amd_fp6_linear itself and `workspace` may be NULL); ao_amd_fp6_linear_ws_parts the number of parts.  Same product as
+ * torchao::quant_llm_linear (torchao/csrc/cuda/fp6_llm/fp6_linear.cu:139-200); it stands where the reference's operator
+ * takes `splitK` and allocates its [splitK, M, N] fp32 reduction workspace (fp6_linear.cu:104-111, 167-168,
+ * SplitK_Reduction in kernel_reduction.cuh:44), with the part count chosen by the library instead of the caller.
+ * Calls that share a workspace must not overlap. */
+int ao_amd_fp6_linear_ws_bytes(int64_t M, int64_t K, int64_t N, int64_t* bytes);
+int ao_amd_fp6_linear_ws_parts(int64_t M, int64_t K, int64_t N);
+int ao_amd_fp6_linear_ws(const void* x_f16, int64_t M, int64_t K, const void* weights_native, const void* scale_f16, int64_t N,
+                         int ebits, int mbits, void* out_f16, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Which kernel instantiation the FPx linear entry points run for a problem, without launching anything: writes a name
  * such as "fp6_gemm_kernel<1,1,4,4,4>" (e3m2 flag, then the tile variant) or "fp6_gemv_kernel<8,1,0>" to `out`.  The
  * flags say which fused variant is meant (RMSNorm on the activations, residual / gate epilogue, two weights).  The test

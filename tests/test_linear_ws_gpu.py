@@ -107,3 +107,66 @@ def test_workspace_linear_refusals_and_fallbacks():
     # the operator takes the same route: same bits as the C call with a workspace
     rc, y_ws, _ = _ws_call(x, packed, qp, N, g, None, False)
     assert rc == 0 and bool(torch.equal(ops.int4wo_linear(x, packed, qp, g, N), y_ws))
+
+
+# (N, K, M, parts the rule gives) for ao_amd_fp6_linear_ws
+FP6_CASES = [
+    (4096, 14336, 16, 4), (4096, 14336, 32, 4), (4096, 14336, 64, 4), (4096, 14336, 100, 2), (4096, 14336, 256, 1),
+    (4096, 4096, 32, 4), (4096, 4096, 64, 4), (4096, 4096, 128, 1), (4096, 4096, 16, 1),
+    (6144, 4096, 32, 2), (6144, 4096, 64, 1), (1024, 4096, 40, 4), (1024, 4096, 256, 4), (14336, 4096, 32, 1),
+    (4096, 8192 + 64, 32, 1),
+]
+
+
+@pytest.mark.parametrize("ebits,mbits", [(3, 2), (2, 3)])
+@pytest.mark.parametrize("N,K,M,parts", FP6_CASES)
+def test_fp6_workspace_linear(N, K, M, parts, ebits, mbits):
+    """ao_amd_fp6_linear_ws (where torchao::quant_llm_linear takes splitK and a [splitK, M, N] workspace,
+    torchao/csrc/cuda/fp6_llm/fp6_linear.cu:104-111, 167-168): <= 1e-3 relative L2 of the fp32 product with the dequantized
+    weight rounded to fp16, one-hot rows bit for bit, and against the plain entry point.  K = 8256 is not a multiple of
+    128: no split."""
+    from ao_amd import _lib, ops
+    print(f"case fp6_linear_ws N={N} K={K} M={M} parts={parts} e{ebits}m{mbits}", flush=True)
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    assert L.ao_amd_fp6_linear_ws_parts(M, K, N) == parts
+    gen = torch.Generator().manual_seed(N + K + M)
+    w = (torch.randn(N, K, generator=gen) * 0.05).half().to(dev)
+    tc, scale = ops.fp6_quantize_pack(w, ebits, mbits)
+    native = ops.fp6_repack(tc, 1 + ebits + mbits)
+    wd = ops.fp6_dequantize(tc, scale, ebits, mbits).half()      # the kernels multiply fp16(value * scale)
+    x = torch.randn(M, K, generator=gen).half().to(dev)
+    st = torch.cuda.current_stream().cuda_stream
+
+    def run(xin):
+        need = ctypes.c_int64(-1)
+        _lib.check(L.ao_amd_fp6_linear_ws_bytes(M, K, N, ctypes.byref(need)))
+        assert need.value == (parts * M * N * 4 if parts > 1 else 0)
+        ws = torch.empty(max(need.value // 4, 1), dtype=torch.float32, device=dev)
+        y = torch.empty(M, N, dtype=torch.float16, device=dev)
+        _lib.check(L.ao_amd_fp6_linear_ws(xin.data_ptr(), M, K, native.data_ptr(), scale.data_ptr(), N, ebits, mbits, y.data_ptr(),
+                                          ws.data_ptr() if need.value else None, need.value, st))
+        return y
+
+    y = run(x)
+    ref = (x.float() @ wd.float().t()).half().float()
+    err = float((y.float() - ref).norm() / ref.norm())
+    assert err <= 1e-3, err
+    y0 = torch.empty_like(y)
+    _lib.check(L.ao_amd_fp6_linear(x.data_ptr(), M, K, native.data_ptr(), scale.data_ptr(), N, ebits, mbits, y0.data_ptr(), st))
+    if parts == 1:
+        same = bool(torch.equal(y, y0))
+        assert same
+    else:
+        d = float((y.float() - y0.float()).norm() / y0.float().norm())
+        assert d <= 1e-3, d
+        # the operator takes the same route
+        same = bool(torch.equal(ops.fp6_linear_native(ebits, mbits, x, native, scale), y))
+        assert same
+    ks = torch.randint(0, K, (M,), generator=gen)
+    ks[0], ks[-1] = 0, K - 1
+    xh = torch.zeros(M, K, dtype=torch.float16)
+    xh[torch.arange(M), ks] = 1.0
+    yh = run(xh.to(dev))
+    exact = bool(torch.equal(yh, wd[:, ks.to(dev)].t().contiguous()))
+    assert exact
