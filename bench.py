@@ -357,6 +357,31 @@ def _time_linear(L, launch, iters, armed=True):
     return durs[len(durs) // 2]
 
 
+def replayed_us(fn, n, reps):
+    """Device time per call of fn(0) .. fn(n - 1) from a replayed HIP graph of the n calls (no host dispatch in the figure)."""
+    import torch
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(n):
+                fn(i)
+    for _ in range(2):
+        graph.replay()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        graph.replay()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / (reps * n)
+
+
 def sweep(kind, iters=100):
     """Per-kernel lines for the shapes of the other benchmark configurations: int4 GEMV (M in 1, 4; g in 64, 128),
     int4 GEMM (M in 16 .. 2048, g=64), the FP6 e3m2 linear (M in 1, 16, 128, 512) and the int8 weight-only linear
@@ -469,6 +494,64 @@ def sweep(kind, iters=100):
                                   "GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
                                   "TFLOPs": round(tfs, 2), "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
             del wq
+    elif kind == "ws":
+        # The linears with a caller-owned workspace beside the plain entry points on the shapes where the library splits K
+        # over workgroups (two launches: tiles + finish), both from replayed HIP graphs over rotating weight copies.
+        def stream():
+            return torch.cuda.current_stream().cuda_stream
+
+        for N, K in [(4096, 4096), (6144, 4096), (4096, 14336), (1024, 4096)]:
+            g = 64
+            _, _, pb, qb = _lib.packed_shape(N, K, g)
+            w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).bfloat16()
+            copies = max(2, -(-SWEEP_ROTATE_BYTES // pb))
+            packed = torch.empty(copies, pb // 4, dtype=torch.int32, device=dev)
+            qp = torch.empty(copies, qb // 4, dtype=torch.int32, device=dev)
+            _lib.check(L.ao_amd_int4wo_quantize_pack(w.data_ptr(), N, K, K, g, packed.data_ptr(), qp.data_ptr(), st))
+            packed[1:] = packed[0]
+            qp[1:] = qp[0]
+            wh = w.half()
+            tc = torch.empty(N * K * 3 // 4, dtype=torch.uint8, device=dev)
+            sc = torch.empty(N, dtype=torch.float16, device=dev)
+            _lib.check(L.ao_amd_fp6_quantize_pack(wh.data_ptr(), _lib.F16, N, K, 3, 2, tc.data_ptr(), sc.data_ptr(), st))
+            nbytes = ctypes.c_int64()
+            _lib.check(L.ao_amd_fp6_native_bytes(N, K, ctypes.byref(nbytes)))
+            copies6 = max(2, -(-SWEEP_ROTATE_BYTES // nbytes.value))
+            native = torch.empty(copies6, nbytes.value, dtype=torch.uint8, device=dev)
+            _lib.check(L.ao_amd_fp6_repack(tc.data_ptr(), N, K, 6, native.data_ptr(), st))
+            native[1:] = native[0]
+            for M in (16, 32, 64, 128):
+                x = torch.randn(M, K, device=dev, generator=gen).bfloat16()
+                y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+                parts = L.ao_amd_int4wo_linear_ws_parts(M, K, N, g)
+                if parts > 1:
+                    ws = torch.empty(parts * M * N, dtype=torch.float32, device=dev)
+                    plain = replayed_us(lambda i: _lib.check(L.ao_amd_int4wo_linear(
+                        x.data_ptr(), M, K, K, packed[i % copies].data_ptr(), qp[i % copies].data_ptr(), N, g, None, y.data_ptr(),
+                        _lib.BF16, N, stream())), copies, 4)
+                    split = replayed_us(lambda i: _lib.check(L.ao_amd_int4wo_linear_ws(
+                        x.data_ptr(), M, K, K, packed[i % copies].data_ptr(), qp[i % copies].data_ptr(), N, g, None, y.data_ptr(),
+                        _lib.BF16, N, ws.data_ptr(), ws.numel() * 4, stream())), copies, 4)
+                    tfs = 2.0 * M * N * K / split / 1e6
+                    print(json.dumps({"kernel": "int4wo_linear_ws", "N": N, "K": K, "M": M, "group": g, "parts": parts,
+                                      "us": round(split, 2), "us_plain": round(plain, 2), "TFLOPs": round(tfs, 2),
+                                      "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
+                parts6 = L.ao_amd_fp6_linear_ws_parts(M, K, N)
+                if parts6 > 1:
+                    xh = x.half()
+                    yh = torch.empty(M, N, dtype=torch.float16, device=dev)
+                    ws = torch.empty(parts6 * M * N, dtype=torch.float32, device=dev)
+                    plain = replayed_us(lambda i: _lib.check(L.ao_amd_fp6_linear(
+                        xh.data_ptr(), M, K, native[i % copies6].data_ptr(), sc.data_ptr(), N, 3, 2, yh.data_ptr(), stream())),
+                        copies6, 4)
+                    split = replayed_us(lambda i: _lib.check(L.ao_amd_fp6_linear_ws(
+                        xh.data_ptr(), M, K, native[i % copies6].data_ptr(), sc.data_ptr(), N, 3, 2, yh.data_ptr(), ws.data_ptr(),
+                        ws.numel() * 4, stream())), copies6, 4)
+                    tfs = 2.0 * M * N * K / split / 1e6
+                    print(json.dumps({"kernel": "fp6_linear_ws_e3m2", "N": N, "K": K, "M": M, "parts": parts6,
+                                      "us": round(split, 2), "us_plain": round(plain, 2), "TFLOPs": round(tfs, 2),
+                                      "mfma_frac": round(tfs / MFMA_PEAK_TFLOPS, 4)}), flush=True)
+            del w, wh, packed, qp, tc, native
     elif kind == "tinygemm":
         # The operator the reference's int4 weight-only linear dispatches to (torchao/dtypes/affine_quantized_tensor.py:631 ->
         # aten._weight_int4pack_mm), as this PyTorch-ROCm build implements it, beside torch.ops.torchao.int4wo_linear
@@ -476,27 +559,6 @@ def sweep(kind, iters=100):
         # figure is device time per launch with cold weights and no host dispatch in it.
         from ao_amd import ops
         from ao_amd.quantization.utils import groupwise_affine_quantize_tensor
-
-        def replayed_us(fn, n, reps):
-            side = torch.cuda.Stream()
-            with torch.cuda.stream(side):
-                for i in range(n):
-                    fn(i)
-                torch.cuda.synchronize()
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, stream=side):
-                    for i in range(n):
-                        fn(i)
-            for _ in range(2):
-                graph.replay()
-            torch.cuda.synchronize()
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            for _ in range(reps):
-                graph.replay()
-            b.record()
-            torch.cuda.synchronize()
-            return a.elapsed_time(b) * 1e3 / (reps * n)
 
         g = 64
         for N, K in [(4096, 4096), (6144, 4096), (14336, 4096), (4096, 14336), (128256, 4096)]:
@@ -606,7 +668,7 @@ def main():
                     help="int4wo-<group> (default: int4wo-<--group>, the headline configuration), int8wo or fp6 (e3m2 on an "
                          "fp16 model): the decode loop of the reference's other weight-only configurations, reported "
                          "without the int4 roofline leg")
-    ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6", "int8", "tinygemm", "quantize"), default=None,
+    ap.add_argument("--sweep", choices=("gemv", "gemm", "fp6", "int8", "ws", "tinygemm", "quantize"), default=None,
                     help="instead of the decode benchmark, print one line per kernel case of the named sweep")
     args = ap.parse_args()
     if args.gpus != 1:
