@@ -122,6 +122,14 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
+// acc + lo * lo + hi * hi of a dword holding two bf16 values, in one instruction (v_dot2c_f32_bf16): the sum of squares of
+// an RMSNorm statistic, whose order of additions is free
+__device__ __forceinline__ float bf16x2_sumsq(uint32_t pair, float acc) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 p;
+    __builtin_memcpy(&p, &pair, 4);
+    return __builtin_amdgcn_fdot2_f32_bf16(p, p, acc, false);
+}
 __device__ __forceinline__ float row16_sum(float v) {
     v += dpp_move<0xB1>(v);
     v += dpp_move<0x4E>(v);

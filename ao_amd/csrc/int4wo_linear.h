@@ -26,6 +26,9 @@ struct LinearArgs {
     int kb_total, kb_per_split;
     uint32_t block_bytes, qblock_bytes;
     int chunks_per_row;
+    // single-row kernels with the fused RMSNorm: K as a float, and 1 / K when that is exact (K a power of two; else 0):
+    // mean = sum * (1 / K) is then the same value as the reference's sum / K without the division sequence
+    float norm_k, norm_inv_k;
 };
 
 __device__ __forceinline__ float silu_bf16(float a) {

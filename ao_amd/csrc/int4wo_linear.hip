@@ -1204,7 +1204,7 @@ static int linear_dispatch(const void* x_bf16, int64_t M, int64_t K, int64_t ldx
                  (const uint16_t*)residual_bf16, ldres, y, y_dtype == AO_F32, ldy,
                  (const uint16_t*)norm_weight_bf16, norm_eps, ksplit, pair8 ? 1 : 0,
                  (int)KB_all, (int)((KB_all + ksplit - 1) / ksplit), (uint32_t)(KB_all * 1024), (uint32_t)(Kp / g * 64),
-                 (int)(Kp / 8)};
+                 (int)(Kp / 8), (float)K, (K & (K - 1)) == 0 ? 1.0f / (float)K : 0.f};
     hipStream_t st = (hipStream_t)stream;
     // the fused RMSNorm lives in the activation staging of the GEMV kernel only
     AO_REQUIRE(!norm_weight_bf16 || (xmode == X_LDS && M <= 16 && (((uintptr_t)norm_weight_bf16) & 15) == 0),
