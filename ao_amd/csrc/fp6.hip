@@ -984,9 +984,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp6_gemv_kernel(const Fp6GemvArgs 
                     const uint32_t u[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        float lo, hi;
-                        halves(u[j], lo, hi);
-                        ss += lo * lo + hi * hi;
+                        // ss + lo * lo + hi * hi of the fp16 pair in one instruction (v_dot2c_f32_f16)
+                        f16x2_t pr;
+                        __builtin_memcpy(&pr, &u[j], 4);
+                        ss = __builtin_amdgcn_fdot2(pr, pr, ss, false);
                     }
                 }
                 ss = wave_sum(ss);

@@ -76,10 +76,7 @@ __device__ __forceinline__ float chunk_sumsq(const uint4& v) {
     const uint32_t u[4] = {v.x, v.y, v.z, v.w};
     float t = 0.f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const float lo = __uint_as_float(u[j] << 16), hi = __uint_as_float(u[j] & 0xffff0000u);
-        t += lo * lo + hi * hi;
-    }
+    for (int j = 0; j < 4; ++j) t = bf16x2_sumsq(u[j], t);
     return t;
 }
 // RMSNorm of one chunk (torchao/_models/llama/model.py:232-244): bf16(bf16(x * rs) * w)
