@@ -261,9 +261,8 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     lmax = wave_max(lmax);
     if (lane == 0) red[wave] = lmax;
     __syncthreads();
-    float gmax = red[0];
-#pragma unroll
-    for (int w = 1; w < 16; ++w) gmax = fmaxf(gmax, red[w]);
+    // the 16 wave maxima: one per lane of a 16-lane row, combined across the row (one LDS read instead of 16)
+    const float gmax = row16_max(red[lane & 15]);
     const float gsub = gmax == -INFINITY ? 0.f : gmax;  // a workgroup without positions (split mode, short context)
     float lsum = 0.f;
     for (int li = tid; li < npass * 64; li += ATT_THREADS) {
@@ -274,9 +273,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
     lsum = wave_sum(lsum);
     if (lane == 0) red[16 + wave] = lsum;
     __syncthreads();  // probabilities and the partial sums are visible
-    float tot = 0.f;
-#pragma unroll
-    for (int w = 0; w < 16; ++w) tot += red[16 + w];
+    const float tot = row16_sum(red[16 + (lane & 15)]);
     const float inv = 1.0f / tot;
 
     // out[d] = sum_t p_t * V[t][d]: same thread mapping (one position per 16-lane group, 8 values of d per lane)
