@@ -317,10 +317,20 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attention_kernel(const uin
         dst[1] = make_float4(oacc[4], oacc[5], oacc[6], oacc[7]);
     }
     __syncthreads();
+    // the 64 rows are added in two steps of 8 (a chain of 16 additions instead of 64): every thread adds the 8 rows of
+    // group tid / 128 at column tid % 128 into the group's first row, then 128 threads add the 8 group rows
+    {
+        const int d = tid & (HD - 1), g8 = (tid >> 7) * 8;
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) s += po[(g8 + w) * HD + d];
+        po[g8 * HD + d] = s;
+    }
+    __syncthreads();
     if (tid < HD) {
         float o = 0.f;
-#pragma unroll 16
-        for (int w = 0; w < 64; ++w) o += po[w * HD + tid];
+#pragma unroll
+        for (int g = 0; g < 8; ++g) o += po[g * 8 * HD + tid];
         if (nsplit == 1) {
             out[(int64_t)h * HD + tid] = E::to_bits(o * inv);
         } else {
