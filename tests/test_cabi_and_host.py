@@ -276,3 +276,17 @@ def test_torchao_alias_package_resolves_to_this_library():
     import torchao._models.llama.model as m
 
     assert m is ao_amd._models.llama.model
+    # the legacy subclass through both import paths is one class object (isinstance checks on weights made by
+    # change_linear_weights_to_int4_woqtensors hold whichever path the caller imported), and no module of the library
+    # is loaded a second time under the torchao name
+    import sys
+
+    from torchao.quantization.subclass import Int4WeightOnlyQuantizedLinearWeight as via_alias
+
+    from ao_amd.quantization.subclass import Int4WeightOnlyQuantizedLinearWeight as direct
+
+    assert via_alias is direct is torchao.quantization.Int4WeightOnlyQuantizedLinearWeight
+    for name, mod in list(sys.modules.items()):
+        if name.startswith("torchao.") and mod is not None:
+            twin = sys.modules.get("ao_amd." + name[len("torchao."):])
+            assert twin is None or twin is mod, name
