@@ -194,3 +194,76 @@ def test_module_api_on_random_layers(seed):
         err = _rel_l2(y, ref)
         # the 16-bit roundings of the chains (product, scale, bias; fp16 products for FPx) against an fp32 reference
         assert bool(torch.isfinite(y.float()).all()) and err <= 8e-3, (seed, i, kind, N, K, lead, dt, err)
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_hqq_matrix_core_product_on_random_shapes(seed):
+    """Both products of the HQQ mixed matmul (1-64 rows) over random shapes, dtypes, signedness and group sizes against
+    the float64 product with the dequantized weight, rounded to the output dtype (1.5e-3: one rounding of the result)."""
+    from ao_amd import ops
+    from ao_amd.prototype.hqq import pack_2xint4
+
+    dev = torch.device("cuda:0")
+    rng = random.Random(seed)
+    torch.manual_seed(seed)
+    for i in range(24):
+        transposed = rng.random() < 0.5
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        signed = rng.random() < 0.5
+        M = rng.randint(1, 64)
+        if transposed:
+            N, g = 16 * rng.randint(1, 80), 2 * rng.choice([1, 4, 16, 32, 64])
+        else:
+            N, g = 4 * rng.randint(1, 300), 8 * rng.choice([1, 2, 4, 8, 16])
+        K = g * rng.randint(1, 40)
+        print(f"case {i} hqq transposed={transposed} {dtype} signed={signed} M={M} N={N} K={K} g={g}", flush=True)
+        lo, hi = (-8, 8) if signed else (0, 16)
+        W_q = torch.randint(lo, hi, (K, N)).to(torch.int8 if signed else torch.uint8)
+        s = (torch.rand(K // g, N) * 0.02 + 1e-3).to(dtype).to(dev)
+        z = (torch.rand(K // g, N) * 6 + (-3 if signed else 5)).to(dtype).to(dev)
+        packed = pack_2xint4(W_q).to(dev)
+        # (q - zero) * scale, each op rounded to the storage dtype (the reference kernel's formula)
+        w = ((W_q.to(dev).to(dtype).reshape(K // g, g, N) - z[:, None, :]) * s[:, None, :]).reshape(K, N)
+        x = torch.randn(M, N if transposed else K, dtype=dtype, device=dev)
+        y = ops.hqq_mixed_mm_mfma(x, packed, s, z, g, transposed)
+        ref = (x.double() @ (w.double().t() if transposed else w.double())).to(dtype)
+        err = _rel_l2(y, ref)
+        assert err <= 1.5e-3, err
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_workspace_linears_on_random_shapes(seed):
+    """The operators at 16-256 rows on narrow weights, where they may split K over workgroups through a workspace
+    (int4 and the Quant-LLM formats), against the product with the dequantized weight."""
+    from ao_amd import _lib, ops
+
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    rng = random.Random(seed)
+    torch.manual_seed(seed)
+    for i in range(16):
+        M = rng.randint(16, 256)
+        K = 256 * rng.randint(4, 60)
+        if rng.random() < 0.5:
+            g = rng.choice([32, 64, 128, 256])
+            N = rng.choice([1000, 1024, 2048, 4096, 4100, 6144])
+            print(f"case {i} int4 M={M} N={N} K={K} g={g} parts={L.ao_amd_int4wo_linear_ws_parts(M, K, N, g)}", flush=True)
+            w = (torch.randn(N, K) * 0.02).bfloat16().to(dev)
+            packed, qp = ops.int4wo_quantize_pack(w, g)
+            dq = ops.int4wo_dequantize(packed, qp, N, K, g)
+            x = torch.randn(M, K).bfloat16().to(dev)
+            y = ops.int4wo_linear(x, packed, qp, g, N)
+            ref = (x.float() @ dq.float().t()).bfloat16()
+        else:
+            e, m = rng.choice([(3, 2), (2, 3), (2, 2), (3, 1)])
+            N = 64 * rng.randint(4, 100)
+            print(f"case {i} fp{1 + e + m} e{e}m{m} M={M} N={N} K={K} parts={L.ao_amd_fp6_linear_ws_parts(M, K, N)}", flush=True)
+            w = (torch.randn(N, K) * 0.05).half().to(dev)
+            tc, scale = ops.fp6_quantize_pack(w, e, m)
+            native = ops.fp6_repack(tc, 1 + e + m)
+            wd = ops.fp6_dequantize(tc, scale, e, m).half()
+            x = torch.randn(M, K).half().to(dev)
+            y = ops.fp6_linear_native(e, m, x, native, scale)
+            ref = (x.float() @ wd.float().t()).half()
+        err = _rel_l2(y, ref)
+        assert err <= 1e-3, err
